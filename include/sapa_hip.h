@@ -1,0 +1,196 @@
+/* C ABI of libsapa_hip.so: SAPA's upsampling operators as hand-written HIP
+ * kernels for gfx950 (MI355X).
+ *
+ * This is the native boundary that the reference's four pybind11 extension
+ * modules (qk_ext, av_ext, dqk, dav) occupy; each entry point below names the
+ * reference function it stands in for.  Plain pointers and sizes only.
+ *
+ * Conventions, shared by every entry point:
+ *   - every tensor is a DEVICE pointer to an NCHW-contiguous array of `dtype`
+ *     elements (the reference's CHECK_CONTIGUOUS contract,
+ *     sapa/sapa/src/cuda/qk_cuda.cpp:34-39);
+ *   - H, W are the LOW-RES extents (key / value); the high-res extents are
+ *     s*H, s*W (sapa/sapa/sapa_func.py:15-16);
+ *   - buffers are borrowed for the duration of the asynchronous launch on
+ *     `stream` (a hipStream_t; NULL = the default stream) and are never
+ *     allocated, freed or retained by the library;
+ *   - forward outputs are fully overwritten; gradient buffers are
+ *     overwritten too, EXCEPT the low-res gradients of the sampled (deform)
+ *     operators, which are accumulated with atomics and must arrive
+ *     zero-filled, as the reference's callers provide them
+ *     (deformsapa/deformsapa/deform_func.py:49-51);
+ *   - the return value is SAPA_OK or a negative sapa_status; nothing here
+ *     calls exit() or throws (the reference exits on a launch failure,
+ *     qk_cuda_kernel.cu:92-96);
+ *   - the library keeps no global state between calls: entry points are
+ *     re-entrant and may be called from several host threads.
+ *   - the device that is current on the calling thread must be the one that
+ *     owns the buffers and `stream`.
+ */
+#ifndef SAPA_HIP_H
+#define SAPA_HIP_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum sapa_dtype {
+    SAPA_F32 = 0,
+    SAPA_F64 = 1,
+    SAPA_F16 = 2,
+    SAPA_BF16 = 3
+} sapa_dtype;
+
+typedef enum sapa_status {
+    SAPA_OK = 0,
+    SAPA_ERR_INVALID_ARGUMENT = -1, /* null pointer, non-positive extent, even K, ... */
+    SAPA_ERR_UNSUPPORTED = -2,      /* valid request this build has no kernel for */
+    SAPA_ERR_TOO_LARGE = -3,        /* an extent or element count exceeds the kernels' index range */
+    SAPA_ERR_LAUNCH = -4            /* HIP reported a launch error; see sapa_hip_last_hip_error() */
+} sapa_status;
+
+/* Version of this ABI (bumped on any signature change). */
+int sapa_hip_abi_version(void);
+/* Static, human-readable text for a sapa_status. */
+const char *sapa_hip_status_string(int status);
+/* Text of the HIP error behind the calling thread's most recent
+ * SAPA_ERR_LAUNCH ("" if none). */
+const char *sapa_hip_last_hip_error(void);
+
+/* ------------------------------------------------------------------ SAPA-B */
+
+/* Local query-key similarity.
+ *   out[n, ky*K+kx, ph, pw] = sum_{c<d} key[n,c,ph/s-r+ky,pw/s-r+kx] * query[n,c,ph,pw],
+ *   r = (K-1)/2; the whole sum is 0 where the neighbour is out of range.
+ * query [B,d,sH,sW], key [B,d,H,W] -> out [B,K*K,sH,sW].
+ * Replaces qk_ext.forward = qk_forward (sapa/sapa/src/qk_ext.cpp:22-34) ->
+ * qk_forward_cuda (src/cuda/qk_cuda.cpp:41-60) -> QKForward
+ * (src/cuda/qk_cuda_kernel.cu:30-68).  fp32 results are bit-identical to that
+ * kernel's arithmetic (one FMA per channel, channels in order). */
+int sapa_qk_forward(const void *query, const void *key, void *out,
+                    int B, int d, int H, int W, int K, int s,
+                    int dtype, void *stream);
+
+/* Gradients of sapa_qk_forward.  grad_out [B,K*K,sH,sW] -> grad_query
+ * [B,d,sH,sW], grad_key [B,d,H,W], both overwritten; either may be NULL to
+ * skip it.  Gather formulation: deterministic, no atomics.
+ * Replaces qk_ext.backward = qk_backward (qk_ext.cpp:36-50) -> QKBackward
+ * (qk_cuda_kernel.cu:101-137). */
+int sapa_qk_backward(const void *grad_out, const void *query, const void *key,
+                     void *grad_query, void *grad_key,
+                     int B, int d, int H, int W, int K, int s,
+                     int dtype, void *stream);
+
+/* Attention-value aggregation.
+ *   out[n,c,ph,pw] = sum_{ky,kx} value[n,c,ph/s-r+ky,pw/s-r+kx] * attn[n,ky*K+kx,ph,pw],
+ *   out-of-range neighbours skipped.
+ * attn [B,K*K,sH,sW], value [B,C,H,W] -> out [B,C,sH,sW].
+ * Replaces av_ext.forward = av_forward (sapa/sapa/src/av_ext.cpp:18-30) ->
+ * av_forward_cuda (src/cuda/av_cuda.cpp:28-47) -> AVForward
+ * (src/cuda/av_cuda_kernel.cu:30-75).  fp32 results are bit-identical to that
+ * kernel's arithmetic (one FMA per neighbour, ky-major order). */
+int sapa_av_forward(const void *attn, const void *value, void *out,
+                    int B, int C, int H, int W, int K, int s,
+                    int dtype, void *stream);
+
+/* Gradients of sapa_av_forward.  grad_out [B,C,sH,sW] -> grad_attn
+ * [B,K*K,sH,sW], grad_value [B,C,H,W], both overwritten; either may be NULL.
+ * Replaces av_ext.backward = av_backward (av_ext.cpp:32-46) -> AVBackward
+ * (av_cuda_kernel.cu:103-148). */
+int sapa_av_backward(const void *grad_out, const void *attn, const void *value,
+                     void *grad_attn, void *grad_value,
+                     int B, int C, int H, int W, int K, int s,
+                     int dtype, void *stream);
+
+/* Softmax over the middle axis of x [N,R,M] -> y [N,R,M] (max-subtracted,
+ * fp32 arithmetic for 16-bit types).  Covers the reference's
+ * F.softmax(logits, dim=1) on [B,K*K,sH,sW] (sapa_base.py:39: N=B, R=K*K,
+ * M=sH*sW) and F.softmax(logits, dim=2) on [B,G,P,sH,sW]
+ * (sapa_deform.py:52: N=B*G, R=P, M=sH*sW).  x == y (in place) is allowed. */
+int sapa_softmax_forward(const void *x, void *y, long long N, int R, long long M,
+                         int dtype, void *stream);
+
+/* Fused sapa_qk_forward -> softmax over K*K -> sapa_av_forward in one launch:
+ * the [B,K*K,sH,sW] logits/weights never touch HBM.  Out-of-range
+ * neighbours have logit 0 and DO take part in the softmax denominator, as in
+ * the three-launch composition SAPA.attention (sapa_base.py:38-40).
+ * query [B,d,sH,sW], key [B,d,H,W], value [B,C,H,W] -> out [B,C,sH,sW].
+ * Logits and weights are kept in fp32 (fp64 for SAPA_F64) whatever `dtype`.
+ * K*K must not exceed 121 (SAPA_ERR_UNSUPPORTED otherwise). */
+int sapa_fused_forward(const void *query, const void *key, const void *value,
+                       void *out, int B, int d, int C, int H, int W,
+                       int K, int s, int dtype, void *stream);
+
+/* sapa_qk_forward -> softmax in one launch, writing the attention weights
+ * attn [B,K*K,sH,sW] (what a training step keeps for the backward pass). */
+int sapa_qk_softmax_forward(const void *query, const void *key, void *attn,
+                            int B, int d, int H, int W, int K, int s,
+                            int dtype, void *stream);
+
+/* ------------------------------------------------------------------ SAPA-D */
+
+/* Offset-sampled query-key similarity.
+ *   out[b,g,p,qh,qw] = sum_{c<d} query[b,g*d+c,qh,qw] * bilinear(key[b,g*d+c]; kh, kw),
+ *   kh = qh/s + offset[b,2*(g*P+p)+1,qh,qw], kw = qw/s + offset[b,2*(g*P+p),qh,qw]
+ *   (offsets in low-res pixels, added to the integer parent coordinate);
+ *   0 unless kh > -1 && kh < H && kw > -1 && kw < W; each of the four corners
+ *   is zero-padded on its own.  d = Cq / G.
+ * query [B,Cq,sH,sW], key [B,Cq,H,W], offset [B,2*G*P,sH,sW] -> out [B,G,P,sH,sW].
+ * Replaces dqk.forward = deform_qk_forward
+ * (deformsapa/deformsapa/src/deform_qk.cpp:32-48) -> deform_qk_forward_cuda
+ * (src/cuda/deform_qk_cuda.cpp:45-68) -> DeformQKForward
+ * (src/cuda/deform_qk_cuda_kernel.cu:139-197, bilinear :23-68).  Coordinates,
+ * floor and the guard are evaluated in `dtype`'s arithmetic (fp32 for 16-bit
+ * types), so fp32 corner indices are bit-exact with the reference's. */
+int sapa_deform_qk_forward(const void *query, const void *key, const void *offset,
+                           void *out, int B, int Cq, int H, int W,
+                           int P, int s, int G, int dtype, void *stream);
+
+/* Gradients of sapa_deform_qk_forward.  grad_query and grad_offset are
+ * overwritten; grad_key is ACCUMULATED with atomics and must be zero-filled
+ * by the caller.  Any of the three may be NULL.  SAPA_F32 / SAPA_F64 only.
+ * Replaces dqk.backward = deform_qk_backward (deform_qk.cpp:50-70) ->
+ * DeformQKBackward (deform_qk_cuda_kernel.cu:233-296, col2im :70-137). */
+int sapa_deform_qk_backward(const void *grad_out, const void *query,
+                            const void *key, const void *offset,
+                            void *grad_query, void *grad_key, void *grad_offset,
+                            int B, int Cq, int H, int W, int P, int s, int G,
+                            int dtype, void *stream);
+
+/* Offset-sampled attention-value aggregation.
+ *   out[b,c,qh,qw] = sum_{p<P} attn[b,g(c),p,qh,qw] * bilinear(value[b,c]; kh, kw),
+ *   g(c) = c / (C/G), same coordinates and guard as above.
+ * attn [B,G,P,sH,sW], value [B,C,H,W], offset [B,2*G*P,sH,sW] -> out [B,C,sH,sW].
+ * Replaces dav.forward = deform_av_forward
+ * (deformsapa/deformsapa/src/deform_av.cpp:32-48) -> DeformAVForward
+ * (src/cuda/deform_av_cuda_kernel.cu:139-195). */
+int sapa_deform_av_forward(const void *attn, const void *value, const void *offset,
+                           void *out, int B, int C, int H, int W,
+                           int P, int s, int G, int dtype, void *stream);
+
+/* Gradients of sapa_deform_av_forward.  grad_attn and grad_offset are
+ * overwritten; grad_value is ACCUMULATED with atomics and must be
+ * zero-filled by the caller.  Any may be NULL.  SAPA_F32 / SAPA_F64 only.
+ * Replaces dav.backward = deform_av_backward (deform_av.cpp:50-70) ->
+ * DeformAVBackward (deform_av_cuda_kernel.cu:230-292). */
+int sapa_deform_av_backward(const void *grad_out, const void *attn,
+                            const void *value, const void *offset,
+                            void *grad_attn, void *grad_value, void *grad_offset,
+                            int B, int C, int H, int W, int P, int s, int G,
+                            int dtype, void *stream);
+
+/* Fused sapa_deform_qk_forward -> softmax over P -> sapa_deform_av_forward in
+ * one launch (SAPADeform.attention, sapa_deform.py:51-53).  Sample positions
+ * and bilinear weights are computed once per (pixel, group, point) and shared
+ * by the similarity and the aggregation.  P must not exceed 64.
+ * query [B,Cq,sH,sW], key [B,Cq,H,W], value [B,C,H,W],
+ * offset [B,2*G*P,sH,sW] -> out [B,C,sH,sW]. */
+int sapa_deform_fused_forward(const void *query, const void *key,
+                              const void *value, const void *offset, void *out,
+                              int B, int Cq, int C, int H, int W,
+                              int P, int s, int G, int dtype, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SAPA_HIP_H */

@@ -1,0 +1,114 @@
+"""ctypes binding of libsapa_hip.so (C ABI in include/sapa_hip.h).
+
+The library is loaded from sapa_amd/lib/, where `python -m sapa_amd.build`
+puts it.  There is no fallback: if the library is missing or a call fails,
+the operators raise.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, 'lib', 'libsapa_hip.so')
+
+ABI_VERSION = 1
+
+DTYPES = {torch.float32: 0, torch.float64: 1, torch.float16: 2, torch.bfloat16: 3}
+
+_vp, _i, _ll = ctypes.c_void_p, ctypes.c_int, ctypes.c_longlong
+# name -> argtypes, in the order of include/sapa_hip.h
+SIGNATURES = {
+    'sapa_qk_forward': [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
+    'sapa_qk_backward': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
+    'sapa_av_forward': [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
+    'sapa_av_backward': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
+    'sapa_softmax_forward': [_vp, _vp, _ll, _i, _ll, _i, _vp],
+    'sapa_fused_forward': [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
+    'sapa_qk_softmax_forward': [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
+    'sapa_deform_qk_forward': [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
+    'sapa_deform_qk_backward': [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
+    'sapa_deform_av_forward': [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
+    'sapa_deform_av_backward': [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
+    'sapa_deform_fused_forward': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
+}
+
+_lib = None
+
+
+class SapaHipError(RuntimeError):
+    """A libsapa_hip.so entry point returned a negative status."""
+
+
+def lib():
+    """The loaded library (loaded on first use)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f'{LIB_PATH} is missing: build it with `python -m sapa_amd.build` '
+                '(hipcc, gfx950).  There is no fallback implementation.')
+        handle = ctypes.CDLL(LIB_PATH)
+        handle.sapa_hip_abi_version.restype = _i
+        handle.sapa_hip_abi_version.argtypes = []
+        if handle.sapa_hip_abi_version() != ABI_VERSION:
+            raise RuntimeError(f'{LIB_PATH}: ABI version {handle.sapa_hip_abi_version()}, '
+                               f'this package expects {ABI_VERSION}; rebuild the library')
+        handle.sapa_hip_status_string.restype = ctypes.c_char_p
+        handle.sapa_hip_status_string.argtypes = [_i]
+        handle.sapa_hip_last_hip_error.restype = ctypes.c_char_p
+        handle.sapa_hip_last_hip_error.argtypes = []
+        for name, argtypes in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = _i
+            fn.argtypes = argtypes
+        _lib = handle
+    return _lib
+
+
+def check(status, what):
+    if status == 0:
+        return
+    handle = lib()
+    msg = handle.sapa_hip_status_string(status).decode()
+    if status == -4:
+        msg += ': ' + handle.sapa_hip_last_hip_error().decode()
+    raise SapaHipError(f'{what}: {msg} (status {status})')
+
+
+def ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def dtype_code(t):
+    try:
+        return DTYPES[t.dtype]
+    except KeyError:
+        raise TypeError(f'unsupported dtype {t.dtype}; supported: {list(DTYPES)}') from None
+
+
+def require_cuda_contiguous(**tensors):
+    """The reference's CHECK_INPUT (sapa/sapa/src/cuda/qk_cuda.cpp:34-39):
+    device tensors, contiguous, and here also one device and one dtype."""
+    first = None
+    for name, t in tensors.items():
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError(f'{name} must be a CUDA tensor')
+        if not t.is_contiguous():
+            raise RuntimeError(f'{name} must be contiguous')
+        if first is None:
+            first = (name, t)
+        else:
+            if t.device != first[1].device:
+                raise RuntimeError(f'{name} is on {t.device}, {first[0]} on {first[1].device}')
+            if t.dtype != first[1].dtype:
+                raise RuntimeError(f'{name} is {t.dtype}, {first[0]} is {first[1].dtype}')
+
+
+def call(name, device, *args):
+    """Run entry point `name` on `device`'s current torch stream."""
+    with torch.cuda.device(device):
+        stream = torch.cuda.current_stream(device).cuda_stream
+        check(getattr(lib(), name)(*args, stream), name)

@@ -1,0 +1,269 @@
+// extern "C" entry points of libsapa_hip.so (declared in include/sapa_hip.h):
+// argument validation, kernel selection, error mapping.  No allocation, no
+// global state apart from a thread-local copy of the last HIP error text.
+#include "../../include/sapa_hip.h"
+
+#include <string.h>
+
+#include "kernels.hpp"
+
+using namespace sapa;
+
+namespace {
+
+thread_local char g_hip_error[256] = "";
+
+int fail_hip(hipError_t e) {
+    strncpy(g_hip_error, hipGetErrorString(e), sizeof(g_hip_error) - 1);
+    g_hip_error[sizeof(g_hip_error) - 1] = 0;
+    return SAPA_ERR_LAUNCH;
+}
+
+int finish(hipError_t e) { return e == hipSuccess ? SAPA_OK : fail_hip(e); }
+
+bool dtype_ok(int dt) { return dt >= SAPA_F32 && dt <= SAPA_BF16; }
+
+// element counts stay below 2^40 and extents below 2^24 so that the kernels'
+// 64-bit flat indices and 32-bit in-plane indices cannot overflow
+const long long kMaxElems = 1LL << 40;
+
+int check_window_args(int B, int c1, int c2, int H, int W, int K, int s, int dtype) {
+    if (!dtype_ok(dtype)) return SAPA_ERR_INVALID_ARGUMENT;
+    if (B < 0 || c1 <= 0 || c2 <= 0 || H <= 0 || W <= 0 || s < 1 || K < 1 || (K - 1) % 2 != 0)
+        return SAPA_ERR_INVALID_ARGUMENT;
+    if (K > 255 || (long long)H * s >= (1 << 24) || (long long)W * s >= (1 << 24) ||
+        (long long)H * s * W * s >= (1LL << 31))
+        return SAPA_ERR_TOO_LARGE;
+    const long long hi = (long long)B * H * s * W * s;
+    const int cmax = c1 > c2 ? c1 : c2;
+    if (hi * cmax >= kMaxElems || hi * K * K >= kMaxElems) return SAPA_ERR_TOO_LARGE;
+    return SAPA_OK;
+}
+
+int check_deform_args(int B, int Cq, int C, int H, int W, int P, int s, int G, int dtype) {
+    if (!dtype_ok(dtype)) return SAPA_ERR_INVALID_ARGUMENT;
+    if (B < 0 || Cq <= 0 || C <= 0 || H <= 0 || W <= 0 || s < 1 || P < 1 || G < 1 ||
+        Cq % G != 0 || C % G != 0)
+        return SAPA_ERR_INVALID_ARGUMENT;
+    if ((long long)H * s >= (1 << 24) || (long long)W * s >= (1 << 24) ||
+        (long long)H * s * W * s >= (1LL << 31))
+        return SAPA_ERR_TOO_LARGE;
+    const long long hi = (long long)B * H * s * W * s;
+    const int cmax = Cq > C ? Cq : C;
+    if (hi * cmax >= kMaxElems || hi * 2 * G * P >= kMaxElems) return SAPA_ERR_TOO_LARGE;
+    return SAPA_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int sapa_hip_abi_version(void) { return 1; }
+
+const char *sapa_hip_status_string(int status) {
+    switch (status) {
+        case SAPA_OK: return "ok";
+        case SAPA_ERR_INVALID_ARGUMENT: return "invalid argument";
+        case SAPA_ERR_UNSUPPORTED: return "unsupported configuration";
+        case SAPA_ERR_TOO_LARGE: return "tensor too large for the kernels' index range";
+        case SAPA_ERR_LAUNCH: return "HIP launch error";
+        default: return "unknown status";
+    }
+}
+
+const char *sapa_hip_last_hip_error(void) { return g_hip_error; }
+
+int sapa_qk_forward(const void *query, const void *key, void *out, int B, int d, int H, int W,
+                    int K, int s, int dtype, void *stream) {
+    const int rc = check_window_args(B, d, d, H, W, K, s, dtype);
+    if (rc != SAPA_OK) return rc;
+    if (B == 0) return SAPA_OK;
+    if (!query || !key || !out) return SAPA_ERR_INVALID_ARGUMENT;
+    hipStream_t st = (hipStream_t)stream;
+    hipError_t e = sapa_b_tiled_launch(TILED_QK, query, key, nullptr, nullptr, out, B, d, 0, H, W,
+                                       K, s, dtype, st);
+    if (e == hipErrorNotSupported)
+        e = qk_forward_generic_launch(query, key, out, B, d, H, W, K, s, dtype, st);
+    return finish(e);
+}
+
+int sapa_av_forward(const void *attn, const void *value, void *out, int B, int C, int H, int W,
+                    int K, int s, int dtype, void *stream) {
+    const int rc = check_window_args(B, C, C, H, W, K, s, dtype);
+    if (rc != SAPA_OK) return rc;
+    if (B == 0) return SAPA_OK;
+    if (!attn || !value || !out) return SAPA_ERR_INVALID_ARGUMENT;
+    hipStream_t st = (hipStream_t)stream;
+    hipError_t e = sapa_b_tiled_launch(TILED_AV, nullptr, nullptr, attn, value, out, B, 0, C, H, W,
+                                       K, s, dtype, st);
+    if (e == hipErrorNotSupported)
+        e = av_forward_generic_launch(attn, value, out, B, C, H, W, K, s, dtype, st);
+    return finish(e);
+}
+
+int sapa_qk_backward(const void *grad_out, const void *query, const void *key, void *grad_query,
+                     void *grad_key, int B, int d, int H, int W, int K, int s, int dtype,
+                     void *stream) {
+    const int rc = check_window_args(B, d, d, H, W, K, s, dtype);
+    if (rc != SAPA_OK) return rc;
+    if (B == 0) return SAPA_OK;
+    if (!grad_out || !query || !key) return SAPA_ERR_INVALID_ARGUMENT;
+    hipStream_t st = (hipStream_t)stream;
+    // grad_query[n,c,ph,pw] = sum_k key[n,c,nbr_k] * grad_out[n,k,ph,pw]: the
+    // aggregation with key in the value's place.
+    if (grad_query) {
+        const int r2 = sapa_av_forward(grad_out, key, grad_query, B, d, H, W, K, s, dtype, stream);
+        if (r2 != SAPA_OK) return r2;
+    }
+    if (grad_key) {
+        const hipError_t e =
+            lowres_grad_generic_launch(query, grad_out, grad_key, B, d, H, W, K, s, dtype, st);
+        if (e != hipSuccess) return fail_hip(e);
+    }
+    return SAPA_OK;
+}
+
+int sapa_av_backward(const void *grad_out, const void *attn, const void *value, void *grad_attn,
+                     void *grad_value, int B, int C, int H, int W, int K, int s, int dtype,
+                     void *stream) {
+    const int rc = check_window_args(B, C, C, H, W, K, s, dtype);
+    if (rc != SAPA_OK) return rc;
+    if (B == 0) return SAPA_OK;
+    if (!grad_out || !attn || !value) return SAPA_ERR_INVALID_ARGUMENT;
+    hipStream_t st = (hipStream_t)stream;
+    // grad_attn[n,k,ph,pw] = sum_c value[n,c,nbr_k] * grad_out[n,c,ph,pw]: the
+    // similarity with grad_out as the query and value as the key.
+    if (grad_attn) {
+        const int r2 = sapa_qk_forward(grad_out, value, grad_attn, B, C, H, W, K, s, dtype, stream);
+        if (r2 != SAPA_OK) return r2;
+    }
+    if (grad_value) {
+        const hipError_t e =
+            lowres_grad_generic_launch(grad_out, attn, grad_value, B, C, H, W, K, s, dtype, st);
+        if (e != hipSuccess) return fail_hip(e);
+    }
+    return SAPA_OK;
+}
+
+int sapa_softmax_forward(const void *x, void *y, long long N, int R, long long M, int dtype,
+                         void *stream) {
+    if (!dtype_ok(dtype) || N < 0 || R < 1 || M < 0) return SAPA_ERR_INVALID_ARGUMENT;
+    if (N == 0 || M == 0) return SAPA_OK;
+    if (!x || !y) return SAPA_ERR_INVALID_ARGUMENT;
+    if (N * M >= kMaxElems / R) return SAPA_ERR_TOO_LARGE;
+    return finish(softmax_generic_launch(x, y, (long)N, R, (long)M, dtype, (hipStream_t)stream));
+}
+
+static int fused_common(int attn_only, const void *query, const void *key, const void *value,
+                        void *out, int B, int d, int C, int H, int W, int K, int s, int dtype,
+                        void *stream) {
+    const int rc = check_window_args(B, d, C, H, W, K, s, dtype);
+    if (rc != SAPA_OK) return rc;
+    if (K * K > 121) return SAPA_ERR_UNSUPPORTED;
+    if (B == 0) return SAPA_OK;
+    if (!query || !key || !out || (!attn_only && !value)) return SAPA_ERR_INVALID_ARGUMENT;
+    hipStream_t st = (hipStream_t)stream;
+    hipError_t e = sapa_b_tiled_launch(attn_only ? TILED_QK_SOFTMAX : TILED_FUSED, query, key,
+                                       nullptr, value, out, B, d, attn_only ? 0 : C, H, W, K, s,
+                                       dtype, st);
+    if (e == hipErrorNotSupported)
+        e = fused_pixel_launch(query, key, value, out, B, d, C, H, W, K, s, attn_only, dtype, st);
+    if (e == hipErrorNotSupported) return SAPA_ERR_UNSUPPORTED;
+    return finish(e);
+}
+
+int sapa_fused_forward(const void *query, const void *key, const void *value, void *out, int B,
+                       int d, int C, int H, int W, int K, int s, int dtype, void *stream) {
+    return fused_common(0, query, key, value, out, B, d, C, H, W, K, s, dtype, stream);
+}
+
+int sapa_qk_softmax_forward(const void *query, const void *key, void *attn, int B, int d, int H,
+                            int W, int K, int s, int dtype, void *stream) {
+    return fused_common(1, query, key, nullptr, attn, B, d, d, H, W, K, s, dtype, stream);
+}
+
+int sapa_deform_qk_forward(const void *query, const void *key, const void *offset, void *out,
+                           int B, int Cq, int H, int W, int P, int s, int G, int dtype,
+                           void *stream) {
+    const int rc = check_deform_args(B, Cq, Cq, H, W, P, s, G, dtype);
+    if (rc != SAPA_OK) return rc;
+    if (B == 0) return SAPA_OK;
+    if (!query || !key || !offset || !out) return SAPA_ERR_INVALID_ARGUMENT;
+    return finish(deform_qk_forward_launch(query, key, offset, out, B, Cq, H, W, P, s, G, dtype,
+                                           (hipStream_t)stream));
+}
+
+int sapa_deform_av_forward(const void *attn, const void *value, const void *offset, void *out,
+                           int B, int C, int H, int W, int P, int s, int G, int dtype,
+                           void *stream) {
+    const int rc = check_deform_args(B, C, C, H, W, P, s, G, dtype);
+    if (rc != SAPA_OK) return rc;
+    if (B == 0) return SAPA_OK;
+    if (!attn || !value || !offset || !out) return SAPA_ERR_INVALID_ARGUMENT;
+    return finish(deform_av_forward_launch(attn, value, offset, out, B, C, H, W, P, s, G, dtype,
+                                           (hipStream_t)stream));
+}
+
+int sapa_deform_fused_forward(const void *query, const void *key, const void *value,
+                              const void *offset, void *out, int B, int Cq, int C, int H, int W,
+                              int P, int s, int G, int dtype, void *stream) {
+    const int rc = check_deform_args(B, Cq, C, H, W, P, s, G, dtype);
+    if (rc != SAPA_OK) return rc;
+    if (P > 64) return SAPA_ERR_UNSUPPORTED;
+    if (B == 0) return SAPA_OK;
+    if (!query || !key || !value || !offset || !out) return SAPA_ERR_INVALID_ARGUMENT;
+    return finish(deform_fused_forward_launch(query, key, value, offset, out, B, Cq, C, H, W, P, s,
+                                              G, dtype, (hipStream_t)stream));
+}
+
+int sapa_deform_qk_backward(const void *grad_out, const void *query, const void *key,
+                            const void *offset, void *grad_query, void *grad_key,
+                            void *grad_offset, int B, int Cq, int H, int W, int P, int s, int G,
+                            int dtype, void *stream) {
+    const int rc = check_deform_args(B, Cq, Cq, H, W, P, s, G, dtype);
+    if (rc != SAPA_OK) return rc;
+    if (dtype != SAPA_F32 && dtype != SAPA_F64) return SAPA_ERR_UNSUPPORTED;
+    if (B == 0) return SAPA_OK;
+    if (!grad_out || !query || !key || !offset) return SAPA_ERR_INVALID_ARGUMENT;
+    hipStream_t st = (hipStream_t)stream;
+    // grad_query[b,g*d+c] = sum_p grad_out[b,g,p] * bilinear(key[b,g*d+c]): the
+    // sampled aggregation with key in the value's place.
+    if (grad_query) {
+        const hipError_t e = deform_av_forward_launch(grad_out, key, offset, grad_query, B, Cq, H,
+                                                      W, P, s, G, dtype, st);
+        if (e != hipSuccess) return fail_hip(e);
+    }
+    if (grad_key || grad_offset) {
+        const hipError_t e = deform_lowgrad_launch(query, grad_out, key, offset, grad_key,
+                                                   grad_offset, B, Cq, H, W, P, s, G, dtype, st);
+        if (e != hipSuccess) return fail_hip(e);
+    }
+    return SAPA_OK;
+}
+
+int sapa_deform_av_backward(const void *grad_out, const void *attn, const void *value,
+                            const void *offset, void *grad_attn, void *grad_value,
+                            void *grad_offset, int B, int C, int H, int W, int P, int s, int G,
+                            int dtype, void *stream) {
+    const int rc = check_deform_args(B, C, C, H, W, P, s, G, dtype);
+    if (rc != SAPA_OK) return rc;
+    if (dtype != SAPA_F32 && dtype != SAPA_F64) return SAPA_ERR_UNSUPPORTED;
+    if (B == 0) return SAPA_OK;
+    if (!grad_out || !attn || !value || !offset) return SAPA_ERR_INVALID_ARGUMENT;
+    hipStream_t st = (hipStream_t)stream;
+    // grad_attn[b,g,p] = sum_{c in g} grad_out[b,c] * bilinear(value[b,c]): the
+    // sampled similarity with grad_out as the query and value as the key.
+    if (grad_attn) {
+        const hipError_t e = deform_qk_forward_launch(grad_out, value, offset, grad_attn, B, C, H,
+                                                      W, P, s, G, dtype, st);
+        if (e != hipSuccess) return fail_hip(e);
+    }
+    if (grad_value || grad_offset) {
+        const hipError_t e = deform_lowgrad_launch(grad_out, attn, value, offset, grad_value,
+                                                   grad_offset, B, C, H, W, P, s, G, dtype, st);
+        if (e != hipSuccess) return fail_hip(e);
+    }
+    return SAPA_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,59 @@
+// Shared device helpers for the SAPA HIP kernels (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace sapa {
+
+typedef _Float16 f16_t;
+typedef __bf16 bf16_t;
+
+// Arithmetic type for a storage type: 16-bit tensors compute in fp32.
+template <typename T> struct Acc { typedef float type; };
+template <> struct Acc<double> { typedef double type; };
+
+__device__ __forceinline__ float fma_(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+__device__ __forceinline__ double fma_(double a, double b, double c) { return __builtin_fma(a, b, c); }
+__device__ __forceinline__ float floor_(float a) { return __builtin_floorf(a); }
+__device__ __forceinline__ double floor_(double a) { return __builtin_floor(a); }
+
+template <typename T>
+__device__ __forceinline__ typename Acc<T>::type ld(const T *p) {
+    return (typename Acc<T>::type)(*p);
+}
+
+// exp(x) for x <= 0 in fp32 to ~1 ulp: hardware exp2 on the high part of
+// x*log2(e), first-order correction for the part the product rounds away.
+__device__ __forceinline__ float exp_(float x) {
+    const float l2e_hi = 1.44269502162933349609375f;    // fl(log2 e)
+    const float l2e_lo = 1.925963033500011e-8f;         // log2 e - l2e_hi
+    const float t = x * l2e_hi;
+    float e = __builtin_fmaf(x, l2e_hi, -t);
+    e = __builtin_fmaf(x, l2e_lo, e);
+    const float r = __builtin_amdgcn_exp2f(t);
+    return __builtin_fmaf(r, e * 0.693147182464599609375f, r);
+}
+__device__ __forceinline__ double exp_(double x) { return exp(x); }
+
+__device__ __forceinline__ float max_(float a, float b) { return __builtin_fmaxf(a, b); }
+__device__ __forceinline__ double max_(double a, double b) { return __builtin_fmax(a, b); }
+
+// In-register softmax of v[0..N): max-subtracted, sum in index order,
+// one correctly rounded reciprocal, then a multiply per element.
+template <typename A, int N>
+__device__ __forceinline__ void softmax_inplace(A (&v)[N]) {
+    A m = v[0];
+#pragma unroll
+    for (int i = 1; i < N; ++i) m = max_(m, v[i]);
+    A sum = 0;
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        v[i] = exp_(v[i] - m);
+        sum += v[i];
+    }
+    const A inv = (A)1 / sum;
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] *= inv;
+}
+
+}  // namespace sapa

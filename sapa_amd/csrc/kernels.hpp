@@ -1,0 +1,51 @@
+// Internal launch interface between the C ABI (capi.hip) and the kernel files.
+// Every launcher enqueues on `st` and returns the HIP status of the launch;
+// arguments are validated by the caller.  `dtype` is the sapa_dtype value.
+#pragma once
+#include "common.hpp"
+
+namespace sapa {
+
+// sapa_b_generic.hip: any K, s, dtype
+hipError_t qk_forward_generic_launch(const void *q, const void *key, void *out, int B, int d,
+                                     int H, int W, int K, int s, int dtype, hipStream_t st);
+hipError_t av_forward_generic_launch(const void *attn, const void *value, void *out, int B, int C,
+                                     int H, int W, int K, int s, int dtype, hipStream_t st);
+hipError_t lowres_grad_generic_launch(const void *hi, const void *w, void *out, int B, int C,
+                                      int H, int W, int K, int s, int dtype, hipStream_t st);
+hipError_t softmax_generic_launch(const void *x, void *y, long N, int R, long M, int dtype,
+                                  hipStream_t st);
+// K in {1,3,5,7,9,11}; hipErrorNotSupported otherwise
+hipError_t fused_pixel_launch(const void *q, const void *key, const void *value, void *out,
+                              int B, int d, int C, int H, int W, int K, int s, int attn_only,
+                              int dtype, hipStream_t st);
+
+// sapa_b_tiled.hip: LDS-tiled kernels.  `mode` selects the stages:
+enum TiledMode { TILED_QK = 0, TILED_QK_SOFTMAX = 1, TILED_AV = 2, TILED_FUSED = 3 };
+// Returns hipErrorNotSupported when no tiled kernel covers (K, s, dtype, shape);
+// the caller then takes the generic path.
+hipError_t sapa_b_tiled_launch(int mode, const void *q, const void *key, const void *attn_in,
+                               const void *value, void *out, int B, int d, int C, int H, int W,
+                               int K, int s, int dtype, hipStream_t st);
+
+// sapa_d.hip
+hipError_t deform_qk_forward_launch(const void *q, const void *key, const void *offset, void *out,
+                                    int B, int Cq, int H, int W, int P, int s, int G, int dtype,
+                                    hipStream_t st);
+hipError_t deform_av_forward_launch(const void *attn, const void *value, const void *offset,
+                                    void *out, int B, int C, int H, int W, int P, int s, int G,
+                                    int dtype, hipStream_t st);
+// P <= 64; hipErrorNotSupported otherwise
+hipError_t deform_fused_forward_launch(const void *q, const void *key, const void *value,
+                                       const void *offset, void *out, int B, int Cq, int C, int H,
+                                       int W, int P, int s, int G, int dtype, hipStream_t st);
+// grad_low (atomic accumulate, may be null) and grad_offset (store, may be
+// null) of either sampled op: hi = per-channel high-res tensor [B,Cx,sH,sW],
+// sc = per-point tensor [B,G,P,sH,sW], low = sampled tensor [B,Cx,H,W].
+// dtype f32 / f64 only.
+hipError_t deform_lowgrad_launch(const void *hi, const void *sc, const void *low,
+                                 const void *offset, void *grad_low, void *grad_offset, int B,
+                                 int Cx, int H, int W, int P, int s, int G, int dtype,
+                                 hipStream_t st);
+
+}  // namespace sapa

@@ -1,0 +1,342 @@
+// LDS-tiled SAPA-B kernels for gfx950: qk, qk+softmax, av and the fused
+// qk -> softmax -> av forward, all from one template.
+//
+// Work decomposition (NCHW tensors, so the contiguous axis is W):
+//   * a workgroup owns a tile of TW x TH = 16 x (4*NWY) low-res parent cells
+//     of one image; a wave owns 16 x 4 of them, lane = (lx 0..15, ly 0..3);
+//   * a thread owns CY x S of the S x S high-res children of its parent
+//     (CY = S: all of them; CY < S: S/CY waves share the parent rows), and
+//     keeps their K*K logits / weights in registers (CY*S*K*K values);
+//   * the low-res key (then value) window of the tile, tile + (K-1) halo, is
+//     staged through LDS in chunks of CH channels, double-buffered, with the
+//     next chunk's global loads in flight during the current chunk's FMAs.
+//     Every staged value is reused by the CY*S children in registers and by
+//     up to K*K parents through LDS;
+//   * q is read and the output written exactly once, as S-wide vectors that
+//     are contiguous across the 16 lanes of a row (S*16 elements per row).
+// LDS layout: window rows of WW <= 24 floats at a row stride of 48 floats,
+// two channels side by side in one row (columns 0..23 and 24..47).  A stride
+// that is 16 mod 32 puts the four 16-lane rows of a wave on disjoint banks,
+// so the window reads (row ly+ky, column lx+kx) are conflict-free.
+//
+// Arithmetic is the reference kernels' own, term by term: one FMA per
+// channel in channel order for the logits (qk_cuda_kernel.cu:55-66), one FMA
+// per neighbour in ky-major order for the aggregation
+// (av_cuda_kernel.cu:57-72).  Out-of-range neighbours are zeros in LDS: they
+// leave a logit at exactly 0 (and that 0 takes part in the softmax) and add
+// exactly 0 to the aggregation, which is what the reference's `continue`
+// does.  16-bit tensors are widened to fp32 on the way into LDS/registers.
+#include "kernels.hpp"
+
+namespace sapa {
+
+template <typename T, int N>
+struct alignas(sizeof(T) * N) Vec {
+    T v[N];
+};
+
+template <typename T, int K, int S, int CY, int NWY, int MODE>
+__global__ void __launch_bounds__(64 * NWY * (S / CY)) __attribute__((amdgpu_waves_per_eu(3, 3)))
+sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
+                    const T *__restrict__ attn_in, const T *__restrict__ value,
+                    T *__restrict__ out, int d, int C, int H, int W, int tiles_x, int tiles_y,
+                    int nblocks, int per_xcd) {
+    typedef float A;
+    constexpr int KK = K * K, R = (K - 1) / 2;
+    constexpr int NSUB = S / CY;           // waves sharing one band of parent rows
+    constexpr int NT = 64 * NWY * NSUB;    // threads per workgroup
+    constexpr int TW = 16, TH = 4 * NWY;   // parents per workgroup
+    constexpr int WW = TW + K - 1, WH = TH + K - 1;
+    constexpr int HALF = 24, STRIDE = 48;
+    constexpr int CH = 8;                  // channels per staged chunk
+    constexpr int WIN = WH * WW;           // window positions per channel
+    constexpr int NPOS = (WIN + NT - 1) / NT;  // positions staged by one thread
+    constexpr int NSTAGE = CH * NPOS;
+    constexpr int BUF = (CH / 2) * WH * STRIDE;
+    constexpr int NJ = CY * S;             // children per thread
+    constexpr bool DO_QK = MODE != TILED_AV;
+    constexpr bool DO_SOFTMAX = MODE == TILED_QK_SOFTMAX || MODE == TILED_FUSED;
+    constexpr bool DO_AV = MODE == TILED_AV || MODE == TILED_FUSED;
+    static_assert(WW < HALF, "window row plus one padding column must fit half an LDS row");
+    static_assert(S % CY == 0, "CY must divide S");
+    typedef Vec<T, S> VecS;
+
+    __shared__ A lds[2 * BUF];
+
+    // Workgroups are handed to the 8 XCDs round-robin; give each XCD a
+    // contiguous run of tiles so that neighbouring tiles (which share halo
+    // rows) meet in the same L2.
+    const int logical = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
+    if (logical >= nblocks) return;
+    const int tx = logical % tiles_x;
+    const int ty = (logical / tiles_x) % tiles_y;
+    const int n = logical / (tiles_x * tiles_y);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int lx = lane & 15, ly = (wave / NSUB) * 4 + (lane >> 4);
+    const int sub = wave % NSUB;
+    const int x0 = tx * TW, y0 = ty * TH;          // tile origin (parents)
+    const int px = x0 + lx, py = y0 + ly;
+    const bool active = px < W && py < H;
+    const int hH = H * S, hW = W * S;
+    const long lplane = (long)H * W, hplane = (long)hH * hW;
+    // first child of this thread; idle threads of a partial tile read (never
+    // write) through the clamped copy, so their loads need no branch
+    const long hpix = (long)(py * S + sub * CY) * hW + (long)px * S;
+    const long hpix_ld =
+        (long)((py < H ? py : H - 1) * S + sub * CY) * hW + (long)(px < W ? px : W - 1) * S;
+
+    const int nKc = DO_QK ? (d + CH - 1) / CH : 0;
+    const int nVc = DO_AV ? (C + CH - 1) / CH : 0;
+    const int ntot = nKc + nVc;
+
+    // Staging map: thread t carries window positions t, t+NT, ... of every
+    // channel of a chunk, so the per-thread part of each address (in-plane
+    // offset, LDS offset, inside-the-image flag) is fixed for the whole
+    // kernel and the per-channel part is wave-uniform.
+    int g_off[NPOS], l_off[NPOS];
+    unsigned g_mask[NPOS];
+#pragma unroll
+    for (int i = 0; i < NPOS; ++i) {
+        const int pos = tid + i * NT;
+        const int row = pos / WW, col = pos % WW;
+        const int gy = y0 - R + row, gx = x0 - R + col;
+        const bool l_ok = WIN % NT == 0 || pos < WIN;
+        const bool g_ok = l_ok && gy >= 0 && gy < H && gx >= 0 && gx < W;
+        const int yy = gy < 0 ? 0 : (gy < H ? gy : H - 1);
+        const int xx = gx < 0 ? 0 : (gx < W ? gx : W - 1);
+        g_off[i] = yy * W + xx;             // clamped: always a legal address
+        g_mask[i] = g_ok ? 0xffffffffu : 0u;
+        // surplus positions land in the unread padding column of row 0
+        l_off[i] = l_ok ? row * STRIDE + col : WW;
+    }
+    A st[NSTAGE];
+    // global -> registers for staged chunk j (key chunks first, then value)
+    auto stage_load = [&](int j) {
+        const bool is_key = j < nKc;
+        const T *src = is_key ? key : value;
+        const int nch = is_key ? d : C;
+        const int c0 = (is_key ? j : j - nKc) * CH;
+        const T *base = src + (long)n * nch * lplane;
+#pragma unroll
+        for (int ch = 0; ch < CH; ++ch) {
+            const int c = c0 + ch;
+            const T *plane = base + (long)(c < nch ? c : nch - 1) * lplane;
+#pragma unroll
+            for (int i = 0; i < NPOS; ++i) {
+                // unconditional load from the clamped address; the value is
+                // masked when it is stored to LDS, so that the load stays in
+                // flight across the FMAs of the current chunk
+                st[ch * NPOS + i] = (A)plane[g_off[i]];
+            }
+        }
+    };
+    // registers -> LDS buffer j&1, zeroing what lies outside the image or
+    // past the last channel
+    auto stage_store = [&](int j) {
+        const bool is_key = j < nKc;
+        const int nch = is_key ? d : C;
+        const int c0 = (is_key ? j : j - nKc) * CH;
+        A *dst = lds + (j & 1) * BUF;
+#pragma unroll
+        for (int ch = 0; ch < CH; ++ch)
+#pragma unroll
+            for (int i = 0; i < NPOS; ++i)
+                dst[(ch >> 1) * WH * STRIDE + (ch & 1) * HALF + l_off[i]] = __uint_as_float(
+                    __float_as_uint(st[ch * NPOS + i]) & (c0 + ch < nch ? g_mask[i] : 0u));
+    };
+
+    A a[NJ][KK];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+        for (int k = 0; k < KK; ++k) a[j][k] = 0;
+
+    stage_load(0);
+    if (MODE == TILED_AV && active) {
+        const T *ap = attn_in + (long)n * KK * hplane + hpix;
+#pragma unroll
+        for (int k = 0; k < KK; ++k)
+#pragma unroll
+            for (int cy = 0; cy < CY; ++cy) {
+                const VecS v = *(const VecS *)(ap + (long)k * hplane + (long)cy * hW);
+#pragma unroll
+                for (int cx = 0; cx < S; ++cx) a[cy * S + cx][k] = (A)v.v[cx];
+            }
+    }
+    stage_store(0);
+    __syncthreads();
+
+    const A *win = lds + ly * STRIDE + lx;  // this thread's window origin in buffer 0
+
+    if (DO_QK) {
+        const T *qp = q + (long)n * d * hplane + hpix_ld;
+        const unsigned qmask = active ? 0xffffffffu : 0u;
+        // q is fetched PF channels ahead of its use (a ring of PF x NJ
+        // registers), so HBM latency hides behind the FMAs of PF channels.
+        constexpr int PF = 4;
+        static_assert(CH % PF == 0, "prefetch ring must divide the chunk");
+        A qr[PF][NJ];
+        auto load_q = [&](int c, A (&dst)[NJ]) {
+#pragma unroll
+            for (int cy = 0; cy < CY; ++cy) {
+                const VecS v =
+                    *(const VecS *)(qp + (long)(c < d ? c : d - 1) * hplane + (long)cy * hW);
+#pragma unroll
+                for (int cx = 0; cx < S; ++cx) dst[cy * S + cx] = (A)v.v[cx];
+            }
+        };
+#pragma unroll
+        for (int u = 0; u < PF; ++u) load_q(u, qr[u]);
+        for (int j = 0; j < nKc; ++j) {
+            if (j + 1 < ntot) stage_load(j + 1);
+            const int c0 = j * CH;
+            const A *wb = win + (j & 1) * BUF;
+#pragma unroll 1
+            for (int ch0 = 0; ch0 < CH; ch0 += PF) {
+#pragma unroll
+                for (int u = 0; u < PF; ++u) {
+                    const int ch = ch0 + u;
+                    // ring values are raw loads from clamped addresses: zero
+                    // them for idle threads and past the last channel here
+                    const unsigned m = c0 + ch < d ? qmask : 0u;
+                    A qv[NJ];
+#pragma unroll
+                    for (int jj = 0; jj < NJ; ++jj)
+                        qv[jj] = __uint_as_float(__float_as_uint(qr[u][jj]) & m);
+                    load_q(c0 + ch + PF, qr[u]);
+                    const A *wc = wb + (ch >> 1) * WH * STRIDE + (ch & 1) * HALF;
+#pragma unroll
+                    for (int ky = 0; ky < K; ++ky)
+#pragma unroll
+                        for (int kx = 0; kx < K; ++kx) {
+                            const A kv = wc[ky * STRIDE + kx];
+#pragma unroll
+                            for (int jj = 0; jj < NJ; ++jj)
+                                a[jj][ky * K + kx] = fma_(kv, qv[jj], a[jj][ky * K + kx]);
+                        }
+                    // keep the next channel's window reads from being hoisted
+                    // over this channel's FMAs (register pressure)
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            if (j + 1 < ntot) stage_store(j + 1);
+            __syncthreads();
+        }
+        if (DO_SOFTMAX) {
+#pragma unroll
+            for (int jj = 0; jj < NJ; ++jj) softmax_inplace<A, KK>(a[jj]);
+        }
+        if (!DO_AV && active) {
+            T *op = out + (long)n * KK * hplane + hpix;
+#pragma unroll
+            for (int k = 0; k < KK; ++k)
+#pragma unroll
+                for (int cy = 0; cy < CY; ++cy) {
+                    VecS v;
+#pragma unroll
+                    for (int cx = 0; cx < S; ++cx) v.v[cx] = (T)a[cy * S + cx][k];
+                    *(VecS *)(op + (long)k * hplane + (long)cy * hW) = v;
+                }
+        }
+    }
+
+    if (DO_AV) {
+        T *op = out + (long)n * C * hplane + hpix;
+        for (int j = nKc; j < ntot; ++j) {
+            if (j + 1 < ntot) stage_load(j + 1);
+            const int c0 = (j - nKc) * CH;
+            const A *wb = win + (j & 1) * BUF;
+#pragma unroll 1
+            for (int ch = 0; ch < CH; ++ch) {
+                {
+                    const int c = c0 + ch;
+                    const A *wc = wb + (ch >> 1) * WH * STRIDE + (ch & 1) * HALF;
+                    A o[NJ];
+#pragma unroll
+                    for (int jj = 0; jj < NJ; ++jj) o[jj] = 0;
+#pragma unroll
+                    for (int ky = 0; ky < K; ++ky)
+#pragma unroll
+                        for (int kx = 0; kx < K; ++kx) {
+                            const A vv = wc[ky * STRIDE + kx];
+#pragma unroll
+                            for (int jj = 0; jj < NJ; ++jj)
+                                o[jj] = fma_(vv, a[jj][ky * K + kx], o[jj]);
+                        }
+                    if (active && c < C) {
+#pragma unroll
+                        for (int cy = 0; cy < CY; ++cy) {
+                            VecS v;
+#pragma unroll
+                            for (int cx = 0; cx < S; ++cx) v.v[cx] = (T)o[cy * S + cx];
+                            *(VecS *)(op + (long)c * hplane + (long)cy * hW) = v;
+                        }
+                    }
+                }
+            }
+            if (j + 1 < ntot) stage_store(j + 1);
+            __syncthreads();
+        }
+    }
+}
+
+// ------------------------------------------------------------------ launcher
+template <typename T, int K, int S, int CY, int NWY>
+static hipError_t launch_mode(int mode, const void *q, const void *key, const void *attn_in,
+                              const void *value, void *out, int B, int d, int C, int H, int W,
+                              hipStream_t st) {
+    constexpr int TW = 16, TH = 4 * NWY, NT = 64 * NWY * (S / CY);
+    const int tiles_x = (W + TW - 1) / TW, tiles_y = (H + TH - 1) / TH;
+    const long nb = (long)tiles_x * tiles_y * B;
+    if (nb > (1L << 30)) return hipErrorNotSupported;
+    const int per_xcd = (int)((nb + 7) / 8);
+    const dim3 grid(per_xcd * 8), block(NT);
+#define SAPA_TM_CASE(M)                                                                       \
+    case M:                                                                                   \
+        hipLaunchKernelGGL((sapa_b_tiled_kernel<T, K, S, CY, NWY, M>), grid, block, 0, st,    \
+                           (const T *)q, (const T *)key, (const T *)attn_in,                  \
+                           (const T *)value, (T *)out, d, C, H, W, tiles_x, tiles_y, (int)nb, \
+                           per_xcd);                                                          \
+        break;
+    switch (mode) {
+        SAPA_TM_CASE(TILED_QK) SAPA_TM_CASE(TILED_QK_SOFTMAX) SAPA_TM_CASE(TILED_AV)
+        SAPA_TM_CASE(TILED_FUSED)
+        default: return hipErrorInvalidValue;
+    }
+#undef SAPA_TM_CASE
+    return hipGetLastError();
+}
+
+template <typename T>
+static hipError_t launch_t(int mode, const void *q, const void *key, const void *attn_in,
+                           const void *value, void *out, int B, int d, int C, int H, int W, int K,
+                           int s, hipStream_t st) {
+    // vector accesses of s elements on the high-res tensors
+    const uintptr_t align = (uintptr_t)(sizeof(T) * s);
+    const void *hi_ptrs[3] = {q, attn_in, out};
+    for (int i = 0; i < 3; ++i)
+        if (hi_ptrs[i] && ((uintptr_t)hi_ptrs[i] % align) != 0) return hipErrorNotSupported;
+    if (K == 5 && s == 2) {
+        // tall tiles amortise the halo; short ones leave fewer idle rows
+        const int waste4 = ((H + 15) / 16) * 16 - H, waste2 = ((H + 7) / 8) * 8 - H;
+        if (waste4 <= waste2)
+            return launch_mode<T, 5, 2, 2, 4>(mode, q, key, attn_in, value, out, B, d, C, H, W, st);
+        return launch_mode<T, 5, 2, 2, 2>(mode, q, key, attn_in, value, out, B, d, C, H, W, st);
+    }
+    return hipErrorNotSupported;
+}
+
+hipError_t sapa_b_tiled_launch(int mode, const void *q, const void *key, const void *attn_in,
+                               const void *value, void *out, int B, int d, int C, int H, int W,
+                               int K, int s, int dtype, hipStream_t st) {
+    switch (dtype) {
+        case 0: return launch_t<float>(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, st);
+        case 2: return launch_t<f16_t>(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, st);
+        case 3: return launch_t<bf16_t>(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, st);
+        default: return hipErrorNotSupported;
+    }
+}
+
+}  // namespace sapa

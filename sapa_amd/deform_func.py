@@ -1,0 +1,202 @@
+"""SAPA-D operators: autograd API of the reference on top of libsapa_hip.so.
+
+Mirrors deformsapa/deformsapa/deform_func.py of the reference
+(DeformQKFunction :7-59, DeformAVFunction :62-114): same names, argument
+order, assertions, output allocation and error behaviour, so
+`from deformsapa import deform_qk, deform_av` callers such as
+SAPADeform.attention (sapa_deform.py:51-53) run unchanged.
+`deform_sapa_fused` is an addition.
+"""
+import torch
+from torch.autograd import Function
+
+from . import _lib
+
+
+def _compute_dtype(t):
+    # the backward kernels exist for fp32 / fp64; 16-bit tensors take the
+    # fp32 kernels and the gradients are rounded back
+    return t.dtype if t.dtype in (torch.float32, torch.float64) else torch.float32
+
+
+def _deform_qk_backward(grad_output, query, key, offset, P, s, G, needs=(True, True, True)):
+    cdt = _compute_dtype(query)
+    go, q, k, off = (t.contiguous().to(cdt) for t in (grad_output, query, key, offset))
+    gq = torch.zeros_like(q) if needs[0] else None
+    gk = torch.zeros_like(k) if needs[1] else None
+    goff = torch.zeros_like(off) if needs[2] else None
+    _lib.require_cuda_contiguous(grad_output=go, query=q, key=k, offset=off)
+    n, c, h, w = k.size()
+    _lib.call('sapa_deform_qk_backward', k.device, _lib.ptr(go), _lib.ptr(q), _lib.ptr(k),
+              _lib.ptr(off), _lib.ptr(gq), _lib.ptr(gk), _lib.ptr(goff), n, c, h, w, P, s, G,
+              _lib.dtype_code(k))
+    return tuple(None if g is None else g.to(t.dtype)
+                 for g, t in ((gq, query), (gk, key), (goff, offset)))
+
+
+def _deform_av_backward(grad_output, attn, value, offset, P, s, G, needs=(True, True, True)):
+    cdt = _compute_dtype(value)
+    go, a, v, off = (t.contiguous().to(cdt) for t in (grad_output, attn, value, offset))
+    ga = torch.zeros_like(a) if needs[0] else None
+    gv = torch.zeros_like(v) if needs[1] else None
+    goff = torch.zeros_like(off) if needs[2] else None
+    _lib.require_cuda_contiguous(grad_output=go, attn=a, value=v, offset=off)
+    n, c, h, w = v.size()
+    _lib.call('sapa_deform_av_backward', v.device, _lib.ptr(go), _lib.ptr(a), _lib.ptr(v),
+              _lib.ptr(off), _lib.ptr(ga), _lib.ptr(gv), _lib.ptr(goff), n, c, h, w, P, s, G,
+              _lib.dtype_code(v))
+    return tuple(None if g is None else g.to(t.dtype)
+                 for g, t in ((ga, attn), (gv, value), (goff, offset)))
+
+
+class DeformQKFunction(Function):
+
+    @staticmethod
+    def forward(ctx, query, key, offset, num_point, scale_factor, groups):
+        assert scale_factor >= 1
+        assert query.size(0) == key.size(0)
+        assert query.size(1) == key.size(1)
+        assert query.size(2) == key.size(2) * scale_factor
+        assert query.size(3) == key.size(3) * scale_factor
+        assert offset.size(0) == key.size(0)
+        assert offset.size(1) == groups * num_point * 2
+        assert offset.size(2) == key.size(2) * scale_factor
+        assert offset.size(3) == key.size(3) * scale_factor
+        assert query.size(1) % groups == 0
+        assert num_point >= 1
+        ctx.num_point = num_point
+        ctx.scale_factor = scale_factor
+        ctx.groups = groups
+        ctx.query_size = query.size()
+        ctx.key_size = key.size()
+        ctx.offset_size = offset.size()
+
+        n, c, h, w = query.size()
+        output = query.new_zeros((n, groups, num_point, h, w))
+        if query.is_cuda:
+            _lib.require_cuda_contiguous(query=query, key=key, offset=offset)
+            _lib.call('sapa_deform_qk_forward', query.device, _lib.ptr(query), _lib.ptr(key),
+                      _lib.ptr(offset), _lib.ptr(output), n, c, key.size(2), key.size(3),
+                      num_point, scale_factor, groups, _lib.dtype_code(query))
+        else:
+            raise NotImplementedError
+
+        if query.requires_grad or key.requires_grad or offset.requires_grad:
+            ctx.save_for_backward(query, key, offset)
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        assert grad_output.is_cuda
+        query, key, offset = ctx.saved_tensors
+        gq, gk, goff = _deform_qk_backward(grad_output, query, key, offset, ctx.num_point,
+                                           ctx.scale_factor, ctx.groups)
+        return gq, gk, goff, None, None, None
+
+
+deform_qk = DeformQKFunction.apply
+
+
+class DeformAVFunction(Function):
+
+    @staticmethod
+    def forward(ctx, attn, value, offset, num_point, scale_factor, groups):
+        assert scale_factor >= 1
+        assert attn.size(0) == value.size(0)
+        assert attn.size(1) == groups
+        assert attn.size(2) == num_point
+        assert attn.size(3) == value.size(2) * scale_factor
+        assert attn.size(4) == value.size(3) * scale_factor
+        assert offset.size(0) == value.size(0)
+        assert offset.size(1) == groups * num_point * 2
+        assert offset.size(2) == value.size(2) * scale_factor
+        assert offset.size(3) == value.size(3) * scale_factor
+        assert value.size(1) % groups == 0
+        assert num_point >= 1
+        ctx.num_point = num_point
+        ctx.scale_factor = scale_factor
+        ctx.groups = groups
+        ctx.attn_size = attn.size()
+        ctx.value_size = value.size()
+        ctx.offset_size = offset.size()
+
+        n, c, h, w = value.size()
+        output = value.new_zeros((n, c, scale_factor * h, scale_factor * w))
+        if attn.is_cuda:
+            _lib.require_cuda_contiguous(attn=attn, value=value, offset=offset)
+            _lib.call('sapa_deform_av_forward', value.device, _lib.ptr(attn), _lib.ptr(value),
+                      _lib.ptr(offset), _lib.ptr(output), n, c, h, w, num_point, scale_factor,
+                      groups, _lib.dtype_code(value))
+        else:
+            raise NotImplementedError
+
+        if attn.requires_grad or value.requires_grad or offset.requires_grad:
+            ctx.save_for_backward(attn, value, offset)
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        assert grad_output.is_cuda
+        attn, value, offset = ctx.saved_tensors
+        ga, gv, goff = _deform_av_backward(grad_output, attn, value, offset, ctx.num_point,
+                                           ctx.scale_factor, ctx.groups)
+        return ga, gv, goff, None, None, None
+
+
+deform_av = DeformAVFunction.apply
+
+
+class DeformSAPAFusedFunction(Function):
+    """deform_av(softmax(deform_qk(query, key, offset), dim=2), value, offset)
+    -- SAPADeform.attention (sapa_deform.py:51-53) -- as one launch in the
+    forward pass; the backward pass recomputes the weights and chains the
+    three operators' gradients (the offset receives both paths' gradients)."""
+
+    @staticmethod
+    def forward(ctx, query, key, value, offset, num_point, scale_factor, groups):
+        assert scale_factor >= 1
+        assert query.size(0) == key.size(0) == value.size(0) == offset.size(0)
+        assert query.size(1) == key.size(1)
+        assert query.size(2) == key.size(2) * scale_factor
+        assert query.size(3) == key.size(3) * scale_factor
+        assert value.size(2) == key.size(2) and value.size(3) == key.size(3)
+        assert offset.size(1) == groups * num_point * 2
+        assert offset.size(2) == key.size(2) * scale_factor
+        assert offset.size(3) == key.size(3) * scale_factor
+        assert query.size(1) % groups == 0 and value.size(1) % groups == 0
+        assert num_point >= 1
+        ctx.num_point = num_point
+        ctx.scale_factor = scale_factor
+        ctx.groups = groups
+
+        n, c, h, w = value.size()
+        output = value.new_zeros((n, c, scale_factor * h, scale_factor * w))
+        if value.is_cuda:
+            _lib.require_cuda_contiguous(query=query, key=key, value=value, offset=offset)
+            _lib.call('sapa_deform_fused_forward', value.device, _lib.ptr(query),
+                      _lib.ptr(key), _lib.ptr(value), _lib.ptr(offset), _lib.ptr(output), n,
+                      key.size(1), c, h, w, num_point, scale_factor, groups,
+                      _lib.dtype_code(value))
+        else:
+            raise NotImplementedError
+
+        if any(t.requires_grad for t in (query, key, value, offset)):
+            ctx.save_for_backward(query, key, value, offset)
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        assert grad_output.is_cuda
+        query, key, value, offset = ctx.saved_tensors
+        P, s, G = ctx.num_point, ctx.scale_factor, ctx.groups
+        with torch.no_grad():
+            logits = DeformQKFunction.apply(query, key, offset, P, s, G)
+            attn = torch.softmax(logits.float(), dim=2).to(logits.dtype)
+        ga, gv, goff_av = _deform_av_backward(grad_output, attn, value, offset, P, s, G)
+        a32, g32 = attn.float(), ga.float()
+        grad_logits = (a32 * (g32 - (g32 * a32).sum(dim=2, keepdim=True))).to(attn.dtype)
+        gq, gk, goff_qk = _deform_qk_backward(grad_logits, query, key, offset, P, s, G)
+        return gq, gk, gv, goff_av + goff_qk, None, None, None
+
+
+deform_sapa_fused = DeformSAPAFusedFunction.apply

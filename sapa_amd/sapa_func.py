@@ -1,0 +1,216 @@
+"""SAPA-B operators: autograd API of the reference on top of libsapa_hip.so.
+
+Mirrors sapa/sapa/sapa_func.py of the reference (QKFunction :9-51,
+AVFunction :54-96): same names, argument order, assertions, output
+allocation and error behaviour (CPU tensors raise NotImplementedError), so
+`from sapa import qk, av` callers such as SAPA.attention (sapa_base.py:38-40)
+run unchanged.  `sapa_fused`, `qk_softmax` and `softmax_k` are additions.
+"""
+import torch
+from torch.autograd import Function
+
+from . import _lib
+
+
+def _check_odd_kernel(kernel_size):
+    assert (kernel_size - 1) % 2 == 0 and kernel_size >= 1
+
+
+def _qk_backward(grad_output, query, key, kernel_size, scale_factor, need_q=True, need_k=True):
+    grad_output = grad_output.contiguous()
+    grad_query = torch.zeros_like(query) if need_q else None
+    grad_key = torch.zeros_like(key) if need_k else None
+    _lib.require_cuda_contiguous(grad_output=grad_output, query=query, key=key)
+    n, c, h, w = key.size()
+    _lib.call('sapa_qk_backward', key.device, _lib.ptr(grad_output), _lib.ptr(query),
+              _lib.ptr(key), _lib.ptr(grad_query), _lib.ptr(grad_key), n, c, h, w,
+              kernel_size, scale_factor, _lib.dtype_code(key))
+    return grad_query, grad_key
+
+
+def _av_backward(grad_output, attn, value, kernel_size, scale_factor, need_a=True, need_v=True):
+    grad_output = grad_output.contiguous()
+    grad_attn = torch.zeros_like(attn) if need_a else None
+    grad_value = torch.zeros_like(value) if need_v else None
+    _lib.require_cuda_contiguous(grad_output=grad_output, attn=attn, value=value)
+    n, c, h, w = value.size()
+    _lib.call('sapa_av_backward', value.device, _lib.ptr(grad_output), _lib.ptr(attn),
+              _lib.ptr(value), _lib.ptr(grad_attn), _lib.ptr(grad_value), n, c, h, w,
+              kernel_size, scale_factor, _lib.dtype_code(value))
+    return grad_attn, grad_value
+
+
+class QKFunction(Function):
+
+    @staticmethod
+    def forward(ctx, query, key, kernel_size, scale_factor):
+        assert scale_factor >= 1
+        assert query.size(0) == key.size(0)
+        assert query.size(1) == key.size(1)
+        assert query.size(-1) == key.size(-1) * scale_factor
+        assert query.size(-2) == key.size(-2) * scale_factor
+        _check_odd_kernel(kernel_size)
+        ctx.kernel_size = kernel_size
+        ctx.scale_factor = scale_factor
+        ctx.query_size = query.size()
+        ctx.key_size = key.size()
+
+        n, c, h, w = key.size()
+        output = key.new_zeros((n, kernel_size ** 2, h * scale_factor, w * scale_factor))
+        if key.is_cuda:
+            _lib.require_cuda_contiguous(key=key, query=query)
+            _lib.call('sapa_qk_forward', key.device, _lib.ptr(query), _lib.ptr(key),
+                      _lib.ptr(output), n, c, h, w, kernel_size, scale_factor,
+                      _lib.dtype_code(key))
+        else:
+            raise NotImplementedError
+
+        if query.requires_grad or key.requires_grad:
+            ctx.save_for_backward(query, key)
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        assert grad_output.is_cuda
+        query, key = ctx.saved_tensors
+        grad_query, grad_key = _qk_backward(grad_output, query, key, ctx.kernel_size,
+                                            ctx.scale_factor)
+        return grad_query, grad_key, None, None
+
+
+qk = QKFunction.apply
+
+
+class AVFunction(Function):
+
+    @staticmethod
+    def forward(ctx, attn, value, kernel_size, scale_factor):
+        assert scale_factor >= 1
+        assert attn.size(0) == value.size(0)
+        assert attn.size(1) == kernel_size * kernel_size
+        assert attn.size(-1) == value.size(-1) * scale_factor
+        assert attn.size(-2) == value.size(-2) * scale_factor
+        _check_odd_kernel(kernel_size)
+        ctx.kernel_size = kernel_size
+        ctx.scale_factor = scale_factor
+        ctx.attn_size = attn.size()
+        ctx.value_size = value.size()
+
+        n, c, h, w = value.size()
+        output = value.new_zeros((n, c, h * scale_factor, w * scale_factor))
+        if value.is_cuda:
+            _lib.require_cuda_contiguous(value=value, attn=attn)
+            _lib.call('sapa_av_forward', value.device, _lib.ptr(attn), _lib.ptr(value),
+                      _lib.ptr(output), n, c, h, w, kernel_size, scale_factor,
+                      _lib.dtype_code(value))
+        else:
+            raise NotImplementedError
+
+        if attn.requires_grad or value.requires_grad:
+            ctx.save_for_backward(attn, value)
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        assert grad_output.is_cuda
+        attn, value = ctx.saved_tensors
+        grad_attn, grad_value = _av_backward(grad_output, attn, value, ctx.kernel_size,
+                                             ctx.scale_factor)
+        return grad_attn, grad_value, None, None
+
+
+av = AVFunction.apply
+
+
+def softmax_k(logits, dim=1):
+    """Softmax over `dim` with the library's kernel (no autograd): the
+    stand-alone form of the F.softmax calls in sapa_base.py:39 (dim=1) and
+    sapa_deform.py:52 (dim=2)."""
+    if not logits.is_cuda:
+        raise NotImplementedError
+    _lib.require_cuda_contiguous(logits=logits)
+    dim = dim % logits.dim()
+    N = 1
+    for v in logits.shape[:dim]:
+        N *= v
+    M = 1
+    for v in logits.shape[dim + 1:]:
+        M *= v
+    out = torch.empty_like(logits)
+    _lib.call('sapa_softmax_forward', logits.device, _lib.ptr(logits), _lib.ptr(out), N,
+              logits.shape[dim], M, _lib.dtype_code(logits))
+    return out
+
+
+def _qk_softmax_forward(query, key, kernel_size, scale_factor):
+    n, c, h, w = key.size()
+    attn = key.new_empty((n, kernel_size ** 2, h * scale_factor, w * scale_factor))
+    _lib.call('sapa_qk_softmax_forward', key.device, _lib.ptr(query), _lib.ptr(key),
+              _lib.ptr(attn), n, c, h, w, kernel_size, scale_factor, _lib.dtype_code(key))
+    return attn
+
+
+def qk_softmax(query, key, kernel_size, scale_factor):
+    """softmax(qk(query, key), dim=1) in one launch (no autograd)."""
+    assert query.size(0) == key.size(0) and query.size(1) == key.size(1)
+    assert query.size(-1) == key.size(-1) * scale_factor
+    assert query.size(-2) == key.size(-2) * scale_factor
+    _check_odd_kernel(kernel_size)
+    if not key.is_cuda:
+        raise NotImplementedError
+    _lib.require_cuda_contiguous(key=key, query=query)
+    return _qk_softmax_forward(query, key, kernel_size, scale_factor)
+
+
+class SAPAFusedFunction(Function):
+    """av(softmax(qk(query, key), dim=1), value) -- SAPA.attention
+    (sapa_base.py:38-40) -- as one launch in the forward pass.  The backward
+    pass recomputes the attention weights (one launch) instead of keeping the
+    [B,K*K,sH,sW] tensor alive, then chains the three operators' gradients."""
+
+    @staticmethod
+    def forward(ctx, query, key, value, kernel_size, scale_factor):
+        assert scale_factor >= 1
+        assert query.size(0) == key.size(0) == value.size(0)
+        assert query.size(1) == key.size(1)
+        assert query.size(-1) == key.size(-1) * scale_factor
+        assert query.size(-2) == key.size(-2) * scale_factor
+        assert value.size(-1) == key.size(-1) and value.size(-2) == key.size(-2)
+        _check_odd_kernel(kernel_size)
+        ctx.kernel_size = kernel_size
+        ctx.scale_factor = scale_factor
+
+        n, d, h, w = key.size()
+        c = value.size(1)
+        output = value.new_zeros((n, c, h * scale_factor, w * scale_factor))
+        if value.is_cuda:
+            _lib.require_cuda_contiguous(value=value, key=key, query=query)
+            _lib.call('sapa_fused_forward', value.device, _lib.ptr(query), _lib.ptr(key),
+                      _lib.ptr(value), _lib.ptr(output), n, d, c, h, w, kernel_size,
+                      scale_factor, _lib.dtype_code(value))
+        else:
+            raise NotImplementedError
+
+        if query.requires_grad or key.requires_grad or value.requires_grad:
+            ctx.save_for_backward(query, key, value)
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        assert grad_output.is_cuda
+        query, key, value = ctx.saved_tensors
+        K, s = ctx.kernel_size, ctx.scale_factor
+        need_q, need_k, need_v = ctx.needs_input_grad[:3]
+        attn = _qk_softmax_forward(query, key, K, s)
+        grad_attn, grad_value = _av_backward(grad_output, attn, value, K, s,
+                                             need_a=need_q or need_k, need_v=need_v)
+        grad_query = grad_key = None
+        if need_q or need_k:
+            # softmax backward in fp32: g_logit = attn * (g_attn - sum_k g_attn * attn)
+            a32, g32 = attn.float(), grad_attn.float()
+            grad_logits = (a32 * (g32 - (g32 * a32).sum(dim=1, keepdim=True))).to(attn.dtype)
+            grad_query, grad_key = _qk_backward(grad_logits, query, key, K, s, need_q, need_k)
+        return grad_query, grad_key, grad_value, None, None
+
+
+sapa_fused = SAPAFusedFunction.apply

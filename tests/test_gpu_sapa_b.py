@@ -1,0 +1,263 @@
+"""GPU parity of the SAPA-B operators (qk, softmax, av, fused) against the
+CPU oracle, through the Python API and so through the C ABI.
+
+Bars: fp32 qk/av bit-exact against the oracle in the reference kernels' own
+arithmetic (same FMA order); fused fp32 within 1e-5 rel / 1e-6 abs; bf16
+within 1e-2 (relative to max(|b|, rms)); integer-valued inputs exact.
+"""
+import pytest
+import torch
+import torch.nn.functional as F
+
+import sapa_amd
+from helpers import (BF16_REL, F16_REL, assert_f32_close, assert_rel_rms_close, gen, golden,
+                     randn, ulp_report)
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda:0'
+
+# B, d, C, H, W, K, s -- K=5,s=2 takes the LDS-tiled kernels, the rest the
+# generic ones; extents are ragged against the 16x16 and 16x8 tiles
+SHAPES = [
+    (2, 6, 5, 9, 19, 5, 2), (1, 32, 64, 32, 32, 5, 2), (2, 8, 8, 16, 16, 5, 2),
+    (1, 3, 2, 1, 1, 5, 2), (1, 9, 7, 17, 33, 5, 2), (3, 64, 16, 24, 40, 5, 2),
+    (1, 4, 3, 5, 6, 3, 3), (1, 3, 2, 6, 7, 7, 1), (2, 5, 4, 4, 4, 1, 1),
+    (1, 4, 6, 7, 5, 9, 2), (1, 2, 2, 3, 3, 11, 4), (1, 3, 3, 8, 8, 3, 2),
+]
+IDS = ['-'.join(map(str, s)) for s in SHAPES]
+
+
+def dev(*ts):
+    return [t.to(DEV) for t in ts]
+
+
+@pytest.mark.parametrize('shape', SHAPES, ids=IDS)
+def test_qk_fp32_bit_exact(coracle, shape):
+    B, d, C, H, W, K, s = shape
+    g = gen(100)
+    q, key = randn(g, B, d, H * s, W * s), randn(g, B, d, H, W)
+    got = sapa_amd.qk(*dev(q, key), K, s).cpu()
+    want = coracle.qk(q, key, K, s, 'f32')
+    assert got.shape == want.shape and got.dtype == torch.float32
+    assert torch.equal(got, want), f'max ulp {ulp_report(got, want)}'
+    if d <= 9:  # short sums: also within the bar of the float64-accumulated value
+        assert_f32_close(got, coracle.qk(q, key, K, s, 'f32a64'), 'qk vs f64 accumulation')
+
+
+@pytest.mark.parametrize('shape', SHAPES, ids=IDS)
+def test_av_fp32_bit_exact(coracle, shape):
+    B, d, C, H, W, K, s = shape
+    g = gen(101)
+    attn, v = randn(g, B, K * K, H * s, W * s), randn(g, B, C, H, W)
+    got = sapa_amd.av(*dev(attn, v), K, s).cpu()
+    want = coracle.av(attn, v, K, s, 'f32')
+    assert torch.equal(got, want), f'max ulp {ulp_report(got, want)}'
+
+
+@pytest.mark.parametrize('shape', SHAPES, ids=IDS)
+def test_fused_fp32(coracle, shape):
+    B, d, C, H, W, K, s = shape
+    g = gen(102)
+    q, key, v = randn(g, B, d, H * s, W * s), randn(g, B, d, H, W), randn(g, B, C, H, W)
+    got = sapa_amd.sapa_fused(*dev(q, key, v), K, s).cpu()
+    assert_f32_close(got, coracle.sapa_fused(q, key, v, K, s, 'f32'), 'fused vs kernel-arithmetic oracle')
+    assert_f32_close(got, coracle.sapa_fused(q, key, v, K, s, 'f32a64'), 'fused vs f64-accumulated oracle')
+    # and the attention weights on their own
+    attn = sapa_amd.qk_softmax(*dev(q, key), K, s).cpu()
+    want = coracle.softmax(coracle.qk(q, key, K, s, 'f32'), 1, 'f32')
+    torch.testing.assert_close(attn, want, rtol=1e-5, atol=1e-7)
+    torch.testing.assert_close(attn.sum(1), torch.ones(B, H * s, W * s), rtol=1e-5, atol=0)
+
+
+@pytest.mark.parametrize('shape', SHAPES, ids=IDS)
+def test_integer_inputs_exact(coracle, shape):
+    """Integer-valued tensors: every product and sum is exact in fp32, so any
+    indexing error is a hard mismatch whatever the summation order."""
+    B, d, C, H, W, K, s = shape
+    g = gen(103)
+    ri = lambda *sh: torch.randint(-4, 5, sh, generator=g).float()
+    q, key, v, attn = ri(B, d, H * s, W * s), ri(B, d, H, W), ri(B, C, H, W), ri(B, K * K, H * s, W * s)
+    assert torch.equal(sapa_amd.qk(*dev(q, key), K, s).cpu(), coracle.qk(q, key, K, s, 'f32a64').float())
+    assert torch.equal(sapa_amd.av(*dev(attn, v), K, s).cpu(), coracle.av(attn, v, K, s, 'f32a64').float())
+
+
+def test_golden_vectors():
+    G = golden()
+    t = lambda a: torch.from_numpy(a)
+    for tag in ('b_k5s2', 'b_k3s3', 'b_k7s1'):
+        B, d, C, H, W, K, s = (int(v) for v in G[f'{tag}.cfg'])
+        q, key, v, attn = (t(G[f'{tag}.{n}']) for n in ('q', 'key', 'v', 'attn'))
+        assert torch.equal(sapa_amd.qk(*dev(q, key), K, s).cpu(), t(G[f'{tag}.qk'])), tag
+        assert torch.equal(sapa_amd.av(*dev(attn, v), K, s).cpu(), t(G[f'{tag}.av'])), tag
+        got = sapa_amd.sapa_fused(*dev(q, key, v), K, s).cpu()
+        assert_f32_close(got, t(G[f'{tag}.fused']), tag)
+        assert_f32_close(got, t(G[f'{tag}.fused64']), tag)
+
+
+def test_reference_forward_check_shape(coracle):
+    """sapa/sapa/forward_check.py:27-46 with its own tolerance (atol=1e-5),
+    against the unfold-based restatement."""
+    from oracle import torch_oracle as T
+    g = gen(104)
+    b, h, w, c, K, s = 4, 10, 12, 8, 5, 2
+    q, k = randn(g, b, c, s * h, s * w), randn(g, b, c, h, w)
+    assert torch.allclose(T.qk(q, k, K, s), sapa_amd.qk(*dev(q, k), K, s).cpu(), atol=1e-5)
+    attn, v = randn(g, b, K * K, s * h, s * w), randn(g, b, c, h, w)
+    assert torch.allclose(T.av(attn, v, K, s), sapa_amd.av(*dev(attn, v), K, s).cpu(), atol=1e-5)
+
+
+def test_softmax_kernel(coracle):
+    g = gen(105)
+    x = randn(g, 2, 25, 14, 22) * 4
+    got = sapa_amd.softmax_k(x.to(DEV), 1).cpu()
+    torch.testing.assert_close(got, coracle.softmax(x, 1, 'f32'), rtol=1e-5, atol=1e-7)
+    torch.testing.assert_close(got, F.softmax(x.double(), 1).float(), rtol=1e-5, atol=1e-7)
+    x5 = randn(g, 2, 4, 9, 6, 10)
+    got = sapa_amd.softmax_k(x5.to(DEV), 2).cpu()
+    torch.testing.assert_close(got, F.softmax(x5, 2), rtol=1e-5, atol=1e-7)
+    xd = x.double()
+    torch.testing.assert_close(sapa_amd.softmax_k(xd.to(DEV), 1).cpu(), F.softmax(xd, 1), rtol=1e-12, atol=1e-15)
+
+
+def test_fused_zero_query_box_filter():
+    """q == 0: uniform weights 1/K^2 everywhere, out-of-range neighbours
+    included in the denominator: the zero-padded box filter of the value."""
+    g = gen(106)
+    B, d, C, H, W, K, s = 2, 8, 6, 21, 37, 5, 2
+    key, v = randn(g, B, d, H, W), randn(g, B, C, H, W)
+    q = torch.zeros(B, d, H * s, W * s)
+    got = sapa_amd.sapa_fused(*dev(q, key, v), K, s).cpu()
+    want = F.avg_pool2d(v.double(), K, 1, K // 2, count_include_pad=True)
+    want = want.repeat_interleave(s, -2).repeat_interleave(s, -1)
+    assert_f32_close(got, want, 'box filter')
+
+
+@pytest.mark.parametrize('dtype,rel', [(torch.bfloat16, BF16_REL), (torch.float16, F16_REL)])
+@pytest.mark.parametrize('shape', [SHAPES[0], SHAPES[5], SHAPES[6], SHAPES[9]],
+                         ids=[IDS[0], IDS[5], IDS[6], IDS[9]])
+def test_16bit_dtypes(coracle, shape, dtype, rel):
+    """Oracle = fp32-input, float64-accumulated math on the rounded inputs."""
+    B, d, C, H, W, K, s = shape
+    g = gen(107)
+    q, key, v = (randn(g, *sh).to(dtype) for sh in
+                 ((B, d, H * s, W * s), (B, d, H, W), (B, C, H, W)))
+    attn = F.softmax(randn(g, B, K * K, H * s, W * s), 1).to(dtype)
+    qf, kf, vf, af = (x.float() for x in (q, key, v, attn))
+    got = sapa_amd.qk(*dev(q, key), K, s)
+    assert got.dtype == dtype
+    assert_rel_rms_close(got.float(), coracle.qk(qf, kf, K, s, 'f32a64'), rel, 'qk')
+    got = sapa_amd.av(*dev(attn, v), K, s)
+    assert_rel_rms_close(got.float(), coracle.av(af, vf, K, s, 'f32a64'), rel, 'av')
+    got = sapa_amd.sapa_fused(*dev(q, key, v), K, s)
+    assert got.dtype == dtype
+    assert_rel_rms_close(got.float(), coracle.sapa_fused(qf, kf, vf, K, s, 'f32a64'), rel, 'fused')
+
+
+@pytest.mark.parametrize('shape', [SHAPES[0], SHAPES[6]], ids=[IDS[0], IDS[6]])
+def test_fp64(coracle, shape):
+    B, d, C, H, W, K, s = shape
+    g = gen(108)
+    q, key, v = (randn(g, *sh, dtype=torch.float64) for sh in
+                 ((B, d, H * s, W * s), (B, d, H, W), (B, C, H, W)))
+    attn = randn(g, B, K * K, H * s, W * s, dtype=torch.float64)
+    assert torch.equal(sapa_amd.qk(*dev(q, key), K, s).cpu(), coracle.qk(q, key, K, s, 'f64'))
+    assert torch.equal(sapa_amd.av(*dev(attn, v), K, s).cpu(), coracle.av(attn, v, K, s, 'f64'))
+    torch.testing.assert_close(sapa_amd.sapa_fused(*dev(q, key, v), K, s).cpu(),
+                               coracle.sapa_fused(q, key, v, K, s, 'f64'), rtol=1e-12, atol=1e-13)
+
+
+@pytest.mark.parametrize('shape', [SHAPES[0], SHAPES[6], SHAPES[7]], ids=[IDS[0], IDS[6], IDS[7]])
+def test_backward_vs_oracle(coracle, shape):
+    B, d, C, H, W, K, s = shape
+    g = gen(109)
+    for dt, tol in ((torch.float64, dict(rtol=1e-11, atol=1e-12)), (torch.float32, dict(rtol=1e-4, atol=1e-5))):
+        q = randn(g, B, d, H * s, W * s, dtype=dt)
+        key = randn(g, B, d, H, W, dtype=dt)
+        go = randn(g, B, K * K, H * s, W * s, dtype=dt)
+        qd, kd = (x.to(DEV).requires_grad_() for x in (q, key))
+        sapa_amd.qk(qd, kd, K, s).backward(go.to(DEV))
+        gq, gk = coracle.qk_backward(go.double(), q.double(), key.double(), K, s, 'f64')
+        torch.testing.assert_close(qd.grad.cpu().double(), gq, **tol)
+        torch.testing.assert_close(kd.grad.cpu().double(), gk, **tol)
+
+        attn = randn(g, B, K * K, H * s, W * s, dtype=dt)
+        v = randn(g, B, C, H, W, dtype=dt)
+        go = randn(g, B, C, H * s, W * s, dtype=dt)
+        ad, vd = (x.to(DEV).requires_grad_() for x in (attn, v))
+        sapa_amd.av(ad, vd, K, s).backward(go.to(DEV))
+        ga, gv = coracle.av_backward(go.double(), attn.double(), v.double(), K, s, 'f64')
+        torch.testing.assert_close(ad.grad.cpu().double(), ga, **tol)
+        torch.testing.assert_close(vd.grad.cpu().double(), gv, **tol)
+
+
+def test_gradcheck_reference_shapes():
+    """sapa/sapa/grad_check.py:8-33: float64 gradcheck at its shapes."""
+    from torch.autograd import gradcheck
+    g = gen(110)
+    b, h, w, c, K, s = 2, 3, 4, 16, 5, 2
+    q = torch.rand(b, c, s * h, s * w, generator=g, dtype=torch.float64).to(DEV).requires_grad_()
+    k = torch.rand(b, c, h, w, generator=g, dtype=torch.float64).to(DEV).requires_grad_()
+    assert gradcheck(sapa_amd.qk, (q, k, K, s))
+    a = randn(g, b, K * K, s * h, s * w, dtype=torch.float64).to(DEV).requires_grad_()
+    v = randn(g, b, c, h, w, dtype=torch.float64).to(DEV).requires_grad_()
+    assert gradcheck(sapa_amd.av, (a, v, K, s), eps=1e-4)
+    v3 = randn(g, b, 3, h, w, dtype=torch.float64).to(DEV).requires_grad_()
+    assert gradcheck(sapa_amd.sapa_fused, (q, k, v3, K, s), eps=1e-5, atol=1e-6)
+
+
+def test_fused_backward_matches_composition():
+    g = gen(111)
+    B, d, C, H, W, K, s = 2, 6, 5, 9, 11, 5, 2
+    q, key, v = randn(g, B, d, H * s, W * s), randn(g, B, d, H, W), randn(g, B, C, H, W)
+    go = randn(g, B, C, H * s, W * s).to(DEV)
+    a = [x.to(DEV).requires_grad_() for x in (q, key, v)]
+    b = [x.to(DEV).requires_grad_() for x in (q, key, v)]
+    sapa_amd.sapa_fused(*a, K, s).backward(go)
+    sapa_amd.av(F.softmax(sapa_amd.qk(b[0], b[1], K, s), dim=1), b[2], K, s).backward(go)
+    for x, y in zip(a, b):
+        torch.testing.assert_close(x.grad, y.grad, rtol=1e-4, atol=1e-5)
+
+
+def test_error_behaviour_on_device():
+    """qk_cuda.cpp:34-39: non-contiguous tensors are refused, not copied."""
+    q = torch.randn(1, 4, 8, 16, device=DEV)[:, :, :, ::2]
+    k = torch.randn(1, 4, 4, 4, device=DEV)
+    with pytest.raises(RuntimeError):
+        sapa_amd.qk(q, k, 5, 2)
+    with pytest.raises(RuntimeError):
+        sapa_amd.qk(torch.randn(1, 4, 8, 8, device=DEV).double(), k, 5, 2)  # dtype mismatch
+    out = sapa_amd.qk(torch.randn(1, 4, 8, 8, device=DEV), k, 5, 2)
+    assert out.shape == (1, 25, 8, 8) and out.dtype == torch.float32 and out.is_cuda
+
+
+def test_sapa_module_forward_and_drop_in_import(coracle):
+    """The reference's own caller pattern: `from sapa import qk, av`, then
+    av(softmax(qk(q, k)), v) (sapa_base.py:4,38-40); and the SAPA module at
+    BASELINE config 1 (1x64x32x32 -> 64x64, d=32, K=5)."""
+    from sapa import av, qk
+    g = gen(112)
+    torch.manual_seed(0)
+    m = sapa_amd.SAPA(64, embedding_dim=32).to(DEV)
+    y, x = randn(g, 1, 64, 64, 64), randn(g, 1, 64, 32, 32)
+    with torch.no_grad():
+        out = m(y.to(DEV), x.to(DEV))
+        qd, kd = m.q(m.norm_y(y.to(DEV))), m.k(m.norm_x(x.to(DEV)))
+        out3 = av(F.softmax(qk(qd, kd, 5, 2), dim=1), x.to(DEV), 5, 2)
+    assert out.shape == (1, 64, 64, 64)
+    want = coracle.sapa_fused(qd.cpu(), kd.cpu(), x, 5, 2, 'f32a64')
+    assert_f32_close(out.cpu(), want, 'SAPA module (fused)')
+    assert_f32_close(out3.cpu(), want, 'reference three-step composition')
+    m.fused = False
+    with torch.no_grad():
+        assert_f32_close(m(y.to(DEV), x.to(DEV)).cpu(), want, 'SAPA module (three-step)')
+
+
+def test_module_trains():
+    torch.manual_seed(1)
+    m = sapa_amd.SAPA(32, embedding_dim=16).to(DEV)
+    y = torch.randn(2, 32, 16, 24, device=DEV)
+    x = torch.randn(2, 32, 8, 12, device=DEV, requires_grad=True)
+    m(y, x).square().mean().backward()
+    for n, p in m.named_parameters():
+        assert p.grad is not None and torch.isfinite(p.grad).all(), n
+    assert x.grad is not None and x.grad.abs().sum() > 0

@@ -1,0 +1,222 @@
+"""GPU parity of the SAPA-D operators (deform_qk, deform_av, fused) against
+the CPU oracle, through the Python API and so through the C ABI.
+
+fp32 results are compared bit-for-bit with the oracle in the reference
+kernels' arithmetic: that pins the floor / guard / corner indexing exactly.
+"""
+import pytest
+import torch
+import torch.nn.functional as F
+
+import sapa_amd
+from helpers import (BF16_REL, F16_REL, assert_f32_close, assert_rel_rms_close, gen, golden,
+                     randn, ulp_report)
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda:0'
+
+# B, G, dq (query/key channels per group), cg (value channels per group), H, W, P, s
+SHAPES = [
+    (2, 4, 2, 3, 7, 9, 5, 2), (1, 2, 3, 2, 5, 5, 9, 1), (1, 4, 8, 16, 12, 20, 9, 2),
+    (2, 1, 4, 5, 6, 4, 25, 2), (1, 3, 2, 2, 4, 5, 3, 3), (1, 2, 5, 9, 8, 8, 17, 2),
+    (1, 1, 2, 2, 3, 3, 40, 2), (1, 4, 32, 64, 16, 16, 5, 2),
+]
+IDS = ['-'.join(map(str, s)) for s in SHAPES]
+
+
+def dev(*ts):
+    return [t.to(DEV) for t in ts]
+
+
+def make(g, shape, dtype=torch.float32, off_scale=1.5):
+    B, G, dq, cg, H, W, P, s = shape
+    q = randn(g, B, G * dq, H * s, W * s, dtype=dtype)
+    key = randn(g, B, G * dq, H, W, dtype=dtype)
+    v = randn(g, B, G * cg, H, W, dtype=dtype)
+    off = randn(g, B, 2 * G * P, H * s, W * s, dtype=dtype) * off_scale
+    attn = randn(g, B, G, P, H * s, W * s, dtype=dtype)
+    return q, key, v, off, attn
+
+
+@pytest.mark.parametrize('shape', SHAPES, ids=IDS)
+def test_deform_qk_av_fp32_bit_exact(coracle, shape):
+    B, G, dq, cg, H, W, P, s = shape
+    q, key, v, off, attn = make(gen(200), shape)
+    got = sapa_amd.deform_qk(*dev(q, key, off), P, s, G).cpu()
+    want = coracle.deform_qk(q, key, off, P, s, G, 'f32')
+    assert got.shape == (B, G, P, H * s, W * s)
+    assert torch.equal(got, want), f'deform_qk max ulp {ulp_report(got, want)}'
+    got = sapa_amd.deform_av(*dev(attn, v, off), P, s, G).cpu()
+    want = coracle.deform_av(attn, v, off, P, s, G, 'f32')
+    assert torch.equal(got, want), f'deform_av max ulp {ulp_report(got, want)}'
+
+
+@pytest.mark.parametrize('shape', SHAPES, ids=IDS)
+def test_deform_fused_fp32(coracle, shape):
+    B, G, dq, cg, H, W, P, s = shape
+    q, key, v, off, _ = make(gen(201), shape)
+    got = sapa_amd.deform_sapa_fused(*dev(q, key, v, off), P, s, G).cpu()
+    assert_f32_close(got, coracle.deform_sapa_fused(q, key, v, off, P, s, G, 'f32'), 'deform fused')
+    want64 = coracle.deform_sapa_fused(q.double(), key.double(), v.double(), off.double(), P, s, G, 'f64')
+    torch.testing.assert_close(got.double(), want64, rtol=1e-4, atol=1e-5)
+
+
+def test_golden_vectors():
+    G = golden()
+    t = lambda a: torch.from_numpy(a)
+    for tag in ('d_p5s2', 'd_p9s1'):
+        B, Gr, dq, cg, H, W, P, s = (int(v) for v in G[f'{tag}.cfg'])
+        q, key, v, off, attn = (t(G[f'{tag}.{n}']) for n in ('q', 'key', 'v', 'off', 'attn'))
+        assert torch.equal(sapa_amd.deform_qk(*dev(q, key, off), P, s, Gr).cpu(), t(G[f'{tag}.dqk'])), tag
+        assert torch.equal(sapa_amd.deform_av(*dev(attn, v, off), P, s, Gr).cpu(), t(G[f'{tag}.dav'])), tag
+        assert_f32_close(sapa_amd.deform_sapa_fused(*dev(q, key, v, off), P, s, Gr).cpu(),
+                         t(G[f'{tag}.dfused']), tag)
+
+
+def test_regular_grid_offsets_reduce_to_sapa_b():
+    """G=1, P=K*K, integer offsets on the window grid: the sampled operators
+    equal the window operators bit for bit (weights are exactly 1,0,0,0)."""
+    g = gen(202)
+    B, d, C, H, W, K, s = 2, 6, 5, 9, 11, 5, 2
+    q, key, v = randn(g, B, d, H * s, W * s), randn(g, B, d, H, W), randn(g, B, C, H, W)
+    attn = randn(g, B, K * K, H * s, W * s)
+    off = torch.zeros(B, 2 * K * K, H * s, W * s)
+    for ky in range(K):
+        for kx in range(K):
+            off[:, 2 * (ky * K + kx)] = kx - K // 2
+            off[:, 2 * (ky * K + kx) + 1] = ky - K // 2
+    a = sapa_amd.deform_qk(*dev(q, key, off), K * K, s, 1)
+    assert torch.equal(a.view(B, K * K, H * s, W * s), sapa_amd.qk(*dev(q, key), K, s))
+    b = sapa_amd.deform_av(attn.view(B, 1, K * K, H * s, W * s).to(DEV), v.to(DEV), off.to(DEV), K * K, s, 1)
+    assert torch.equal(b, sapa_amd.av(*dev(attn, v), K, s))
+    c = sapa_amd.deform_sapa_fused(*dev(q, key, v, off), K * K, s, 1)
+    assert_f32_close(c.cpu(), sapa_amd.sapa_fused(*dev(q, key, v), K, s).cpu(), 'fused families')
+
+
+def test_guard_and_borders(coracle):
+    """Offsets that push samples across every border, onto exact integers and
+    onto the guard's edges (-1 and H): indices must still match exactly."""
+    g = gen(203)
+    shape = (1, 2, 3, 2, 5, 6, 8, 2)
+    B, G, dq, cg, H, W, P, s = shape
+    q, key, v, off, attn = make(g, shape, off_scale=4.0)
+    off[:, :, ::3, ::2] = torch.round(off[:, :, ::3, ::2])          # exact integers
+    off[0, 0] = -1.0 - torch.arange(W * s).div(s, rounding_mode='floor').float()  # kw == -1 exactly
+    off[0, 3] = float(H)                                             # kh >= H
+    got = sapa_amd.deform_qk(*dev(q, key, off), P, s, G).cpu()
+    assert torch.equal(got, coracle.deform_qk(q, key, off, P, s, G, 'f32'))
+    assert torch.count_nonzero(got[0, 0, 0]) == 0
+    got = sapa_amd.deform_av(*dev(attn, v, off), P, s, G).cpu()
+    assert torch.equal(got, coracle.deform_av(attn, v, off, P, s, G, 'f32'))
+
+
+@pytest.mark.parametrize('dtype,rel', [(torch.bfloat16, BF16_REL), (torch.float16, F16_REL)])
+def test_16bit_dtypes(coracle, dtype, rel):
+    shape = SHAPES[2]
+    B, G, dq, cg, H, W, P, s = shape
+    q, key, v, off, attn = (x.to(dtype) for x in make(gen(204), shape))
+    attn = F.softmax(attn.float(), 2).to(dtype)
+    qf, kf, vf, of, af = (x.float() for x in (q, key, v, off, attn))
+    got = sapa_amd.deform_qk(*dev(q, key, off), P, s, G)
+    assert got.dtype == dtype
+    assert_rel_rms_close(got.float(), coracle.deform_qk(qf, kf, of, P, s, G, 'f32a64'), rel, 'dqk')
+    got = sapa_amd.deform_av(*dev(attn, v, off), P, s, G)
+    assert_rel_rms_close(got.float(), coracle.deform_av(af, vf, of, P, s, G, 'f32a64'), rel, 'dav')
+    got = sapa_amd.deform_sapa_fused(*dev(q, key, v, off), P, s, G)
+    want = coracle.deform_sapa_fused(qf, kf, vf, of, P, s, G, 'f32')
+    assert_rel_rms_close(got.float(), want, rel, 'dfused')
+
+
+def test_fp64(coracle):
+    shape = SHAPES[0]
+    B, G, dq, cg, H, W, P, s = shape
+    q, key, v, off, attn = make(gen(205), shape, dtype=torch.float64)
+    assert torch.equal(sapa_amd.deform_qk(*dev(q, key, off), P, s, G).cpu(),
+                       coracle.deform_qk(q, key, off, P, s, G, 'f64'))
+    assert torch.equal(sapa_amd.deform_av(*dev(attn, v, off), P, s, G).cpu(),
+                       coracle.deform_av(attn, v, off, P, s, G, 'f64'))
+    torch.testing.assert_close(sapa_amd.deform_sapa_fused(*dev(q, key, v, off), P, s, G).cpu(),
+                               coracle.deform_sapa_fused(q, key, v, off, P, s, G, 'f64'),
+                               rtol=1e-12, atol=1e-13)
+
+
+@pytest.mark.parametrize('shape', [SHAPES[0], SHAPES[4]], ids=[IDS[0], IDS[4]])
+def test_backward_vs_oracle(coracle, shape):
+    B, G, dq, cg, H, W, P, s = shape
+    for dt, tol in ((torch.float64, dict(rtol=1e-10, atol=1e-11)), (torch.float32, dict(rtol=1e-4, atol=1e-4))):
+        g = gen(206)
+        q, key, v, off, attn = make(g, shape, dtype=dt)
+        go = randn(g, B, G, P, H * s, W * s, dtype=dt)
+        qd, kd, od = (x.to(DEV).requires_grad_() for x in (q, key, off))
+        sapa_amd.deform_qk(qd, kd, od, P, s, G).backward(go.to(DEV))
+        gq, gk, goff = coracle.deform_qk_backward(go.double(), q.double(), key.double(), off.double(), P, s, G, 'f64')
+        if dt == torch.float64:
+            torch.testing.assert_close(qd.grad.cpu().double(), gq, **tol)
+            torch.testing.assert_close(kd.grad.cpu().double(), gk, **tol)
+            torch.testing.assert_close(od.grad.cpu().double(), goff, **tol)
+        else:
+            # fp32 coordinates differ from float64 ones in the last bit: compare
+            # with the oracle run in fp32 arithmetic instead
+            gq32, gk32, goff32 = coracle.deform_qk_backward(go, q, key, off, P, s, G, 'f32')
+            torch.testing.assert_close(qd.grad.cpu(), gq32, **tol)
+            torch.testing.assert_close(kd.grad.cpu(), gk32, **tol)
+            torch.testing.assert_close(od.grad.cpu(), goff32, **tol)
+
+        go = randn(g, B, G * cg, H * s, W * s, dtype=dt)
+        ad, vd, od = (x.to(DEV).requires_grad_() for x in (attn, v, off))
+        sapa_amd.deform_av(ad, vd, od, P, s, G).backward(go.to(DEV))
+        mode = 'f64' if dt == torch.float64 else 'f32'
+        ga, gv, goff = coracle.deform_av_backward(go, attn, v, off, P, s, G, mode)
+        torch.testing.assert_close(ad.grad.cpu(), ga, **tol)
+        torch.testing.assert_close(vd.grad.cpu(), gv, **tol)
+        torch.testing.assert_close(od.grad.cpu(), goff, **tol)
+
+
+def test_gradcheck_reference_shapes():
+    """deformsapa/deformsapa/grad_check.py:8-35: float64 gradcheck at its
+    shapes, offsets in [0,1) so no sample sits on a bilinear kink."""
+    from torch.autograd import gradcheck
+    g = gen(207)
+    b, h, w, c, P, s, G = 2, 3, 4, 16, 5, 2, 4
+    r = lambda *sh: torch.rand(*sh, generator=g, dtype=torch.float64).to(DEV).requires_grad_()
+    q, k, o = r(b, c, s * h, s * w), r(b, c, h, w), r(b, G * P * 2, s * h, s * w)
+    assert gradcheck(sapa_amd.deform_qk, (q, k, o, P, s, G))
+    a = randn(g, b, G, P, s * h, s * w, dtype=torch.float64).to(DEV).requires_grad_()
+    v = randn(g, b, c, h, w, dtype=torch.float64).to(DEV).requires_grad_()
+    assert gradcheck(sapa_amd.deform_av, (a, v, o, P, s, G))
+    assert gradcheck(sapa_amd.deform_sapa_fused, (q, k, v, o, P, s, G), eps=1e-5, atol=1e-6)
+
+
+def test_sapa_deform_module(coracle):
+    """SAPADeform at the module's defaults (P=9, G=4, pixel-shuffled offsets,
+    sapa_deform.py:8-9,44-45), fused and three-step, against the oracle fed
+    with the same projections."""
+    from deformsapa import deform_av, deform_qk
+    g = gen(208)
+    torch.manual_seed(2)
+    m = sapa_amd.SAPADeform(16, embedding_dim=8).to(DEV)
+    torch.nn.init.normal_(m.offset.weight, std=0.3)   # spread the samples out
+    y, x = randn(g, 2, 16, 12, 20), randn(g, 2, 16, 6, 10)
+    with torch.no_grad():
+        out = m(y.to(DEV), x.to(DEV))
+        q, k = m.q(y.to(DEV)), m.k(x.to(DEV))
+        off = F.pixel_shuffle(m.offset(x.to(DEV)), 2).contiguous()
+        out3 = deform_av(F.softmax(deform_qk(q, k, off, 9, 2, 4), dim=2), x.to(DEV), off, 9, 2, 4)
+    assert out.shape == (2, 16, 12, 20)
+    want = coracle.deform_sapa_fused(q.cpu(), k.cpu(), x, off.cpu(), 9, 2, 4, 'f32')
+    assert_f32_close(out.cpu(), want, 'SAPADeform fused')
+    assert_f32_close(out3.cpu(), want, 'SAPADeform three-step')
+    m2 = sapa_amd.SAPADeform(16, embedding_dim=8, high_offset=False, norm=False, fused=False).to(DEV)
+    with torch.no_grad():
+        assert m2(y.to(DEV), x.to(DEV)).shape == (2, 16, 12, 20)
+
+
+def test_module_trains():
+    torch.manual_seed(3)
+    m = sapa_amd.SAPADeform(16, embedding_dim=8).to(DEV)
+    y = torch.randn(2, 16, 12, 16, device=DEV)
+    x = torch.randn(2, 16, 6, 8, device=DEV, requires_grad=True)
+    m(y, x).square().mean().backward()
+    for n, p in m.named_parameters():
+        assert p.grad is not None and torch.isfinite(p.grad).all(), n
+    assert x.grad is not None and x.grad.abs().sum() > 0
