@@ -163,10 +163,13 @@ def main():
         # the timed GPU output for the same image, against the CPU result
         got = out[:1].float().cpu()
         err = (got - ref).abs()
-        tol = (1e-6 + 1e-5 * ref.abs()) if args.dtype == 'fp32' else \
+        # the CPU path sums in another order (einsum), so this is fp32-vs-fp32
+        # at the reference's own check tolerance, allclose(atol=1e-5)
+        tol = (1e-5 + 1e-5 * ref.abs()) if args.dtype == 'fp32' else \
             1e-2 * torch.maximum(ref.abs(), ref.pow(2).mean().sqrt())
         rec['parity_vs_cpu_sample'] = {'max_abs_err': err.max().item(),
-                                       'violations': int((err > 3 * tol).sum().item())}
+                                       'outside_tolerance': int((err > tol).sum().item()),
+                                       'elements': err.numel()}
     print(json.dumps(rec))
 
 
