@@ -86,6 +86,10 @@ def main():
     ap.add_argument('--dtype', default='fp32', choices=['fp32', 'bf16'])
     ap.add_argument('--workload', default='fpn_large', choices=sorted(WORKLOADS))
     ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--calibration-copy', action='store_true',
+                    help='after the timed region, run 5 device copies of 1 GiB (a kernel of '
+                         'known traffic: 1 GiB read + 1 GiB written) for scaling profiler '
+                         'byte counters')
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit('bench.py: this build measures one GPU only (the operators are '
@@ -124,6 +128,14 @@ def main():
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
     ms = e0.elapsed_time(e1) / args.steps
+
+    if args.calibration_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     pix = B * H * s * W * s
     esize = out.element_size()

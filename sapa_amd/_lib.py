@@ -10,7 +10,8 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, 'lib', 'libsapa_hip.so')
+# SAPA_HIP_LIBRARY points at another build of the same ABI (e.g. a tuning build)
+LIB_PATH = os.environ.get('SAPA_HIP_LIBRARY') or os.path.join(_HERE, 'lib', 'libsapa_hip.so')
 
 ABI_VERSION = 1
 

@@ -2,8 +2,9 @@
 // qk -> softmax -> av forward, all from one template.
 //
 // Work decomposition (NCHW tensors, so the contiguous axis is W):
-//   * a workgroup owns a tile of TW x TH = 16 x (4*NWY) low-res parent cells
-//     of one image; a wave owns 16 x 4 of them, lane = (lx 0..15, ly 0..3);
+//   * a workgroup owns a tile of TW x TH = (16*NWX) x (4*NWY) low-res parent
+//     cells of one image; a wave owns 16 x 4 of them, lane = (lx 0..15,
+//     ly 0..3);
 //   * a thread owns CY x S of the S x S high-res children of its parent
 //     (CY = S: all of them; CY < S: S/CY waves share the parent rows), and
 //     keeps their K*K logits / weights in registers (CY*S*K*K values);
@@ -14,10 +15,14 @@
 //     up to K*K parents through LDS;
 //   * q is read and the output written exactly once, as S-wide vectors that
 //     are contiguous across the 16 lanes of a row (S*16 elements per row).
-// LDS layout: window rows of WW <= 24 floats at a row stride of 48 floats,
-// two channels side by side in one row (columns 0..23 and 24..47).  A stride
-// that is 16 mod 32 puts the four 16-lane rows of a wave on disjoint banks,
-// so the window reads (row ly+ky, column lx+kx) are conflict-free.
+// LDS layout: two channels side by side in one LDS row, each in HALF >= WW+1
+// floats with HALF = 8 mod 16, so the row stride 2*HALF is 16 mod 32 (48 for
+// a 16-wide tile).  That puts the four 16-lane rows of a wave on disjoint
+// banks, so the window reads (row ly+ky, column lx+kx) are conflict-free.
+// What bounds the kernel on MI355X is the number of 64-byte requests between
+// a CU's vector L1 and L2, not HBM bytes: a window row that starts 2 floats
+// left of a 64-byte boundary costs a whole extra line per side, which is why
+// wider tiles (NWX = 2) win even though they idle more lanes on ragged widths.
 //
 // Arithmetic is the reference kernels' own, term by term: one FMA per
 // channel in channel order for the logits (qk_cuda_kernel.cu:55-66), one FMA
@@ -35,8 +40,41 @@ struct alignas(sizeof(T) * N) Vec {
     T v[N];
 };
 
-template <typename T, int K, int S, int CY, int NWY, int MODE>
-__global__ void __launch_bounds__(64 * NWY * (S / CY)) __attribute__((amdgpu_waves_per_eu(3, 3)))
+// Unsigned integer of NB bytes, as the carrier of a streaming access.
+template <int NB> struct Bits;
+template <> struct Bits<2> { typedef unsigned short type; };
+template <> struct Bits<4> { typedef unsigned type; };
+template <> struct Bits<8> { typedef unsigned type __attribute__((ext_vector_type(2))); };
+template <> struct Bits<16> { typedef unsigned type __attribute__((ext_vector_type(4))); };
+
+// The high-res tensors are touched exactly once (q read, output written), so
+// both go around the caches as non-temporal accesses: that leaves L2 to the
+// low-res windows, which neighbouring tiles re-read, and lets partial-line
+// output writes drain without allocating.
+#ifndef SAPA_STREAM_LOADS
+#define SAPA_STREAM_LOADS 1
+#endif
+template <typename T, int N>
+__device__ __forceinline__ Vec<T, N> load_stream(const T *p) {
+    typedef typename Bits<sizeof(T) * N>::type B;
+    union { B b; Vec<T, N> v; } u;
+#if SAPA_STREAM_LOADS
+    u.b = __builtin_nontemporal_load((const B *)p);
+#else
+    u.b = *(const B *)p;
+#endif
+    return u.v;
+}
+template <typename T, int N>
+__device__ __forceinline__ void store_stream(T *p, const Vec<T, N> &v) {
+    typedef typename Bits<sizeof(T) * N>::type B;
+    union { B b; Vec<T, N> v; } u;
+    u.v = v;
+    __builtin_nontemporal_store(u.b, (B *)p);
+}
+
+template <typename T, int K, int S, int CY, int NWX, int NWY, int CH, int MODE>
+__global__ void __launch_bounds__(64 * NWX * NWY * (S / CY)) __attribute__((amdgpu_waves_per_eu(3, 3)))
 sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
                     const T *__restrict__ attn_in, const T *__restrict__ value,
                     T *__restrict__ out, int d, int C, int H, int W, int tiles_x, int tiles_y,
@@ -44,11 +82,12 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
     typedef float A;
     constexpr int KK = K * K, R = (K - 1) / 2;
     constexpr int NSUB = S / CY;           // waves sharing one band of parent rows
-    constexpr int NT = 64 * NWY * NSUB;    // threads per workgroup
-    constexpr int TW = 16, TH = 4 * NWY;   // parents per workgroup
+    constexpr int NT = 64 * NWX * NWY * NSUB;    // threads per workgroup
+    constexpr int TW = 16 * NWX, TH = 4 * NWY;   // parents per workgroup
     constexpr int WW = TW + K - 1, WH = TH + K - 1;
-    constexpr int HALF = 24, STRIDE = 48;
-    constexpr int CH = 8;                  // channels per staged chunk
+    // LDS row: two channels side by side, each HALF >= WW + 1 floats wide
+    // (one padding column) with HALF = 8 mod 16, so the row stride is 16 mod 32
+    constexpr int HALF = ((WW + 1 - 8 + 15) / 16) * 16 + 8, STRIDE = 2 * HALF;
     constexpr int WIN = WH * WW;           // window positions per channel
     constexpr int NPOS = (WIN + NT - 1) / NT;  // positions staged by one thread
     constexpr int NSTAGE = CH * NPOS;
@@ -57,7 +96,8 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
     constexpr bool DO_QK = MODE != TILED_AV;
     constexpr bool DO_SOFTMAX = MODE == TILED_QK_SOFTMAX || MODE == TILED_FUSED;
     constexpr bool DO_AV = MODE == TILED_AV || MODE == TILED_FUSED;
-    static_assert(WW < HALF, "window row plus one padding column must fit half an LDS row");
+    static_assert(WW < HALF && STRIDE % 32 == 16, "LDS row layout");
+    static_assert(CH % 2 == 0, "channels are staged in pairs");
     static_assert(S % CY == 0, "CY must divide S");
     typedef Vec<T, S> VecS;
 
@@ -74,8 +114,8 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
-    const int lx = lane & 15, ly = (wave / NSUB) * 4 + (lane >> 4);
-    const int sub = wave % NSUB;
+    const int sub = wave % NSUB, wxy = wave / NSUB;
+    const int lx = (wxy % NWX) * 16 + (lane & 15), ly = (wxy / NWX) * 4 + (lane >> 4);
     const int x0 = tx * TW, y0 = ty * TH;          // tile origin (parents)
     const int px = x0 + lx, py = y0 + ly;
     const bool active = px < W && py < H;
@@ -175,14 +215,14 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
         const unsigned qmask = active ? 0xffffffffu : 0u;
         // q is fetched PF channels ahead of its use (a ring of PF x NJ
         // registers), so HBM latency hides behind the FMAs of PF channels.
-        constexpr int PF = 4;
+        constexpr int PF = CH < 4 ? CH : 4;
         static_assert(CH % PF == 0, "prefetch ring must divide the chunk");
         A qr[PF][NJ];
         auto load_q = [&](int c, A (&dst)[NJ]) {
 #pragma unroll
             for (int cy = 0; cy < CY; ++cy) {
                 const VecS v =
-                    *(const VecS *)(qp + (long)(c < d ? c : d - 1) * hplane + (long)cy * hW);
+                    load_stream<T, S>(qp + (long)(c < d ? c : d - 1) * hplane + (long)cy * hW);
 #pragma unroll
                 for (int cx = 0; cx < S; ++cx) dst[cy * S + cx] = (A)v.v[cx];
             }
@@ -271,7 +311,7 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
                             VecS v;
 #pragma unroll
                             for (int cx = 0; cx < S; ++cx) v.v[cx] = (T)o[cy * S + cx];
-                            *(VecS *)(op + (long)c * hplane + (long)cy * hW) = v;
+                            store_stream<T, S>(op + (long)c * hplane + (long)cy * hW, v);
                         }
                     }
                 }
@@ -283,11 +323,11 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
 }
 
 // ------------------------------------------------------------------ launcher
-template <typename T, int K, int S, int CY, int NWY>
+template <typename T, int K, int S, int CY, int NWX, int NWY, int CH>
 static hipError_t launch_mode(int mode, const void *q, const void *key, const void *attn_in,
                               const void *value, void *out, int B, int d, int C, int H, int W,
                               hipStream_t st) {
-    constexpr int TW = 16, TH = 4 * NWY, NT = 64 * NWY * (S / CY);
+    constexpr int TW = 16 * NWX, TH = 4 * NWY, NT = 64 * NWX * NWY * (S / CY);
     const int tiles_x = (W + TW - 1) / TW, tiles_y = (H + TH - 1) / TH;
     const long nb = (long)tiles_x * tiles_y * B;
     if (nb > (1L << 30)) return hipErrorNotSupported;
@@ -295,7 +335,7 @@ static hipError_t launch_mode(int mode, const void *q, const void *key, const vo
     const dim3 grid(per_xcd * 8), block(NT);
 #define SAPA_TM_CASE(M)                                                                       \
     case M:                                                                                   \
-        hipLaunchKernelGGL((sapa_b_tiled_kernel<T, K, S, CY, NWY, M>), grid, block, 0, st,    \
+        hipLaunchKernelGGL((sapa_b_tiled_kernel<T, K, S, CY, NWX, NWY, CH, M>), grid, block, 0, st,    \
                            (const T *)q, (const T *)key, (const T *)attn_in,                  \
                            (const T *)value, (T *)out, d, C, H, W, tiles_x, tiles_y, (int)nb, \
                            per_xcd);                                                          \
@@ -319,11 +359,23 @@ static hipError_t launch_t(int mode, const void *q, const void *key, const void 
     for (int i = 0; i < 3; ++i)
         if (hi_ptrs[i] && ((uintptr_t)hi_ptrs[i] % align) != 0) return hipErrorNotSupported;
     if (K == 5 && s == 2) {
-        // tall tiles amortise the halo; short ones leave fewer idle rows
-        const int waste4 = ((H + 15) / 16) * 16 - H, waste2 = ((H + 7) / 8) * 8 - H;
-        if (waste4 <= waste2)
-            return launch_mode<T, 5, 2, 2, 4>(mode, q, key, attn_in, value, out, B, d, C, H, W, st);
-        return launch_mode<T, 5, 2, 2, 2>(mode, q, key, attn_in, value, out, B, d, C, H, W, st);
+#ifdef SAPA_TUNE_GEOM
+        return launch_mode<T, 5, 2, 2, SAPA_TUNE_GEOM>(mode, q, key, attn_in, value, out, B, d, C, H, W, st);
+#else
+        // Tile geometry: padded parent count times the relative cost per
+        // parent measured at the FPN shapes on MI355X (wider tiles fetch
+        // fewer partial cache lines per window row, taller ones fewer halo
+        // rows; both idle more lanes on ragged extents).
+        auto padded = [&](int tw, int th) {
+            return (double)((W + tw - 1) / tw * tw) * (double)((H + th - 1) / th * th);
+        };
+        const double c12 = padded(16, 8), c14 = 0.96 * padded(16, 16), c22 = 0.88 * padded(32, 8);
+        if (c22 <= c12 && c22 <= c14)
+            return launch_mode<T, 5, 2, 2, 2, 2, 8>(mode, q, key, attn_in, value, out, B, d, C, H, W, st);
+        if (c14 <= c12)
+            return launch_mode<T, 5, 2, 2, 1, 4, 8>(mode, q, key, attn_in, value, out, B, d, C, H, W, st);
+        return launch_mode<T, 5, 2, 2, 1, 2, 8>(mode, q, key, attn_in, value, out, B, d, C, H, W, st);
+#endif
     }
     return hipErrorNotSupported;
 }
@@ -333,8 +385,10 @@ hipError_t sapa_b_tiled_launch(int mode, const void *q, const void *key, const v
                                int K, int s, int dtype, hipStream_t st) {
     switch (dtype) {
         case 0: return launch_t<float>(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, st);
+#ifndef SAPA_TUNE_GEOM
         case 2: return launch_t<f16_t>(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, st);
         case 3: return launch_t<bf16_t>(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, st);
+#endif
         default: return hipErrorNotSupported;
     }
 }

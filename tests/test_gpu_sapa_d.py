@@ -174,17 +174,21 @@ def test_backward_vs_oracle(coracle, shape):
 
 def test_gradcheck_reference_shapes():
     """deformsapa/deformsapa/grad_check.py:8-35: float64 gradcheck at its
-    shapes, offsets in [0,1) so no sample sits on a bilinear kink."""
+    shapes, offsets in [0,1) so no sample sits on a bilinear kink.  The
+    gradient of the sampled tensor is accumulated with atomics (as in the
+    reference, deform_qk_cuda_kernel.cu:105), so two runs may differ in the
+    last bits: nondet_tol allows for that."""
     from torch.autograd import gradcheck
     g = gen(207)
     b, h, w, c, P, s, G = 2, 3, 4, 16, 5, 2, 4
     r = lambda *sh: torch.rand(*sh, generator=g, dtype=torch.float64).to(DEV).requires_grad_()
     q, k, o = r(b, c, s * h, s * w), r(b, c, h, w), r(b, G * P * 2, s * h, s * w)
-    assert gradcheck(sapa_amd.deform_qk, (q, k, o, P, s, G))
+    assert gradcheck(sapa_amd.deform_qk, (q, k, o, P, s, G), nondet_tol=1e-10)
     a = randn(g, b, G, P, s * h, s * w, dtype=torch.float64).to(DEV).requires_grad_()
     v = randn(g, b, c, h, w, dtype=torch.float64).to(DEV).requires_grad_()
-    assert gradcheck(sapa_amd.deform_av, (a, v, o, P, s, G))
-    assert gradcheck(sapa_amd.deform_sapa_fused, (q, k, v, o, P, s, G), eps=1e-5, atol=1e-6)
+    assert gradcheck(sapa_amd.deform_av, (a, v, o, P, s, G), nondet_tol=1e-10)
+    assert gradcheck(sapa_amd.deform_sapa_fused, (q, k, v, o, P, s, G), eps=1e-5, atol=1e-6,
+                     nondet_tol=1e-10)
 
 
 def test_sapa_deform_module(coracle):
