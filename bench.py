@@ -37,7 +37,12 @@ WORKLOADS = {
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE + WRITE_SIZE,
 # scaled by what the same counters read for a plain copy of known size); see
 # the summaries under profiles/.  None = not measured for that case.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {
+    # profiles/sapa_b_fused_fpn_large_fp32.md: (332361.6 * 1.9999 + 1158510.8 * 1.0) KiB
+    ('fpn_large', 'fp32'): 1866974632,
+    # profiles/sapa_b_fused_fpn_large_bf16.md: (161706.3 * 1.9999 + 542299.6 * 1.0) KiB
+    ('fpn_large', 'bf16'): 886480921,
+}
 
 
 def algorithmic_bytes(B, C, d, H, W, s, esize):
