@@ -78,7 +78,7 @@ __global__ void __launch_bounds__(64 * NWX * NWY * (S / CY)) __attribute__((amdg
 sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
                     const T *__restrict__ attn_in, const T *__restrict__ value,
                     T *__restrict__ out, int d, int C, int H, int W, int tiles_x, int tiles_y,
-                    int nblocks, int per_xcd) {
+                    int nblocks, int per_xcd, int cgroups, int cper) {
     typedef float A;
     constexpr int KK = K * K, R = (K - 1) / 2;
     constexpr int NSUB = S / CY;           // waves sharing one band of parent rows
@@ -108,9 +108,16 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
     // rows) meet in the same L2.
     const int logical = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
     if (logical >= nblocks) return;
+    // logical = ((n * cgroups + cg) * tiles_y + ty) * tiles_x + tx; a small
+    // problem is split over `cgroups` slices of `cper` value channels each
+    // (every slice recomputes the logits) so that the chip is still filled
     const int tx = logical % tiles_x;
     const int ty = (logical / tiles_x) % tiles_y;
-    const int n = logical / (tiles_x * tiles_y);
+    const int cg = (logical / (tiles_x * tiles_y)) % cgroups;
+    const int n = logical / (tiles_x * tiles_y * cgroups);
+    const int cbeg = cg * cper;                      // first value channel of this slice
+    const int cend = cbeg + cper < C ? cbeg + cper : C;
+    if (DO_AV && cbeg >= C) return;                  // rounding left this slice empty
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -128,7 +135,7 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
         (long)((py < H ? py : H - 1) * S + sub * CY) * hW + (long)(px < W ? px : W - 1) * S;
 
     const int nKc = DO_QK ? (d + CH - 1) / CH : 0;
-    const int nVc = DO_AV ? (C + CH - 1) / CH : 0;
+    const int nVc = DO_AV ? (cend - cbeg + CH - 1) / CH : 0;
     const int ntot = nKc + nVc;
 
     // Staging map: thread t carries window positions t, t+NT, ... of every
@@ -157,7 +164,7 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
         const bool is_key = j < nKc;
         const T *src = is_key ? key : value;
         const int nch = is_key ? d : C;
-        const int c0 = (is_key ? j : j - nKc) * CH;
+        const int c0 = is_key ? j * CH : cbeg + (j - nKc) * CH;
         const T *base = src + (long)n * nch * lplane;
 #pragma unroll
         for (int ch = 0; ch < CH; ++ch) {
@@ -177,7 +184,7 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
     auto stage_store = [&](int j) {
         const bool is_key = j < nKc;
         const int nch = is_key ? d : C;
-        const int c0 = (is_key ? j : j - nKc) * CH;
+        const int c0 = is_key ? j * CH : cbeg + (j - nKc) * CH;
         A *dst = lds + (j & 1) * BUF;
 #pragma unroll
         for (int ch = 0; ch < CH; ++ch)
@@ -286,7 +293,7 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
         T *op = out + (long)n * C * hplane + hpix;
         for (int j = nKc; j < ntot; ++j) {
             if (j + 1 < ntot) stage_load(j + 1);
-            const int c0 = (j - nKc) * CH;
+            const int c0 = cbeg + (j - nKc) * CH;
             const A *wb = win + (j & 1) * BUF;
 #pragma unroll 1
             for (int ch = 0; ch < CH; ++ch) {
@@ -305,7 +312,7 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
                             for (int jj = 0; jj < NJ; ++jj)
                                 o[jj] = fma_(vv, a[jj][ky * K + kx], o[jj]);
                         }
-                    if (active && c < C) {
+                    if (active && c < cend) {
 #pragma unroll
                         for (int cy = 0; cy < CY; ++cy) {
                             VecS v;
@@ -329,7 +336,21 @@ static hipError_t launch_mode(int mode, const void *q, const void *key, const vo
                               hipStream_t st) {
     constexpr int TW = 16 * NWX, TH = 4 * NWY, NT = 64 * NWX * NWY * (S / CY);
     const int tiles_x = (W + TW - 1) / TW, tiles_y = (H + TH - 1) / TH;
-    const long nb = (long)tiles_x * tiles_y * B;
+    // Few tiles: slice the value channels over several workgroups per tile,
+    // up to two workgroups per CU (256 CUs) -- beyond that the recomputed
+    // logits cost more than the added parallelism gains (measured).  A slice
+    // is a multiple of CH channels and at least 4 chunks long.
+    int cgroups = 1;
+    if (mode == TILED_FUSED || mode == TILED_AV) {
+        const long tiles = (long)tiles_x * tiles_y * B;
+        const int max_groups = C / (4 * CH) > 0 ? C / (4 * CH) : 1;
+        while (cgroups * 2 <= max_groups && tiles * cgroups * 2 <= 512) cgroups *= 2;
+#ifdef SAPA_TUNE_CGROUPS
+        cgroups = SAPA_TUNE_CGROUPS;
+#endif
+    }
+    const int cper = ((C + cgroups - 1) / cgroups + CH - 1) / CH * CH;
+    const long nb = (long)tiles_x * tiles_y * B * cgroups;
     if (nb > (1L << 30)) return hipErrorNotSupported;
     const int per_xcd = (int)((nb + 7) / 8);
     const dim3 grid(per_xcd * 8), block(NT);
@@ -338,7 +359,7 @@ static hipError_t launch_mode(int mode, const void *q, const void *key, const vo
         hipLaunchKernelGGL((sapa_b_tiled_kernel<T, K, S, CY, NWX, NWY, CH, M>), grid, block, 0, st,    \
                            (const T *)q, (const T *)key, (const T *)attn_in,                  \
                            (const T *)value, (T *)out, d, C, H, W, tiles_x, tiles_y, (int)nb, \
-                           per_xcd);                                                          \
+                           per_xcd, cgroups, cper);                                                          \
         break;
     switch (mode) {
         SAPA_TM_CASE(TILED_QK) SAPA_TM_CASE(TILED_QK_SOFTMAX) SAPA_TM_CASE(TILED_AV)

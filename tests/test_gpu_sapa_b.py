@@ -265,3 +265,16 @@ def test_module_trains():
     for n, p in m.named_parameters():
         assert p.grad is not None and torch.isfinite(p.grad).all(), n
     assert x.grad is not None and x.grad.abs().sum() > 0
+
+
+@pytest.mark.parametrize('C', [32, 64, 100, 260])
+def test_fused_and_av_with_sliced_value_channels(coracle, C):
+    """Few tiles and many value channels: the launcher slices the channels
+    over several workgroups per tile (ragged last slice at C=100, 260)."""
+    B, d, H, W, K, s = 1, 8, 10, 20, 5, 2
+    g = gen(113)
+    q, key, v = randn(g, B, d, H * s, W * s), randn(g, B, d, H, W), randn(g, B, C, H, W)
+    attn = F.softmax(randn(g, B, K * K, H * s, W * s), 1)
+    got = sapa_amd.sapa_fused(*dev(q, key, v), K, s).cpu()
+    assert_f32_close(got, coracle.sapa_fused(q, key, v, K, s, 'f32'), f'fused C={C}')
+    assert torch.equal(sapa_amd.av(*dev(attn, v), K, s).cpu(), coracle.av(attn, v, K, s, 'f32'))
