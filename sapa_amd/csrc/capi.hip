@@ -27,6 +27,19 @@ bool dtype_ok(int dt) { return dt >= SAPA_F32 && dt <= SAPA_BF16; }
 // 64-bit flat indices and 32-bit in-plane indices cannot overflow
 const long long kMaxElems = 1LL << 40;
 
+// LDS-tiled SAPA-B kernel for `mode`: the VALU kernel where it has an
+// instance (K = 5, s = 2, where it is the faster one), else the matrix-pipe
+// kernel; hipErrorNotSupported when neither covers the request.
+hipError_t tiled_launch(int mode, const void *q, const void *key, const void *attn_in,
+                        const void *value, void *out, int B, int d, int C, int H, int W, int K,
+                        int s, int dtype, hipStream_t st) {
+    hipError_t e = sapa_b_tiled_launch(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s,
+                                       dtype, st);
+    if (e == hipErrorNotSupported)
+        e = sapa_b_mfma_launch(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, dtype, st);
+    return e;
+}
+
 int check_window_args(int B, int c1, int c2, int H, int W, int K, int s, int dtype) {
     if (!dtype_ok(dtype)) return SAPA_ERR_INVALID_ARGUMENT;
     if (B < 0 || c1 <= 0 || c2 <= 0 || H <= 0 || W <= 0 || s < 1 || K < 1 || (K - 1) % 2 != 0)
@@ -80,7 +93,7 @@ int sapa_qk_forward(const void *query, const void *key, void *out, int B, int d,
     if (B == 0) return SAPA_OK;
     if (!query || !key || !out) return SAPA_ERR_INVALID_ARGUMENT;
     hipStream_t st = (hipStream_t)stream;
-    hipError_t e = sapa_b_tiled_launch(TILED_QK, query, key, nullptr, nullptr, out, B, d, 0, H, W,
+    hipError_t e = tiled_launch(TILED_QK, query, key, nullptr, nullptr, out, B, d, 0, H, W,
                                        K, s, dtype, st);
     if (e == hipErrorNotSupported)
         e = qk_forward_generic_launch(query, key, out, B, d, H, W, K, s, dtype, st);
@@ -94,7 +107,7 @@ int sapa_av_forward(const void *attn, const void *value, void *out, int B, int C
     if (B == 0) return SAPA_OK;
     if (!attn || !value || !out) return SAPA_ERR_INVALID_ARGUMENT;
     hipStream_t st = (hipStream_t)stream;
-    hipError_t e = sapa_b_tiled_launch(TILED_AV, nullptr, nullptr, attn, value, out, B, 0, C, H, W,
+    hipError_t e = tiled_launch(TILED_AV, nullptr, nullptr, attn, value, out, B, 0, C, H, W,
                                        K, s, dtype, st);
     if (e == hipErrorNotSupported)
         e = av_forward_generic_launch(attn, value, out, B, C, H, W, K, s, dtype, st);
@@ -163,7 +176,7 @@ static int fused_common(int attn_only, const void *query, const void *key, const
     if (B == 0) return SAPA_OK;
     if (!query || !key || !out || (!attn_only && !value)) return SAPA_ERR_INVALID_ARGUMENT;
     hipStream_t st = (hipStream_t)stream;
-    hipError_t e = sapa_b_tiled_launch(attn_only ? TILED_QK_SOFTMAX : TILED_FUSED, query, key,
+    hipError_t e = tiled_launch(attn_only ? TILED_QK_SOFTMAX : TILED_FUSED, query, key,
                                        nullptr, value, out, B, d, attn_only ? 0 : C, H, W, K, s,
                                        dtype, st);
     if (e == hipErrorNotSupported)

@@ -28,6 +28,12 @@ hipError_t sapa_b_tiled_launch(int mode, const void *q, const void *key, const v
                                const void *value, void *out, int B, int d, int C, int H, int W,
                                int K, int s, int dtype, hipStream_t st);
 
+// sapa_b_mfma.hip: the same four modes on the matrix pipe (4x4x1 MFMA, one
+// block per parent); hipErrorNotSupported when (K, s, dtype) has no instance.
+hipError_t sapa_b_mfma_launch(int mode, const void *q, const void *key, const void *attn_in,
+                              const void *value, void *out, int B, int d, int C, int H, int W,
+                              int K, int s, int dtype, hipStream_t st);
+
 // sapa_d.hip
 hipError_t deform_qk_forward_launch(const void *q, const void *key, const void *offset, void *out,
                                     int B, int Cq, int H, int W, int P, int s, int G, int dtype,

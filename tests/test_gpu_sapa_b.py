@@ -23,6 +23,9 @@ SHAPES = [
     (1, 3, 2, 1, 1, 5, 2), (1, 9, 7, 17, 33, 5, 2), (3, 64, 16, 24, 40, 5, 2),
     (1, 4, 3, 5, 6, 3, 3), (1, 3, 2, 6, 7, 7, 1), (2, 5, 4, 4, 4, 1, 1),
     (1, 4, 6, 7, 5, 9, 2), (1, 2, 2, 3, 3, 11, 4), (1, 3, 3, 8, 8, 3, 2),
+    # the matrix-pipe kernel: K in {3,5,7} x s in {2,4} except K=5, s=2
+    (1, 5, 6, 9, 37, 7, 2), (2, 4, 5, 7, 18, 3, 4), (1, 6, 8, 6, 35, 5, 4), (1, 4, 9, 5, 17, 7, 4),
+    (2, 9, 13, 11, 34, 3, 2), (1, 64, 40, 16, 16, 7, 4),
 ]
 IDS = ['-'.join(map(str, s)) for s in SHAPES]
 
@@ -137,8 +140,8 @@ def test_fused_zero_query_box_filter():
 
 
 @pytest.mark.parametrize('dtype,rel', [(torch.bfloat16, BF16_REL), (torch.float16, F16_REL)])
-@pytest.mark.parametrize('shape', [SHAPES[0], SHAPES[5], SHAPES[6], SHAPES[9]],
-                         ids=[IDS[0], IDS[5], IDS[6], IDS[9]])
+@pytest.mark.parametrize('shape', [SHAPES[0], SHAPES[5], SHAPES[6], SHAPES[9], SHAPES[12], SHAPES[15]],
+                         ids=[IDS[0], IDS[5], IDS[6], IDS[9], IDS[12], IDS[15]])
 def test_16bit_dtypes(coracle, shape, dtype, rel):
     """Oracle = fp32-input, float64-accumulated math on the rounded inputs."""
     B, d, C, H, W, K, s = shape
