@@ -40,6 +40,26 @@ hipError_t tiled_launch(int mode, const void *q, const void *key, const void *at
     return e;
 }
 
+// The sampled forward ops: LDS-windowed kernel where it applies, else the
+// global-memory kernel.
+hipError_t deform_qk_any(const void *q, const void *key, const void *offset, void *out, int B,
+                         int Cq, int H, int W, int P, int s, int G, int dtype, hipStream_t st) {
+    hipError_t e = deform_lds_launch(0, q, key, nullptr, nullptr, offset, out, B, Cq, Cq, H, W, P,
+                                     s, G, dtype, st);
+    if (e == hipErrorNotSupported)
+        e = deform_qk_forward_launch(q, key, offset, out, B, Cq, H, W, P, s, G, dtype, st);
+    return e;
+}
+
+hipError_t deform_av_any(const void *attn, const void *value, const void *offset, void *out, int B,
+                         int C, int H, int W, int P, int s, int G, int dtype, hipStream_t st) {
+    hipError_t e = deform_lds_launch(1, nullptr, nullptr, attn, value, offset, out, B, C, C, H, W,
+                                     P, s, G, dtype, st);
+    if (e == hipErrorNotSupported)
+        e = deform_av_forward_launch(attn, value, offset, out, B, C, H, W, P, s, G, dtype, st);
+    return e;
+}
+
 int check_window_args(int B, int c1, int c2, int H, int W, int K, int s, int dtype) {
     if (!dtype_ok(dtype)) return SAPA_ERR_INVALID_ARGUMENT;
     if (B < 0 || c1 <= 0 || c2 <= 0 || H <= 0 || W <= 0 || s < 1 || K < 1 || (K - 1) % 2 != 0)
@@ -202,8 +222,8 @@ int sapa_deform_qk_forward(const void *query, const void *key, const void *offse
     if (rc != SAPA_OK) return rc;
     if (B == 0) return SAPA_OK;
     if (!query || !key || !offset || !out) return SAPA_ERR_INVALID_ARGUMENT;
-    return finish(deform_qk_forward_launch(query, key, offset, out, B, Cq, H, W, P, s, G, dtype,
-                                           (hipStream_t)stream));
+    return finish(deform_qk_any(query, key, offset, out, B, Cq, H, W, P, s, G, dtype,
+                                (hipStream_t)stream));
 }
 
 int sapa_deform_av_forward(const void *attn, const void *value, const void *offset, void *out,
@@ -213,8 +233,8 @@ int sapa_deform_av_forward(const void *attn, const void *value, const void *offs
     if (rc != SAPA_OK) return rc;
     if (B == 0) return SAPA_OK;
     if (!attn || !value || !offset || !out) return SAPA_ERR_INVALID_ARGUMENT;
-    return finish(deform_av_forward_launch(attn, value, offset, out, B, C, H, W, P, s, G, dtype,
-                                           (hipStream_t)stream));
+    return finish(deform_av_any(attn, value, offset, out, B, C, H, W, P, s, G, dtype,
+                                (hipStream_t)stream));
 }
 
 int sapa_deform_fused_forward(const void *query, const void *key, const void *value,
@@ -225,8 +245,12 @@ int sapa_deform_fused_forward(const void *query, const void *key, const void *va
     if (P > 64) return SAPA_ERR_UNSUPPORTED;
     if (B == 0) return SAPA_OK;
     if (!query || !key || !value || !offset || !out) return SAPA_ERR_INVALID_ARGUMENT;
-    return finish(deform_fused_forward_launch(query, key, value, offset, out, B, Cq, C, H, W, P, s,
-                                              G, dtype, (hipStream_t)stream));
+    hipError_t e = deform_lds_launch(2, query, key, nullptr, value, offset, out, B, Cq, C, H, W, P,
+                                     s, G, dtype, (hipStream_t)stream);
+    if (e == hipErrorNotSupported)
+        e = deform_fused_forward_launch(query, key, value, offset, out, B, Cq, C, H, W, P, s, G,
+                                        dtype, (hipStream_t)stream);
+    return finish(e);
 }
 
 int sapa_deform_qk_backward(const void *grad_out, const void *query, const void *key,
@@ -242,8 +266,8 @@ int sapa_deform_qk_backward(const void *grad_out, const void *query, const void 
     // grad_query[b,g*d+c] = sum_p grad_out[b,g,p] * bilinear(key[b,g*d+c]): the
     // sampled aggregation with key in the value's place.
     if (grad_query) {
-        const hipError_t e = deform_av_forward_launch(grad_out, key, offset, grad_query, B, Cq, H,
-                                                      W, P, s, G, dtype, st);
+        const hipError_t e =
+            deform_av_any(grad_out, key, offset, grad_query, B, Cq, H, W, P, s, G, dtype, st);
         if (e != hipSuccess) return fail_hip(e);
     }
     if (grad_key || grad_offset) {
@@ -267,8 +291,8 @@ int sapa_deform_av_backward(const void *grad_out, const void *attn, const void *
     // grad_attn[b,g,p] = sum_{c in g} grad_out[b,c] * bilinear(value[b,c]): the
     // sampled similarity with grad_out as the query and value as the key.
     if (grad_attn) {
-        const hipError_t e = deform_qk_forward_launch(grad_out, value, offset, grad_attn, B, C, H,
-                                                      W, P, s, G, dtype, st);
+        const hipError_t e =
+            deform_qk_any(grad_out, value, offset, grad_attn, B, C, H, W, P, s, G, dtype, st);
         if (e != hipSuccess) return fail_hip(e);
     }
     if (grad_value || grad_offset) {

@@ -34,6 +34,14 @@ hipError_t sapa_b_mfma_launch(int mode, const void *q, const void *key, const vo
                               const void *value, void *out, int B, int d, int C, int H, int W,
                               int K, int s, int dtype, hipStream_t st);
 
+// sapa_d_lds.hip: the SAPA-D forward ops gathering from an LDS-resident
+// window; mode 0 = deform_qk (out = logits), 1 = deform_av (attn_in given),
+// 2 = fused.  hipErrorNotSupported when (s, dtype, P) has no instance / does
+// not fit LDS; the caller then takes the global-memory kernels below.
+hipError_t deform_lds_launch(int mode, const void *q, const void *key, const void *attn_in,
+                             const void *value, const void *offset, void *out, int B, int Cq, int C,
+                             int H, int W, int P, int s, int G, int dtype, hipStream_t st);
+
 // sapa_d.hip
 hipError_t deform_qk_forward_launch(const void *q, const void *key, const void *offset, void *out,
                                     int B, int Cq, int H, int W, int P, int s, int G, int dtype,

@@ -6,6 +6,7 @@
 // Coordinates, floor and weights are evaluated in the tensor's arithmetic
 // type (fp32 for 16-bit tensors), so the corner indices are the reference's.
 #include "kernels.hpp"
+#include "deform_tap.hpp"
 
 namespace sapa {
 
@@ -13,56 +14,6 @@ static inline int grid_for(long total, int block) {
     long g = (total + block - 1) / block;
     const long cap = 256L * 64;
     return (int)(g < cap ? (g > 0 ? g : 1) : cap);
-}
-
-// One bilinear sample position: four weights, four plane offsets, four
-// per-corner validity flags (deform_qk_cuda_kernel.cu:30-64).
-template <typename A>
-struct Tap {
-    A w1, w2, w3, w4;
-    A lh, lw, hh, hw;
-    int i1, i2, i3, i4;
-    bool m1, m2, m3, m4;
-};
-
-// False when the position fails the guard kh > -1 && kh < H && kw > -1 &&
-// kw < W (deform_qk_cuda_kernel.cu:187): the sample then contributes nothing.
-template <typename A>
-__device__ __forceinline__ bool tap_setup(A kh, A kw, int H, int W, Tap<A> &t) {
-    if (!(kh > (A)-1 && kh < (A)H && kw > (A)-1 && kw < (A)W)) return false;
-    const int h_low = (int)floor_(kh), w_low = (int)floor_(kw);
-    const int h_high = h_low + 1, w_high = w_low + 1;
-    t.lh = kh - (A)h_low;
-    t.lw = kw - (A)w_low;
-    t.hh = (A)1 - t.lh;
-    t.hw = (A)1 - t.lw;
-    t.m1 = h_low >= 0 && w_low >= 0;
-    t.m2 = h_low >= 0 && w_high <= W - 1;
-    t.m3 = h_high <= H - 1 && w_low >= 0;
-    t.m4 = h_high <= H - 1 && w_high <= W - 1;
-    t.i1 = t.m1 ? h_low * W + w_low : 0;
-    t.i2 = t.m2 ? h_low * W + w_high : 0;
-    t.i3 = t.m3 ? h_high * W + w_low : 0;
-    t.i4 = t.m4 ? h_high * W + w_high : 0;
-    t.w1 = t.hh * t.hw;
-    t.w2 = t.hh * t.lw;
-    t.w3 = t.lh * t.hw;
-    t.w4 = t.lh * t.lw;
-    return true;
-}
-
-// w1*v1 + w2*v2 + w3*v3 + w4*v4, evaluated left to right with FMAs.
-template <typename T, typename A>
-__device__ __forceinline__ A tap_sample(const T *plane, const Tap<A> &t) {
-    const A v1 = t.m1 ? ld(plane + t.i1) : (A)0;
-    const A v2 = t.m2 ? ld(plane + t.i2) : (A)0;
-    const A v3 = t.m3 ? ld(plane + t.i3) : (A)0;
-    const A v4 = t.m4 ? ld(plane + t.i4) : (A)0;
-    A val = t.w1 * v1;
-    val = fma_(t.w2, v2, val);
-    val = fma_(t.w3, v3, val);
-    val = fma_(t.w4, v4, val);
-    return val;
 }
 
 // out[b,g,p,qh,qw] = sum_{c<d} q[b,g*d+c,qh,qw] * bilinear(key[b,g*d+c])

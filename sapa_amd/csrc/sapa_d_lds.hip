@@ -1,0 +1,251 @@
+// SAPA-D kernels that gather from an LDS-resident window instead of global
+// memory: deform_qk, deform_av and the fused deform_qk -> softmax -> deform_av.
+//
+// A workgroup owns a TPW x TPH tile of low-res parent cells of one (image,
+// group) pair; a thread owns one high-res query pixel of it.  The sampled
+// tensor's window -- the tile plus HR = 4 cells on every side, one more on the
+// high side for the +1 bilinear corners -- is staged in LDS CH channels at a
+// time, zero-filled outside the image, so a sample whose floor() corner lies
+// in the window reads its four corners from LDS and needs no border masks
+// (a zero there is exactly the reference's per-corner zero padding,
+// deformsapa/deformsapa/src/cuda/deform_qk_cuda_kernel.cu:39-62).  A sample
+// that leaves the window -- offsets beyond +-4 cells -- takes the same taps
+// from global memory, so any offset is handled.  The P logits / weights of a
+// pixel live in LDS as well ([P][thread], conflict-free), which keeps the
+// loop over sample points a run-time loop: any P, no register arrays.
+//
+// Arithmetic is the reference kernels' own (fp32 for 16-bit tensors):
+// coordinates parent + offset, floor, strict guard, weights hh*hw.., the
+// value w1*v1 + w2*v2 + w3*v3 + w4*v4 left to right, one FMA per channel in
+// channel order for a logit (deform_qk_cuda_kernel.cu:180-193), one FMA per
+// sample point in point order for an output (deform_av_cuda_kernel.cu:178-192).
+#include "deform_tap.hpp"
+#include "kernels.hpp"
+
+namespace sapa {
+
+enum DeformMode { DEFORM_QK = 0, DEFORM_AV = 1, DEFORM_FUSED = 2 };
+
+template <typename T, int S, int TPW, int TPH, int CH, int MODE>
+__global__ void __launch_bounds__(TPW *TPH *S *S)
+deform_lds_kernel(const T *__restrict__ q, const T *__restrict__ key,
+                  const T *__restrict__ attn_in, const T *__restrict__ value,
+                  const T *__restrict__ offset, T *__restrict__ out, int Cq, int C, int H, int W,
+                  int P, int G, int tiles_x, int tiles_y, int nblocks, int per_xcd) {
+    typedef float A;
+    constexpr int HR = 4;                           // window reach in low-res cells
+    constexpr int NT = TPW * TPH * S * S;
+    constexpr int WW = TPW + 2 * HR + 1, WH = TPH + 2 * HR + 1;
+    constexpr int RS = WW | 1;                      // odd row stride
+    constexpr int CS = WH * RS;
+    constexpr int WIN = WH * WW;
+    constexpr int TXP = TPW * S;                    // tile width in pixels
+    constexpr bool DO_QK = MODE != DEFORM_AV, DO_AV = MODE != DEFORM_QK;
+
+    extern __shared__ float smem[];
+    A *win = smem;                                  // [CH][WH][RS]
+    A *lg = smem + CH * CS;                         // [P][NT]
+
+    const int logical = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
+    if (logical >= nblocks) return;
+    const int tx = logical % tiles_x;
+    const int ty = (logical / tiles_x) % tiles_y;
+    const int g = (logical / (tiles_x * tiles_y)) % G;
+    const int b = logical / (tiles_x * tiles_y * G);
+
+    const int tid = threadIdx.x;
+    const int hH = H * S, hW = W * S, GP = G * P, d = Cq / G, cg = C / G;
+    const long lplane = (long)H * W, hplane = (long)hH * hW;
+    const int qw = tx * TXP + tid % TXP, qh = ty * TPH * S + tid / TXP;
+    const bool active = qw < hW && qh < hH;
+    // idle threads of a partial tile read through clamped coordinates
+    const long pix = (long)(qh < hH ? qh : hH - 1) * hW + (qw < hW ? qw : hW - 1);
+    const A ph = (A)((qh < hH ? qh : hH - 1) / S), pw = (A)((qw < hW ? qw : hW - 1) / S);
+    const int wx0 = tx * TPW - HR, wy0 = ty * TPH - HR;
+    const T *op = offset + ((((long)b * GP + (long)g * P)) << 1) * hplane + pix;
+    A *lgt = lg + tid;
+
+    // window of `nvalid` channels starting at plane `src` -> LDS, zero-filled
+    // outside the image and past the last channel
+    auto stage = [&](const T *src, int nvalid) {
+        for (int idx = tid; idx < CH * WIN; idx += NT) {
+            const int ch = idx / WIN, pos = idx % WIN;
+            const int row = pos / WW, col = pos % WW;
+            const int gy = wy0 + row, gx = wx0 + col;
+            A v = 0;
+            if (ch < nvalid && gy >= 0 && gy < H && gx >= 0 && gx < W)
+                v = (A)src[(long)ch * lplane + (long)gy * W + gx];
+            win[ch * CS + row * RS + col] = v;
+        }
+    };
+
+    // `fn(wp)` with wp = LDS address of the tap's low corner if the tap is
+    // inside the window; otherwise `fg()` (global-memory taps)
+    if (DO_QK) {
+        const long ch0 = (long)b * Cq + (long)g * d;
+        for (int c0 = 0; c0 < d; c0 += CH) {
+            const int nvalid = d - c0 < CH ? d - c0 : CH;
+            A qv[CH];
+#pragma unroll
+            for (int ch = 0; ch < CH; ++ch)
+                qv[ch] = (active && ch < nvalid) ? (A)q[(ch0 + c0 + ch) * hplane + pix] : (A)0;
+            __syncthreads();                       // the previous chunk's readers are done
+            stage(key + (ch0 + c0) * lplane, nvalid);
+            __syncthreads();
+            for (int p = 0; p < P; ++p) {
+                const A kw = pw + (A)op[(long)(2 * p) * hplane];
+                const A kh = ph + (A)op[(long)(2 * p + 1) * hplane];
+                A acc = c0 == 0 ? (A)0 : lgt[p * NT];
+                Tap<A> tap;
+                if (tap_setup(kh, kw, H, W, tap)) {
+                    const int hl = (int)floor_(kh) - wy0, wl = (int)floor_(kw) - wx0;
+                    if (hl >= 0 && hl <= WH - 2 && wl >= 0 && wl <= WW - 2) {
+                        const A *wp = win + hl * RS + wl;
+#pragma unroll
+                        for (int ch = 0; ch < CH; ++ch) {
+                            A val = tap.w1 * wp[ch * CS];
+                            val = fma_(tap.w2, wp[ch * CS + 1], val);
+                            val = fma_(tap.w3, wp[ch * CS + RS], val);
+                            val = fma_(tap.w4, wp[ch * CS + RS + 1], val);
+                            acc = fma_(val, qv[ch], acc);
+                        }
+                    } else {
+                        const T *kp = key + (ch0 + c0) * lplane;
+                        for (int ch = 0; ch < nvalid; ++ch)
+                            acc = fma_(tap_sample(kp + (long)ch * lplane, tap), qv[ch], acc);
+                    }
+                }
+                lgt[p * NT] = acc;
+            }
+        }
+        if (MODE == DEFORM_FUSED) {
+            // softmax over the P points of this pixel (guard failures keep
+            // logit 0 and take part, as in softmax(deform_qk(...), dim=2))
+            A m = lgt[0];
+            for (int p = 1; p < P; ++p) m = max_(m, lgt[p * NT]);
+            A sum = 0;
+            for (int p = 0; p < P; ++p) {
+                const A e = exp_(lgt[p * NT] - m);
+                lgt[p * NT] = e;
+                sum += e;
+            }
+            const A inv = (A)1 / sum;
+            for (int p = 0; p < P; ++p) lgt[p * NT] *= inv;
+        } else if (active) {
+            T *o = out + ((long)b * GP + (long)g * P) * hplane + pix;
+            for (int p = 0; p < P; ++p) o[(long)p * hplane] = (T)lgt[p * NT];
+        }
+    } else {
+        const T *ap = attn_in + ((long)b * GP + (long)g * P) * hplane + pix;
+        for (int p = 0; p < P; ++p) lgt[p * NT] = (A)ap[(long)p * hplane];
+    }
+
+    if (DO_AV) {
+        const long ch0 = (long)b * C + (long)g * cg;
+        for (int c0 = 0; c0 < cg; c0 += CH) {
+            const int nvalid = cg - c0 < CH ? cg - c0 : CH;
+            __syncthreads();
+            stage(value + (ch0 + c0) * lplane, nvalid);
+            __syncthreads();
+            A o[CH];
+#pragma unroll
+            for (int ch = 0; ch < CH; ++ch) o[ch] = 0;
+            for (int p = 0; p < P; ++p) {
+                const A kw = pw + (A)op[(long)(2 * p) * hplane];
+                const A kh = ph + (A)op[(long)(2 * p + 1) * hplane];
+                const A wa = lgt[p * NT];
+                Tap<A> tap;
+                if (tap_setup(kh, kw, H, W, tap)) {
+                    const int hl = (int)floor_(kh) - wy0, wl = (int)floor_(kw) - wx0;
+                    if (hl >= 0 && hl <= WH - 2 && wl >= 0 && wl <= WW - 2) {
+                        const A *wp = win + hl * RS + wl;
+#pragma unroll
+                        for (int ch = 0; ch < CH; ++ch) {
+                            A val = tap.w1 * wp[ch * CS];
+                            val = fma_(tap.w2, wp[ch * CS + 1], val);
+                            val = fma_(tap.w3, wp[ch * CS + RS], val);
+                            val = fma_(tap.w4, wp[ch * CS + RS + 1], val);
+                            o[ch] = fma_(val, wa, o[ch]);
+                        }
+                    } else {
+                        const T *vp = value + (ch0 + c0) * lplane;
+#pragma unroll
+                        for (int ch = 0; ch < CH; ++ch)
+                            if (ch < nvalid)
+                                o[ch] = fma_(tap_sample(vp + (long)ch * lplane, tap), wa, o[ch]);
+                    }
+                }
+            }
+            if (active) {
+                T *dst = out + (ch0 + c0) * hplane + pix;
+#pragma unroll
+                for (int ch = 0; ch < CH; ++ch)
+                    if (ch < nvalid) dst[(long)ch * hplane] = (T)o[ch];
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------ launcher
+template <typename T, int S, int TPW, int TPH, int CH>
+static hipError_t launch_geom(int mode, const void *q, const void *key, const void *attn_in,
+                              const void *value, const void *offset, void *out, int B, int Cq,
+                              int C, int H, int W, int P, int G, hipStream_t st) {
+    constexpr int HR = 4, NT = TPW * TPH * S * S;
+    constexpr int WW = TPW + 2 * HR + 1, WH = TPH + 2 * HR + 1, RS = WW | 1, CS = WH * RS;
+    const size_t smem = ((size_t)CH * CS + (size_t)P * NT) * sizeof(float);
+    if (smem > 64 * 1024) return hipErrorNotSupported;   // the default dynamic-LDS limit
+    const int tiles_x = (W + TPW - 1) / TPW, tiles_y = (H + TPH - 1) / TPH;
+    const long nb = (long)tiles_x * tiles_y * G * B;
+    if (nb > (1L << 30)) return hipErrorNotSupported;
+    const int per_xcd = (int)((nb + 7) / 8);
+    const dim3 grid(per_xcd * 8), block(NT);
+#define SAPA_DL_CASE(M)                                                                       \
+    case M:                                                                                   \
+        hipLaunchKernelGGL((deform_lds_kernel<T, S, TPW, TPH, CH, M>), grid, block, smem, st, \
+                           (const T *)q, (const T *)key, (const T *)attn_in,                  \
+                           (const T *)value, (const T *)offset, (T *)out, Cq, C, H, W, P, G,  \
+                           tiles_x, tiles_y, (int)nb, per_xcd);                               \
+        break;
+    switch (mode) {
+        SAPA_DL_CASE(DEFORM_QK) SAPA_DL_CASE(DEFORM_AV) SAPA_DL_CASE(DEFORM_FUSED)
+        default: return hipErrorInvalidValue;
+    }
+#undef SAPA_DL_CASE
+    return hipGetLastError();
+}
+
+template <typename T>
+static hipError_t launch_t(int mode, const void *q, const void *key, const void *attn_in,
+                           const void *value, const void *offset, void *out, int B, int Cq, int C,
+                           int H, int W, int P, int s, int G, hipStream_t st) {
+#ifdef SAPA_DLDS_TUNE
+    if (s == 2) return launch_geom<T, 2, SAPA_DLDS_TUNE>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, G, st);
+    return hipErrorNotSupported;
+#else
+    switch (s) {
+        case 1: return launch_geom<T, 1, 16, 16, 8>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, G, st);
+        case 2: return launch_geom<T, 2, 8, 8, 16>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, G, st);
+        case 4: return launch_geom<T, 4, 4, 4, 16>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, G, st);
+        default: return hipErrorNotSupported;
+    }
+#endif
+}
+
+// mode: 0 = deform_qk (out = logits), 1 = deform_av (attn_in given),
+// 2 = fused.  hipErrorNotSupported: no instance for (s, dtype) or P too large
+// for the LDS budget; the caller then takes the global-memory kernels.
+hipError_t deform_lds_launch(int mode, const void *q, const void *key, const void *attn_in,
+                             const void *value, const void *offset, void *out, int B, int Cq, int C,
+                             int H, int W, int P, int s, int G, int dtype, hipStream_t st) {
+    switch (dtype) {
+        case 0: return launch_t<float>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, s, G, st);
+#ifndef SAPA_DLDS_TUNE
+        case 2: return launch_t<f16_t>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, s, G, st);
+        case 3: return launch_t<bf16_t>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, s, G, st);
+#endif
+        default: return hipErrorNotSupported;
+    }
+}
+
+}  // namespace sapa
