@@ -73,7 +73,7 @@ __device__ __forceinline__ void store_stream(T *p, const Vec<T, N> &v) {
     __builtin_nontemporal_store(u.b, (B *)p);
 }
 
-template <typename T, int K, int S, int CY, int NWX, int NWY, int CH, int MODE>
+template <typename T, int K, int S, int CY, int NWX, int NWY, int CH, int VEC, int MODE>
 __global__ void __launch_bounds__(64 * NWX * NWY * (S / CY)) __attribute__((amdgpu_waves_per_eu(3, 3)))
 sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
                     const T *__restrict__ attn_in, const T *__restrict__ value,
@@ -84,24 +84,36 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
     constexpr int NSUB = S / CY;           // waves sharing one band of parent rows
     constexpr int NT = 64 * NWX * NWY * NSUB;    // threads per workgroup
     constexpr int TW = 16 * NWX, TH = 4 * NWY;   // parents per workgroup
-    constexpr int WW = TW + K - 1, WH = TH + K - 1;
-    // LDS row: two channels side by side, each HALF >= WW + 1 floats wide
-    // (one padding column) with HALF = 8 mod 16, so the row stride is 16 mod 32
-    constexpr int HALF = ((WW + 1 - 8 + 15) / 16) * 16 + 8, STRIDE = 2 * HALF;
-    constexpr int WIN = WH * WW;           // window positions per channel
-    constexpr int NPOS = (WIN + NT - 1) / NT;  // positions staged by one thread
-    constexpr int NSTAGE = CH * NPOS;
+    // The window is staged as VEC-wide vectors (VEC = 1, 2 or 4 elements):
+    // its left edge is moved out to a multiple of VEC and its width rounded up.
+    constexpr int HL = (R + VEC - 1) / VEC * VEC;                 // left halo, staged
+    constexpr int WW = (HL + TW + R + VEC - 1) / VEC * VEC;       // staged window width
+    constexpr int WH = TH + K - 1;
+    // LDS row: two channels side by side, each HALF > WW floats wide (spare
+    // columns absorb surplus staging lanes) with HALF = 8 mod 16, so the row
+    // stride is 16 mod 32
+    constexpr int HALF = ((WW + VEC - 8 + 15) / 16) * 16 + 8, STRIDE = 2 * HALF;
+    constexpr int NVR = WW / VEC, NVP = WH * NVR;   // vectors per row / per channel
+    // staging threads are split into NSL slices that take every NSL-th channel
+    constexpr int NSL = (CH % 4 == 0 && NT >= 4 * NVP && NT % 256 == 0) ? 4
+                        : (NT >= 2 * NVP && NT % 128 == 0) ? 2 : 1;
+    constexpr int TPC = NT / NSL;                   // threads per slice (whole waves)
+    constexpr int NPOS = (NVP + TPC - 1) / TPC;     // vectors per thread and channel
+    constexpr int CPT = CH / NSL;                   // channels per thread
+    constexpr int NSTAGE = CPT * NPOS * VEC;
     constexpr int BUF = (CH / 2) * WH * STRIDE;
     constexpr int NJ = CY * S;             // children per thread
     constexpr bool DO_QK = MODE != TILED_AV;
     constexpr bool DO_SOFTMAX = MODE == TILED_QK_SOFTMAX || MODE == TILED_FUSED;
     constexpr bool DO_AV = MODE == TILED_AV || MODE == TILED_FUSED;
-    static_assert(WW < HALF && STRIDE % 32 == 16, "LDS row layout");
+    static_assert(WW + VEC <= HALF && STRIDE % 32 == 16, "LDS row layout");
+    static_assert(TPC % 64 == 0 && CH % NSL == 0, "staging slices are whole waves");
+    typedef Vec<T, VEC> VecV;
     static_assert(CH % 2 == 0, "channels are staged in pairs");
     static_assert(S % CY == 0, "CY must divide S");
     typedef Vec<T, S> VecS;
 
-    __shared__ A lds[2 * BUF];
+    __shared__ __attribute__((aligned(16))) A lds[2 * BUF];
 
     // Workgroups are handed to the 8 XCDs round-robin; give each XCD a
     // contiguous run of tiles so that neighbouring tiles (which share halo
@@ -138,24 +150,26 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
     const int nVc = DO_AV ? (cend - cbeg + CH - 1) / CH : 0;
     const int ntot = nKc + nVc;
 
-    // Staging map: thread t carries window positions t, t+NT, ... of every
-    // channel of a chunk, so the per-thread part of each address (in-plane
-    // offset, LDS offset, inside-the-image flag) is fixed for the whole
-    // kernel and the per-channel part is wave-uniform.
+    // Staging map: thread t of slice sl carries vectors t, t+TPC, ... of the
+    // window of channels sl, sl+NSL, ... of a chunk, so the per-thread part
+    // of each address (in-plane offset, LDS offset, inside-the-image mask) is
+    // fixed for the whole kernel and the channel part is wave-uniform.
+    const int sl = tid / TPC, vt = tid % TPC;
     int g_off[NPOS], l_off[NPOS];
     unsigned g_mask[NPOS];
 #pragma unroll
     for (int i = 0; i < NPOS; ++i) {
-        const int pos = tid + i * NT;
-        const int row = pos / WW, col = pos % WW;
-        const int gy = y0 - R + row, gx = x0 - R + col;
-        const bool l_ok = WIN % NT == 0 || pos < WIN;
-        const bool g_ok = l_ok && gy >= 0 && gy < H && gx >= 0 && gx < W;
+        const int v = vt + i * TPC;
+        const int row = v / NVR, col = (v % NVR) * VEC;
+        const int gy = y0 - R + row, gx = x0 - HL + col;
+        const bool l_ok = NVP % TPC == 0 || v < NVP;
+        // W is a multiple of VEC and gx too: a vector is all inside or all outside
+        const bool g_ok = l_ok && gy >= 0 && gy < H && gx >= 0 && gx + VEC <= W;
         const int yy = gy < 0 ? 0 : (gy < H ? gy : H - 1);
-        const int xx = gx < 0 ? 0 : (gx < W ? gx : W - 1);
+        const int xx = gx < 0 ? 0 : (gx + VEC <= W ? gx : W - VEC);
         g_off[i] = yy * W + xx;             // clamped: always a legal address
         g_mask[i] = g_ok ? 0xffffffffu : 0u;
-        // surplus positions land in the unread padding column of row 0
+        // surplus vectors land in the unread spare columns of row 0
         l_off[i] = l_ok ? row * STRIDE + col : WW;
     }
     A st[NSTAGE];
@@ -167,15 +181,17 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
         const int c0 = is_key ? j * CH : cbeg + (j - nKc) * CH;
         const T *base = src + (long)n * nch * lplane;
 #pragma unroll
-        for (int ch = 0; ch < CH; ++ch) {
-            const int c = c0 + ch;
+        for (int ci = 0; ci < CPT; ++ci) {
+            const int c = c0 + sl + ci * NSL;
             const T *plane = base + (long)(c < nch ? c : nch - 1) * lplane;
 #pragma unroll
             for (int i = 0; i < NPOS; ++i) {
                 // unconditional load from the clamped address; the value is
                 // masked when it is stored to LDS, so that the load stays in
                 // flight across the FMAs of the current chunk
-                st[ch * NPOS + i] = (A)plane[g_off[i]];
+                const VecV v = *(const VecV *)(plane + g_off[i]);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) st[(ci * NPOS + i) * VEC + e] = (A)v.v[e];
             }
         }
     };
@@ -187,11 +203,19 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
         const int c0 = is_key ? j * CH : cbeg + (j - nKc) * CH;
         A *dst = lds + (j & 1) * BUF;
 #pragma unroll
-        for (int ch = 0; ch < CH; ++ch)
+        for (int ci = 0; ci < CPT; ++ci) {
+            const int ch = sl + ci * NSL;
+            A *dc = dst + (ch >> 1) * WH * STRIDE + (ch & 1) * HALF;
 #pragma unroll
-            for (int i = 0; i < NPOS; ++i)
-                dst[(ch >> 1) * WH * STRIDE + (ch & 1) * HALF + l_off[i]] = __uint_as_float(
-                    __float_as_uint(st[ch * NPOS + i]) & (c0 + ch < nch ? g_mask[i] : 0u));
+            for (int i = 0; i < NPOS; ++i) {
+                const unsigned m = c0 + ch < nch ? g_mask[i] : 0u;
+                Vec<A, VEC> o;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e)
+                    o.v[e] = __uint_as_float(__float_as_uint(st[(ci * NPOS + i) * VEC + e]) & m);
+                *(Vec<A, VEC> *)(dc + l_off[i]) = o;
+            }
+        }
     };
 
     A a[NJ][KK];
@@ -215,7 +239,8 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
     stage_store(0);
     __syncthreads();
 
-    const A *win = lds + ly * STRIDE + lx;  // this thread's window origin in buffer 0
+    // this thread's window origin in buffer 0 (its neighbour kx = 0 column)
+    const A *win = lds + ly * STRIDE + lx + (HL - R);
 
     if (DO_QK) {
         const T *qp = q + (long)n * d * hplane + hpix_ld;
@@ -330,7 +355,7 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
 }
 
 // ------------------------------------------------------------------ launcher
-template <typename T, int K, int S, int CY, int NWX, int NWY, int CH>
+template <typename T, int K, int S, int CY, int NWX, int NWY, int CH, int VEC>
 static hipError_t launch_mode(int mode, const void *q, const void *key, const void *attn_in,
                               const void *value, void *out, int B, int d, int C, int H, int W,
                               hipStream_t st) {
@@ -356,7 +381,7 @@ static hipError_t launch_mode(int mode, const void *q, const void *key, const vo
     const dim3 grid(per_xcd * 8), block(NT);
 #define SAPA_TM_CASE(M)                                                                       \
     case M:                                                                                   \
-        hipLaunchKernelGGL((sapa_b_tiled_kernel<T, K, S, CY, NWX, NWY, CH, M>), grid, block, 0, st,    \
+        hipLaunchKernelGGL((sapa_b_tiled_kernel<T, K, S, CY, NWX, NWY, CH, VEC, M>), grid, block, 0, st,    \
                            (const T *)q, (const T *)key, (const T *)attn_in,                  \
                            (const T *)value, (T *)out, d, C, H, W, tiles_x, tiles_y, (int)nb, \
                            per_xcd, cgroups, cper);                                                          \
@@ -391,11 +416,19 @@ static hipError_t launch_t(int mode, const void *q, const void *key, const void 
             return (double)((W + tw - 1) / tw * tw) * (double)((H + th - 1) / th * th);
         };
         const double c12 = padded(16, 8), c14 = 0.96 * padded(16, 16), c22 = 0.88 * padded(32, 8);
-        if (c22 <= c12 && c22 <= c14)
-            return launch_mode<T, 5, 2, 2, 2, 2, 8>(mode, q, key, attn_in, value, out, B, d, C, H, W, st);
-        if (c14 <= c12)
-            return launch_mode<T, 5, 2, 2, 1, 4, 8>(mode, q, key, attn_in, value, out, B, d, C, H, W, st);
-        return launch_mode<T, 5, 2, 2, 1, 2, 8>(mode, q, key, attn_in, value, out, B, d, C, H, W, st);
+        // The low-res windows are staged with 4- or 2-element vector loads
+        // when rows and base pointers allow it (scalar loads otherwise).
+        auto aligned = [&](int vec) {
+            const uintptr_t a = (uintptr_t)(sizeof(T) * vec);
+            return W % vec == 0 && (!key || (uintptr_t)key % a == 0) &&
+                   (!value || (uintptr_t)value % a == 0);
+        };
+#define SAPA_GEOM(NWX, NWY, VEC) \
+    launch_mode<T, 5, 2, 2, NWX, NWY, 8, VEC>(mode, q, key, attn_in, value, out, B, d, C, H, W, st)
+        if (c22 <= c12 && c22 <= c14) return aligned(4) ? SAPA_GEOM(2, 2, 4) : SAPA_GEOM(2, 2, 1);
+        if (c14 <= c12) return aligned(2) ? SAPA_GEOM(1, 4, 2) : SAPA_GEOM(1, 4, 1);
+        return aligned(2) ? SAPA_GEOM(1, 2, 2) : SAPA_GEOM(1, 2, 1);
+#undef SAPA_GEOM
 #endif
     }
     return hipErrorNotSupported;

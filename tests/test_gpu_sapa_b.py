@@ -281,3 +281,24 @@ def test_fused_and_av_with_sliced_value_channels(coracle, C):
     got = sapa_amd.sapa_fused(*dev(q, key, v), K, s).cpu()
     assert_f32_close(got, coracle.sapa_fused(q, key, v, K, s, 'f32'), f'fused C={C}')
     assert torch.equal(sapa_amd.av(*dev(attn, v), K, s).cpu(), coracle.av(attn, v, K, s, 'f32'))
+
+
+@pytest.mark.parametrize('W', [20, 22, 21, 36, 34, 33])
+def test_window_staging_vector_widths(coracle, W):
+    """Row lengths that are multiples of 4, of 2 only, and odd select the
+    4-, 2- and 1-element staging loads of the tiled kernel; a sliced view
+    shifts the base pointer off 16-byte alignment."""
+    B, d, C, H, K, s = 2, 8, 8, 9, 5, 2
+    g = gen(114)
+    q, key, v = randn(g, B, d, H * s, W * s), randn(g, B, d, H, W), randn(g, B, C + 1, H, W)
+    vd = v.to(DEV)[:, 1:].contiguous()
+    got = sapa_amd.sapa_fused(q.to(DEV), key.to(DEV), vd, K, s).cpu()
+    assert_f32_close(got, coracle.sapa_fused(q, key, v[:, 1:].contiguous(), K, s, 'f32'), f'W={W}')
+    # an unaligned (but contiguous) value tensor: flat storage offset of one element
+    flat = torch.empty(B * C * H * W + 1, device=DEV)
+    vu = flat[1:].view(B, C, H, W)
+    vu.copy_(v[:, 1:])
+    got = sapa_amd.sapa_fused(q.to(DEV), key.to(DEV), vu, K, s).cpu()
+    assert_f32_close(got, coracle.sapa_fused(q, key, v[:, 1:].contiguous(), K, s, 'f32'), f'W={W} unaligned')
+    logits = sapa_amd.qk(q.to(DEV), key.to(DEV), K, s).cpu()
+    assert torch.equal(logits, coracle.qk(q, key, K, s, 'f32'))
