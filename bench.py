@@ -3,7 +3,8 @@
 one MI355X, on the workload BASELINE.json's metric is quoted on.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype fp32|bf16]
-                    [--workload fpn_large|fpn_mid|fpn_small|stress] [--no-cpu-baseline]
+                    [--workload fpn_large|fpn_mid|fpn_small|stress|deform_p25|deform_p9|deform_p5]
+                    [--no-cpu-baseline]
 
 A step is one fused forward over the whole synthetic batch, inputs already
 resident in HBM.  Prints ONE JSON line: output Gpix/s, the HBM roofline of
@@ -33,6 +34,13 @@ WORKLOADS = {
     'fpn_small': (16, 256, 64, 25, 42, 5, 2),
     'stress': (4, 512, 64, 64, 64, 7, 4),
 }
+# SAPA-D (fused deform_qk -> softmax -> deform_av), BASELINE config 4:
+# name -> (B, C, d, G, H, W, P, s); offsets ~N(0, 0.75) clipped to +-4 cells
+DEFORM_WORKLOADS = {
+    'deform_p25': (8, 256, 32, 4, 64, 64, 25, 2),
+    'deform_p9': (8, 256, 32, 4, 64, 64, 9, 2),
+    'deform_p5': (8, 256, 32, 4, 64, 64, 5, 2),
+}
 
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE + WRITE_SIZE,
 # scaled by what the same counters read for a plain copy of known size); see
@@ -61,26 +69,47 @@ def make_inputs(cfg, dtype, device, seed=0):
     return q.to(dtype).contiguous(), key.to(dtype).contiguous(), v.to(dtype).contiguous()
 
 
+def deform_algorithmic_bytes(B, C, d, G, H, W, P, s, esize):
+    """Read q, key, value, offset once, write the output once."""
+    hi, lo = B * H * s * W * s, B * H * W
+    return esize * (hi * (G * d + 2 * G * P + C) + lo * (G * d + C))
+
+
+def make_deform_inputs(cfg, dtype, device, seed=0):
+    B, C, d, G, H, W, P, s = cfg
+    g = torch.Generator(device=device).manual_seed(seed)
+    q = torch.randn(B, G * d, H * s, W * s, generator=g, device=device)
+    key = torch.randn(B, G * d, H, W, generator=g, device=device)
+    v = torch.randn(B, C, H, W, generator=g, device=device)
+    off = (0.75 * torch.randn(B, 2 * G * P, H * s, W * s, generator=g, device=device)).clamp(-4, 4)
+    return tuple(t.to(dtype).contiguous() for t in (q, key, v, off))
+
+
+def timed_median(fn, budget_s):
+    """Median wall time of fn() over at least 3 runs within the budget."""
+    fn()  # warm-up
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 3 or (time.perf_counter() - t_start < budget_s and len(times) < 20):
+        t0 = time.perf_counter()
+        out = fn()
+        times.append(time.perf_counter() - t0)
+        if time.perf_counter() - t_start > 3 * budget_s:
+            break
+    times.sort()
+    return times[len(times) // 2], len(times), out
+
+
 def cpu_baseline(q, key, v, K, s, budget_s=20.0):
     """Time the unfold-based CPU math on image 0 of the batch (repeated while
     the budget lasts); returns (Gpix/s, cores, description, output)."""
     from oracle import torch_oracle
     q0, k0, v0 = (t[:1].float().cpu() for t in (q, key, v))
     cores = torch.get_num_threads()
-    out = torch_oracle.sapa_fused(q0, k0, v0, K, s)  # warm-up
-    times = []
-    t_start = time.perf_counter()
-    while len(times) < 3 or (time.perf_counter() - t_start < budget_s and len(times) < 20):
-        t0 = time.perf_counter()
-        out = torch_oracle.sapa_fused(q0, k0, v0, K, s)
-        times.append(time.perf_counter() - t0)
-        if time.perf_counter() - t_start > 3 * budget_s:
-            break
-    times.sort()
-    med = times[len(times) // 2]
+    med, runs, out = timed_median(lambda: torch_oracle.sapa_fused(q0, k0, v0, K, s), budget_s)
     pix = q0.shape[2] * q0.shape[3]
     return pix / med / 1e9, cores, (f'image 0 of the batch (1x{q0.shape[1]}x{q0.shape[2]}x{q0.shape[3]} '
-                                    f'query), fp32, median of {len(times)} runs'), out
+                                    f'query), fp32, median of {runs} runs'), out
 
 
 def main():
@@ -89,7 +118,8 @@ def main():
     ap.add_argument('--steps', type=int, default=100)
     ap.add_argument('--warmup', type=int, default=10)
     ap.add_argument('--dtype', default='fp32', choices=['fp32', 'bf16'])
-    ap.add_argument('--workload', default='fpn_large', choices=sorted(WORKLOADS))
+    ap.add_argument('--workload', default='fpn_large',
+                    choices=sorted(WORKLOADS) + sorted(DEFORM_WORKLOADS))
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--calibration-copy', action='store_true',
                     help='after the timed region, run 5 device copies of 1 GiB (a kernel of '
@@ -107,18 +137,30 @@ def main():
 
     dev = torch.device('cuda:0')
     torch.cuda.set_device(dev)
-    cfg = WORKLOADS[args.workload]
-    B, C, d, H, W, K, s = cfg
     dtype = {'fp32': torch.float32, 'bf16': torch.bfloat16}[args.dtype]
-    q, key, v = make_inputs(cfg, dtype, dev)
+    stream = torch.cuda.current_stream(dev)
+    deform = args.workload in DEFORM_WORKLOADS
+    if deform:
+        cfg = DEFORM_WORKLOADS[args.workload]
+        B, C, d, G, H, W, P, s = cfg
+        q, key, v, off = make_deform_inputs(cfg, dtype, dev)
+    else:
+        cfg = WORKLOADS[args.workload]
+        B, C, d, H, W, K, s = cfg
+        q, key, v = make_inputs(cfg, dtype, dev)
     out = torch.empty(B, C, H * s, W * s, dtype=dtype, device=dev)
     code = _lib.dtype_code(out)
-    stream = torch.cuda.current_stream(dev)
 
-    def step():
-        _lib.check(lib.sapa_fused_forward(q.data_ptr(), key.data_ptr(), v.data_ptr(),
-                                          out.data_ptr(), B, d, C, H, W, K, s, code,
-                                          stream.cuda_stream), 'sapa_fused_forward')
+    if deform:
+        def step():
+            _lib.check(lib.sapa_deform_fused_forward(
+                q.data_ptr(), key.data_ptr(), v.data_ptr(), off.data_ptr(), out.data_ptr(), B,
+                G * d, C, H, W, P, s, G, code, stream.cuda_stream), 'sapa_deform_fused_forward')
+    else:
+        def step():
+            _lib.check(lib.sapa_fused_forward(q.data_ptr(), key.data_ptr(), v.data_ptr(),
+                                              out.data_ptr(), B, d, C, H, W, K, s, code,
+                                              stream.cuda_stream), 'sapa_fused_forward')
 
     for _ in range(args.warmup):
         step()
@@ -144,10 +186,22 @@ def main():
 
     pix = B * H * s * W * s
     esize = out.element_size()
-    abytes = algorithmic_bytes(B, C, d, H, W, s, esize)
+    if deform:
+        abytes = deform_algorithmic_bytes(B, C, d, G, H, W, P, s, esize)
+        what = 'fused SAPA-D forward (deform_qk->softmax->deform_av)'
+        wl = (f'{args.workload}: SAPA-D B={B} C={C} d={d} G={G} P={P} {H}x{W}->{H * s}x{W * s} '
+              f's={s} {args.dtype}, NCHW, offsets ~N(0,0.75) clipped to +-4')
+        kern = 'deform_lds_kernel (fused mode)'
+    else:
+        abytes = algorithmic_bytes(B, C, d, H, W, s, esize)
+        what = 'fused SAPA-B forward (qk->softmax->av)'
+        wl = (f'{args.workload}: SAPA-B FPN-style B={B} C={C} d={d} '
+              f'{H}x{W}->{H * s}x{W * s} K={K} s={s} {args.dtype}, NCHW')
+        kern = ('sapa_b_tiled_kernel (fused mode)' if (K, s) == (5, 2)
+                else 'sapa_b_mfma_kernel (fused mode)')
     achieved = abytes / (ms * 1e-3) / 1e9
     rec = {
-        'metric': 'upsampled Gpix/s, fused SAPA-B forward (qk->softmax->av), 1 GPU',
+        'metric': f'upsampled Gpix/s, {what}, 1 GPU',
         'value': pix / (ms * 1e-3) / 1e9,
         'unit': 'Gpix/s',
         'n_gpus': 1,
@@ -160,8 +214,7 @@ def main():
         'vs_baseline': None,
         'dtype': 'f32' if args.dtype == 'fp32' else 'bf16',
         'data': 'synthetic',
-        'config': {'workload': f'{args.workload}: SAPA-B FPN-style B={B} C={C} d={d} '
-                               f'{H}x{W}->{H * s}x{W * s} K={K} s={s} {args.dtype}, NCHW'},
+        'config': {'workload': wl},
         'roofline': {
             'bound': 'hbm',
             'achieved': achieved,
@@ -170,11 +223,19 @@ def main():
             'frac': achieved / HBM_PEAK_GBS,
             'traffic': MEASURED_TRAFFIC_BYTES.get((args.workload, args.dtype)),
             'algorithmic_bytes': abytes,
-            'kernel': 'sapa_b_tiled_kernel (fused mode)',
+            'kernel': kern,
         },
     }
     if not args.no_cpu_baseline:
-        gpix, cores, sample, ref = cpu_baseline(q, key, v, K, s)
+        if deform:
+            from oracle import torch_oracle
+            q0, k0, v0, o0 = (t[:1].float().cpu() for t in (q, key, v, off))
+            med, runs, ref = timed_median(
+                lambda: torch_oracle.deform_sapa_fused(q0, k0, v0, o0, P, s, G), 20.0)
+            gpix, cores = q0.shape[2] * q0.shape[3] / med / 1e9, torch.get_num_threads()
+            sample = (f'image 0 of the batch (grid_sample formulation, fp32), median of {runs} runs')
+        else:
+            gpix, cores, sample, ref = cpu_baseline(q, key, v, K, s)
         rec['cpu_baseline'] = {'value': gpix, 'unit': 'Gpix/s', 'cores': cores, 'kind': 'port',
                                'sample': sample}
         # the timed GPU output for the same image, against the CPU result
@@ -182,8 +243,14 @@ def main():
         err = (got - ref).abs()
         # the CPU path sums in another order (einsum), so this is fp32-vs-fp32
         # at the reference's own check tolerance, allclose(atol=1e-5)
-        tol = (1e-5 + 1e-5 * ref.abs()) if args.dtype == 'fp32' else \
-            1e-2 * torch.maximum(ref.abs(), ref.pow(2).mean().sqrt())
+        if args.dtype != 'fp32':
+            tol = 1e-2 * torch.maximum(ref.abs(), ref.pow(2).mean().sqrt())
+        elif deform:
+            # grid_sample normalises and de-normalises the coordinates in fp32,
+            # which moves each sample by a few 1e-7 cells
+            tol = 1e-4 + 1e-4 * ref.abs()
+        else:
+            tol = 1e-5 + 1e-5 * ref.abs()
         rec['parity_vs_cpu_sample'] = {'max_abs_err': err.max().item(),
                                        'outside_tolerance': int((err > tol).sum().item()),
                                        'elements': err.numel()}
