@@ -41,6 +41,16 @@ typedef enum sapa_dtype {
     SAPA_BF16 = 3
 } sapa_dtype;
 
+/* Where the sampled operators read the offsets from (the *_from entry points).
+ * SAPADeform builds the hi-res offset tensor from a low-res 1x1-conv output,
+ * by pixel_shuffle or by nearest interpolation (sapa_deform.py:44-47); the
+ * last two values read that conv output in place instead. */
+typedef enum sapa_offset_layout {
+    SAPA_OFFSET_HIRES = 0,         /* [B, 2*G*P, sH, sW], as the reference's extensions take it */
+    SAPA_OFFSET_PIXEL_SHUFFLE = 1, /* [B, 2*G*P*s*s, H, W]: hi[c][qh][qw] = lo[c*s*s + (qh%s)*s + qw%s][qh/s][qw/s] */
+    SAPA_OFFSET_NEAREST = 2        /* [B, 2*G*P, H, W]: hi[c][qh][qw] = lo[c][qh/s][qw/s] */
+} sapa_offset_layout;
+
 typedef enum sapa_status {
     SAPA_OK = 0,
     SAPA_ERR_INVALID_ARGUMENT = -1, /* null pointer, non-positive extent, even K, ... */
@@ -189,6 +199,24 @@ int sapa_deform_fused_forward(const void *query, const void *key,
                               const void *value, const void *offset, void *out,
                               int B, int Cq, int C, int H, int W,
                               int P, int s, int G, int dtype, void *stream);
+
+/* The three sampled forward operators reading the offsets in the layout
+ * `offset_layout` (sapa_offset_layout) names; with SAPA_OFFSET_HIRES they are
+ * the functions above.  They replace
+ *   F.pixel_shuffle(self.offset(x_), s)  /  F.interpolate(self.offset(x_), scale_factor=s)
+ * followed by dqk.forward / dav.forward (sapa_deform.py:44-53): the hi-res
+ * offset tensor is never written.  Results are bit-identical to materialising
+ * it first. */
+int sapa_deform_qk_forward_from(const void *query, const void *key, const void *offset,
+                                void *out, int B, int Cq, int H, int W, int P, int s, int G,
+                                int offset_layout, int dtype, void *stream);
+int sapa_deform_av_forward_from(const void *attn, const void *value, const void *offset,
+                                void *out, int B, int C, int H, int W, int P, int s, int G,
+                                int offset_layout, int dtype, void *stream);
+int sapa_deform_fused_forward_from(const void *query, const void *key, const void *value,
+                                   const void *offset, void *out, int B, int Cq, int C,
+                                   int H, int W, int P, int s, int G, int offset_layout,
+                                   int dtype, void *stream);
 
 #ifdef __cplusplus
 }

@@ -43,20 +43,35 @@ hipError_t tiled_launch(int mode, const void *q, const void *key, const void *at
 // The sampled forward ops: LDS-windowed kernel where it applies, else the
 // global-memory kernel.
 hipError_t deform_qk_any(const void *q, const void *key, const void *offset, void *out, int B,
-                         int Cq, int H, int W, int P, int s, int G, int dtype, hipStream_t st) {
+                         int Cq, int H, int W, int P, int s, int G, int olayout, int dtype,
+                         hipStream_t st) {
     hipError_t e = deform_lds_launch(0, q, key, nullptr, nullptr, offset, out, B, Cq, Cq, H, W, P,
-                                     s, G, dtype, st);
+                                     s, G, olayout, dtype, st);
     if (e == hipErrorNotSupported)
-        e = deform_qk_forward_launch(q, key, offset, out, B, Cq, H, W, P, s, G, dtype, st);
+        e = deform_qk_forward_launch(q, key, offset, out, B, Cq, H, W, P, s, G, olayout, dtype,
+                                     st);
     return e;
 }
 
 hipError_t deform_av_any(const void *attn, const void *value, const void *offset, void *out, int B,
-                         int C, int H, int W, int P, int s, int G, int dtype, hipStream_t st) {
+                         int C, int H, int W, int P, int s, int G, int olayout, int dtype,
+                         hipStream_t st) {
     hipError_t e = deform_lds_launch(1, nullptr, nullptr, attn, value, offset, out, B, C, C, H, W,
-                                     P, s, G, dtype, st);
+                                     P, s, G, olayout, dtype, st);
     if (e == hipErrorNotSupported)
-        e = deform_av_forward_launch(attn, value, offset, out, B, C, H, W, P, s, G, dtype, st);
+        e = deform_av_forward_launch(attn, value, offset, out, B, C, H, W, P, s, G, olayout,
+                                     dtype, st);
+    return e;
+}
+
+hipError_t deform_fused_any(const void *q, const void *key, const void *value, const void *offset,
+                            void *out, int B, int Cq, int C, int H, int W, int P, int s, int G,
+                            int olayout, int dtype, hipStream_t st) {
+    hipError_t e = deform_lds_launch(2, q, key, nullptr, value, offset, out, B, Cq, C, H, W, P, s,
+                                     G, olayout, dtype, st);
+    if (e == hipErrorNotSupported)
+        e = deform_fused_forward_launch(q, key, value, offset, out, B, Cq, C, H, W, P, s, G,
+                                        olayout, dtype, st);
     return e;
 }
 
@@ -215,42 +230,63 @@ int sapa_qk_softmax_forward(const void *query, const void *key, void *attn, int 
     return fused_common(1, query, key, nullptr, attn, B, d, d, H, W, K, s, dtype, stream);
 }
 
+int sapa_deform_qk_forward_from(const void *query, const void *key, const void *offset,
+                                void *out, int B, int Cq, int H, int W, int P, int s, int G,
+                                int offset_layout, int dtype, void *stream) {
+    const int rc = check_deform_args(B, Cq, Cq, H, W, P, s, G, dtype);
+    if (rc != SAPA_OK) return rc;
+    if (offset_layout < 0 || offset_layout > 2) return SAPA_ERR_INVALID_ARGUMENT;
+    if (B == 0) return SAPA_OK;
+    if (!query || !key || !offset || !out) return SAPA_ERR_INVALID_ARGUMENT;
+    return finish(deform_qk_any(query, key, offset, out, B, Cq, H, W, P, s, G, offset_layout,
+                                dtype, (hipStream_t)stream));
+}
+
 int sapa_deform_qk_forward(const void *query, const void *key, const void *offset, void *out,
                            int B, int Cq, int H, int W, int P, int s, int G, int dtype,
                            void *stream) {
-    const int rc = check_deform_args(B, Cq, Cq, H, W, P, s, G, dtype);
+    return sapa_deform_qk_forward_from(query, key, offset, out, B, Cq, H, W, P, s, G,
+                                       SAPA_OFFSET_HIRES, dtype, stream);
+}
+
+int sapa_deform_av_forward_from(const void *attn, const void *value, const void *offset,
+                                void *out, int B, int C, int H, int W, int P, int s, int G,
+                                int offset_layout, int dtype, void *stream) {
+    const int rc = check_deform_args(B, C, C, H, W, P, s, G, dtype);
     if (rc != SAPA_OK) return rc;
+    if (offset_layout < 0 || offset_layout > 2) return SAPA_ERR_INVALID_ARGUMENT;
     if (B == 0) return SAPA_OK;
-    if (!query || !key || !offset || !out) return SAPA_ERR_INVALID_ARGUMENT;
-    return finish(deform_qk_any(query, key, offset, out, B, Cq, H, W, P, s, G, dtype,
-                                (hipStream_t)stream));
+    if (!attn || !value || !offset || !out) return SAPA_ERR_INVALID_ARGUMENT;
+    return finish(deform_av_any(attn, value, offset, out, B, C, H, W, P, s, G, offset_layout,
+                                dtype, (hipStream_t)stream));
 }
 
 int sapa_deform_av_forward(const void *attn, const void *value, const void *offset, void *out,
                            int B, int C, int H, int W, int P, int s, int G, int dtype,
                            void *stream) {
-    const int rc = check_deform_args(B, C, C, H, W, P, s, G, dtype);
+    return sapa_deform_av_forward_from(attn, value, offset, out, B, C, H, W, P, s, G,
+                                       SAPA_OFFSET_HIRES, dtype, stream);
+}
+
+int sapa_deform_fused_forward_from(const void *query, const void *key, const void *value,
+                                   const void *offset, void *out, int B, int Cq, int C, int H,
+                                   int W, int P, int s, int G, int offset_layout, int dtype,
+                                   void *stream) {
+    const int rc = check_deform_args(B, Cq, C, H, W, P, s, G, dtype);
     if (rc != SAPA_OK) return rc;
+    if (offset_layout < 0 || offset_layout > 2) return SAPA_ERR_INVALID_ARGUMENT;
+    if (P > 64) return SAPA_ERR_UNSUPPORTED;
     if (B == 0) return SAPA_OK;
-    if (!attn || !value || !offset || !out) return SAPA_ERR_INVALID_ARGUMENT;
-    return finish(deform_av_any(attn, value, offset, out, B, C, H, W, P, s, G, dtype,
-                                (hipStream_t)stream));
+    if (!query || !key || !value || !offset || !out) return SAPA_ERR_INVALID_ARGUMENT;
+    return finish(deform_fused_any(query, key, value, offset, out, B, Cq, C, H, W, P, s, G,
+                                   offset_layout, dtype, (hipStream_t)stream));
 }
 
 int sapa_deform_fused_forward(const void *query, const void *key, const void *value,
                               const void *offset, void *out, int B, int Cq, int C, int H, int W,
                               int P, int s, int G, int dtype, void *stream) {
-    const int rc = check_deform_args(B, Cq, C, H, W, P, s, G, dtype);
-    if (rc != SAPA_OK) return rc;
-    if (P > 64) return SAPA_ERR_UNSUPPORTED;
-    if (B == 0) return SAPA_OK;
-    if (!query || !key || !value || !offset || !out) return SAPA_ERR_INVALID_ARGUMENT;
-    hipError_t e = deform_lds_launch(2, query, key, nullptr, value, offset, out, B, Cq, C, H, W, P,
-                                     s, G, dtype, (hipStream_t)stream);
-    if (e == hipErrorNotSupported)
-        e = deform_fused_forward_launch(query, key, value, offset, out, B, Cq, C, H, W, P, s, G,
-                                        dtype, (hipStream_t)stream);
-    return finish(e);
+    return sapa_deform_fused_forward_from(query, key, value, offset, out, B, Cq, C, H, W, P, s, G,
+                                          SAPA_OFFSET_HIRES, dtype, stream);
 }
 
 int sapa_deform_qk_backward(const void *grad_out, const void *query, const void *key,
@@ -267,7 +303,8 @@ int sapa_deform_qk_backward(const void *grad_out, const void *query, const void 
     // sampled aggregation with key in the value's place.
     if (grad_query) {
         const hipError_t e =
-            deform_av_any(grad_out, key, offset, grad_query, B, Cq, H, W, P, s, G, dtype, st);
+            deform_av_any(grad_out, key, offset, grad_query, B, Cq, H, W, P, s, G, SAPA_OFFSET_HIRES,
+                          dtype, st);
         if (e != hipSuccess) return fail_hip(e);
     }
     if (grad_key || grad_offset) {
@@ -292,7 +329,8 @@ int sapa_deform_av_backward(const void *grad_out, const void *attn, const void *
     // sampled similarity with grad_out as the query and value as the key.
     if (grad_attn) {
         const hipError_t e =
-            deform_qk_any(grad_out, value, offset, grad_attn, B, C, H, W, P, s, G, dtype, st);
+            deform_qk_any(grad_out, value, offset, grad_attn, B, C, H, W, P, s, G, SAPA_OFFSET_HIRES,
+                          dtype, st);
         if (e != hipSuccess) return fail_hip(e);
     }
     if (grad_value || grad_offset) {

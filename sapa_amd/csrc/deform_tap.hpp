@@ -6,6 +6,43 @@
 
 namespace sapa {
 
+// Where the kernels read a pixel's sampling offsets from.  The module that
+// owns these operators produces the hi-res offset tensor [B, 2GP, sH, sW]
+// from a low-res 1x1-conv output, either by pixel_shuffle of [B, 2GP*s*s, H, W]
+// or by nearest interpolation of [B, 2GP, H, W] (sapa_deform.py:44-47); the
+// last two layouts read that low-res tensor in place, which saves writing and
+// re-reading the hi-res copy.
+enum OffsetLayout { OFFSET_HIRES = 0, OFFSET_PIXEL_SHUFFLE = 1, OFFSET_NEAREST = 2 };
+
+// Channel j (0 = x of the first point, 1 = y, 2 = x of the next point ...)
+// of one pixel's offsets is base[j * stride].
+template <typename T>
+struct OffsetRef {
+    const T *base;
+    long stride;
+};
+
+// k0 = b * G * P + g * P + p: the first sample point wanted.
+// pixel_shuffle: hi[b, c, qh, qw] = lo[b, c*s*s + (qh%s)*s + qw%s, qh/s, qw/s].
+template <typename T>
+__device__ __forceinline__ OffsetRef<T> offset_ref(const T *offset, int layout, long k0, int qh,
+                                                   int qw, int s, int H, int W) {
+    const long lplane = (long)H * W;
+    OffsetRef<T> r;
+    if (layout == OFFSET_HIRES) {
+        r.stride = lplane * s * s;
+        r.base = offset + (k0 << 1) * r.stride + (long)qh * (W * s) + qw;
+    } else if (layout == OFFSET_PIXEL_SHUFFLE) {
+        r.stride = lplane * s * s;
+        r.base = offset + (k0 << 1) * r.stride + (long)((qh % s) * s + qw % s) * lplane +
+                 (long)(qh / s) * W + qw / s;
+    } else {
+        r.stride = lplane;
+        r.base = offset + (k0 << 1) * lplane + (long)(qh / s) * W + qw / s;
+    }
+    return r;
+}
+
 // One bilinear sample position: four weights, four plane offsets, four
 // per-corner validity flags (deform_qk_cuda_kernel.cu:30-64).
 template <typename A>

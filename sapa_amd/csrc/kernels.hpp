@@ -40,19 +40,22 @@ hipError_t sapa_b_mfma_launch(int mode, const void *q, const void *key, const vo
 // not fit LDS; the caller then takes the global-memory kernels below.
 hipError_t deform_lds_launch(int mode, const void *q, const void *key, const void *attn_in,
                              const void *value, const void *offset, void *out, int B, int Cq, int C,
-                             int H, int W, int P, int s, int G, int dtype, hipStream_t st);
+                             int H, int W, int P, int s, int G, int olayout, int dtype,
+                             hipStream_t st);
 
-// sapa_d.hip
+// sapa_d.hip.  olayout (OffsetLayout in deform_tap.hpp) says whether `offset`
+// is the hi-res tensor or the low-res tensor it is produced from.
 hipError_t deform_qk_forward_launch(const void *q, const void *key, const void *offset, void *out,
-                                    int B, int Cq, int H, int W, int P, int s, int G, int dtype,
-                                    hipStream_t st);
+                                    int B, int Cq, int H, int W, int P, int s, int G, int olayout,
+                                    int dtype, hipStream_t st);
 hipError_t deform_av_forward_launch(const void *attn, const void *value, const void *offset,
                                     void *out, int B, int C, int H, int W, int P, int s, int G,
-                                    int dtype, hipStream_t st);
+                                    int olayout, int dtype, hipStream_t st);
 // P <= 64; hipErrorNotSupported otherwise
 hipError_t deform_fused_forward_launch(const void *q, const void *key, const void *value,
                                        const void *offset, void *out, int B, int Cq, int C, int H,
-                                       int W, int P, int s, int G, int dtype, hipStream_t st);
+                                       int W, int P, int s, int G, int olayout, int dtype,
+                                       hipStream_t st);
 // grad_low (atomic accumulate, may be null) and grad_offset (store, may be
 // null) of either sampled op: hi = per-channel high-res tensor [B,Cx,sH,sW],
 // sc = per-point tensor [B,G,P,sH,sW], low = sampled tensor [B,Cx,H,W].

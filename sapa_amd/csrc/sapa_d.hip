@@ -21,7 +21,7 @@ template <typename T>
 __global__ void __launch_bounds__(256)
 deform_qk_forward_kernel(const T *__restrict__ q, const T *__restrict__ key,
                          const T *__restrict__ offset, T *__restrict__ out, int B, int Cq, int H,
-                         int W, int P, int s, int G) {
+                         int W, int P, int s, int G, int olayout) {
     typedef typename Acc<T>::type A;
     const int hH = H * s, hW = W * s, GP = G * P, d = Cq / G;
     const long lplane = (long)H * W, hplane = (long)hH * hW;
@@ -36,8 +36,8 @@ deform_qk_forward_kernel(const T *__restrict__ q, const T *__restrict__ key,
         const int b = (int)(t / GP);
         const int g = k / P;
         const long pix = (long)qh * hW + qw;
-        const long oi = (((long)b * GP + k) << 1) * hplane + pix;
-        const A off_w = ld(offset + oi), off_h = ld(offset + oi + hplane);
+        const OffsetRef<T> op = offset_ref(offset, olayout, (long)b * GP + k, qh, qw, s, H, W);
+        const A off_w = ld(op.base), off_h = ld(op.base + op.stride);
         const A kh = (A)(qh / s) + off_h, kw = (A)(qw / s) + off_w;
         Tap<A> tap;
         A acc = 0;
@@ -57,7 +57,7 @@ template <typename T>
 __global__ void __launch_bounds__(256)
 deform_av_forward_kernel(const T *__restrict__ attn, const T *__restrict__ value,
                          const T *__restrict__ offset, T *__restrict__ out, int B, int C, int H,
-                         int W, int P, int s, int G) {
+                         int W, int P, int s, int G, int olayout) {
     typedef typename Acc<T>::type A;
     const int hH = H * s, hW = W * s, GP = G * P, cg = C / G;
     const long lplane = (long)H * W, hplane = (long)hH * hW;
@@ -74,12 +74,13 @@ deform_av_forward_kernel(const T *__restrict__ attn, const T *__restrict__ value
         const long pix = (long)qh * hW + qw;
         const long k0 = (long)b * GP + (long)g * P;
         const T *ap = attn + k0 * hplane + pix;
-        const T *op = offset + (k0 << 1) * hplane + pix;
+        const OffsetRef<T> op = offset_ref(offset, olayout, k0, qh, qw, s, H, W);
         const T *plane = value + ((long)b * C + c) * lplane;
         const A ph = (A)(qh / s), pw = (A)(qw / s);
         A acc = 0;
         for (int ip = 0; ip < P; ++ip) {
-            const A off_w = ld(op + (2 * ip) * hplane), off_h = ld(op + (2 * ip + 1) * hplane);
+            const A off_w = ld(op.base + (2 * ip) * op.stride);
+            const A off_h = ld(op.base + (2 * ip + 1) * op.stride);
             const A wa = ld(ap + ip * hplane);
             Tap<A> tap;
             if (tap_setup(ph + off_h, pw + off_w, H, W, tap))
@@ -98,7 +99,7 @@ __global__ void __launch_bounds__(256)
 deform_fused_forward_kernel(const T *__restrict__ q, const T *__restrict__ key,
                             const T *__restrict__ value, const T *__restrict__ offset,
                             T *__restrict__ out, int B, int Cq, int C, int H, int W, int P, int s,
-                            int G) {
+                            int G, int olayout) {
     typedef typename Acc<T>::type A;
     constexpr int CC = 8;  // value channels accumulated together
     const int hH = H * s, hW = W * s, GP = G * P, d = Cq / G, cg = C / G;
@@ -114,7 +115,7 @@ deform_fused_forward_kernel(const T *__restrict__ q, const T *__restrict__ key,
         const int b = (int)(t / G);
         const long pix = (long)qh * hW + qw;
         const long k0 = (long)b * GP + (long)g * P;
-        const T *op = offset + (k0 << 1) * hplane + pix;
+        const OffsetRef<T> op = offset_ref(offset, olayout, k0, qh, qw, s, H, W);
         const A ph = (A)(qh / s), pw = (A)(qw / s);
         const T *qp = q + ((long)b * Cq + (long)g * d) * hplane + pix;
         const T *kp = key + ((long)b * Cq + (long)g * d) * lplane;
@@ -123,8 +124,8 @@ deform_fused_forward_kernel(const T *__restrict__ q, const T *__restrict__ key,
 #pragma unroll
         for (int ip = 0; ip < PMAX; ++ip) {
             if (ip < P) {
-                kw[ip] = pw + ld(op + (2 * ip) * hplane);
-                kh[ip] = ph + ld(op + (2 * ip + 1) * hplane);
+                kw[ip] = pw + ld(op.base + (2 * ip) * op.stride);
+                kh[ip] = ph + ld(op.base + (2 * ip + 1) * op.stride);
                 Tap<A> tap;
                 A acc = 0;
                 if (tap_setup(kh[ip], kw[ip], H, W, tap))
@@ -250,35 +251,35 @@ deform_lowgrad_kernel(const T *__restrict__ hi, const T *__restrict__ sc,
     }
 
 hipError_t deform_qk_forward_launch(const void *q, const void *key, const void *offset, void *out,
-                                    int B, int Cq, int H, int W, int P, int s, int G, int dtype,
-                                    hipStream_t st) {
+                                    int B, int Cq, int H, int W, int P, int s, int G, int olayout,
+                                    int dtype, hipStream_t st) {
     const long total = (long)B * G * P * H * s * W * s;
     SAPA_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(deform_qk_forward_kernel<T>,
         dim3(grid_for(total, 256)), dim3(256), 0, st, (const T *)q, (const T *)key,
-        (const T *)offset, (T *)out, B, Cq, H, W, P, s, G));
+        (const T *)offset, (T *)out, B, Cq, H, W, P, s, G, olayout));
     return hipGetLastError();
 }
 
 hipError_t deform_av_forward_launch(const void *attn, const void *value, const void *offset,
                                     void *out, int B, int C, int H, int W, int P, int s, int G,
-                                    int dtype, hipStream_t st) {
+                                    int olayout, int dtype, hipStream_t st) {
     const long total = (long)B * C * H * s * W * s;
     SAPA_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(deform_av_forward_kernel<T>,
         dim3(grid_for(total, 256)), dim3(256), 0, st, (const T *)attn, (const T *)value,
-        (const T *)offset, (T *)out, B, C, H, W, P, s, G));
+        (const T *)offset, (T *)out, B, C, H, W, P, s, G, olayout));
     return hipGetLastError();
 }
 
 template <typename T>
 static hipError_t deform_fused_t(const void *q, const void *key, const void *value,
                                  const void *offset, void *out, int B, int Cq, int C, int H, int W,
-                                 int P, int s, int G, hipStream_t st) {
+                                 int P, int s, int G, int olayout, hipStream_t st) {
     const long total = (long)B * G * H * s * W * s;
     const dim3 grid(grid_for(total, 256)), block(256);
 #define SAPA_DF_CASE(PM)                                                                       \
     hipLaunchKernelGGL((deform_fused_forward_kernel<T, PM>), grid, block, 0, st, (const T *)q, \
                        (const T *)key, (const T *)value, (const T *)offset, (T *)out, B, Cq,   \
-                       C, H, W, P, s, G)
+                       C, H, W, P, s, G, olayout)
     if (P <= 8) SAPA_DF_CASE(8);
     else if (P <= 16) SAPA_DF_CASE(16);
     else if (P <= 32) SAPA_DF_CASE(32);
@@ -290,9 +291,10 @@ static hipError_t deform_fused_t(const void *q, const void *key, const void *val
 
 hipError_t deform_fused_forward_launch(const void *q, const void *key, const void *value,
                                        const void *offset, void *out, int B, int Cq, int C, int H,
-                                       int W, int P, int s, int G, int dtype, hipStream_t st) {
+                                       int W, int P, int s, int G, int olayout, int dtype,
+                                       hipStream_t st) {
     SAPA_DISPATCH_DTYPE(dtype, return (deform_fused_t<T>(q, key, value, offset, out, B, Cq, C, H,
-                                                         W, P, s, G, st)));
+                                                         W, P, s, G, olayout, st)));
     return hipSuccess;
 }
 

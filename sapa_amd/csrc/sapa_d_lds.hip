@@ -31,7 +31,7 @@ __global__ void __launch_bounds__(TPW *TPH *S *S)
 deform_lds_kernel(const T *__restrict__ q, const T *__restrict__ key,
                   const T *__restrict__ attn_in, const T *__restrict__ value,
                   const T *__restrict__ offset, T *__restrict__ out, int Cq, int C, int H, int W,
-                  int P, int G, int tiles_x, int tiles_y, int nblocks, int per_xcd) {
+                  int P, int G, int olayout, int tiles_x, int tiles_y, int nblocks, int per_xcd) {
     typedef float A;
     constexpr int HR = 4;                           // window reach in low-res cells
     constexpr int NT = TPW * TPH * S * S;
@@ -62,7 +62,8 @@ deform_lds_kernel(const T *__restrict__ q, const T *__restrict__ key,
     const long pix = (long)(qh < hH ? qh : hH - 1) * hW + (qw < hW ? qw : hW - 1);
     const A ph = (A)((qh < hH ? qh : hH - 1) / S), pw = (A)((qw < hW ? qw : hW - 1) / S);
     const int wx0 = tx * TPW - HR, wy0 = ty * TPH - HR;
-    const T *op = offset + ((((long)b * GP + (long)g * P)) << 1) * hplane + pix;
+    const OffsetRef<T> op = offset_ref(offset, olayout, (long)b * GP + (long)g * P,
+                                       qh < hH ? qh : hH - 1, qw < hW ? qw : hW - 1, S, H, W);
     A *lgt = lg + tid;
 
     // window of `nvalid` channels starting at plane `src` -> LDS, zero-filled
@@ -93,8 +94,8 @@ deform_lds_kernel(const T *__restrict__ q, const T *__restrict__ key,
             stage(key + (ch0 + c0) * lplane, nvalid);
             __syncthreads();
             for (int p = 0; p < P; ++p) {
-                const A kw = pw + (A)op[(long)(2 * p) * hplane];
-                const A kh = ph + (A)op[(long)(2 * p + 1) * hplane];
+                const A kw = pw + (A)op.base[(long)(2 * p) * op.stride];
+                const A kh = ph + (A)op.base[(long)(2 * p + 1) * op.stride];
                 A acc = c0 == 0 ? (A)0 : lgt[p * NT];
                 Tap<A> tap;
                 if (tap_setup(kh, kw, H, W, tap)) {
@@ -151,8 +152,8 @@ deform_lds_kernel(const T *__restrict__ q, const T *__restrict__ key,
 #pragma unroll
             for (int ch = 0; ch < CH; ++ch) o[ch] = 0;
             for (int p = 0; p < P; ++p) {
-                const A kw = pw + (A)op[(long)(2 * p) * hplane];
-                const A kh = ph + (A)op[(long)(2 * p + 1) * hplane];
+                const A kw = pw + (A)op.base[(long)(2 * p) * op.stride];
+                const A kh = ph + (A)op.base[(long)(2 * p + 1) * op.stride];
                 const A wa = lgt[p * NT];
                 Tap<A> tap;
                 if (tap_setup(kh, kw, H, W, tap)) {
@@ -190,7 +191,7 @@ deform_lds_kernel(const T *__restrict__ q, const T *__restrict__ key,
 template <typename T, int S, int TPW, int TPH, int CH>
 static hipError_t launch_geom(int mode, const void *q, const void *key, const void *attn_in,
                               const void *value, const void *offset, void *out, int B, int Cq,
-                              int C, int H, int W, int P, int G, hipStream_t st) {
+                              int C, int H, int W, int P, int G, int olayout, hipStream_t st) {
     constexpr int HR = 4, NT = TPW * TPH * S * S;
     constexpr int WW = TPW + 2 * HR + 1, WH = TPH + 2 * HR + 1, RS = WW | 1, CS = WH * RS;
     const size_t smem = ((size_t)CH * CS + (size_t)P * NT) * sizeof(float);
@@ -205,7 +206,7 @@ static hipError_t launch_geom(int mode, const void *q, const void *key, const vo
         hipLaunchKernelGGL((deform_lds_kernel<T, S, TPW, TPH, CH, M>), grid, block, smem, st, \
                            (const T *)q, (const T *)key, (const T *)attn_in,                  \
                            (const T *)value, (const T *)offset, (T *)out, Cq, C, H, W, P, G,  \
-                           tiles_x, tiles_y, (int)nb, per_xcd);                               \
+                           olayout, tiles_x, tiles_y, (int)nb, per_xcd);                      \
         break;
     switch (mode) {
         SAPA_DL_CASE(DEFORM_QK) SAPA_DL_CASE(DEFORM_AV) SAPA_DL_CASE(DEFORM_FUSED)
@@ -218,15 +219,15 @@ static hipError_t launch_geom(int mode, const void *q, const void *key, const vo
 template <typename T>
 static hipError_t launch_t(int mode, const void *q, const void *key, const void *attn_in,
                            const void *value, const void *offset, void *out, int B, int Cq, int C,
-                           int H, int W, int P, int s, int G, hipStream_t st) {
+                           int H, int W, int P, int s, int G, int olayout, hipStream_t st) {
 #ifdef SAPA_DLDS_TUNE
-    if (s == 2) return launch_geom<T, 2, SAPA_DLDS_TUNE>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, G, st);
+    if (s == 2) return launch_geom<T, 2, SAPA_DLDS_TUNE>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, G, olayout, st);
     return hipErrorNotSupported;
 #else
     switch (s) {
-        case 1: return launch_geom<T, 1, 16, 16, 8>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, G, st);
-        case 2: return launch_geom<T, 2, 8, 8, 16>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, G, st);
-        case 4: return launch_geom<T, 4, 4, 4, 16>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, G, st);
+        case 1: return launch_geom<T, 1, 16, 16, 8>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, G, olayout, st);
+        case 2: return launch_geom<T, 2, 8, 8, 16>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, G, olayout, st);
+        case 4: return launch_geom<T, 4, 4, 4, 16>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, G, olayout, st);
         default: return hipErrorNotSupported;
     }
 #endif
@@ -237,12 +238,13 @@ static hipError_t launch_t(int mode, const void *q, const void *key, const void 
 // for the LDS budget; the caller then takes the global-memory kernels.
 hipError_t deform_lds_launch(int mode, const void *q, const void *key, const void *attn_in,
                              const void *value, const void *offset, void *out, int B, int Cq, int C,
-                             int H, int W, int P, int s, int G, int dtype, hipStream_t st) {
+                             int H, int W, int P, int s, int G, int olayout, int dtype,
+                             hipStream_t st) {
     switch (dtype) {
-        case 0: return launch_t<float>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, s, G, st);
+        case 0: return launch_t<float>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, s, G, olayout, st);
 #ifndef SAPA_DLDS_TUNE
-        case 2: return launch_t<f16_t>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, s, G, st);
-        case 3: return launch_t<bf16_t>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, s, G, st);
+        case 2: return launch_t<f16_t>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, s, G, olayout, st);
+        case 3: return launch_t<bf16_t>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, s, G, olayout, st);
 #endif
         default: return hipErrorNotSupported;
     }

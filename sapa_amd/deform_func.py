@@ -8,6 +8,7 @@ SAPADeform.attention (sapa_deform.py:51-53) run unchanged.
 `deform_sapa_fused` is an addition.
 """
 import torch
+import torch.nn.functional as F
 from torch.autograd import Function
 
 from . import _lib
@@ -146,37 +147,92 @@ class DeformAVFunction(Function):
 deform_av = DeformAVFunction.apply
 
 
+OFFSET_LAYOUTS = {'hires': 0, 'pixel_shuffle': 1, 'nearest': 2}
+
+
+def expand_offset(offset, scale_factor, layout):
+    """The hi-res offset tensor [B, 2GP, sH, sW] that a low-res offset tensor
+    in `layout` stands for (sapa_deform.py:44-47)."""
+    if layout == 'hires':
+        return offset
+    if layout == 'pixel_shuffle':
+        return F.pixel_shuffle(offset, scale_factor)
+    if layout == 'nearest':
+        return F.interpolate(offset, scale_factor=scale_factor)
+    raise ValueError('offset_layout must be one of %s' % sorted(OFFSET_LAYOUTS))
+
+
+def _reduce_offset_grad(grad_hi, scale_factor, layout):
+    # adjoint of expand_offset
+    if layout == 'hires':
+        return grad_hi
+    if layout == 'pixel_shuffle':
+        return F.pixel_unshuffle(grad_hi, scale_factor)
+    b, c, hh, hw = grad_hi.shape
+    s = scale_factor
+    return grad_hi.view(b, c, hh // s, s, hw // s, s).sum(dim=(3, 5))
+
+
+def _deform_fused_backward(grad_output, query, key, value, offset, P, s, G, offset_layout):
+    """Gradients of deform_av(softmax(deform_qk(q, k, off), dim=2), v, off)
+    with respect to q, k, v and the offset tensor in its own layout."""
+    with torch.no_grad():
+        offset = expand_offset(offset, s, offset_layout).contiguous()
+        logits = DeformQKFunction.apply(query, key, offset, P, s, G)
+        attn = torch.softmax(logits.float(), dim=2).to(logits.dtype)
+        ga, gv, goff_av = _deform_av_backward(grad_output, attn, value, offset, P, s, G)
+        a32, g32 = attn.float(), ga.float()
+        grad_logits = (a32 * (g32 - (g32 * a32).sum(dim=2, keepdim=True))).to(attn.dtype)
+        gq, gk, goff_qk = _deform_qk_backward(grad_logits, query, key, offset, P, s, G)
+        goff = _reduce_offset_grad(goff_av + goff_qk, s, offset_layout)
+    return gq, gk, gv, goff
+
+
 class DeformSAPAFusedFunction(Function):
     """deform_av(softmax(deform_qk(query, key, offset), dim=2), value, offset)
     -- SAPADeform.attention (sapa_deform.py:51-53) -- as one launch in the
     forward pass; the backward pass recomputes the weights and chains the
-    three operators' gradients (the offset receives both paths' gradients)."""
+    three operators' gradients (the offset receives both paths' gradients).
+
+    `offset_layout` 'pixel_shuffle' / 'nearest' takes the low-res output of the
+    offset convolution itself ([B, 2GP*s*s, H, W] / [B, 2GP, H, W]) and reads it
+    in place, so F.pixel_shuffle / F.interpolate (sapa_deform.py:44-47) and the
+    hi-res offset tensor disappear from the forward pass."""
 
     @staticmethod
-    def forward(ctx, query, key, value, offset, num_point, scale_factor, groups):
+    def forward(ctx, query, key, value, offset, num_point, scale_factor, groups,
+                offset_layout='hires'):
+        if offset_layout not in OFFSET_LAYOUTS:
+            raise ValueError('offset_layout must be one of %s' % sorted(OFFSET_LAYOUTS))
         assert scale_factor >= 1
         assert query.size(0) == key.size(0) == value.size(0) == offset.size(0)
         assert query.size(1) == key.size(1)
         assert query.size(2) == key.size(2) * scale_factor
         assert query.size(3) == key.size(3) * scale_factor
         assert value.size(2) == key.size(2) and value.size(3) == key.size(3)
-        assert offset.size(1) == groups * num_point * 2
-        assert offset.size(2) == key.size(2) * scale_factor
-        assert offset.size(3) == key.size(3) * scale_factor
+        if offset_layout == 'hires':
+            assert offset.size(1) == groups * num_point * 2
+            assert offset.size(2) == key.size(2) * scale_factor
+            assert offset.size(3) == key.size(3) * scale_factor
+        else:
+            per_cell = scale_factor ** 2 if offset_layout == 'pixel_shuffle' else 1
+            assert offset.size(1) == groups * num_point * 2 * per_cell
+            assert offset.size(2) == key.size(2) and offset.size(3) == key.size(3)
         assert query.size(1) % groups == 0 and value.size(1) % groups == 0
         assert num_point >= 1
         ctx.num_point = num_point
         ctx.scale_factor = scale_factor
         ctx.groups = groups
+        ctx.offset_layout = offset_layout
 
         n, c, h, w = value.size()
         output = value.new_zeros((n, c, scale_factor * h, scale_factor * w))
         if value.is_cuda:
             _lib.require_cuda_contiguous(query=query, key=key, value=value, offset=offset)
-            _lib.call('sapa_deform_fused_forward', value.device, _lib.ptr(query),
+            _lib.call('sapa_deform_fused_forward_from', value.device, _lib.ptr(query),
                       _lib.ptr(key), _lib.ptr(value), _lib.ptr(offset), _lib.ptr(output), n,
                       key.size(1), c, h, w, num_point, scale_factor, groups,
-                      _lib.dtype_code(value))
+                      OFFSET_LAYOUTS[offset_layout], _lib.dtype_code(value))
         else:
             raise NotImplementedError
 
@@ -188,15 +244,13 @@ class DeformSAPAFusedFunction(Function):
     def backward(ctx, grad_output):
         assert grad_output.is_cuda
         query, key, value, offset = ctx.saved_tensors
-        P, s, G = ctx.num_point, ctx.scale_factor, ctx.groups
-        with torch.no_grad():
-            logits = DeformQKFunction.apply(query, key, offset, P, s, G)
-            attn = torch.softmax(logits.float(), dim=2).to(logits.dtype)
-        ga, gv, goff_av = _deform_av_backward(grad_output, attn, value, offset, P, s, G)
-        a32, g32 = attn.float(), ga.float()
-        grad_logits = (a32 * (g32 - (g32 * a32).sum(dim=2, keepdim=True))).to(attn.dtype)
-        gq, gk, goff_qk = _deform_qk_backward(grad_logits, query, key, offset, P, s, G)
-        return gq, gk, gv, goff_av + goff_qk, None, None, None
+        gq, gk, gv, goff = _deform_fused_backward(
+            grad_output, query, key, value, offset, ctx.num_point, ctx.scale_factor, ctx.groups,
+            ctx.offset_layout)
+        return gq, gk, gv, goff, None, None, None, None
 
 
-deform_sapa_fused = DeformSAPAFusedFunction.apply
+def deform_sapa_fused(query, key, value, offset, num_point, scale_factor, groups,
+                      offset_layout='hires'):
+    return DeformSAPAFusedFunction.apply(query, key, value, offset, num_point, scale_factor,
+                                         groups, offset_layout)

@@ -82,6 +82,12 @@ class SAPADeform(nn.Module):
         if self.norm:
             y = self.norm_y(y)
         q, k = self.q(y), self.k(x_)
+        if self.fused:
+            # the kernel reads the offset convolution's output in place
+            return deform_sapa_fused(q.contiguous(), k.contiguous(), x.contiguous(),
+                                     self.offset(x_).contiguous(), self.num_point,
+                                     self.up_factor, self.groups,
+                                     'pixel_shuffle' if self.high_offset else 'nearest')
         if self.high_offset:
             offset = F.pixel_shuffle(self.offset(x_), upscale_factor=self.up_factor)
         else:

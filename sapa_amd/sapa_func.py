@@ -162,6 +162,22 @@ def qk_softmax(query, key, kernel_size, scale_factor):
     return _qk_softmax_forward(query, key, kernel_size, scale_factor)
 
 
+def _fused_backward(grad_output, query, key, value, K, s, needs=(True, True, True)):
+    """Gradients of av(softmax(qk(query, key)), value): the attention weights
+    are recomputed (one launch), then the three operators' gradients chain."""
+    need_q, need_k, need_v = needs
+    attn = _qk_softmax_forward(query, key, K, s)
+    grad_attn, grad_value = _av_backward(grad_output, attn, value, K, s,
+                                         need_a=need_q or need_k, need_v=need_v)
+    grad_query = grad_key = None
+    if need_q or need_k:
+        # softmax backward in fp32: g_logit = attn * (g_attn - sum_k g_attn * attn)
+        a32, g32 = attn.float(), grad_attn.float()
+        grad_logits = (a32 * (g32 - (g32 * a32).sum(dim=1, keepdim=True))).to(attn.dtype)
+        grad_query, grad_key = _qk_backward(grad_logits, query, key, K, s, need_q, need_k)
+    return grad_query, grad_key, grad_value
+
+
 class SAPAFusedFunction(Function):
     """av(softmax(qk(query, key), dim=1), value) -- SAPA.attention
     (sapa_base.py:38-40) -- as one launch in the forward pass.  The backward
@@ -199,17 +215,9 @@ class SAPAFusedFunction(Function):
     def backward(ctx, grad_output):
         assert grad_output.is_cuda
         query, key, value = ctx.saved_tensors
-        K, s = ctx.kernel_size, ctx.scale_factor
-        need_q, need_k, need_v = ctx.needs_input_grad[:3]
-        attn = _qk_softmax_forward(query, key, K, s)
-        grad_attn, grad_value = _av_backward(grad_output, attn, value, K, s,
-                                             need_a=need_q or need_k, need_v=need_v)
-        grad_query = grad_key = None
-        if need_q or need_k:
-            # softmax backward in fp32: g_logit = attn * (g_attn - sum_k g_attn * attn)
-            a32, g32 = attn.float(), grad_attn.float()
-            grad_logits = (a32 * (g32 - (g32 * a32).sum(dim=1, keepdim=True))).to(attn.dtype)
-            grad_query, grad_key = _qk_backward(grad_logits, query, key, K, s, need_q, need_k)
+        grad_query, grad_key, grad_value = _fused_backward(
+            grad_output, query, key, value, ctx.kernel_size, ctx.scale_factor,
+            ctx.needs_input_grad[:3])
         return grad_query, grad_key, grad_value, None, None
 
 

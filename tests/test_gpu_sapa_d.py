@@ -210,9 +210,15 @@ def test_sapa_deform_module(coracle):
     want = coracle.deform_sapa_fused(q.cpu(), k.cpu(), x, off.cpu(), 9, 2, 4, 'f32')
     assert_f32_close(out.cpu(), want, 'SAPADeform fused')
     assert_f32_close(out3.cpu(), want, 'SAPADeform three-step')
+    # nearest-interpolated offsets: the fused module reads the low-res tensor in place
     m2 = sapa_amd.SAPADeform(16, embedding_dim=8, high_offset=False, norm=False, fused=False).to(DEV)
+    torch.nn.init.normal_(m2.offset.weight, std=0.3)
     with torch.no_grad():
-        assert m2(y.to(DEV), x.to(DEV)).shape == (2, 16, 12, 20)
+        out2 = m2(y.to(DEV), x.to(DEV))
+        m2.fused = True
+        out2f = m2(y.to(DEV), x.to(DEV))
+    assert out2.shape == (2, 16, 12, 20)
+    assert_f32_close(out2f.cpu(), out2.cpu(), 'SAPADeform nearest offsets, fused vs three-step')
 
 
 def test_module_trains():
@@ -224,3 +230,97 @@ def test_module_trains():
     for n, p in m.named_parameters():
         assert p.grad is not None and torch.isfinite(p.grad).all(), n
     assert x.grad is not None and x.grad.abs().sum() > 0
+
+
+def _lowres_offsets(g, shape, layout, dtype=torch.float32):
+    B, G, dq, cg, H, W, P, s = shape
+    ch = 2 * G * P * (s * s if layout == 'pixel_shuffle' else 1)
+    return randn(g, B, ch, H, W, dtype=dtype) * 1.5
+
+
+@pytest.mark.parametrize('layout', ['pixel_shuffle', 'nearest'])
+@pytest.mark.parametrize('shape', [SHAPES[0], SHAPES[2], SHAPES[4], SHAPES[6]],
+                         ids=[IDS[0], IDS[2], IDS[4], IDS[6]])
+def test_offsets_read_in_place_match_materialised(layout, shape):
+    """Offsets read from the low-res convolution output (sapa_deform.py:44-47)
+    give the very bits of pixel_shuffle / interpolate followed by the
+    hi-res-offset operators, for all three forward entry points and for both
+    the LDS-windowed (s in 1, 2, 4) and the global-memory kernels (s = 3)."""
+    from sapa_amd import _lib
+    from sapa_amd.deform_func import OFFSET_LAYOUTS, expand_offset
+    B, G, dq, cg, H, W, P, s = shape
+    g = gen(300 + s)
+    q, key, v, _, attn = make(g, shape)
+    lo = _lowres_offsets(g, shape, layout)
+    q, key, v, attn, lo = dev(q, key, v, attn, lo)
+    hi = expand_offset(lo, s, layout).contiguous()
+    code = OFFSET_LAYOUTS[layout]
+    dt = _lib.dtype_code(q)
+
+    want = sapa_amd.deform_qk(q, key, hi, P, s, G)
+    got = torch.empty_like(want)
+    _lib.call('sapa_deform_qk_forward_from', q.device, _lib.ptr(q), _lib.ptr(key), _lib.ptr(lo),
+              _lib.ptr(got), B, G * dq, H, W, P, s, G, code, dt)
+    assert torch.equal(got, want), 'deform_qk ' + layout
+
+    want = sapa_amd.deform_av(attn, v, hi, P, s, G)
+    got = torch.empty_like(want)
+    _lib.call('sapa_deform_av_forward_from', q.device, _lib.ptr(attn), _lib.ptr(v), _lib.ptr(lo),
+              _lib.ptr(got), B, G * cg, H, W, P, s, G, code, dt)
+    assert torch.equal(got, want), 'deform_av ' + layout
+
+    want = sapa_amd.deform_sapa_fused(q, key, v, hi, P, s, G)
+    got = sapa_amd.deform_sapa_fused(q, key, v, lo, P, s, G, layout)
+    assert torch.equal(got, want), 'fused ' + layout
+
+
+def test_offsets_read_in_place_fp64_and_bf16():
+    from sapa_amd.deform_func import expand_offset
+    shape = SHAPES[2]
+    B, G, dq, cg, H, W, P, s = shape
+    for dtype in (torch.float64, torch.bfloat16):
+        g = gen(310)
+        q, key, v, _, _ = make(g, shape, dtype=dtype)
+        lo = _lowres_offsets(g, shape, 'pixel_shuffle', dtype=dtype)
+        q, key, v, lo = dev(q, key, v, lo)
+        want = sapa_amd.deform_sapa_fused(q, key, v, expand_offset(lo, s, 'pixel_shuffle').contiguous(),
+                                          P, s, G)
+        got = sapa_amd.deform_sapa_fused(q, key, v, lo, P, s, G, 'pixel_shuffle')
+        assert torch.equal(got, want), str(dtype)
+
+
+@pytest.mark.parametrize('layout', ['pixel_shuffle', 'nearest'])
+def test_offsets_read_in_place_gradients(layout):
+    """Gradients with respect to the low-res offset tensor equal autograd
+    through pixel_shuffle / interpolate into the hi-res-offset operator."""
+    from sapa_amd.deform_func import expand_offset
+    shape = (1, 2, 3, 2, 4, 5, 4, 2)
+    B, G, dq, cg, H, W, P, s = shape
+    g = gen(320)
+    q, key, v, _, _ = make(g, shape, dtype=torch.float64)
+    lo = _lowres_offsets(g, shape, layout, dtype=torch.float64)
+    q, key, v, lo = dev(q, key, v, lo)
+    up = randn(g, B, G * cg, H * s, W * s, dtype=torch.float64).to(DEV)
+    grads = []
+    for direct in (True, False):
+        ts = [t.clone().requires_grad_(True) for t in (q, key, v, lo)]
+        if direct:
+            out = sapa_amd.deform_sapa_fused(ts[0], ts[1], ts[2], ts[3], P, s, G, layout)
+        else:
+            out = sapa_amd.deform_sapa_fused(ts[0], ts[1], ts[2],
+                                             expand_offset(ts[3], s, layout).contiguous(), P, s, G)
+        (out * up).sum().backward()
+        grads.append([t.grad for t in ts])
+    for a, b, name in zip(grads[0], grads[1], ('q', 'key', 'value', 'offset')):
+        assert a.shape == b.shape
+        torch.testing.assert_close(a, b, rtol=1e-10, atol=1e-12, msg=name + ' ' + layout)
+
+
+def test_offset_layout_is_validated():
+    g = gen(330)
+    q, key, v, off, _ = make(g, SHAPES[0])
+    q, key, v, off = dev(q, key, v, off)
+    with pytest.raises(ValueError):
+        sapa_amd.deform_sapa_fused(q, key, v, off, 5, 2, 4, 'bilinear')
+    with pytest.raises(AssertionError):
+        sapa_amd.deform_sapa_fused(q, key, v, off, 5, 2, 4, 'nearest')   # hi-res shape, low-res layout
