@@ -40,6 +40,16 @@ hipError_t tiled_launch(int mode, const void *q, const void *key, const void *at
     return e;
 }
 
+// Low-res gradient of qk / av: tiled scatter where it applies, else the
+// gather kernel.
+hipError_t lowres_grad_any(const void *hi, const void *w, void *out, int B, int C, int H, int W,
+                           int K, int s, int dtype, hipStream_t st) {
+    hipError_t e = lowres_grad_tiled_launch(hi, w, out, B, C, H, W, K, s, dtype, st);
+    if (e == hipErrorNotSupported)
+        e = lowres_grad_generic_launch(hi, w, out, B, C, H, W, K, s, dtype, st);
+    return e;
+}
+
 // The sampled forward ops: LDS-windowed kernel where it applies, else the
 // global-memory kernel.
 hipError_t deform_qk_any(const void *q, const void *key, const void *offset, void *out, int B,
@@ -165,7 +175,7 @@ int sapa_qk_backward(const void *grad_out, const void *query, const void *key, v
     }
     if (grad_key) {
         const hipError_t e =
-            lowres_grad_generic_launch(query, grad_out, grad_key, B, d, H, W, K, s, dtype, st);
+            lowres_grad_any(query, grad_out, grad_key, B, d, H, W, K, s, dtype, st);
         if (e != hipSuccess) return fail_hip(e);
     }
     return SAPA_OK;
@@ -187,7 +197,7 @@ int sapa_av_backward(const void *grad_out, const void *attn, const void *value, 
     }
     if (grad_value) {
         const hipError_t e =
-            lowres_grad_generic_launch(grad_out, attn, grad_value, B, C, H, W, K, s, dtype, st);
+            lowres_grad_any(grad_out, attn, grad_value, B, C, H, W, K, s, dtype, st);
         if (e != hipSuccess) return fail_hip(e);
     }
     return SAPA_OK;

@@ -34,6 +34,12 @@ hipError_t sapa_b_mfma_launch(int mode, const void *q, const void *key, const vo
                               const void *value, void *out, int B, int d, int C, int H, int W,
                               int K, int s, int dtype, hipStream_t st);
 
+// sapa_b_lowgrad.hip: grad_key / grad_value as an LDS-tiled gather (no
+// atomics, `out` fully overwritten).  hipErrorNotSupported unless fp32,
+// s = 2, K in {3, 5}.
+hipError_t lowres_grad_tiled_launch(const void *hi, const void *w, void *out, int B, int C, int H,
+                                    int W, int K, int s, int dtype, hipStream_t st);
+
 // sapa_d_lds.hip: the SAPA-D forward ops gathering from an LDS-resident
 // window; mode 0 = deform_qk (out = logits), 1 = deform_av (attn_in given),
 // 2 = fused.  hipErrorNotSupported when (s, dtype, P) has no instance / does

@@ -1,0 +1,210 @@
+// Gradient of the SAPA-B operators with respect to their low-res operand
+// (grad_key of qk, grad_value of av) as an LDS-tiled gather:
+//
+//   out[n,c,y,x] = sum over window entries k = (ky,kx), i.e. over the parents
+//                  (py,px) = (y + r - ky, x + r - kx) that see cell (y,x) as
+//                  their entry k, and over their S*S children j, of
+//                  w[n, k, child j] * hi[n, c, child j]
+//
+// (w = grad of the logits and hi = query for grad_key; w = attention weights
+// and hi = grad of the output for grad_value).  The reference scatters the
+// same products with one global atomicAdd each
+// (sapa/sapa/src/cuda/qk_cuda_kernel.cu:120-135, av_cuda_kernel.cu:128-145);
+// here every output element is owned by one thread, so there are no atomics,
+// the output needs no zero-fill and the result is the same on every run.
+// (Scattering into LDS was measured too: LDS float atomics run at a small
+// fraction of the plain LDS rate on this part, and tile-level global atomics
+// alone cost more than this whole kernel.)
+//
+// A workgroup owns a tile of TW x TH = (16*NWX) x (4*NWY) low-res cells of one
+// image; a thread owns one cell and keeps the K*K x S*S weights that multiply
+// into it in registers for the whole launch (they do not depend on the
+// channel).  The high-res window of `hi` that the tile's cells draw from --
+// the children of the tile's parents plus r parents on every side -- is staged
+// through LDS CH channels at a time, double-buffered, with the next chunk's
+// global loads in flight during the current chunk's FMAs; a thread reads the
+// S children of a parent row with one S-wide LDS access.  Each child row has
+// its own running sum over k in ascending order, one FMA per term; the row
+// sums are added at the end.
+#include "kernels.hpp"
+
+namespace sapa {
+
+namespace {
+
+template <int N> struct FVec;
+template <> struct FVec<2> { typedef float type __attribute__((ext_vector_type(2))); };
+template <> struct FVec<4> { typedef float type __attribute__((ext_vector_type(4))); };
+
+template <int K, int S, int NWX, int NWY, int CH, int VEC>
+__global__ void __launch_bounds__(64 * NWX *NWY) __attribute__((amdgpu_waves_per_eu(3, 3)))
+lowgrad_gather_kernel(const float *__restrict__ hi, const float *__restrict__ w,
+                      float *__restrict__ out, int C, int H, int W, int tiles_x, int tiles_y,
+                      int nblocks, int per_xcd, int cgroups, int cper) {
+    static_assert(S == 2, "children are read as 2-wide vectors");
+    constexpr int TW = 16 * NWX, TH = 4 * NWY, NT = 64 * NWX * NWY;
+    constexpr int KK = K * K, R = (K - 1) / 2, NJ = S * S;
+    constexpr int WPW = TW + 2 * R, WPH = TH + 2 * R;   // window in parents
+    constexpr int WW = WPW * S, WH = WPH * S;            // window in high-res pixels
+    constexpr int RS = WW;                               // LDS row stride (floats)
+    constexpr int PS = WH * RS;                          // one channel's plane
+    constexpr int NV = WH * (WW / VEC);                  // vector loads per channel
+    constexpr int NLD = (CH * NV + NT - 1) / NT;         // per thread and chunk
+    static_assert(WW % VEC == 0 && (R * S) % VEC == 0, "window rows must be whole aligned vectors");
+    static_assert(NLD <= 32, "validity mask is 32 bits");
+    typedef typename FVec<VEC>::type V;
+    typedef typename FVec<S>::type V2;
+
+    __shared__ __attribute__((aligned(16))) float win[2 * CH * PS];
+
+    const int logical = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
+    if (logical >= nblocks) return;
+    const int tx = logical % tiles_x;
+    const int ty = (logical / tiles_x) % tiles_y;
+    const int cg = (logical / (tiles_x * tiles_y)) % cgroups;
+    const int n = logical / (tiles_x * tiles_y * cgroups);
+    const int cbeg = cg * cper, cend = cbeg + cper < C ? cbeg + cper : C;
+
+    const int tid = threadIdx.x, lane = tid % 64, wv = tid / 64;
+    const int lx = (wv % NWX) * 16 + lane % 16, ly = (wv / NWX) * 4 + lane / 16;
+    const int x = tx * TW + lx, y = ty * TH + ly;
+    const int hW = W * S, hH = H * S;
+    const long hplane = (long)hH * hW;
+
+    // weights of the terms that flow into cell (y, x); parents outside the
+    // image contribute nothing
+    float wr[KK][NJ];
+    {
+        const float *wp = w + (long)n * KK * hplane;
+#pragma unroll
+        for (int k = 0; k < KK; ++k) {
+            const int py = y + R - k / K, px = x + R - k % K;
+            const bool ok = py >= 0 && py < H && px >= 0 && px < W;
+            const long base = (long)k * hplane + (long)((ok ? py : 0) * S) * hW + (ok ? px : 0) * S;
+#pragma unroll
+            for (int cy = 0; cy < S; ++cy) {
+                const V2 v = *(const V2 *)(wp + base + (long)cy * hW);
+#pragma unroll
+                for (int cx = 0; cx < S; ++cx) wr[k][cy * S + cx] = ok ? v[cx] : 0.f;
+            }
+        }
+    }
+
+    // staging: element e of a chunk = (channel, window row, vector in the row)
+    const int wy0 = (ty * TH - R) * S, wx0 = (tx * TW - R) * S;   // window origin, high-res
+    const float *hp = hi + (long)n * C * hplane;
+    V stage[NLD];
+    unsigned okmask = 0;
+    auto issue = [&](int c0) {
+        okmask = 0;
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            const int e = tid + i * NT;
+            const int ch = e / NV, rem = e % NV;
+            const int row = rem / (WW / VEC), col = rem % (WW / VEC) * VEC;
+            const int gy = wy0 + row, gx = wx0 + col;
+            // a vector is either all inside or all outside the image: gx and
+            // the image width are both multiples of VEC
+            const bool ok =
+                e < CH * NV && c0 + ch < cend && gy >= 0 && gy < hH && gx >= 0 && gx < hW;
+            const long off = ok ? (long)(c0 + ch) * hplane + (long)gy * hW + gx : 0;
+            stage[i] = *(const V *)(hp + off);
+            okmask |= (unsigned)ok << i;
+        }
+    };
+    auto commit = [&](float *buf) {
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            const int e = tid + i * NT;
+            if (e < CH * NV) {
+                const int ch = e / NV, rem = e % NV;
+                const int row = rem / (WW / VEC), col = rem % (WW / VEC) * VEC;
+                V v = stage[i];
+                if (!((okmask >> i) & 1)) v = (V)(0.f);
+                *(V *)(buf + ch * PS + row * RS + col) = v;
+            }
+        }
+    };
+
+    issue(cbeg);
+    commit(win);
+    __syncthreads();
+
+    // the children of window parent (ly + 2r - ky, lx + 2r - kx) feed entry k
+    const float *base = win + (ly + 2 * R) * S * RS + (lx + 2 * R) * S;
+    const bool live = x < W && y < H;
+    const long lplane = (long)H * W;
+    float *op = out + (long)n * C * lplane + (long)(y < H ? y : 0) * W + (x < W ? x : 0);
+    int parity = 0;
+    for (int c0 = cbeg; c0 < cend; c0 += CH, parity ^= 1) {
+        const bool more = c0 + CH < cend;
+        if (more) issue(c0 + CH);
+        const float *buf = base + parity * CH * PS;
+#pragma unroll 1
+        for (int ch = 0; ch < CH; ++ch) {
+            float acc[S];   // one running sum per child row: two shorter FMA chains
+#pragma unroll
+            for (int cy = 0; cy < S; ++cy) acc[cy] = 0.f;
+#pragma unroll
+            for (int k = 0; k < KK; ++k)
+#pragma unroll
+                for (int cy = 0; cy < S; ++cy) {
+                    const V2 h =
+                        *(const V2 *)(buf + ch * PS + (cy - (k / K) * S) * RS - (k % K) * S);
+                    acc[cy] = __builtin_fmaf(wr[k][cy * S], h[0], acc[cy]);
+                    acc[cy] = __builtin_fmaf(wr[k][cy * S + 1], h[1], acc[cy]);
+                }
+            if (live && c0 + ch < cend) op[(long)(c0 + ch) * lplane] = acc[0] + acc[1];
+        }
+        if (more) commit(win + (parity ^ 1) * CH * PS);
+        __syncthreads();
+    }
+}
+
+template <int K, int S, int NWX, int NWY, int CH, int VEC>
+hipError_t launch_geom(const void *hi, const void *w, void *out, int B, int C, int H, int W,
+                       hipStream_t st) {
+    constexpr int TW = 16 * NWX, TH = 4 * NWY, NT = 64 * NWX * NWY;
+    const int tiles_x = (W + TW - 1) / TW, tiles_y = (H + TH - 1) / TH;
+    const long tiles = (long)tiles_x * tiles_y * B;
+    // few tiles: slice the channels over several workgroups per tile (each
+    // re-reads the tile's weights, which is small against C channels of hi)
+    int cgroups = 1;
+    const int max_groups = C / (4 * CH) > 0 ? C / (4 * CH) : 1;
+    while (cgroups * 2 <= max_groups && tiles * cgroups * 2 <= 1024) cgroups *= 2;
+    const int cper = ((C + cgroups - 1) / cgroups + CH - 1) / CH * CH;
+    const long nb = tiles * cgroups;
+    if (nb > (1L << 30)) return hipErrorNotSupported;
+    const int per_xcd = (int)((nb + 7) / 8);
+    hipLaunchKernelGGL((lowgrad_gather_kernel<K, S, NWX, NWY, CH, VEC>), dim3(per_xcd * 8),
+                       dim3(NT), 0, st, (const float *)hi, (const float *)w, (float *)out, C, H, W,
+                       tiles_x, tiles_y, (int)nb, per_xcd, cgroups, cper);
+    return hipGetLastError();
+}
+
+template <int K, int VEC>
+hipError_t launch_k(const void *hi, const void *w, void *out, int B, int C, int H, int W,
+                    hipStream_t st) {
+    const bool wide = (W + 31) / 32 * 32 * 0.9 <= (W + 15) / 16 * 16;
+    return wide ? launch_geom<K, 2, 2, 2, 2, VEC>(hi, w, out, B, C, H, W, st)
+                : launch_geom<K, 2, 1, 2, 2, VEC>(hi, w, out, B, C, H, W, st);
+}
+
+}  // namespace
+
+// fp32, (K, s) in {(3, 2), (5, 2)}, hi / w aligned to s elements;
+// hipErrorNotSupported otherwise (the caller then takes the generic kernel).
+// `out` is fully overwritten.
+hipError_t lowres_grad_tiled_launch(const void *hi, const void *w, void *out, int B, int C, int H,
+                                    int W, int K, int s, int dtype, hipStream_t st) {
+    if (dtype != 0 || s != 2 || (K != 3 && K != 5)) return hipErrorNotSupported;
+    if ((uintptr_t)hi % 8 || (uintptr_t)w % 8) return hipErrorNotSupported;
+    if (K == 3) return launch_k<3, 2>(hi, w, out, B, C, H, W, st);
+    // 16-byte staging loads when the rows of hi allow it (the window starts
+    // r * s = 4 pixels left of a tile, which keeps them aligned)
+    const bool v4 = (uintptr_t)hi % 16 == 0 && W % 2 == 0;
+    return v4 ? launch_k<5, 4>(hi, w, out, B, C, H, W, st)
+              : launch_k<5, 2>(hi, w, out, B, C, H, W, st);
+}
+
+}  // namespace sapa

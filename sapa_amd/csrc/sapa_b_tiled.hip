@@ -73,8 +73,11 @@ __device__ __forceinline__ void store_stream(T *p, const Vec<T, N> &v) {
     __builtin_nontemporal_store(u.b, (B *)p);
 }
 
+#ifndef SAPA_TILED_WPE
+#define SAPA_TILED_WPE 3
+#endif
 template <typename T, int K, int S, int CY, int NWX, int NWY, int CH, int VEC, int MODE>
-__global__ void __launch_bounds__(64 * NWX * NWY * (S / CY)) __attribute__((amdgpu_waves_per_eu(3, 3)))
+__global__ void __launch_bounds__(64 * NWX * NWY * (S / CY)) __attribute__((amdgpu_waves_per_eu(SAPA_TILED_WPE, SAPA_TILED_WPE)))
 sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
                     const T *__restrict__ attn_in, const T *__restrict__ value,
                     T *__restrict__ out, int d, int C, int H, int W, int tiles_x, int tiles_y,
@@ -406,7 +409,7 @@ static hipError_t launch_t(int mode, const void *q, const void *key, const void 
         if (hi_ptrs[i] && ((uintptr_t)hi_ptrs[i] % align) != 0) return hipErrorNotSupported;
     if (K == 5 && s == 2) {
 #ifdef SAPA_TUNE_GEOM
-        return launch_mode<T, 5, 2, 2, SAPA_TUNE_GEOM>(mode, q, key, attn_in, value, out, B, d, C, H, W, st);
+        return launch_mode<T, 5, 2, SAPA_TUNE_GEOM>(mode, q, key, attn_in, value, out, B, d, C, H, W, st);
 #else
         // Tile geometry: padded parent count times the relative cost per
         // parent measured at the FPN shapes on MI355X (wider tiles fetch

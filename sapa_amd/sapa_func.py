@@ -16,7 +16,18 @@ def _check_odd_kernel(kernel_size):
     assert (kernel_size - 1) % 2 == 0 and kernel_size >= 1
 
 
+def _wide(*tensors):
+    # the tiled gradient kernels are fp32; 16-bit tensors take them and the
+    # gradients are rounded back
+    return [t.float() if t.dtype in (torch.float16, torch.bfloat16) else t for t in tensors]
+
+
 def _qk_backward(grad_output, query, key, kernel_size, scale_factor, need_q=True, need_k=True):
+    if key.dtype in (torch.float16, torch.bfloat16):
+        gq, gk = _qk_backward(*_wide(grad_output, query, key), kernel_size, scale_factor,
+                              need_q, need_k)
+        return (None if gq is None else gq.to(query.dtype),
+                None if gk is None else gk.to(key.dtype))
     grad_output = grad_output.contiguous()
     grad_query = torch.zeros_like(query) if need_q else None
     grad_key = torch.zeros_like(key) if need_k else None
@@ -29,6 +40,11 @@ def _qk_backward(grad_output, query, key, kernel_size, scale_factor, need_q=True
 
 
 def _av_backward(grad_output, attn, value, kernel_size, scale_factor, need_a=True, need_v=True):
+    if value.dtype in (torch.float16, torch.bfloat16):
+        ga, gv = _av_backward(*_wide(grad_output, attn, value), kernel_size, scale_factor,
+                              need_a, need_v)
+        return (None if ga is None else ga.to(attn.dtype),
+                None if gv is None else gv.to(value.dtype))
     grad_output = grad_output.contiguous()
     grad_attn = torch.zeros_like(attn) if need_a else None
     grad_value = torch.zeros_like(value) if need_v else None
@@ -166,6 +182,11 @@ def _fused_backward(grad_output, query, key, value, K, s, needs=(True, True, Tru
     """Gradients of av(softmax(qk(query, key)), value): the attention weights
     are recomputed (one launch), then the three operators' gradients chain."""
     need_q, need_k, need_v = needs
+    if value.dtype in (torch.float16, torch.bfloat16):
+        # the whole chain in fp32, one rounding at the end
+        grads = _fused_backward(*_wide(grad_output, query, key, value), K, s, needs)
+        return tuple(None if g is None else g.to(t.dtype)
+                     for g, t in zip(grads, (query, key, value)))
     attn = _qk_softmax_forward(query, key, K, s)
     grad_attn, grad_value = _av_backward(grad_output, attn, value, K, s,
                                          need_a=need_q or need_k, need_v=need_v)

@@ -197,6 +197,83 @@ def test_backward_vs_oracle(coracle, shape):
         torch.testing.assert_close(vd.grad.cpu().double(), gv, **tol)
 
 
+# B, d, C, H, W, K: more than one tile in x and y, ragged edges, channel counts
+# that are not a multiple of the kernel's chunk, channel slicing (few tiles,
+# many channels)
+LOWGRAD_SHAPES = [(2, 5, 11, 19, 45, 5), (1, 40, 70, 9, 17, 5), (1, 3, 9, 21, 70, 3),
+                  (2, 16, 8, 8, 32, 5), (1, 2, 1, 1, 1, 5)]
+
+
+@pytest.mark.parametrize('shape', LOWGRAD_SHAPES, ids=['-'.join(map(str, s)) for s in LOWGRAD_SHAPES])
+def test_tiled_lowres_gradients_vs_oracle(coracle, shape):
+    """grad_key / grad_value from the tiled scatter kernel (fp32, s = 2)
+    against the float64 oracle, twice in a row into dirty buffers' successors
+    (the kernel zero-fills its output itself)."""
+    B, d, C, H, W, K = shape
+    s = 2
+    g = gen(150)
+    q, key = randn(g, B, d, H * s, W * s), randn(g, B, d, H, W)
+    go = randn(g, B, K * K, H * s, W * s)
+    attn, v = randn(g, B, K * K, H * s, W * s), randn(g, B, C, H, W)
+    go2 = randn(g, B, C, H * s, W * s)
+    _, gk = coracle.qk_backward(go.double(), q.double(), key.double(), K, s, 'f64')
+    _, gv = coracle.av_backward(go2.double(), attn.double(), v.double(), K, s, 'f64')
+    from sapa_amd import _lib
+    qd, kd, god, ad, vd, go2d = dev(q, key, go, attn, v, go2)
+    for fill in (7.0, -3.0):
+        out_k = torch.full_like(kd, fill)
+        _lib.call('sapa_qk_backward', kd.device, _lib.ptr(god), _lib.ptr(qd), _lib.ptr(kd), None,
+                  _lib.ptr(out_k), B, d, H, W, K, s, 0)
+        torch.testing.assert_close(out_k.cpu().double(), gk, rtol=1e-4, atol=2e-5)
+        out_v = torch.full_like(vd, fill)
+        _lib.call('sapa_av_backward', vd.device, _lib.ptr(go2d), _lib.ptr(ad), _lib.ptr(vd), None,
+                  _lib.ptr(out_v), B, C, H, W, K, s, 0)
+        torch.testing.assert_close(out_v.cpu().double(), gv, rtol=1e-4, atol=2e-5)
+
+
+def test_tiled_lowres_gradient_integer_inputs_exact():
+    """Integer-valued inputs make every product and sum exact in fp32, so any
+    order of the atomic adds gives the same bits: an index error cannot hide."""
+    g = gen(151)
+    B, C, H, W, K, s = 2, 10, 13, 37, 5, 2
+    attn = torch.randint(-3, 4, (B, K * K, H * s, W * s), generator=g).float()
+    go = torch.randint(-3, 4, (B, C, H * s, W * s), generator=g).float()
+    v = torch.zeros(B, C, H, W)
+    ad, vd, god = dev(attn, v, go)
+    ad.requires_grad_(False)
+    vd.requires_grad_()
+    sapa_amd.av(ad, vd, K, s).backward(god)
+    want = torch.zeros(B, C, H, W, dtype=torch.float64)
+    r = K // 2
+    a6 = attn.double().view(B, K, K, H, s, W, s)
+    g6 = go.double().view(B, C, H, s, W, s)
+    for ky in range(K):
+        for kx in range(K):
+            contrib = torch.einsum('bhiwj,bchiwj->bchw', a6[:, ky, kx], g6)   # per parent
+            dy, dx = ky - r, kx - r                                          # cell = parent + (dy, dx)
+            ys, xs = slice(max(0, -dy), H - max(0, dy)), slice(max(0, -dx), W - max(0, dx))
+            yd, xd = slice(max(0, dy), H + min(0, dy)), slice(max(0, dx), W + min(0, dx))
+            want[:, :, yd, xd] += contrib[:, :, ys, xs]
+    assert torch.equal(vd.grad.cpu().double(), want)
+
+
+def test_backward_16bit_tensors():
+    """16-bit tensors: gradients come back in the tensors' dtype and agree
+    with the fp32 gradients at the same (rounded) inputs."""
+    g = gen(152)
+    B, d, C, H, W, K, s = 1, 8, 12, 10, 20, 5, 2
+    q, key, v = randn(g, B, d, H * s, W * s), randn(g, B, d, H, W), randn(g, B, C, H, W)
+    go = randn(g, B, C, H * s, W * s)
+    for dt, rel in ((torch.bfloat16, 3e-2), (torch.float16, 5e-3)):
+        ts = [t.to(DEV).to(dt).requires_grad_() for t in (q, key, v)]
+        sapa_amd.sapa_fused(*ts, K, s).backward(go.to(DEV).to(dt))
+        ref = [t.detach().float().requires_grad_() for t in ts]
+        sapa_amd.sapa_fused(*ref, K, s).backward(go.to(DEV).to(dt).float())
+        for a, b in zip(ts, ref):
+            assert a.grad.dtype == dt
+            assert_rel_rms_close(a.grad.float().cpu(), b.grad.cpu(), rel, str(dt))
+
+
 def test_gradcheck_reference_shapes():
     """sapa/sapa/grad_check.py:8-33: float64 gradcheck at its shapes."""
     from torch.autograd import gradcheck
