@@ -40,6 +40,29 @@ hipError_t tiled_launch(int mode, const void *q, const void *key, const void *at
     return e;
 }
 
+// grad_low / grad_offset of a sampled op (hi = per-channel high-res tensor,
+// sc = per-point scalar tensor, low = sampled tensor): the LDS kernels where
+// they apply, the per-term kernel for whatever they leave.
+hipError_t deform_lowgrad_any(const void *hi, const void *sc, const void *low, const void *offset,
+                              void *grad_low, void *grad_offset, int B, int Cx, int H, int W,
+                              int P, int s, int G, int dtype, hipStream_t st) {
+    if (grad_offset) {
+        const hipError_t e = deform_lds_launch(3, hi, low, sc, nullptr, offset, grad_offset, B, Cx,
+                                               Cx, H, W, P, s, G, SAPA_OFFSET_HIRES, dtype, st);
+        if (e == hipSuccess) grad_offset = nullptr;
+        else if (e != hipErrorNotSupported) return e;
+    }
+    if (grad_low) {
+        const hipError_t e =
+            deform_lowgrad_lds_launch(hi, sc, offset, grad_low, B, Cx, H, W, P, s, G, dtype, st);
+        if (e == hipSuccess) grad_low = nullptr;
+        else if (e != hipErrorNotSupported) return e;
+    }
+    if (!grad_low && !grad_offset) return hipSuccess;
+    return deform_lowgrad_launch(hi, sc, low, offset, grad_low, grad_offset, B, Cx, H, W, P, s, G,
+                                 dtype, st);
+}
+
 // Low-res gradient of qk / av: tiled scatter where it applies, else the
 // gather kernel.
 hipError_t lowres_grad_any(const void *hi, const void *w, void *out, int B, int C, int H, int W,
@@ -318,7 +341,7 @@ int sapa_deform_qk_backward(const void *grad_out, const void *query, const void 
         if (e != hipSuccess) return fail_hip(e);
     }
     if (grad_key || grad_offset) {
-        const hipError_t e = deform_lowgrad_launch(query, grad_out, key, offset, grad_key,
+        const hipError_t e = deform_lowgrad_any(query, grad_out, key, offset, grad_key,
                                                    grad_offset, B, Cq, H, W, P, s, G, dtype, st);
         if (e != hipSuccess) return fail_hip(e);
     }
@@ -344,7 +367,7 @@ int sapa_deform_av_backward(const void *grad_out, const void *attn, const void *
         if (e != hipSuccess) return fail_hip(e);
     }
     if (grad_value || grad_offset) {
-        const hipError_t e = deform_lowgrad_launch(grad_out, attn, value, offset, grad_value,
+        const hipError_t e = deform_lowgrad_any(grad_out, attn, value, offset, grad_value,
                                                    grad_offset, B, C, H, W, P, s, G, dtype, st);
         if (e != hipSuccess) return fail_hip(e);
     }

@@ -62,6 +62,14 @@ hipError_t deform_fused_forward_launch(const void *q, const void *key, const voi
                                        const void *offset, void *out, int B, int Cq, int C, int H,
                                        int W, int P, int s, int G, int olayout, int dtype,
                                        hipStream_t st);
+// sapa_d_lowgrad.hip: grad_low of either sampled op (hi, sc as below) summed
+// in LDS windows first (64-bit fixed point, integer atomics), one global float
+// atomic per touched window cell.  fp32, s in {1, 2, 4}; hipErrorNotSupported
+// otherwise.  Accumulates into grad_low.
+hipError_t deform_lowgrad_lds_launch(const void *hi, const void *sc, const void *offset,
+                                     void *grad_low, int B, int Cx, int H, int W, int P, int s,
+                                     int G, int dtype, hipStream_t st);
+
 // grad_low (atomic accumulate, may be null) and grad_offset (store, may be
 // null) of either sampled op: hi = per-channel high-res tensor [B,Cx,sH,sW],
 // sc = per-point tensor [B,G,P,sH,sW], low = sampled tensor [B,Cx,H,W].

@@ -24,7 +24,7 @@
 
 namespace sapa {
 
-enum DeformMode { DEFORM_QK = 0, DEFORM_AV = 1, DEFORM_FUSED = 2 };
+enum DeformMode { DEFORM_QK = 0, DEFORM_AV = 1, DEFORM_FUSED = 2, DEFORM_OFFGRAD = 3 };
 
 template <typename T, int S, int TPW, int TPH, int CH, int MODE>
 __global__ void __launch_bounds__(TPW *TPH *S *S)
@@ -40,7 +40,8 @@ deform_lds_kernel(const T *__restrict__ q, const T *__restrict__ key,
     constexpr int CS = WH * RS;
     constexpr int WIN = WH * WW;
     constexpr int TXP = TPW * S;                    // tile width in pixels
-    constexpr bool DO_QK = MODE != DEFORM_AV, DO_AV = MODE != DEFORM_QK;
+    constexpr bool DO_QK = MODE == DEFORM_QK || MODE == DEFORM_FUSED;
+    constexpr bool DO_AV = MODE == DEFORM_AV || MODE == DEFORM_FUSED;
 
     extern __shared__ float smem[];
     A *win = smem;                                  // [CH][WH][RS]
@@ -79,6 +80,72 @@ deform_lds_kernel(const T *__restrict__ q, const T *__restrict__ key,
             win[ch * CS + row * RS + col] = v;
         }
     };
+
+    if (MODE == DEFORM_OFFGRAD) {
+        // Gradient with respect to the offsets of either sampled operator
+        // (deform_qk_cuda_kernel.cu:98-133): q = the per-channel high-res
+        // tensor (query, or grad of the output), key = the sampled tensor,
+        // attn_in = the per-point scalar (grad of the logits, or the
+        // attention weights), out = grad_offset [B,2GP,sH,sW].  Per point the
+        // two running sums live in LDS next to each other ([2P][thread]).
+        const long ch0 = (long)b * Cq + (long)g * d;
+        const T *sp = attn_in + ((long)b * GP + (long)g * P) * hplane + pix;
+        for (int c0 = 0; c0 < d; c0 += CH) {
+            const int nvalid = d - c0 < CH ? d - c0 : CH;
+            A qv[CH];
+#pragma unroll
+            for (int ch = 0; ch < CH; ++ch)
+                qv[ch] = (active && ch < nvalid) ? (A)q[(ch0 + c0 + ch) * hplane + pix] : (A)0;
+            __syncthreads();
+            stage(key + (ch0 + c0) * lplane, nvalid);
+            __syncthreads();
+            for (int p = 0; p < P; ++p) {
+                const A kw = pw + (A)op.base[(long)(2 * p) * op.stride];
+                const A kh = ph + (A)op.base[(long)(2 * p + 1) * op.stride];
+                const A scv = (A)sp[(long)p * hplane];
+                A gw = c0 == 0 ? (A)0 : lgt[(2 * p) * NT];
+                A gh = c0 == 0 ? (A)0 : lgt[(2 * p + 1) * NT];
+                Tap<A> tap;
+                if (tap_setup(kh, kw, H, W, tap)) {
+                    const int hl = (int)floor_(kh) - wy0, wl = (int)floor_(kw) - wx0;
+                    if (hl >= 0 && hl <= WH - 2 && wl >= 0 && wl <= WW - 2) {
+                        const A *wp = win + hl * RS + wl;
+#pragma unroll
+                        for (int ch = 0; ch < CH; ++ch) {
+                            const A tv = qv[ch] * scv;
+                            const A v1 = wp[ch * CS], v2 = wp[ch * CS + 1];
+                            const A v3 = wp[ch * CS + RS], v4 = wp[ch * CS + RS + 1];
+                            const A ghc = -tap.hw * v1 - tap.lw * v2 + tap.hw * v3 + tap.lw * v4;
+                            const A gwc = -tap.hh * v1 + tap.hh * v2 - tap.lh * v3 + tap.lh * v4;
+                            gh = fma_(ghc, tv, gh);
+                            gw = fma_(gwc, tv, gw);
+                        }
+                    } else {
+                        const T *kp = key + (ch0 + c0) * lplane;
+                        for (int ch = 0; ch < nvalid; ++ch) {
+                            const T *plane = kp + (long)ch * lplane;
+                            const A tv = qv[ch] * scv;
+                            const A v1 = tap.m1 ? ld(plane + tap.i1) : (A)0;
+                            const A v2 = tap.m2 ? ld(plane + tap.i2) : (A)0;
+                            const A v3 = tap.m3 ? ld(plane + tap.i3) : (A)0;
+                            const A v4 = tap.m4 ? ld(plane + tap.i4) : (A)0;
+                            const A ghc = -tap.hw * v1 - tap.lw * v2 + tap.hw * v3 + tap.lw * v4;
+                            const A gwc = -tap.hh * v1 + tap.hh * v2 - tap.lh * v3 + tap.lh * v4;
+                            gh = fma_(ghc, tv, gh);
+                            gw = fma_(gwc, tv, gw);
+                        }
+                    }
+                }
+                lgt[(2 * p) * NT] = gw;
+                lgt[(2 * p + 1) * NT] = gh;
+            }
+        }
+        if (active) {
+            T *o = out + ((((long)b * GP + (long)g * P)) << 1) * hplane + pix;
+            for (int p = 0; p < 2 * P; ++p) o[(long)p * hplane] = (T)lgt[p * NT];
+        }
+        return;
+    }
 
     // `fn(wp)` with wp = LDS address of the tap's low corner if the tap is
     // inside the window; otherwise `fg()` (global-memory taps)
@@ -194,8 +261,10 @@ static hipError_t launch_geom(int mode, const void *q, const void *key, const vo
                               int C, int H, int W, int P, int G, int olayout, hipStream_t st) {
     constexpr int HR = 4, NT = TPW * TPH * S * S;
     constexpr int WW = TPW + 2 * HR + 1, WH = TPH + 2 * HR + 1, RS = WW | 1, CS = WH * RS;
-    const size_t smem = ((size_t)CH * CS + (size_t)P * NT) * sizeof(float);
-    if (smem > 64 * 1024) return hipErrorNotSupported;   // the default dynamic-LDS limit
+    const size_t smem =
+        ((size_t)CH * CS + (size_t)(mode == DEFORM_OFFGRAD ? 2 : 1) * P * NT) * sizeof(float);
+    if (smem > 160 * 1024) return hipErrorNotSupported;  // LDS of one CU
+    const bool big = smem > 64 * 1024;                   // beyond the default dynamic-LDS limit
     const int tiles_x = (W + TPW - 1) / TPW, tiles_y = (H + TPH - 1) / TPH;
     const long nb = (long)tiles_x * tiles_y * G * B;
     if (nb > (1L << 30)) return hipErrorNotSupported;
@@ -203,6 +272,12 @@ static hipError_t launch_geom(int mode, const void *q, const void *key, const vo
     const dim3 grid(per_xcd * 8), block(NT);
 #define SAPA_DL_CASE(M)                                                                       \
     case M:                                                                                   \
+        if (big && hipFuncSetAttribute(                                                       \
+                       reinterpret_cast<const void *>(&deform_lds_kernel<T, S, TPW, TPH, CH, M>), \
+                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) { \
+            (void)hipGetLastError();                                                          \
+            return hipErrorNotSupported;                                                      \
+        }                                                                                     \
         hipLaunchKernelGGL((deform_lds_kernel<T, S, TPW, TPH, CH, M>), grid, block, smem, st, \
                            (const T *)q, (const T *)key, (const T *)attn_in,                  \
                            (const T *)value, (const T *)offset, (T *)out, Cq, C, H, W, P, G,  \
@@ -210,6 +285,7 @@ static hipError_t launch_geom(int mode, const void *q, const void *key, const vo
         break;
     switch (mode) {
         SAPA_DL_CASE(DEFORM_QK) SAPA_DL_CASE(DEFORM_AV) SAPA_DL_CASE(DEFORM_FUSED)
+        SAPA_DL_CASE(DEFORM_OFFGRAD)
         default: return hipErrorInvalidValue;
     }
 #undef SAPA_DL_CASE
@@ -234,7 +310,8 @@ static hipError_t launch_t(int mode, const void *q, const void *key, const void 
 }
 
 // mode: 0 = deform_qk (out = logits), 1 = deform_av (attn_in given),
-// 2 = fused.  hipErrorNotSupported: no instance for (s, dtype) or P too large
+// 2 = fused, 3 = gradient of the offsets (q = per-channel high-res tensor,
+// key = sampled tensor, attn_in = per-point scalar, out = grad_offset).  hipErrorNotSupported: no instance for (s, dtype) or P too large
 // for the LDS budget; the caller then takes the global-memory kernels.
 hipError_t deform_lds_launch(int mode, const void *q, const void *key, const void *attn_in,
                              const void *value, const void *offset, void *out, int B, int Cq, int C,

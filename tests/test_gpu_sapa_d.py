@@ -324,3 +324,86 @@ def test_offset_layout_is_validated():
         sapa_amd.deform_sapa_fused(q, key, v, off, 5, 2, 4, 'bilinear')
     with pytest.raises(AssertionError):
         sapa_amd.deform_sapa_fused(q, key, v, off, 5, 2, 4, 'nearest')   # hi-res shape, low-res layout
+
+
+# B, G, dq, cg, H, W, P, s: several tiles per image, ragged edges, every scale
+# factor with an LDS instance, many points (larger dynamic LDS)
+LDS_GRAD_SHAPES = [(1, 2, 5, 9, 19, 21, 9, 2), (1, 1, 3, 4, 6, 7, 25, 2), (1, 2, 4, 4, 17, 18, 4, 1),
+                   (1, 2, 3, 3, 5, 6, 6, 4), (2, 4, 8, 16, 9, 9, 9, 2)]
+
+
+@pytest.mark.parametrize('off_scale', [1.5, 4.0], ids=['offsets1.5', 'offsets4'])
+@pytest.mark.parametrize('shape', LDS_GRAD_SHAPES, ids=['-'.join(map(str, s)) for s in LDS_GRAD_SHAPES])
+def test_lds_gradient_kernels_vs_oracle(coracle, shape, off_scale):
+    """fp32 gradients of both sampled operators from the LDS kernels (offset
+    gradient by gather, low-res gradient by fixed-point scatter) against the
+    float64 oracle; offsets of scale 4 push many taps out of the LDS window
+    onto the per-term path."""
+    B, G, dq, cg, H, W, P, s = shape
+    g = gen(340)
+    q, key, v, off, attn = make(g, shape, off_scale=off_scale)
+    go_qk = randn(g, B, G, P, H * s, W * s)
+    go_av = randn(g, B, G * cg, H * s, W * s)
+    qd, kd, od = (x.to(DEV).requires_grad_() for x in (q, key, off))
+    sapa_amd.deform_qk(qd, kd, od, P, s, G).backward(go_qk.to(DEV))
+    gq, gk, goff = coracle.deform_qk_backward(go_qk.double(), q.double(), key.double(),
+                                              off.double(), P, s, G, 'f64')
+    tol = dict(rtol=1e-4, atol=5e-5)
+    torch.testing.assert_close(qd.grad.cpu().double(), gq, **tol)
+    torch.testing.assert_close(kd.grad.cpu().double(), gk, **tol)
+    torch.testing.assert_close(od.grad.cpu().double(), goff, **tol)
+    ad, vd, od = (x.to(DEV).requires_grad_() for x in (attn, v, off))
+    sapa_amd.deform_av(ad, vd, od, P, s, G).backward(go_av.to(DEV))
+    ga, gv, goff = coracle.deform_av_backward(go_av.double(), attn.double(), v.double(),
+                                              off.double(), P, s, G, 'f64')
+    torch.testing.assert_close(ad.grad.cpu().double(), ga, **tol)
+    torch.testing.assert_close(vd.grad.cpu().double(), gv, **tol)
+    torch.testing.assert_close(od.grad.cpu().double(), goff, **tol)
+
+
+@pytest.mark.parametrize('magnitude', [1e-12, 1.0, 1e12])
+def test_lowres_gradient_fixed_point_scaling(coracle, magnitude):
+    """The fixed-point window sums rescale themselves to the data: the
+    relative accuracy of grad_value does not depend on the magnitude of the
+    incoming gradient, and one huge element does not wipe out the rest."""
+    shape = (1, 2, 4, 8, 9, 10, 9, 2)
+    B, G, dq, cg, H, W, P, s = shape
+    g = gen(341)
+    _, _, v, off, attn = make(g, shape)
+    attn = torch.softmax(attn, dim=2)
+    go = randn(g, B, G * cg, H * s, W * s) * magnitude
+    go[0, 3, 5, 7] = 1e4 * magnitude
+    ad, vd, od = (x.to(DEV).requires_grad_() for x in (attn, v, off))
+    sapa_amd.deform_av(ad, vd, od, P, s, G).backward(go.to(DEV))
+    _, gv, _ = coracle.deform_av_backward(go.double(), attn.double(), v.double(), off.double(),
+                                          P, s, G, 'f64')
+    got = vd.grad.cpu().double()
+    scale = gv.abs().max()
+    # per element: fp32 resolution of the element itself plus 2^-30 of the
+    # largest magnitude in play
+    err = (got - gv).abs()
+    bound = 1e-5 * gv.abs() + 1e-9 * scale
+    assert (err <= bound).all(), float((err - bound).max() / scale)
+
+
+def test_lowres_gradient_integer_inputs_exact(coracle):
+    """Integer-valued tensors with half-integer offsets: every term is a
+    multiple of 1/4 and every sum is exact in fp32 and in the fixed-point
+    window, so the result does not depend on the order of any add."""
+    shape = (1, 2, 3, 4, 11, 13, 6, 2)
+    B, G, dq, cg, H, W, P, s = shape
+    g = gen(342)
+    attn = torch.randint(-2, 3, (B, G, P, H * s, W * s), generator=g).float()
+    go = torch.randint(-2, 3, (B, G * cg, H * s, W * s), generator=g).float()
+    off = torch.randint(-7, 8, (B, 2 * G * P, H * s, W * s), generator=g).float() * 0.5
+    v = torch.zeros(B, G * cg, H, W)
+    runs = []
+    for _ in range(2):
+        ad, vd, od = (x.to(DEV) for x in (attn, v, off))
+        vd.requires_grad_()
+        sapa_amd.deform_av(ad, vd, od, P, s, G).backward(go.to(DEV))
+        runs.append(vd.grad.cpu())
+    _, gv, _ = coracle.deform_av_backward(go.double(), attn.double(), v.double(), off.double(),
+                                          P, s, G, 'f64')
+    assert torch.equal(runs[0].double(), gv)
+    assert torch.equal(runs[0], runs[1])
