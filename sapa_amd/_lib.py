@@ -80,6 +80,21 @@ def check(status, what):
     raise SapaHipError(f'{what}: {msg} (status {status})')
 
 
+# SAPA_AMD_POISON=1 fills every buffer the kernels are meant to overwrite with
+# NaN first, so that a skipped element shows up in any comparison (test aid).
+_POISON = os.environ.get('SAPA_AMD_POISON', '') not in ('', '0')
+
+
+def new_out(like, shape=None):
+    """A buffer that a kernel overwrites completely.  The reference allocates
+    these zero-filled (new_zeros, sapa/sapa/sapa_func.py:24); since every
+    element is written, the fill is skipped here."""
+    shape = like.shape if shape is None else shape
+    if _POISON:
+        return like.new_full(shape, float('nan'))
+    return like.new_empty(shape)
+
+
 def ptr(t):
     return None if t is None else t.data_ptr()
 

@@ -23,9 +23,9 @@ def _compute_dtype(t):
 def _deform_qk_backward(grad_output, query, key, offset, P, s, G, needs=(True, True, True)):
     cdt = _compute_dtype(query)
     go, q, k, off = (t.contiguous().to(cdt) for t in (grad_output, query, key, offset))
-    gq = torch.zeros_like(q) if needs[0] else None
+    gq = _lib.new_out(q) if needs[0] else None
     gk = torch.zeros_like(k) if needs[1] else None
-    goff = torch.zeros_like(off) if needs[2] else None
+    goff = _lib.new_out(off) if needs[2] else None
     _lib.require_cuda_contiguous(grad_output=go, query=q, key=k, offset=off)
     n, c, h, w = k.size()
     _lib.call('sapa_deform_qk_backward', k.device, _lib.ptr(go), _lib.ptr(q), _lib.ptr(k),
@@ -38,9 +38,9 @@ def _deform_qk_backward(grad_output, query, key, offset, P, s, G, needs=(True, T
 def _deform_av_backward(grad_output, attn, value, offset, P, s, G, needs=(True, True, True)):
     cdt = _compute_dtype(value)
     go, a, v, off = (t.contiguous().to(cdt) for t in (grad_output, attn, value, offset))
-    ga = torch.zeros_like(a) if needs[0] else None
+    ga = _lib.new_out(a) if needs[0] else None
     gv = torch.zeros_like(v) if needs[1] else None
-    goff = torch.zeros_like(off) if needs[2] else None
+    goff = _lib.new_out(off) if needs[2] else None
     _lib.require_cuda_contiguous(grad_output=go, attn=a, value=v, offset=off)
     n, c, h, w = v.size()
     _lib.call('sapa_deform_av_backward', v.device, _lib.ptr(go), _lib.ptr(a), _lib.ptr(v),
@@ -73,7 +73,7 @@ class DeformQKFunction(Function):
         ctx.offset_size = offset.size()
 
         n, c, h, w = query.size()
-        output = query.new_zeros((n, groups, num_point, h, w))
+        output = _lib.new_out(query, (n, groups, num_point, h, w))
         if query.is_cuda:
             _lib.require_cuda_contiguous(query=query, key=key, offset=offset)
             _lib.call('sapa_deform_qk_forward', query.device, _lib.ptr(query), _lib.ptr(key),
@@ -122,7 +122,7 @@ class DeformAVFunction(Function):
         ctx.offset_size = offset.size()
 
         n, c, h, w = value.size()
-        output = value.new_zeros((n, c, scale_factor * h, scale_factor * w))
+        output = _lib.new_out(value, (n, c, scale_factor * h, scale_factor * w))
         if attn.is_cuda:
             _lib.require_cuda_contiguous(attn=attn, value=value, offset=offset)
             _lib.call('sapa_deform_av_forward', value.device, _lib.ptr(attn), _lib.ptr(value),
@@ -226,7 +226,7 @@ class DeformSAPAFusedFunction(Function):
         ctx.offset_layout = offset_layout
 
         n, c, h, w = value.size()
-        output = value.new_zeros((n, c, scale_factor * h, scale_factor * w))
+        output = _lib.new_out(value, (n, c, scale_factor * h, scale_factor * w))
         if value.is_cuda:
             _lib.require_cuda_contiguous(query=query, key=key, value=value, offset=offset)
             _lib.call('sapa_deform_fused_forward_from', value.device, _lib.ptr(query),

@@ -29,8 +29,8 @@ def _qk_backward(grad_output, query, key, kernel_size, scale_factor, need_q=True
         return (None if gq is None else gq.to(query.dtype),
                 None if gk is None else gk.to(key.dtype))
     grad_output = grad_output.contiguous()
-    grad_query = torch.zeros_like(query) if need_q else None
-    grad_key = torch.zeros_like(key) if need_k else None
+    grad_query = _lib.new_out(query) if need_q else None
+    grad_key = _lib.new_out(key) if need_k else None
     _lib.require_cuda_contiguous(grad_output=grad_output, query=query, key=key)
     n, c, h, w = key.size()
     _lib.call('sapa_qk_backward', key.device, _lib.ptr(grad_output), _lib.ptr(query),
@@ -46,8 +46,8 @@ def _av_backward(grad_output, attn, value, kernel_size, scale_factor, need_a=Tru
         return (None if ga is None else ga.to(attn.dtype),
                 None if gv is None else gv.to(value.dtype))
     grad_output = grad_output.contiguous()
-    grad_attn = torch.zeros_like(attn) if need_a else None
-    grad_value = torch.zeros_like(value) if need_v else None
+    grad_attn = _lib.new_out(attn) if need_a else None
+    grad_value = _lib.new_out(value) if need_v else None
     _lib.require_cuda_contiguous(grad_output=grad_output, attn=attn, value=value)
     n, c, h, w = value.size()
     _lib.call('sapa_av_backward', value.device, _lib.ptr(grad_output), _lib.ptr(attn),
@@ -72,7 +72,7 @@ class QKFunction(Function):
         ctx.key_size = key.size()
 
         n, c, h, w = key.size()
-        output = key.new_zeros((n, kernel_size ** 2, h * scale_factor, w * scale_factor))
+        output = _lib.new_out(key, (n, kernel_size ** 2, h * scale_factor, w * scale_factor))
         if key.is_cuda:
             _lib.require_cuda_contiguous(key=key, query=query)
             _lib.call('sapa_qk_forward', key.device, _lib.ptr(query), _lib.ptr(key),
@@ -113,7 +113,7 @@ class AVFunction(Function):
         ctx.value_size = value.size()
 
         n, c, h, w = value.size()
-        output = value.new_zeros((n, c, h * scale_factor, w * scale_factor))
+        output = _lib.new_out(value, (n, c, h * scale_factor, w * scale_factor))
         if value.is_cuda:
             _lib.require_cuda_contiguous(value=value, attn=attn)
             _lib.call('sapa_av_forward', value.device, _lib.ptr(attn), _lib.ptr(value),
@@ -219,7 +219,7 @@ class SAPAFusedFunction(Function):
 
         n, d, h, w = key.size()
         c = value.size(1)
-        output = value.new_zeros((n, c, h * scale_factor, w * scale_factor))
+        output = _lib.new_out(value, (n, c, h * scale_factor, w * scale_factor))
         if value.is_cuda:
             _lib.require_cuda_contiguous(value=value, key=key, query=query)
             _lib.call('sapa_fused_forward', value.device, _lib.ptr(query), _lib.ptr(key),
