@@ -126,6 +126,9 @@ def main():
     ap.add_argument('--dtype', default='fp32', choices=['fp32', 'bf16'])
     ap.add_argument('--workload', default='fpn_large',
                     choices=sorted(WORKLOADS) + sorted(DEFORM_WORKLOADS))
+    ap.add_argument('--pass', dest='direction', default='forward', choices=['forward', 'train'],
+                    help="'train' times the fused forward plus its backward (all input "
+                         'gradients) through the autograd API instead of the forward alone')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--calibration-copy', action='store_true',
                     help='after the timed region, run 5 device copies of 1 GiB (a kernel of '
@@ -168,6 +171,20 @@ def main():
                                               out.data_ptr(), B, d, C, H, W, K, s, code,
                                               stream.cuda_stream), 'sapa_fused_forward')
 
+    train = args.direction == 'train'
+    if train:
+        import sapa_amd
+        go = torch.randn(B, C, H * s, W * s, device=dev).to(dtype)
+        leaves = [t.requires_grad_() for t in ((q, key, v, off) if deform else (q, key, v))]
+        if deform:
+            def step():
+                y = sapa_amd.deform_sapa_fused(q, key, v, off, P, s, G)
+                torch.autograd.grad(y, leaves, go)
+        else:
+            def step():
+                y = sapa_amd.sapa_fused(q, key, v, K, s)
+                torch.autograd.grad(y, leaves, go)
+
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -205,6 +222,15 @@ def main():
               f'{H}x{W}->{H * s}x{W * s} K={K} s={s} {args.dtype}, NCHW')
         kern = ('sapa_b_tiled_kernel (fused mode)' if (K, s) == (5, 2)
                 else 'sapa_b_mfma_kernel (fused mode)')
+    if train:
+        # backward: read grad_out, q, key, value (offset); write every input gradient
+        hi_px, lo_px = B * H * s * W * s, B * H * W
+        qc = G * d if deform else d
+        abytes += esize * (hi_px * (C + 2 * qc) + 2 * lo_px * (qc + C))
+        if deform:
+            abytes += esize * hi_px * 2 * (2 * G * P)
+        what = what.replace('forward', 'forward + backward')
+        kern = 'several (see profiles/)'
     achieved = abytes / (ms * 1e-3) / 1e9
     rec = {
         'metric': f'upsampled Gpix/s, {what}, 1 GPU',
@@ -227,12 +253,12 @@ def main():
             'peak': HBM_PEAK_GBS,
             'unit': 'GB/s',
             'frac': achieved / HBM_PEAK_GBS,
-            'traffic': MEASURED_TRAFFIC_BYTES.get((args.workload, args.dtype)),
+            'traffic': None if train else MEASURED_TRAFFIC_BYTES.get((args.workload, args.dtype)),
             'algorithmic_bytes': abytes,
             'kernel': kern,
         },
     }
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and not train:
         if deform:
             from oracle import torch_oracle
             q0, k0, v0, o0 = (t[:1].float().cpu() for t in (q, key, v, off))

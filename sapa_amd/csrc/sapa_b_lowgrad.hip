@@ -30,8 +30,6 @@
 
 namespace sapa {
 
-namespace {
-
 template <int N> struct FVec;
 template <> struct FVec<2> { typedef float type __attribute__((ext_vector_type(2))); };
 template <> struct FVec<4> { typedef float type __attribute__((ext_vector_type(4))); };
@@ -162,7 +160,7 @@ lowgrad_gather_kernel(const float *__restrict__ hi, const float *__restrict__ w,
 }
 
 template <int K, int S, int NWX, int NWY, int CH, int VEC>
-hipError_t launch_geom(const void *hi, const void *w, void *out, int B, int C, int H, int W,
+static hipError_t lowgrad_launch_geom(const void *hi, const void *w, void *out, int B, int C, int H, int W,
                        hipStream_t st) {
     constexpr int TW = 16 * NWX, TH = 4 * NWY, NT = 64 * NWX * NWY;
     const int tiles_x = (W + TW - 1) / TW, tiles_y = (H + TH - 1) / TH;
@@ -183,14 +181,12 @@ hipError_t launch_geom(const void *hi, const void *w, void *out, int B, int C, i
 }
 
 template <int K, int VEC>
-hipError_t launch_k(const void *hi, const void *w, void *out, int B, int C, int H, int W,
+static hipError_t lowgrad_launch_k(const void *hi, const void *w, void *out, int B, int C, int H, int W,
                     hipStream_t st) {
     const bool wide = (W + 31) / 32 * 32 * 0.9 <= (W + 15) / 16 * 16;
-    return wide ? launch_geom<K, 2, 2, 2, 2, VEC>(hi, w, out, B, C, H, W, st)
-                : launch_geom<K, 2, 1, 2, 2, VEC>(hi, w, out, B, C, H, W, st);
+    return wide ? lowgrad_launch_geom<K, 2, 2, 2, 2, VEC>(hi, w, out, B, C, H, W, st)
+                : lowgrad_launch_geom<K, 2, 1, 2, 2, VEC>(hi, w, out, B, C, H, W, st);
 }
-
-}  // namespace
 
 // fp32, (K, s) in {(3, 2), (5, 2)}, hi / w aligned to s elements;
 // hipErrorNotSupported otherwise (the caller then takes the generic kernel).
@@ -199,12 +195,12 @@ hipError_t lowres_grad_tiled_launch(const void *hi, const void *w, void *out, in
                                     int W, int K, int s, int dtype, hipStream_t st) {
     if (dtype != 0 || s != 2 || (K != 3 && K != 5)) return hipErrorNotSupported;
     if ((uintptr_t)hi % 8 || (uintptr_t)w % 8) return hipErrorNotSupported;
-    if (K == 3) return launch_k<3, 2>(hi, w, out, B, C, H, W, st);
+    if (K == 3) return lowgrad_launch_k<3, 2>(hi, w, out, B, C, H, W, st);
     // 16-byte staging loads when the rows of hi allow it (the window starts
     // r * s = 4 pixels left of a tile, which keeps them aligned)
     const bool v4 = (uintptr_t)hi % 16 == 0 && W % 2 == 0;
-    return v4 ? launch_k<5, 4>(hi, w, out, B, C, H, W, st)
-              : launch_k<5, 2>(hi, w, out, B, C, H, W, st);
+    return v4 ? lowgrad_launch_k<5, 4>(hi, w, out, B, C, H, W, st)
+              : lowgrad_launch_k<5, 2>(hi, w, out, B, C, H, W, st);
 }
 
 }  // namespace sapa

@@ -28,8 +28,6 @@
 
 namespace sapa {
 
-namespace {
-
 template <int S, int TPW, int TPH, int CH>
 __global__ void __launch_bounds__(TPW *TPH *S *S)
 deform_lowgrad_lds_kernel(const float *__restrict__ hi, const float *__restrict__ sc,
@@ -164,7 +162,7 @@ deform_lowgrad_lds_kernel(const float *__restrict__ hi, const float *__restrict_
 }
 
 template <int S, int TPW, int TPH, int CH>
-hipError_t launch_geom(const void *hi, const void *sc, const void *offset, void *grad_low, int B,
+static hipError_t deform_lowgrad_launch_geom(const void *hi, const void *sc, const void *offset, void *grad_low, int B,
                        int Cx, int H, int W, int P, int G, hipStream_t st) {
     constexpr int NT = TPW * TPH * S * S;
     const int tiles_x = (W + TPW - 1) / TPW, tiles_y = (H + TPH - 1) / TPH;
@@ -177,8 +175,6 @@ hipError_t launch_geom(const void *hi, const void *sc, const void *offset, void 
     return hipGetLastError();
 }
 
-}  // namespace
-
 // fp32, s in {1, 2, 4}; hipErrorNotSupported otherwise (the caller then takes
 // the per-term atomic kernel).  grad_low is accumulated into.
 hipError_t deform_lowgrad_lds_launch(const void *hi, const void *sc, const void *offset,
@@ -186,9 +182,9 @@ hipError_t deform_lowgrad_lds_launch(const void *hi, const void *sc, const void 
                                      int G, int dtype, hipStream_t st) {
     if (dtype != 0) return hipErrorNotSupported;
     switch (s) {
-        case 1: return launch_geom<1, 16, 16, 4>(hi, sc, offset, grad_low, B, Cx, H, W, P, G, st);
-        case 2: return launch_geom<2, 8, 8, 8>(hi, sc, offset, grad_low, B, Cx, H, W, P, G, st);
-        case 4: return launch_geom<4, 4, 4, 8>(hi, sc, offset, grad_low, B, Cx, H, W, P, G, st);
+        case 1: return deform_lowgrad_launch_geom<1, 16, 16, 4>(hi, sc, offset, grad_low, B, Cx, H, W, P, G, st);
+        case 2: return deform_lowgrad_launch_geom<2, 8, 8, 8>(hi, sc, offset, grad_low, B, Cx, H, W, P, G, st);
+        case 4: return deform_lowgrad_launch_geom<4, 4, 4, 8>(hi, sc, offset, grad_low, B, Cx, H, W, P, G, st);
         default: return hipErrorNotSupported;
     }
 }
