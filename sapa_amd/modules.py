@@ -6,12 +6,64 @@ sapa_deform.py:7-62, so its checkpoints load.  `x` is the low-res feature
 (source of key and value), `y` the high-res guide (source of the query).
 `fused=True` (default) runs attention as the single fused launch; False
 runs the reference's three-step composition on the separate operators.
+`fold_norm=True` folds the GroupNorms into the 1x1 projections (one batched
+GEMM per projection straight from the un-normalised feature).
 """
+import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
 from .deform_func import deform_av, deform_qk, deform_sapa_fused
 from .sapa_func import av, qk, sapa_fused
+
+
+def norm_project(x, norm, *convs):
+    """conv(norm(x)) for a GroupNorm and one or more 1x1 convolutions fed by
+    it (sapa_base.py:26-36: norm_y -> q, norm_x -> k) without materialising
+    norm(x): the normalisation is affine per (image, channel), so it folds into
+    per-image projection weights
+
+        W'[b,o,c] = W[o,c] * gamma[c] * rstd[b,g(c)]
+        b'[b,o]   = bias[o] + sum_c W[o,c] * (beta[c] - gamma[c] * mean[b,g(c)] * rstd[b,g(c)])
+
+    and each projection becomes one batched GEMM  W'[b] @ x[b]  reading x
+    directly.  That removes the write and re-read of norm(x) (2.2 GB for the
+    largest FPN level in fp32).  Exact in real arithmetic; in floating point it
+    differs from the two-step form by rounding only, with one caveat: the mean
+    is subtracted after the GEMM instead of before it, so it loses accuracy if
+    |mean| exceeds the standard deviation of a group by many orders of magnitude.
+    Statistics are taken in fp32, like GroupNorm's.  Returns a list, one output
+    per convolution, each [B, out, H, W] contiguous."""
+    B, C, H, W = x.shape
+    G = norm.num_groups
+    xg = x.reshape(B, G, -1)
+    if x.dtype in (torch.float16, torch.bfloat16):
+        # fp32 accumulation straight from the 16-bit tensor (no fp32 copy)
+        mean = xg.mean(dim=2, dtype=torch.float32)
+        sq = torch.linalg.vector_norm(xg, dim=2, dtype=torch.float32).square() / xg.shape[2]
+        var = (sq - mean * mean).clamp_min(0)
+    else:
+        var, mean = torch.var_mean(xg.float(), dim=2, unbiased=False)
+    rstd = torch.rsqrt(var + norm.eps)
+    per_c = C // G
+    rstd_c = rstd.repeat_interleave(per_c, dim=1)                    # [B, C]
+    mean_c = mean.repeat_interleave(per_c, dim=1)
+    gamma = norm.weight.float() if norm.weight is not None else x.new_ones(C, dtype=torch.float32)
+    beta = norm.bias.float() if norm.bias is not None else x.new_zeros(C, dtype=torch.float32)
+    scale = gamma.unsqueeze(0) * rstd_c                              # [B, C]
+    shift = beta.unsqueeze(0) - mean_c * scale                       # [B, C]
+    x3 = x.reshape(B, C, H * W)
+    outs = []
+    for conv in convs:
+        assert conv.kernel_size == (1, 1) and conv.groups == 1
+        w = conv.weight.reshape(conv.out_channels, C).float()
+        w_b = (w.unsqueeze(0) * scale.unsqueeze(1)).to(x.dtype)      # [B, O, C]
+        b_b = torch.einsum('oc,bc->bo', w, shift)
+        if conv.bias is not None:
+            b_b = b_b + conv.bias.float().unsqueeze(0)
+        out = torch.baddbmm(b_b.to(x.dtype).unsqueeze(2), w_b, x3)   # [B, O, HW]
+        outs.append(out.view(B, conv.out_channels, H, W))
+    return outs
 
 
 def _init_projection(m):
@@ -24,7 +76,7 @@ def _init_projection(m):
 
 class SAPA(nn.Module):
     def __init__(self, dim_y, dim_x=None, up_factor=2, up_kernel_size=5, embedding_dim=32,
-                 qkv_bias=True, norm=True, fused=True):
+                 qkv_bias=True, norm=True, fused=True, fold_norm=False):
         super().__init__()
         dim_x = dim_y if dim_x is None else dim_x
         self.up_factor = up_factor
@@ -32,6 +84,8 @@ class SAPA(nn.Module):
         self.embedding_dim = embedding_dim
         self.norm = norm
         self.fused = fused
+        # fold_norm: GroupNorm folded into the q / k projections (norm_project)
+        self.fold_norm = fold_norm
         if norm:
             self.norm_y = nn.GroupNorm(32, dim_y)
             self.norm_x = nn.GroupNorm(32, dim_x)
@@ -41,6 +95,9 @@ class SAPA(nn.Module):
 
     def forward(self, y, x):
         # the value is the un-normalised x; only the key sees norm_x(x)
+        if self.norm and self.fold_norm:
+            (q,), (k,) = norm_project(y, self.norm_y, self.q), norm_project(x, self.norm_x, self.k)
+            return self.attention(q, k, x)
         x_ = self.norm_x(x) if self.norm else x
         if self.norm:
             y = self.norm_y(y)
@@ -56,9 +113,10 @@ class SAPA(nn.Module):
 
 class SAPADeform(nn.Module):
     def __init__(self, dim_y, dim_x=None, up_factor=2, num_point=9, groups=4, embedding_dim=32,
-                 qkv_bias=True, high_offset=True, norm=False, fused=True):
+                 qkv_bias=True, high_offset=True, norm=False, fused=True, fold_norm=False):
         super().__init__()
         dim_x = dim_y if dim_x is None else dim_x
+        self.fold_norm = fold_norm
         self.up_factor = up_factor
         self.num_point = num_point
         self.groups = groups
@@ -78,20 +136,24 @@ class SAPADeform(nn.Module):
         self.apply(_init_projection)
 
     def forward(self, y, x):
-        x_ = self.norm_x(x) if self.norm else x
-        if self.norm:
-            y = self.norm_y(y)
-        q, k = self.q(y), self.k(x_)
+        if self.norm and self.fold_norm:
+            (q,) = norm_project(y, self.norm_y, self.q)
+            k, offset_lo = norm_project(x, self.norm_x, self.k, self.offset)
+        else:
+            x_ = self.norm_x(x) if self.norm else x
+            if self.norm:
+                y = self.norm_y(y)
+            q, k, offset_lo = self.q(y), self.k(x_), self.offset(x_)
         if self.fused:
             # the kernel reads the offset convolution's output in place
             return deform_sapa_fused(q.contiguous(), k.contiguous(), x.contiguous(),
-                                     self.offset(x_).contiguous(), self.num_point,
+                                     offset_lo.contiguous(), self.num_point,
                                      self.up_factor, self.groups,
                                      'pixel_shuffle' if self.high_offset else 'nearest')
         if self.high_offset:
-            offset = F.pixel_shuffle(self.offset(x_), upscale_factor=self.up_factor)
+            offset = F.pixel_shuffle(offset_lo, upscale_factor=self.up_factor)
         else:
-            offset = F.interpolate(self.offset(x_), scale_factor=self.up_factor)
+            offset = F.interpolate(offset_lo, scale_factor=self.up_factor)
         return self.attention(q, k, x, offset)
 
     def attention(self, q, k, x, offset):

@@ -379,3 +379,28 @@ def test_window_staging_vector_widths(coracle, W):
     assert_f32_close(got, coracle.sapa_fused(q, key, v[:, 1:].contiguous(), K, s, 'f32'), f'W={W} unaligned')
     logits = sapa_amd.qk(q.to(DEV), key.to(DEV), K, s).cpu()
     assert torch.equal(logits, coracle.qk(q, key, K, s, 'f32'))
+
+
+def test_module_with_folded_groupnorm_matches_two_step():
+    """SAPA(fold_norm=True) = the same module with GroupNorm and the 1x1
+    projections as separate steps (sapa_base.py:26-36), up to rounding."""
+    torch.manual_seed(5)
+    m = sapa_amd.SAPA(64, embedding_dim=16).to(DEV)
+    torch.nn.init.normal_(m.norm_y.weight, 1.0, 0.2)
+    torch.nn.init.normal_(m.norm_x.bias, 0.0, 0.2)
+    torch.nn.init.normal_(m.q.weight, std=0.2)
+    torch.nn.init.normal_(m.k.weight, std=0.2)
+    y = torch.randn(2, 64, 18, 22, device=DEV) + 0.5
+    x = torch.randn(2, 64, 9, 11, device=DEV)
+    with torch.no_grad():
+        want = m(y, x)
+        m.fold_norm = True
+        got = m(y, x)
+    torch.testing.assert_close(got, want, rtol=1e-4, atol=1e-4)
+    md = sapa_amd.SAPADeform(64, embedding_dim=8, norm=True).to(DEV)
+    torch.nn.init.normal_(md.offset.weight, std=0.1)
+    with torch.no_grad():
+        want = md(y, x)
+        md.fold_norm = True
+        got = md(y, x)
+    torch.testing.assert_close(got, want, rtol=1e-4, atol=1e-4)
