@@ -372,7 +372,10 @@ static hipError_t launch_mode(int mode, const void *q, const void *key, const vo
     if (mode == TILED_FUSED || mode == TILED_AV) {
         const long tiles = (long)tiles_x * tiles_y * B;
         const int max_groups = C / (4 * CH) > 0 ? C / (4 * CH) : 1;
-        while (cgroups * 2 <= max_groups && tiles * cgroups * 2 <= 512) cgroups *= 2;
+        // (16-bit tensors: up to four per CU -- their recomputed logits cost
+        // relatively less -- measured on the FPN levels)
+        const long limit = sizeof(T) == 2 ? 1024 : 512;
+        while (cgroups * 2 <= max_groups && tiles * cgroups * 2 <= limit) cgroups *= 2;
 #ifdef SAPA_TUNE_CGROUPS
         cgroups = SAPA_TUNE_CGROUPS;
 #endif
