@@ -112,6 +112,18 @@ int sapa_av_backward(const void *grad_out, const void *attn, const void *value,
                      int B, int C, int H, int W, int K, int s,
                      int dtype, void *stream);
 
+/* Gradient of the logits through the aggregation and the softmax in one
+ * launch:  g = d(loss)/d(attn) = sum_c value[n,c,nbr_k] * grad_out[n,c,ph,pw]  (the
+ * grad_attn of sapa_av_backward), then
+ *   grad_logits[n,k,ph,pw] = attn[n,k,ph,pw] * (g[k] - sum_k' g[k'] * attn[n,k',ph,pw]),
+ * the backward of F.softmax(., dim=1) in SAPA.attention (sapa_base.py:39-40).
+ * grad_out [B,C,sH,sW], attn [B,K*K,sH,sW], value [B,C,H,W] -> grad_logits
+ * [B,K*K,sH,sW].  SAPA_ERR_UNSUPPORTED when no register-tiled kernel covers
+ * (K, s): use sapa_av_backward and a separate softmax backward then. */
+int sapa_av_backward_logits(const void *grad_out, const void *attn, const void *value,
+                            void *grad_logits, int B, int C, int H, int W,
+                            int K, int s, int dtype, void *stream);
+
 /* Softmax over the middle axis of x [N,R,M] -> y [N,R,M] (max-subtracted,
  * fp32 arithmetic for 16-bit types).  Covers the reference's
  * F.softmax(logits, dim=1) on [B,K*K,sH,sW] (sapa_base.py:39: N=B, R=K*K,

@@ -27,6 +27,7 @@ SIGNATURES = {
     'sapa_softmax_forward': [_vp, _vp, _ll, _i, _ll, _i, _vp],
     'sapa_fused_forward': [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_qk_softmax_forward': [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
+    'sapa_av_backward_logits': [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_deform_qk_forward': [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_deform_qk_backward': [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_deform_av_forward': [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
@@ -124,6 +125,20 @@ def require_cuda_contiguous(**tensors):
                 raise RuntimeError(f'{name} is on {t.device}, {first[0]} on {first[1].device}')
             if t.dtype != first[1].dtype:
                 raise RuntimeError(f'{name} is {t.dtype}, {first[0]} is {first[1].dtype}')
+
+
+UNSUPPORTED = -2   # SAPA_ERR_UNSUPPORTED: a valid request this build has no kernel for
+
+
+def call_status(name, device, *args):
+    """Like `call`, but hands back SAPA_ERR_UNSUPPORTED instead of raising on
+    it, for entry points that have a composite fallback."""
+    with torch.cuda.device(device):
+        stream = torch.cuda.current_stream(device).cuda_stream
+        status = getattr(lib(), name)(*args, stream)
+    if status != UNSUPPORTED:
+        check(status, name)
+    return status
 
 
 def call(name, device, *args):

@@ -226,6 +226,21 @@ int sapa_av_backward(const void *grad_out, const void *attn, const void *value, 
     return SAPA_OK;
 }
 
+int sapa_av_backward_logits(const void *grad_out, const void *attn, const void *value,
+                            void *grad_logits, int B, int C, int H, int W, int K, int s, int dtype,
+                            void *stream) {
+    const int rc = check_window_args(B, C, C, H, W, K, s, dtype);
+    if (rc != SAPA_OK) return rc;
+    if (B == 0) return SAPA_OK;
+    if (!grad_out || !attn || !value || !grad_logits) return SAPA_ERR_INVALID_ARGUMENT;
+    // only the register-tiled kernel has this epilogue
+    const hipError_t e =
+        sapa_b_tiled_launch(TILED_QK_SOFTMAX_BWD, grad_out, value, attn, nullptr, grad_logits, B, C,
+                            0, H, W, K, s, dtype, (hipStream_t)stream);
+    if (e == hipErrorNotSupported) return SAPA_ERR_UNSUPPORTED;
+    return finish(e);
+}
+
 int sapa_softmax_forward(const void *x, void *y, long long N, int R, long long M, int dtype,
                          void *stream) {
     if (!dtype_ok(dtype) || N < 0 || R < 1 || M < 0) return SAPA_ERR_INVALID_ARGUMENT;

@@ -21,7 +21,10 @@ hipError_t fused_pixel_launch(const void *q, const void *key, const void *value,
                               int dtype, hipStream_t st);
 
 // sapa_b_tiled.hip: LDS-tiled kernels.  `mode` selects the stages:
-enum TiledMode { TILED_QK = 0, TILED_QK_SOFTMAX = 1, TILED_AV = 2, TILED_FUSED = 3 };
+// TILED_QK_SOFTMAX_BWD: the similarity g = qk(q, key) followed by the softmax
+// backward against the weights in attn_in: out[k] = attn[k] * (g[k] - sum_k' g[k'] * attn[k']).
+enum TiledMode { TILED_QK = 0, TILED_QK_SOFTMAX = 1, TILED_AV = 2, TILED_FUSED = 3,
+                 TILED_QK_SOFTMAX_BWD = 4 };
 // Returns hipErrorNotSupported when no tiled kernel covers (K, s, dtype, shape);
 // the caller then takes the generic path.
 hipError_t sapa_b_tiled_launch(int mode, const void *q, const void *key, const void *attn_in,

@@ -250,7 +250,10 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
         const unsigned qmask = active ? 0xffffffffu : 0u;
         // q is fetched PF channels ahead of its use (a ring of PF x NJ
         // registers), so HBM latency hides behind the FMAs of PF channels.
-        constexpr int PF = CH < 4 ? CH : 4;
+#ifndef SAPA_TILED_PF
+#define SAPA_TILED_PF 4
+#endif
+        constexpr int PF = CH < SAPA_TILED_PF ? CH : SAPA_TILED_PF;
         static_assert(CH % PF == 0, "prefetch ring must divide the chunk");
         A qr[PF][NJ];
         auto load_q = [&](int c, A (&dst)[NJ]) {
@@ -302,6 +305,33 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
         if (DO_SOFTMAX) {
 #pragma unroll
             for (int jj = 0; jj < NJ; ++jj) softmax_inplace<A, KK>(a[jj]);
+        }
+        if (MODE == TILED_QK_SOFTMAX_BWD && active) {
+            // a[][] holds g = d(loss)/d(attn); turn it into d(loss)/d(logits).
+            // The weights are read twice (the second time from cache) rather
+            // than kept in another K*K registers per child.
+            const T *ap = attn_in + (long)n * KK * hplane + hpix;
+            A dot[NJ];
+#pragma unroll
+            for (int jj = 0; jj < NJ; ++jj) dot[jj] = 0;
+#pragma unroll
+            for (int k = 0; k < KK; ++k)
+#pragma unroll
+                for (int cy = 0; cy < CY; ++cy) {
+                    const VecS v = *(const VecS *)(ap + (long)k * hplane + (long)cy * hW);
+#pragma unroll
+                    for (int cx = 0; cx < S; ++cx)
+                        dot[cy * S + cx] = fma_(a[cy * S + cx][k], (A)v.v[cx], dot[cy * S + cx]);
+                }
+#pragma unroll
+            for (int k = 0; k < KK; ++k)
+#pragma unroll
+                for (int cy = 0; cy < CY; ++cy) {
+                    const VecS v = *(const VecS *)(ap + (long)k * hplane + (long)cy * hW);
+#pragma unroll
+                    for (int cx = 0; cx < S; ++cx)
+                        a[cy * S + cx][k] = (A)v.v[cx] * (a[cy * S + cx][k] - dot[cy * S + cx]);
+                }
         }
         if (!DO_AV && active) {
             T *op = out + (long)n * KK * hplane + hpix;
@@ -394,7 +424,7 @@ static hipError_t launch_mode(int mode, const void *q, const void *key, const vo
         break;
     switch (mode) {
         SAPA_TM_CASE(TILED_QK) SAPA_TM_CASE(TILED_QK_SOFTMAX) SAPA_TM_CASE(TILED_AV)
-        SAPA_TM_CASE(TILED_FUSED)
+        SAPA_TM_CASE(TILED_FUSED) SAPA_TM_CASE(TILED_QK_SOFTMAX_BWD)
         default: return hipErrorInvalidValue;
     }
 #undef SAPA_TM_CASE

@@ -188,13 +188,27 @@ def _fused_backward(grad_output, query, key, value, K, s, needs=(True, True, Tru
         return tuple(None if g is None else g.to(t.dtype)
                      for g, t in zip(grads, (query, key, value)))
     attn = _qk_softmax_forward(query, key, K, s)
-    grad_attn, grad_value = _av_backward(grad_output, attn, value, K, s,
-                                         need_a=need_q or need_k, need_v=need_v)
-    grad_query = grad_key = None
+    grad_query = grad_key = grad_logits = None
     if need_q or need_k:
-        # softmax backward in fp32: g_logit = attn * (g_attn - sum_k g_attn * attn)
-        a32, g32 = attn.float(), grad_attn.float()
-        grad_logits = (a32 * (g32 - (g32 * a32).sum(dim=1, keepdim=True))).to(attn.dtype)
+        # grad of the logits through av and softmax in one launch where the
+        # library has it ...
+        grad_output = grad_output.contiguous()
+        _lib.require_cuda_contiguous(grad_output=grad_output, attn=attn, value=value)
+        n, c, h, w = value.size()
+        grad_logits = _lib.new_out(attn)
+        status = _lib.call_status('sapa_av_backward_logits', value.device, _lib.ptr(grad_output),
+                                  _lib.ptr(attn), _lib.ptr(value), _lib.ptr(grad_logits), n, c, h,
+                                  w, K, s, _lib.dtype_code(value))
+        if status == _lib.UNSUPPORTED:
+            grad_logits = None
+    grad_attn, grad_value = _av_backward(
+        grad_output, attn, value, K, s,
+        need_a=(need_q or need_k) and grad_logits is None, need_v=need_v)
+    if need_q or need_k:
+        if grad_logits is None:
+            # ... else softmax backward in fp32: attn * (g_attn - sum_k g_attn * attn)
+            a32, g32 = attn.float(), grad_attn.float()
+            grad_logits = (a32 * (g32 - (g32 * a32).sum(dim=1, keepdim=True))).to(attn.dtype)
         grad_query, grad_key = _qk_backward(grad_logits, query, key, K, s, need_q, need_k)
     return grad_query, grad_key, grad_value
 

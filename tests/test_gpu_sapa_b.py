@@ -404,3 +404,29 @@ def test_module_with_folded_groupnorm_matches_two_step():
         md.fold_norm = True
         got = md(y, x)
     torch.testing.assert_close(got, want, rtol=1e-4, atol=1e-4)
+
+
+def test_av_backward_logits_entry_point(coracle):
+    """sapa_av_backward_logits = softmax backward applied to the grad_attn of
+    the aggregation, against float64 arithmetic on the oracle's grad_attn."""
+    from sapa_amd import _lib
+    g = gen(160)
+    B, C, H, W, K, s = 2, 11, 9, 21, 5, 2
+    attn = torch.softmax(randn(g, B, K * K, H * s, W * s) * 2, dim=1)
+    v, go = randn(g, B, C, H, W), randn(g, B, C, H * s, W * s)
+    ga, _ = coracle.av_backward(go.double(), attn.double(), v.double(), K, s, 'f64')
+    a64 = attn.double()
+    want = a64 * (ga - (ga * a64).sum(dim=1, keepdim=True))
+    ad, vd, god = dev(attn, v, go)
+    got = torch.full_like(ad, float('nan'))
+    status = _lib.call_status('sapa_av_backward_logits', ad.device, _lib.ptr(god), _lib.ptr(ad),
+                              _lib.ptr(vd), _lib.ptr(got), B, C, H, W, K, s, 0)
+    assert status == 0
+    torch.testing.assert_close(got.cpu().double(), want, rtol=1e-4, atol=1e-5)
+    # no register-tiled instance for K = 7, s = 1: the caller is told so
+    a7 = torch.softmax(randn(g, 1, 49, 6, 7), dim=1).to(DEV)
+    out7 = torch.empty_like(a7)
+    status = _lib.call_status('sapa_av_backward_logits', a7.device, _lib.ptr(randn(g, 1, 3, 6, 7).to(DEV)),
+                              _lib.ptr(a7), _lib.ptr(randn(g, 1, 3, 6, 7).to(DEV)), _lib.ptr(out7),
+                              1, 3, 6, 7, 7, 1, 0)
+    assert status == _lib.UNSUPPORTED
