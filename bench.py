@@ -121,8 +121,9 @@ def cpu_baseline(q, key, v, K, s, budget_s=20.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
-    ap.add_argument('--steps', type=int, default=100)
-    ap.add_argument('--warmup', type=int, default=10)
+    ap.add_argument('--steps', type=int, default=200)
+    # the GPU's clocks take ~50 ms of work to settle: warm up for about that long
+    ap.add_argument('--warmup', type=int, default=200)
     ap.add_argument('--dtype', default='fp32', choices=['fp32', 'bf16'])
     ap.add_argument('--workload', default='fpn_large',
                     choices=sorted(WORKLOADS) + sorted(DEFORM_WORKLOADS))

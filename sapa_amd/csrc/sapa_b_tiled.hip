@@ -2,9 +2,9 @@
 // qk -> softmax -> av forward, all from one template.
 //
 // Work decomposition (NCHW tensors, so the contiguous axis is W):
-//   * a workgroup owns a tile of TW x TH = (16*NWX) x (4*NWY) low-res parent
-//     cells of one image; a wave owns 16 x 4 of them, lane = (lx 0..15,
-//     ly 0..3);
+//   * a wave owns WLX x (64/WLX) low-res parent cells of one image (16 x 4 or
+//     32 x 2), lane = (lx 0..WLX-1, ly 0..64/WLX-1); a workgroup owns a tile
+//     of NWX x NWY waves, TW x TH = (WLX*NWX) x ((64/WLX)*NWY) parents;
 //   * a thread owns CY x S of the S x S high-res children of its parent
 //     (CY = S: all of them; CY < S: S/CY waves share the parent rows), and
 //     keeps their K*K logits / weights in registers (CY*S*K*K values);
@@ -14,7 +14,8 @@
 //     Every staged value is reused by the CY*S children in registers and by
 //     up to K*K parents through LDS;
 //   * q is read and the output written exactly once, as S-wide vectors that
-//     are contiguous across the 16 lanes of a row (S*16 elements per row).
+//     are contiguous across the WLX lanes of a row (S*WLX elements per row:
+//     the longer these row segments, the fewer partial cache lines).
 // LDS layout: two channels side by side in one LDS row, each in HALF >= WW+1
 // floats with HALF = 8 mod 16, so the row stride 2*HALF is 16 mod 32 (48 for
 // a 16-wide tile).  That puts the four 16-lane rows of a wave on disjoint
@@ -76,7 +77,7 @@ __device__ __forceinline__ void store_stream(T *p, const Vec<T, N> &v) {
 #ifndef SAPA_TILED_WPE
 #define SAPA_TILED_WPE 3
 #endif
-template <typename T, int K, int S, int CY, int NWX, int NWY, int CH, int VEC, int MODE>
+template <typename T, int K, int S, int CY, int NWX, int NWY, int CH, int VEC, int WLX, int MODE>
 __global__ void __launch_bounds__(64 * NWX * NWY * (S / CY)) __attribute__((amdgpu_waves_per_eu(SAPA_TILED_WPE, SAPA_TILED_WPE)))
 sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
                     const T *__restrict__ attn_in, const T *__restrict__ value,
@@ -86,7 +87,9 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
     constexpr int KK = K * K, R = (K - 1) / 2;
     constexpr int NSUB = S / CY;           // waves sharing one band of parent rows
     constexpr int NT = 64 * NWX * NWY * NSUB;    // threads per workgroup
-    constexpr int TW = 16 * NWX, TH = 4 * NWY;   // parents per workgroup
+    constexpr int WLY = 64 / WLX;                  // a wave owns WLX x WLY parents
+    static_assert(WLX == 16 || WLX == 32 || WLX == 64, "wave shape");
+    constexpr int TW = WLX * NWX, TH = WLY * NWY;   // parents per workgroup
     // The window is staged as VEC-wide vectors (VEC = 1, 2 or 4 elements):
     // its left edge is moved out to a multiple of VEC and its width rounded up.
     constexpr int HL = (R + VEC - 1) / VEC * VEC;                 // left halo, staged
@@ -137,7 +140,7 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int sub = wave % NSUB, wxy = wave / NSUB;
-    const int lx = (wxy % NWX) * 16 + (lane & 15), ly = (wxy / NWX) * 4 + (lane >> 4);
+    const int lx = (wxy % NWX) * WLX + (lane % WLX), ly = (wxy / NWX) * WLY + (lane / WLX);
     const int x0 = tx * TW, y0 = ty * TH;          // tile origin (parents)
     const int px = x0 + lx, py = y0 + ly;
     const bool active = px < W && py < H;
@@ -388,11 +391,11 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
 }
 
 // ------------------------------------------------------------------ launcher
-template <typename T, int K, int S, int CY, int NWX, int NWY, int CH, int VEC>
+template <typename T, int K, int S, int CY, int NWX, int NWY, int CH, int VEC, int WLX>
 static hipError_t launch_mode(int mode, const void *q, const void *key, const void *attn_in,
                               const void *value, void *out, int B, int d, int C, int H, int W,
                               hipStream_t st) {
-    constexpr int TW = 16 * NWX, TH = 4 * NWY, NT = 64 * NWX * NWY * (S / CY);
+    constexpr int TW = WLX * NWX, TH = (64 / WLX) * NWY, NT = 64 * NWX * NWY * (S / CY);
     const int tiles_x = (W + TW - 1) / TW, tiles_y = (H + TH - 1) / TH;
     // Few tiles: slice the value channels over several workgroups per tile,
     // up to two workgroups per CU (256 CUs) -- beyond that the recomputed
@@ -417,7 +420,7 @@ static hipError_t launch_mode(int mode, const void *q, const void *key, const vo
     const dim3 grid(per_xcd * 8), block(NT);
 #define SAPA_TM_CASE(M)                                                                       \
     case M:                                                                                   \
-        hipLaunchKernelGGL((sapa_b_tiled_kernel<T, K, S, CY, NWX, NWY, CH, VEC, M>), grid, block, 0, st,    \
+        hipLaunchKernelGGL((sapa_b_tiled_kernel<T, K, S, CY, NWX, NWY, CH, VEC, WLX, M>), grid, block, 0, st,    \
                            (const T *)q, (const T *)key, (const T *)attn_in,                  \
                            (const T *)value, (T *)out, d, C, H, W, tiles_x, tiles_y, (int)nb, \
                            per_xcd, cgroups, cper);                                                          \
@@ -451,7 +454,9 @@ static hipError_t launch_t(int mode, const void *q, const void *key, const void 
         auto padded = [&](int tw, int th) {
             return (double)((W + tw - 1) / tw * tw) * (double)((H + th - 1) / th * th);
         };
-        const double c12 = padded(16, 8), c14 = 0.96 * padded(16, 16), c22 = 0.88 * padded(32, 8);
+        // 32 x 8 tiles are built from 32 x 2-parent waves: their hi-res row
+        // segments are twice as long as those of 16 x 4-parent waves.
+        const double c12 = padded(16, 8), c14 = 0.96 * padded(16, 16), c22 = 0.81 * padded(32, 8);
         // The low-res windows are staged with 4- or 2-element vector loads
         // when rows and base pointers allow it (scalar loads otherwise).
         auto aligned = [&](int vec) {
@@ -459,11 +464,13 @@ static hipError_t launch_t(int mode, const void *q, const void *key, const void 
             return W % vec == 0 && (!key || (uintptr_t)key % a == 0) &&
                    (!value || (uintptr_t)value % a == 0);
         };
-#define SAPA_GEOM(NWX, NWY, VEC) \
-    launch_mode<T, 5, 2, 2, NWX, NWY, 8, VEC>(mode, q, key, attn_in, value, out, B, d, C, H, W, st)
-        if (c22 <= c12 && c22 <= c14) return aligned(4) ? SAPA_GEOM(2, 2, 4) : SAPA_GEOM(2, 2, 1);
-        if (c14 <= c12) return aligned(2) ? SAPA_GEOM(1, 4, 2) : SAPA_GEOM(1, 4, 1);
-        return aligned(2) ? SAPA_GEOM(1, 2, 2) : SAPA_GEOM(1, 2, 1);
+#define SAPA_GEOM(NWX, NWY, VEC, WLX)                                                            \
+    launch_mode<T, 5, 2, 2, NWX, NWY, 8, VEC, WLX>(mode, q, key, attn_in, value, out, B, d, C, H, \
+                                                   W, st)
+        if (c22 <= c12 && c22 <= c14)
+            return aligned(4) ? SAPA_GEOM(1, 4, 4, 32) : SAPA_GEOM(1, 4, 1, 32);
+        if (c14 <= c12) return aligned(2) ? SAPA_GEOM(1, 4, 2, 16) : SAPA_GEOM(1, 4, 1, 16);
+        return aligned(2) ? SAPA_GEOM(1, 2, 2, 16) : SAPA_GEOM(1, 2, 1, 16);
 #undef SAPA_GEOM
 #endif
     }
@@ -475,7 +482,7 @@ hipError_t sapa_b_tiled_launch(int mode, const void *q, const void *key, const v
                                int K, int s, int dtype, hipStream_t st) {
     switch (dtype) {
         case 0: return launch_t<float>(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, st);
-#ifndef SAPA_TUNE_GEOM
+#if !defined(SAPA_TUNE_GEOM) || defined(SAPA_TUNE_ALLTYPES)
         case 2: return launch_t<f16_t>(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, st);
         case 3: return launch_t<bf16_t>(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, st);
 #endif
