@@ -46,16 +46,16 @@ DEFORM_WORKLOADS = {
 # scaled by what the same counters read for a plain copy of known size); see
 # the summaries under profiles/.  None = not measured for that case.
 MEASURED_TRAFFIC_BYTES = {
-    # profiles/sapa_b_fused_fpn_large_fp32.md: (326480.1 * 2.0000 + 1157602.9 * 1.0000) KiB
-    ('fpn_large', 'fp32'): 1853999908,
-    # profiles/sapa_b_fused_fpn_large_bf16.md: (156402.1 * 2.0000 + 542512.3 * 1.0000) KiB
-    ('fpn_large', 'bf16'): 875836093,
-    # profiles/sapa_b_mfma_fused_stress_bf16.md: (61545.7 * 1.9999 + 304717.3 * 1.0000) KiB
-    ('stress', 'bf16'): 438072935,
-    # profiles/sapa_d_lds_fused_deform_p9_fp32.md: (133133.8 * 1.9999 + 131526.6 * 1.0000) KiB
-    ('deform_p9', 'fp32'): 407334344,
-    # profiles/sapa_d_lds_fused_deform_p25_fp32.md: (343691.2 * 1.9999 + 131078.6 * 1.0000) KiB
-    ('deform_p25', 'fp32'): 838086343,
+    # profiles/sapa_b_fused_fpn_large_fp32.md: (324281.2 * 1.9999 + 1106514.0 * 1.0000) KiB
+    ('fpn_large', 'fp32'): 1797181513,
+    # profiles/sapa_b_fused_fpn_large_bf16.md: (156041.3 * 1.9999 + 541653.7 * 1.0000) KiB
+    ('fpn_large', 'bf16'): 874217926,
+    # profiles/sapa_b_mfma_fused_stress_bf16.md: (61582.7 * 1.9999 + 304782.4 * 1.0000) KiB
+    ('stress', 'bf16'): 438215372,
+    # profiles/sapa_d_lds_fused_deform_p9_fp32.md: (132709.9 * 1.9999 + 131503.8 * 1.0000) KiB
+    ('deform_p9', 'fp32'): 406442924,
+    # profiles/sapa_d_lds_fused_deform_p25_fp32.md: (343906.3 * 1.9999 + 131079.0 * 1.0000) KiB
+    ('deform_p25', 'fp32'): 838527266,
 }
 
 
