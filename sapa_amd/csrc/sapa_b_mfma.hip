@@ -308,8 +308,10 @@ static hipError_t launch_t(int mode, const void *q, const void *key, const void 
     if (K == 5 && s == 2)
         return launch_mode<T, 5, 2, SAPA_MFMA_TUNE>(mode, q, key, attn_in, value, out, B, d, C, H, W, st);
 #else
-    // s = 2: 32x4-parent tiles, 8 waves; s = 4: 16x4-parent tiles, 16 waves
-    // (4 child groups per parent row).  K = 5, s = 2 is left to the VALU
+    // s = 2: 32x4-parent tiles, 8 waves; s = 4: 16x2-parent tiles, 8 waves (4
+    // child groups per parent row) and 16-channel chunks: with s*s = 16
+    // children per parent the low-res halo is cheap, and two workgroups per CU
+    // overlap each other's barriers (a 16-wave workgroup owns the CU alone).  K = 5, s = 2 is left to the VALU
     // kernel, which is the faster one at that size.
 #define SAPA_MM_INST(KV, SV, ...)                                                              \
     if (K == KV && s == SV)                                                                    \
@@ -317,9 +319,13 @@ static hipError_t launch_t(int mode, const void *q, const void *key, const void 
                                                    H, W, st);
     SAPA_MM_INST(3, 2, 2, 4, 8, 5)
     SAPA_MM_INST(7, 2, 2, 4, 8, 4)
-    SAPA_MM_INST(3, 4, 1, 4, 8, 5)
-    SAPA_MM_INST(5, 4, 1, 4, 8, 4)
-    SAPA_MM_INST(7, 4, 1, 4, 8, 4)
+    SAPA_MM_INST(3, 4, 1, 2, 16, 5)
+    SAPA_MM_INST(5, 4, 1, 2, 16, 4)
+#ifdef SAPA_MFMA_TUNE_74
+    SAPA_MM_INST(7, 4, SAPA_MFMA_TUNE_74)
+#else
+    SAPA_MM_INST(7, 4, 1, 2, 16, 4)
+#endif
 #undef SAPA_MM_INST
 #endif
     return hipErrorNotSupported;
