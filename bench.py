@@ -50,8 +50,8 @@ MEASURED_TRAFFIC_BYTES = {
     ('fpn_large', 'fp32'): 1797181513,
     # profiles/sapa_b_fused_fpn_large_bf16.md: (156041.3 * 1.9999 + 541653.7 * 1.0000) KiB
     ('fpn_large', 'bf16'): 874217926,
-    # profiles/sapa_b_mfma_fused_stress_bf16.md: (61582.7 * 1.9999 + 304782.4 * 1.0000) KiB
-    ('stress', 'bf16'): 438215372,
+    # profiles/sapa_b_mfma_fused_stress_bf16.md: (39700.2 * 1.9999 + 292841.7 * 1.0000) KiB
+    ('stress', 'bf16'): 381173848,
     # profiles/sapa_d_lds_fused_deform_p9_fp32.md: (132709.9 * 1.9999 + 131503.8 * 1.0000) KiB
     ('deform_p9', 'fp32'): 406442924,
     # profiles/sapa_d_lds_fused_deform_p25_fp32.md: (343906.3 * 1.9999 + 131079.0 * 1.0000) KiB
