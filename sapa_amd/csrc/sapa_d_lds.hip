@@ -99,9 +99,15 @@ deform_lds_kernel(const T *__restrict__ q, const T *__restrict__ key,
             __syncthreads();
             stage(key + (ch0 + c0) * lplane, nvalid);
             __syncthreads();
+            // the next point's offsets are fetched while this point is evaluated
+            A ow = (A)op.base[0], oh = (A)op.base[op.stride];
             for (int p = 0; p < P; ++p) {
-                const A kw = pw + (A)op.base[(long)(2 * p) * op.stride];
-                const A kh = ph + (A)op.base[(long)(2 * p + 1) * op.stride];
+                const A kw = pw + ow, kh = ph + oh;
+                {
+                    const int pn = p + 1 < P ? p + 1 : p;
+                    ow = (A)op.base[(long)(2 * pn) * op.stride];
+                    oh = (A)op.base[(long)(2 * pn + 1) * op.stride];
+                }
                 const A scv = (A)sp[(long)p * hplane];
                 A gw = c0 == 0 ? (A)0 : lgt[(2 * p) * NT];
                 A gh = c0 == 0 ? (A)0 : lgt[(2 * p + 1) * NT];
@@ -160,9 +166,15 @@ deform_lds_kernel(const T *__restrict__ q, const T *__restrict__ key,
             __syncthreads();                       // the previous chunk's readers are done
             stage(key + (ch0 + c0) * lplane, nvalid);
             __syncthreads();
+            // the next point's offsets are fetched while this point is evaluated
+            A ow = (A)op.base[0], oh = (A)op.base[op.stride];
             for (int p = 0; p < P; ++p) {
-                const A kw = pw + (A)op.base[(long)(2 * p) * op.stride];
-                const A kh = ph + (A)op.base[(long)(2 * p + 1) * op.stride];
+                const A kw = pw + ow, kh = ph + oh;
+                {
+                    const int pn = p + 1 < P ? p + 1 : p;
+                    ow = (A)op.base[(long)(2 * pn) * op.stride];
+                    oh = (A)op.base[(long)(2 * pn + 1) * op.stride];
+                }
                 A acc = c0 == 0 ? (A)0 : lgt[p * NT];
                 Tap<A> tap;
                 if (tap_setup(kh, kw, H, W, tap)) {
@@ -218,9 +230,15 @@ deform_lds_kernel(const T *__restrict__ q, const T *__restrict__ key,
             A o[CH];
 #pragma unroll
             for (int ch = 0; ch < CH; ++ch) o[ch] = 0;
+            // the next point's offsets are fetched while this point is evaluated
+            A ow = (A)op.base[0], oh = (A)op.base[op.stride];
             for (int p = 0; p < P; ++p) {
-                const A kw = pw + (A)op.base[(long)(2 * p) * op.stride];
-                const A kh = ph + (A)op.base[(long)(2 * p + 1) * op.stride];
+                const A kw = pw + ow, kh = ph + oh;
+                {
+                    const int pn = p + 1 < P ? p + 1 : p;
+                    ow = (A)op.base[(long)(2 * pn) * op.stride];
+                    oh = (A)op.base[(long)(2 * pn + 1) * op.stride];
+                }
                 const A wa = lgt[p * NT];
                 Tap<A> tap;
                 if (tap_setup(kh, kw, H, W, tap)) {

@@ -101,10 +101,16 @@ deform_lowgrad_lds_kernel(const float *__restrict__ hi, const float *__restrict_
         for (int ch = 0; ch < CH; ++ch) hs[ch] = (double)hv[ch] * scale;
 
         if (active) {
+            // the next point's offsets and scalar are fetched while this one is scattered
+            float ow = op[0], oh = op[hplane], sn = sp[0];
             for (int p = 0; p < P; ++p) {
-                const float kw = pw + op[(long)(2 * p) * hplane];
-                const float kh = ph + op[(long)(2 * p + 1) * hplane];
-                const float scv = sp[(long)p * hplane];
+                const float kw = pw + ow, kh = ph + oh, scv = sn;
+                {
+                    const int pn = p + 1 < P ? p + 1 : p;
+                    ow = op[(long)(2 * pn) * hplane];
+                    oh = op[(long)(2 * pn + 1) * hplane];
+                    sn = sp[(long)pn * hplane];
+                }
                 Tap<float> tap;
                 if (!tap_setup(kh, kw, H, W, tap)) continue;
                 const int hl = (int)floor_(kh) - wy0, wl = (int)floor_(kw) - wx0;
