@@ -79,6 +79,37 @@ __device__ __forceinline__ bool tap_setup(A kh, A kw, int H, int W, Tap<A> &t) {
     return true;
 }
 
+// The same sample position for a kernel that gathers from an LDS window whose
+// origin is the low-res cell (wy0, wx0) and which is WH x WW cells large:
+// everything is computed unconditionally (no early exit), `guard` is the
+// reference's range test and `inwin` says that all four corners lie in the
+// window, where out-of-image cells hold zeros.  Weights are the expressions of
+// tap_setup, bit for bit.
+template <typename A>
+struct WinTap {
+    A w1, w2, w3, w4;
+    int hl, wl;          // window-relative low corner
+    bool guard, inwin;
+};
+
+template <typename A>
+__device__ __forceinline__ WinTap<A> win_tap(A kh, A kw, int H, int W, int wy0, int wx0, int WH,
+                                             int WW) {
+    WinTap<A> t;
+    t.guard = kh > (A)-1 && kh < (A)H && kw > (A)-1 && kw < (A)W;
+    const A fh = floor_(kh), fw = floor_(kw);
+    t.hl = (int)fh - wy0;
+    t.wl = (int)fw - wx0;
+    t.inwin = t.guard && t.hl >= 0 && t.hl <= WH - 2 && t.wl >= 0 && t.wl <= WW - 2;
+    const A lh = kh - fh, lw = kw - fw;
+    const A hh = (A)1 - lh, hw = (A)1 - lw;
+    t.w1 = hh * hw;
+    t.w2 = hh * lw;
+    t.w3 = lh * hw;
+    t.w4 = lh * lw;
+    return t;
+}
+
 // w1*v1 + w2*v2 + w3*v3 + w4*v4, evaluated left to right with FMAs.
 template <typename T, typename A>
 __device__ __forceinline__ A tap_sample(const T *plane, const Tap<A> &t) {

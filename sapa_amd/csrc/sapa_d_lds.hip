@@ -240,26 +240,29 @@ deform_lds_kernel(const T *__restrict__ q, const T *__restrict__ key,
                     oh = (A)op.base[(long)(2 * pn + 1) * op.stride];
                 }
                 const A wa = lgt[p * NT];
-                Tap<A> tap;
-                if (tap_setup(kh, kw, H, W, tap)) {
-                    const int hl = (int)floor_(kh) - wy0, wl = (int)floor_(kw) - wx0;
-                    if (hl >= 0 && hl <= WH - 2 && wl >= 0 && wl <= WW - 2) {
-                        const A *wp = win + hl * RS + wl;
+                // Straight-line path for the common case (tap inside the
+                // window): same expressions as tap_setup, results kept only
+                // where the guard holds, so that consecutive points can be
+                // interleaved by the scheduler.
+                const WinTap<A> wt = win_tap(kh, kw, H, W, wy0, wx0, WH, WW);
+                const A *wp = win + (wt.inwin ? wt.hl * RS + wt.wl : 0);
 #pragma unroll
-                        for (int ch = 0; ch < CH; ++ch) {
-                            A val = tap.w1 * wp[ch * CS];
-                            val = fma_(tap.w2, wp[ch * CS + 1], val);
-                            val = fma_(tap.w3, wp[ch * CS + RS], val);
-                            val = fma_(tap.w4, wp[ch * CS + RS + 1], val);
-                            o[ch] = fma_(val, wa, o[ch]);
-                        }
-                    } else {
-                        const T *vp = value + (ch0 + c0) * lplane;
+                for (int ch = 0; ch < CH; ++ch) {
+                    A val = wt.w1 * wp[ch * CS];
+                    val = fma_(wt.w2, wp[ch * CS + 1], val);
+                    val = fma_(wt.w3, wp[ch * CS + RS], val);
+                    val = fma_(wt.w4, wp[ch * CS + RS + 1], val);
+                    const A on = fma_(val, wa, o[ch]);
+                    o[ch] = wt.inwin ? on : o[ch];
+                }
+                if (wt.guard && !wt.inwin) {       // rare: the tap left the window
+                    Tap<A> tap;
+                    tap_setup(kh, kw, H, W, tap);
+                    const T *vp = value + (ch0 + c0) * lplane;
 #pragma unroll
-                        for (int ch = 0; ch < CH; ++ch)
-                            if (ch < nvalid)
-                                o[ch] = fma_(tap_sample(vp + (long)ch * lplane, tap), wa, o[ch]);
-                    }
+                    for (int ch = 0; ch < CH; ++ch)
+                        if (ch < nvalid)
+                            o[ch] = fma_(tap_sample(vp + (long)ch * lplane, tap), wa, o[ch]);
                 }
             }
             if (active) {
