@@ -1,10 +1,11 @@
 #!/usr/bin/env python3
 """Benchmark of the fused SAPA-B forward (qk -> softmax -> av, one launch) on
-one MI355X, on the workload BASELINE.json's metric is quoted on.
+one MI355X; the default workload is the largest FPN level (B=16, C=256, d=64,
+K=5, 100x168 -> 200x336, fp32).
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype fp32|bf16]
                     [--workload fpn_large|fpn_mid|fpn_small|stress|deform_p25|deform_p9|deform_p5]
-                    [--no-cpu-baseline]
+                    [--pass forward|train] [--no-cpu-baseline] [--calibration-copy]
 
 A step is one fused forward over the whole synthetic batch, inputs already
 resident in HBM.  Prints ONE JSON line: output Gpix/s, the HBM roofline of
@@ -138,7 +139,8 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit('bench.py: this build measures one GPU only (the operators are '
-                 'single-device; see DESIGN.md for how the path would shard). Use --gpus 1.')
+                 'single-device: a batch shards over GPUs by image, with no communication). '
+                 'Use --gpus 1.')
     if not torch.cuda.is_available():
         sys.exit('bench.py: no GPU visible')
 
