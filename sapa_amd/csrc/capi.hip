@@ -33,8 +33,10 @@ const long long kMaxElems = 1LL << 40;
 hipError_t tiled_launch(int mode, const void *q, const void *key, const void *attn_in,
                         const void *value, void *out, int B, int d, int C, int H, int W, int K,
                         int s, int dtype, hipStream_t st) {
-    hipError_t e = sapa_b_tiled_launch(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s,
-                                       dtype, st);
+    hipError_t e = sapa_b_dot2_launch(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s,
+                                      dtype, st);
+    if (e == hipErrorNotSupported)
+        e = sapa_b_tiled_launch(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, dtype, st);
     if (e == hipErrorNotSupported)
         e = sapa_b_mfma_launch(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, dtype, st);
     return e;

@@ -31,6 +31,13 @@ hipError_t sapa_b_tiled_launch(int mode, const void *q, const void *key, const v
                                const void *value, void *out, int B, int d, int C, int H, int W,
                                int K, int s, int dtype, hipStream_t st);
 
+// sapa_b_dot2.hip: the four forward modes for f16 / bf16 tensors on the
+// two-term dot-product instructions (K = 5, s = 2); hipErrorNotSupported
+// otherwise.
+hipError_t sapa_b_dot2_launch(int mode, const void *q, const void *key, const void *attn_in,
+                              const void *value, void *out, int B, int d, int C, int H, int W,
+                              int K, int s, int dtype, hipStream_t st);
+
 // sapa_b_mfma.hip: the same four modes on the matrix pipe (4x4x1 MFMA, one
 // block per parent); hipErrorNotSupported when (K, s, dtype) has no instance.
 hipError_t sapa_b_mfma_launch(int mode, const void *q, const void *key, const void *attn_in,

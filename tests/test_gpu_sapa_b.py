@@ -160,6 +160,42 @@ def test_16bit_dtypes(coracle, shape, dtype, rel):
     assert_rel_rms_close(got.float(), coracle.sapa_fused(qf, kf, vf, K, s, 'f32a64'), rel, 'fused')
 
 
+# K = 5, s = 2, W a multiple of 4 and at least 32: the 16-bit kernels built on
+# the two-term dot product instructions.  Several tiles in x and y, ragged
+# edges, odd channel counts (the last channel pair / value chunk is partial).
+DOT2_SHAPES = [(2, 7, 11, 13, 36, 5, 2), (1, 16, 8, 8, 32, 5, 2), (1, 33, 20, 9, 68, 5, 2),
+               (1, 5, 3, 3, 100, 5, 2), (1, 1, 1, 1, 32, 5, 2), (2, 18, 70, 17, 44, 5, 2)]
+
+
+@pytest.mark.parametrize('dtype,rel', [(torch.bfloat16, BF16_REL), (torch.float16, F16_REL)])
+@pytest.mark.parametrize('shape', DOT2_SHAPES, ids=['-'.join(map(str, s)) for s in DOT2_SHAPES])
+def test_16bit_dot_product_kernels(coracle, shape, dtype, rel):
+    B, d, C, H, W, K, s = shape
+    g = gen(117)
+    q, key, v = (randn(g, *sh).to(dtype) for sh in
+                 ((B, d, H * s, W * s), (B, d, H, W), (B, C, H, W)))
+    attn = F.softmax(randn(g, B, K * K, H * s, W * s), 1).to(dtype)
+    qf, kf, vf, af = (x.float() for x in (q, key, v, attn))
+    got = sapa_amd.qk(*dev(q, key), K, s)
+    assert got.dtype == dtype
+    # products of 16-bit values are exact in fp32 and the sums are fp32: only
+    # the final rounding to the 16-bit type separates the result from the oracle
+    want = coracle.qk(qf, kf, K, s, 'f32a64')
+    assert_rel_rms_close(got.float(), want, rel, 'qk')
+    if d <= 8:
+        # at most one unit in the last place of the 16-bit type
+        torch.testing.assert_close(got.float().cpu(), want.to(dtype).float(),
+                                   rtol=2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10, atol=1e-6)
+    got = sapa_amd.qk_softmax(*dev(q, key), K, s)
+    want = coracle.softmax(coracle.qk(qf, kf, K, s, 'f32a64').float(), 1, 'f32')
+    assert_rel_rms_close(got.float(), want, rel, 'qk_softmax')
+    got = sapa_amd.av(*dev(attn, v), K, s)
+    assert_rel_rms_close(got.float(), coracle.av(af, vf, K, s, 'f32a64'), rel, 'av')
+    got = sapa_amd.sapa_fused(*dev(q, key, v), K, s)
+    assert got.dtype == dtype
+    assert_rel_rms_close(got.float(), coracle.sapa_fused(qf, kf, vf, K, s, 'f32a64'), rel, 'fused')
+
+
 @pytest.mark.parametrize('shape', [SHAPES[0], SHAPES[6]], ids=[IDS[0], IDS[6]])
 def test_fp64(coracle, shape):
     B, d, C, H, W, K, s = shape
