@@ -49,8 +49,8 @@ DEFORM_WORKLOADS = {
 MEASURED_TRAFFIC_BYTES = {
     # profiles/sapa_b_fused_fpn_large_fp32.md: (324281.2 * 1.9999 + 1106514.0 * 1.0000) KiB
     ('fpn_large', 'fp32'): 1797181513,
-    # profiles/sapa_b_fused_fpn_large_bf16.md: (156041.3 * 1.9999 + 541653.7 * 1.0000) KiB
-    ('fpn_large', 'bf16'): 874217926,
+    # profiles/sapa_b_fused_fpn_large_bf16.md: (174519.2 * 2.0000 + 594522.0 * 1.0000) KiB
+    ('fpn_large', 'bf16'): 966196919,
     # profiles/sapa_b_mfma_fused_stress_bf16.md: (39700.2 * 1.9999 + 292841.7 * 1.0000) KiB
     ('stress', 'bf16'): 381173848,
     # profiles/sapa_d_lds_fused_deform_p9_fp32.md: (132709.9 * 1.9999 + 131503.8 * 1.0000) KiB
@@ -223,8 +223,12 @@ def main():
         what = 'fused SAPA-B forward (qk->softmax->av)'
         wl = (f'{args.workload}: SAPA-B FPN-style B={B} C={C} d={d} '
               f'{H}x{W}->{H * s}x{W * s} K={K} s={s} {args.dtype}, NCHW')
-        kern = ('sapa_b_tiled_kernel (fused mode)' if (K, s) == (5, 2)
-                else 'sapa_b_mfma_kernel (fused mode)')
+        if (K, s) != (5, 2):
+            kern = 'sapa_b_mfma_kernel (fused mode)'
+        elif esize == 2 and W % 4 == 0 and W >= 32:
+            kern = 'sapa_b_dot2_kernel (fused mode)'
+        else:
+            kern = 'sapa_b_tiled_kernel (fused mode)'
     if train:
         # backward: read grad_out, q, key, value (offset); write every input gradient
         hi_px, lo_px = B * H * s * W * s, B * H * W
