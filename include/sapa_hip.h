@@ -149,6 +149,29 @@ int sapa_qk_softmax_forward(const void *query, const void *key, void *attn,
                             int B, int d, int H, int W, int K, int s,
                             int dtype, void *stream);
 
+/* The same four forward operators for tensors in channels-last memory order
+ * (torch.channels_last: a logical [B,C,H,W] tensor stored as [B,H,W,C]):
+ * query [B,sH,sW,d], key [B,H,W,d], value [B,H,W,C], attn [B,sH,sW,K*K],
+ * out [B,sH,sW,C] (qk: [B,sH,sW,K*K]).  The reference requires contiguous
+ * NCHW tensors (CHECK_CONTIGUOUS, sapa/sapa/src/qk_cuda.cpp:35-39); these let
+ * a channels-last model call the operators without a layout copy.  Covered:
+ * SAPA_F32 / F16 / BF16, K in {3, 5}, s = 2, channel counts that are multiples
+ * of 4, tensors aligned to 4 elements; SAPA_ERR_UNSUPPORTED otherwise.  The
+ * channel sums run in tree order: results agree with sapa_*_forward to
+ * rounding (1e-5 relative in fp32), not bit for bit. */
+int sapa_qk_forward_nhwc(const void *query, const void *key, void *out,
+                         int B, int d, int H, int W, int K, int s,
+                         int dtype, void *stream);
+int sapa_qk_softmax_forward_nhwc(const void *query, const void *key, void *attn,
+                                 int B, int d, int H, int W, int K, int s,
+                                 int dtype, void *stream);
+int sapa_av_forward_nhwc(const void *attn, const void *value, void *out,
+                         int B, int C, int H, int W, int K, int s,
+                         int dtype, void *stream);
+int sapa_fused_forward_nhwc(const void *query, const void *key, const void *value,
+                            void *out, int B, int d, int C, int H, int W,
+                            int K, int s, int dtype, void *stream);
+
 /* ------------------------------------------------------------------ SAPA-D */
 
 /* Offset-sampled query-key similarity.

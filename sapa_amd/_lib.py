@@ -28,6 +28,10 @@ SIGNATURES = {
     'sapa_fused_forward': [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_qk_softmax_forward': [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_av_backward_logits': [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
+    'sapa_qk_forward_nhwc': [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
+    'sapa_qk_softmax_forward_nhwc': [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
+    'sapa_av_forward_nhwc': [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
+    'sapa_fused_forward_nhwc': [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_deform_qk_forward': [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_deform_qk_backward': [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_deform_av_forward': [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
@@ -86,14 +90,16 @@ def check(status, what):
 _POISON = os.environ.get('SAPA_AMD_POISON', '') not in ('', '0')
 
 
-def new_out(like, shape=None):
+def new_out(like, shape=None, channels_last=False):
     """A buffer that a kernel overwrites completely.  The reference allocates
     these zero-filled (new_zeros, sapa/sapa/sapa_func.py:24); since every
     element is written, the fill is skipped here."""
     shape = like.shape if shape is None else shape
+    fmt = torch.channels_last if channels_last else torch.contiguous_format
+    out = torch.empty(tuple(shape), dtype=like.dtype, device=like.device, memory_format=fmt)
     if _POISON:
-        return like.new_full(shape, float('nan'))
-    return like.new_empty(shape)
+        out.fill_(float('nan'))
+    return out
 
 
 def ptr(t):
@@ -125,6 +131,35 @@ def require_cuda_contiguous(**tensors):
                 raise RuntimeError(f'{name} is on {t.device}, {first[0]} on {first[1].device}')
             if t.dtype != first[1].dtype:
                 raise RuntimeError(f'{name} is {t.dtype}, {first[0]} is {first[1].dtype}')
+
+
+def memory_layout(**tensors):
+    """'contiguous' when every tensor is contiguous (what the reference
+    requires), 'channels_last' when every tensor is a 4-D device tensor in
+    torch.channels_last order (served without a copy by the *_nhwc entry
+    points); anything else raises like the reference's CHECK_INPUT."""
+    ts = [t for t in tensors.values() if t is not None]
+    if all(t.is_contiguous() for t in ts):
+        require_cuda_contiguous(**tensors)
+        return 'contiguous'
+    if all(t.dim() == 4 and t.is_contiguous(memory_format=torch.channels_last) for t in ts):
+        # same device / dtype checks, on views that are contiguous
+        require_cuda_contiguous(**{k: (None if t is None else t.permute(0, 2, 3, 1))
+                                   for k, t in tensors.items()})
+        return 'channels_last'
+    bad = [k for k, t in tensors.items() if t is not None and not t.is_contiguous()]
+    raise RuntimeError(f'{bad[0]} must be contiguous (or every tensor in torch.channels_last order)')
+
+
+def call_nhwc(name, device, *args):
+    """An *_nhwc entry point; SAPA_ERR_UNSUPPORTED becomes an error that says
+    what the channels-last kernels cover (there is no hidden layout copy)."""
+    status = call_status(name, device, *args)
+    if status == UNSUPPORTED:
+        raise RuntimeError(
+            f'{name}: channels_last tensors are served for float32 / float16 / bfloat16, '
+            'kernel_size 3 or 5, scale_factor 2, channel counts that are multiples of 4; '
+            'call .contiguous() on the inputs for other configurations')
 
 
 UNSUPPORTED = -2   # SAPA_ERR_UNSUPPORTED: a valid request this build has no kernel for

@@ -280,6 +280,44 @@ int sapa_qk_softmax_forward(const void *query, const void *key, void *attn, int 
     return fused_common(1, query, key, nullptr, attn, B, d, d, H, W, K, s, dtype, stream);
 }
 
+// Channels-last memory order: only the kernel of sapa_b_nhwc.hip serves it.
+static int nhwc_common(int mode, const void *query, const void *key, const void *attn,
+                       const void *value, void *out, int B, int d, int C, int H, int W, int K,
+                       int s, int dtype, void *stream) {
+    const int rc = check_window_args(B, d, C, H, W, K, s, dtype);
+    if (rc != SAPA_OK) return rc;
+    if (B == 0) return SAPA_OK;
+    const bool need_qk = mode != TILED_AV, need_av = mode == TILED_AV || mode == TILED_FUSED;
+    if (!out || (need_qk && (!query || !key)) || (need_av && !value) || (mode == TILED_AV && !attn))
+        return SAPA_ERR_INVALID_ARGUMENT;
+    const hipError_t e = sapa_b_nhwc_launch(mode, query, key, attn, value, out, B, d, C, H, W, K, s,
+                                            dtype, (hipStream_t)stream);
+    if (e == hipErrorNotSupported) return SAPA_ERR_UNSUPPORTED;
+    return finish(e);
+}
+
+int sapa_qk_forward_nhwc(const void *query, const void *key, void *out, int B, int d, int H, int W,
+                         int K, int s, int dtype, void *stream) {
+    return nhwc_common(TILED_QK, query, key, nullptr, nullptr, out, B, d, d, H, W, K, s, dtype, stream);
+}
+
+int sapa_qk_softmax_forward_nhwc(const void *query, const void *key, void *attn, int B, int d,
+                                 int H, int W, int K, int s, int dtype, void *stream) {
+    return nhwc_common(TILED_QK_SOFTMAX, query, key, nullptr, nullptr, attn, B, d, d, H, W, K, s,
+                       dtype, stream);
+}
+
+int sapa_av_forward_nhwc(const void *attn, const void *value, void *out, int B, int C, int H,
+                         int W, int K, int s, int dtype, void *stream) {
+    return nhwc_common(TILED_AV, nullptr, nullptr, attn, value, out, B, C, C, H, W, K, s, dtype, stream);
+}
+
+int sapa_fused_forward_nhwc(const void *query, const void *key, const void *value, void *out,
+                            int B, int d, int C, int H, int W, int K, int s, int dtype,
+                            void *stream) {
+    return nhwc_common(TILED_FUSED, query, key, nullptr, value, out, B, d, C, H, W, K, s, dtype, stream);
+}
+
 int sapa_deform_qk_forward_from(const void *query, const void *key, const void *offset,
                                 void *out, int B, int Cq, int H, int W, int P, int s, int G,
                                 int offset_layout, int dtype, void *stream) {

@@ -31,6 +31,13 @@ hipError_t sapa_b_tiled_launch(int mode, const void *q, const void *key, const v
                                const void *value, void *out, int B, int d, int C, int H, int W,
                                int K, int s, int dtype, hipStream_t st);
 
+// sapa_b_nhwc.hip: the four forward modes for tensors in channels-last memory
+// order ([B, H, W, channels]); f32 / f16 / bf16, K in {3, 5}, s = 2, channel
+// counts multiples of 4.  hipErrorNotSupported otherwise.
+hipError_t sapa_b_nhwc_launch(int mode, const void *q, const void *key, const void *attn_in,
+                              const void *value, void *out, int B, int d, int C, int H, int W,
+                              int K, int s, int dtype, hipStream_t st);
+
 // sapa_b_dot2.hip: the four forward modes for f16 / bf16 tensors on the
 // two-term dot-product instructions (K = 5, s = 2); hipErrorNotSupported
 // otherwise.

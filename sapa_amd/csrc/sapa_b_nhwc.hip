@@ -1,0 +1,406 @@
+// SAPA-B for tensors in channels-last memory order (torch.channels_last: the
+// logical [B, C, H, W] tensor stored as [B, H, W, C]): qk, qk+softmax, av and
+// the fused qk -> softmax -> av forward, K in {3, 5}, s = 2.
+//
+// With the channels innermost every access of the operation is a long
+// contiguous run -- a pixel's q is one record of d elements, an output pixel
+// one record of C elements -- so the lanes of a wave run along the CHANNELS:
+//
+//   * a row of 16 lanes owns one low-res parent with its 2 x 2 children; lane i
+//     of the row holds channels 4i .. 4i+3 of the current 64-channel chunk.  A
+//     wave works on 4 parents that are neighbours in x, a workgroup of 4 waves
+//     on a tile of 4 x 4 parents;
+//   * key and value windows (tile + K-1 halo positions) go through LDS as
+//     [position][64 channels], one chunk at a time, double-buffered; a row of
+//     lanes reads one position as 256 contiguous bytes (no bank conflicts);
+//   * logits, one window row (K taps x 4 children = 20 values for K = 5) at a
+//     time: every lane accumulates its 4 channels' part of the products; the 16
+//     lanes of a row are then summed with a 4-step butterfly that halves the
+//     number of live values at every step (the lane keeps the sums whose index
+//     bit matches its lane bit and hands the others to its partner: DPP quad
+//     permutes for lane distances 1 and 2, a cross-lane permute for 4 and 8).
+//     Afterwards lane l holds, for window row ky, the logits with in-row index
+//     16 m + l (index = 4 * kx + child): 100 values in 10 registers per lane;
+//   * softmax per child across the 4 lanes x 10 registers that hold its taps;
+//   * aggregation: the weights stay in those registers; every FMA fetches its
+//     weight from the lane that owns it through a DPP row broadcast
+//     (v_fmac_f32_dpp row_newbcast), so a lane needs 16 accumulators (4 children
+//     x 4 channels) and no copy of the 100 weights.  One 16-byte LDS read feeds
+//     16 FMAs.
+//
+// The channel sums run in tree order, not in the reference kernels' sequential
+// order: results agree with them to rounding (1e-5 relative in fp32), not bit
+// for bit.  Out-of-range window positions are zeros in LDS: logit exactly 0
+// (and part of the softmax), contribution exactly 0.
+#include <utility>
+
+#include "kernels.hpp"
+
+namespace sapa {
+
+namespace nhwc {
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose
+// index is a compile-time constant in the body (DPP controls are immediates)
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+typedef unsigned u32;
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef u32 u32x2 __attribute__((ext_vector_type(2)));
+typedef u32 u32x4 __attribute__((ext_vector_type(4)));
+
+// 4 consecutive elements <-> 4 floats
+template <typename T> struct Quad;
+template <> struct Quad<float> {
+    typedef f32x4 raw;
+    static __device__ __forceinline__ raw buffer_load(__amdgpu_buffer_rsrc_t r, u32 off) {
+        union { u32x4 u; f32x4 f; } x;
+        x.u = __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
+        return x.f;
+    }
+    static __device__ __forceinline__ f32x4 widen(raw v) { return v; }
+    static __device__ __forceinline__ raw narrow(f32x4 v) { return v; }
+};
+template <typename H> struct Quad16 {
+    typedef u32x2 raw;
+    static __device__ __forceinline__ raw buffer_load(__amdgpu_buffer_rsrc_t r, u32 off) {
+        return __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0);
+    }
+    static __device__ __forceinline__ f32x4 widen(raw v) {
+        union { u32x2 u; H h[4]; } x;
+        x.u = v;
+        f32x4 f = {(float)x.h[0], (float)x.h[1], (float)x.h[2], (float)x.h[3]};
+        return f;
+    }
+    static __device__ __forceinline__ raw narrow(f32x4 v) {
+        union { u32x2 u; H h[4]; } x;
+        x.h[0] = (H)v[0];
+        x.h[1] = (H)v[1];
+        x.h[2] = (H)v[2];
+        x.h[3] = (H)v[3];
+        return x.u;
+    }
+};
+template <> struct Quad<f16_t> : Quad16<f16_t> {};
+template <> struct Quad<bf16_t> : Quad16<bf16_t> {};
+
+// value of lane (l ^ D) of the same row of 16 lanes
+template <int D>
+__device__ __forceinline__ float row_xor(float v, int lane) {
+    union { float f; int i; } x, y;
+    x.f = v;
+    if (D == 1) y.i = __builtin_amdgcn_mov_dpp(x.i, 0xB1, 0xf, 0xf, true);        // quad_perm [1,0,3,2]
+    else if (D == 2) y.i = __builtin_amdgcn_mov_dpp(x.i, 0x4E, 0xf, 0xf, true);   // quad_perm [2,3,0,1]
+    else y.i = __builtin_amdgcn_ds_bpermute((lane ^ D) << 2, x.i);
+    return y.f;
+}
+// acc += v * (w of lane SRC of the own row of 16 lanes): one instruction, the
+// weight is fetched through the DPP row broadcast.  The caller keeps two wait
+// states between the last VALU write of w and the first of these.
+template <int SRC>
+__device__ __forceinline__ void fma_bcast(float &acc, float w, float v) {
+    asm("v_fmac_f32_dpp %0, %1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf"
+        : "+v"(acc)
+        : "v"(w), "v"(v), "n"(SRC));
+}
+
+// One butterfly step over lane distance D: n values per lane -> (n + 1) / 2.
+// The lane whose bit D is clear keeps the even-indexed sums, its partner the
+// odd-indexed ones; each adds what the other held of them.
+template <int D, int N>
+__device__ __forceinline__ void halve(const float (&in)[N], float (&out)[(N + 1) / 2], int lane) {
+    const bool hi = lane & D;
+#pragma unroll
+    for (int m = 0; m < (N + 1) / 2; ++m) {
+        const float a = in[2 * m], b = 2 * m + 1 < N ? in[2 * m + 1] : 0.f;
+        const float keep = hi ? b : a, send = hi ? a : b;
+        out[m] = keep + row_xor<D>(send, lane);
+    }
+}
+
+template <typename T, int K, int MODE>
+__global__ void __launch_bounds__(256)
+sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
+                   const T *__restrict__ attn_in, const T *__restrict__ value,
+                   T *__restrict__ out, int d, int C, int H, int W, int tiles_x, int tiles_y,
+                   int nblocks, int per_xcd) {
+    constexpr int S = 2, NJ = 4, KK = K * K, R = (K - 1) / 2;
+    constexpr int TP = 4;                         // tile: TP x TP parents, one row per wave
+    constexpr int WW = TP + K - 1, NPOS = WW * WW;   // window positions
+    constexpr int CHK = 64;                       // channels per chunk: 16 lanes x 4
+    constexpr int BUF = NPOS * CHK;               // floats per LDS buffer
+    constexpr int NT = 256, NPASS = (NPOS * 16 + NT - 1) / NT;   // staging passes (16 quads per position)
+    constexpr int NV = K * NJ;                    // logits of one window row, index = 4 * kx + child
+    constexpr int N1 = (NV + 1) / 2, N2 = (N1 + 1) / 2, N3 = (N2 + 1) / 2;
+    constexpr int RPR = (N3 + 1) / 2, NR = K * RPR;   // registers per window row / in all
+    constexpr bool DO_QK = MODE != TILED_AV;
+    constexpr bool DO_SOFTMAX = MODE == TILED_QK_SOFTMAX || MODE == TILED_FUSED;
+    constexpr bool DO_AV = MODE == TILED_AV || MODE == TILED_FUSED;
+    typedef Quad<T> Q4;
+    typedef typename Q4::raw Raw;
+
+    __shared__ __attribute__((aligned(16))) float lds[2 * BUF];
+
+    const int logical = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
+    if (logical >= nblocks) return;
+    const int tx = logical % tiles_x;
+    const int ty = (logical / tiles_x) % tiles_y;
+    const int n = logical / (tiles_x * tiles_y);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int row = lane >> 4, li = lane & 15;    // parent within the wave, channel quad
+    const int x0 = tx * TP, y0 = ty * TP;
+    const int px = x0 + row, py = y0 + wave;
+    const bool active = px < W && py < H;
+    const int hW = W * S;
+    const long lpix = (long)H * W, hpix = lpix * S * S;
+
+    const int nKc = DO_QK ? (d + CHK - 1) / CHK : 0;
+    const int nVc = DO_AV ? (C + CHK - 1) / CHK : 0;
+    const int ntot = nKc + nVc;
+
+    // ---- staging: pass p, thread t moves channel quad t % 16 of window position
+    // p * 16 + t / 16.  Byte offsets into the image's tensor; 2^31 marks a
+    // position outside the image (beyond every descriptor: zero fill).
+    int spix[NPASS];
+#pragma unroll
+    for (int p = 0; p < NPASS; ++p) {
+        const int pos = p * (NT / 16) + tid / 16;
+        const int gy = y0 - R + pos / WW, gx = x0 - R + pos % WW;
+        spix[p] = (pos < NPOS && gy >= 0 && gy < H && gx >= 0 && gx < W) ? gy * W + gx : -1;
+    }
+    const int sq = tid & 15;                      // channel quad staged by this thread
+    Raw st[NPASS];
+    auto stage_load = [&](int j) {
+        const bool is_key = j < nKc;
+        const int nch = is_key ? d : C;
+        const int c0 = (is_key ? j : j - nKc) * CHK;
+        const T *base = (is_key ? key : value) + (long)n * lpix * nch;
+        const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)base, 0, (int)(lpix * nch * (long)sizeof(T)), 0x00020000);
+        const bool c_ok = c0 + 4 * sq < nch;
+#pragma unroll
+        for (int p = 0; p < NPASS; ++p) {
+            const u32 off = (c_ok && spix[p] >= 0)
+                                ? (u32)(spix[p] * nch + c0 + 4 * sq) * (u32)sizeof(T)
+                                : 0x80000000u;
+            st[p] = Q4::buffer_load(r, off);
+        }
+    };
+    auto stage_store = [&](int j) {
+        float *dst = lds + (j & 1) * BUF;
+#pragma unroll
+        for (int p = 0; p < NPASS; ++p) {
+            const int pos = p * (NT / 16) + tid / 16;
+            if (NPOS % (NT / 16) == 0 || pos < NPOS) *(f32x4 *)(dst + pos * CHK + 4 * sq) = Q4::widen(st[p]);
+        }
+    };
+
+    // this row's window origin: tap (ky, kx) of parent (wave, row) sits at
+    // position (wave + ky) * WW + row + kx
+    const float *win = lds + ((wave * WW + row) * CHK + 4 * li);
+
+    // logits, then weights: w[ky * RPR + m] of lane li is in-row index 16 m + li,
+    // i.e. child li & 3 and kx = 4 m + (li >> 2); ok[m]: that index exists
+    float w[NR];
+    bool ok[RPR];
+#pragma unroll
+    for (int m = 0; m < RPR; ++m) ok[m] = 16 * m + li < NV;
+    const int jl = li & 3, kxl = li >> 2;          // this lane's child and first kx
+    stage_load(0);
+    stage_store(0);
+    __syncthreads();
+
+    if (DO_QK) {
+#pragma unroll
+        for (int i = 0; i < NR; ++i) w[i] = 0.f;
+        const T *qp = q + ((long)n * hpix + (long)(py * S) * hW + (long)px * S) * d;
+        for (int j = 0; j < nKc; ++j) {
+            if (j + 1 < ntot) stage_load(j + 1);
+            const int c0 = j * CHK;
+            // q of the 4 children, this lane's 4 channels (zeros past d and for idle rows)
+            f32x4 qv[NJ];
+            const bool q_ok = active && c0 + 4 * li < d;
+#pragma unroll
+            for (int jj = 0; jj < NJ; ++jj) {
+                Raw raw = {};
+                if (q_ok)
+                    raw = __builtin_nontemporal_load(
+                        (const Raw *)(qp + ((long)(jj >> 1) * hW + (jj & 1)) * d + c0 + 4 * li));
+                qv[jj] = Q4::widen(raw);
+            }
+            const float *wb = win + (j & 1) * BUF;
+#pragma unroll
+            for (int ky = 0; ky < K; ++ky) {
+                float part[NV];
+#pragma unroll
+                for (int kx = 0; kx < K; ++kx) {
+                    const f32x4 kv = *(const f32x4 *)(wb + (ky * WW + kx) * CHK);
+#pragma unroll
+                    for (int jj = 0; jj < NJ; ++jj) {
+                        float a = kv[0] * qv[jj][0];
+#pragma unroll
+                        for (int e = 1; e < 4; ++e) a = fma_(kv[e], qv[jj][e], a);
+                        part[kx * NJ + jj] = a;
+                    }
+                }
+                // sum over the 16 lanes of the row
+                float p1[N1], p2[N2], p3[N3], p4[RPR];
+                halve<1, NV>(part, p1, lane);
+                halve<2, N1>(p1, p2, lane);
+                halve<4, N2>(p2, p3, lane);
+                halve<8, N3>(p3, p4, lane);
+#pragma unroll
+                for (int m = 0; m < RPR; ++m) w[ky * RPR + m] += p4[m];
+            }
+            if (j + 1 < ntot) stage_store(j + 1);
+            __syncthreads();
+        }
+        if (DO_SOFTMAX) {
+            // a child's taps lie in this lane's registers and in the lanes at
+            // distance 4, 8, 12
+            float mx = w[0];                       // in-row index li < NV always
+#pragma unroll
+            for (int i = 1; i < NR; ++i)
+                if (ok[i % RPR]) mx = max_(mx, w[i]);
+            mx = max_(mx, row_xor<4>(mx, lane));
+            mx = max_(mx, row_xor<8>(mx, lane));
+            float sum = 0.f;
+#pragma unroll
+            for (int i = 0; i < NR; ++i) {
+                w[i] = ok[i % RPR] ? exp_(w[i] - mx) : 0.f;
+                sum += w[i];
+            }
+            sum += row_xor<4>(sum, lane);
+            sum += row_xor<8>(sum, lane);
+            const float inv = 1.f / sum;
+#pragma unroll
+            for (int i = 0; i < NR; ++i) w[i] *= inv;
+        }
+        if (!DO_AV && active) {
+            // attn[pixel of child jl][tap]: 4 lanes write 4 consecutive taps
+            T *ap = out + ((long)n * hpix + (long)(py * S + (jl >> 1)) * hW + (long)px * S + (jl & 1)) * KK;
+#pragma unroll
+            for (int i = 0; i < NR; ++i)
+                if (ok[i % RPR]) ap[(i / RPR) * K + 4 * (i % RPR) + kxl] = (T)w[i];
+        }
+    } else {
+        // av(): the weights come from memory, in the same lane layout
+        const T *ap = attn_in + ((long)n * hpix + (long)(py * S + (jl >> 1)) * hW + (long)px * S + (jl & 1)) * KK;
+#pragma unroll
+        for (int i = 0; i < NR; ++i)
+            w[i] = (active && ok[i % RPR]) ? (float)ap[(i / RPR) * K + 4 * (i % RPR) + kxl] : 0.f;
+    }
+
+    if (DO_AV) {
+        asm volatile("s_nop 4");                   // w was just written: DPP reads need two wait states
+        T *op = out + ((long)n * hpix + (long)(py * S) * hW + (long)px * S) * C;
+        for (int j = nKc; j < ntot; ++j) {
+            if (j + 1 < ntot) stage_load(j + 1);
+            const int c0 = (j - nKc) * CHK;
+            const float *wb = win + (j & 1) * BUF;
+            float o[NJ][4];
+#pragma unroll
+            for (int jj = 0; jj < NJ; ++jj)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[jj][e] = 0.f;
+            static_for<K>([&](auto iky) {
+                static_for<K>([&](auto ikx) {
+                    constexpr int ky = decltype(iky)::value, kx = decltype(ikx)::value;
+                    const f32x4 vv = *(const f32x4 *)(wb + (ky * WW + kx) * CHK);
+                    static_for<NJ>([&](auto ijj) {
+                        // the weight lives in register ky * RPR + idx / 16 of lane idx % 16
+                        constexpr int jj = decltype(ijj)::value, idx = kx * NJ + jj;
+                        const float wr = w[ky * RPR + idx / 16];
+                        static_for<4>([&](auto ie) {
+                            constexpr int e = decltype(ie)::value;
+                            fma_bcast<idx % 16>(o[jj][e], wr, vv[e]);
+                        });
+                    });
+                });
+            });
+            if (active && c0 + 4 * li < C) {
+#pragma unroll
+                for (int jj = 0; jj < NJ; ++jj)
+                    __builtin_nontemporal_store(
+                        Q4::narrow(f32x4{o[jj][0], o[jj][1], o[jj][2], o[jj][3]}),
+                        (Raw *)(op + ((long)(jj >> 1) * hW + (jj & 1)) * C + c0 + 4 * li));
+            }
+            if (j + 1 < ntot) stage_store(j + 1);
+            __syncthreads();
+        }
+    }
+}
+
+template <typename T, int K>
+static hipError_t launch_k(int mode, const void *q, const void *key, const void *attn_in,
+                           const void *value, void *out, int B, int d, int C, int H, int W,
+                           hipStream_t st) {
+    const int tiles_x = (W + 3) / 4, tiles_y = (H + 3) / 4;
+    const long nb = (long)tiles_x * tiles_y * B;
+    if (nb > (1L << 30)) return hipErrorNotSupported;
+    const int per_xcd = (int)((nb + 7) / 8);
+    const dim3 grid(per_xcd * 8), block(256);
+#define SAPA_NHWC_CASE(M)                                                                      \
+    case M:                                                                                    \
+        hipLaunchKernelGGL((sapa_b_nhwc_kernel<T, K, M>), grid, block, 0, st, (const T *)q,    \
+                           (const T *)key, (const T *)attn_in, (const T *)value, (T *)out, d,  \
+                           C, H, W, tiles_x, tiles_y, (int)nb, per_xcd);                       \
+        break;
+    switch (mode) {
+        SAPA_NHWC_CASE(TILED_QK) SAPA_NHWC_CASE(TILED_QK_SOFTMAX) SAPA_NHWC_CASE(TILED_AV)
+        SAPA_NHWC_CASE(TILED_FUSED)
+        default: return hipErrorNotSupported;
+    }
+#undef SAPA_NHWC_CASE
+    return hipGetLastError();
+}
+
+template <typename T>
+static hipError_t launch_t(int mode, const void *q, const void *key, const void *attn_in,
+                           const void *value, void *out, int B, int d, int C, int H, int W, int K,
+                           hipStream_t st) {
+    switch (K) {
+        case 3: return launch_k<T, 3>(mode, q, key, attn_in, value, out, B, d, C, H, W, st);
+        case 5: return launch_k<T, 5>(mode, q, key, attn_in, value, out, B, d, C, H, W, st);
+        default: return hipErrorNotSupported;
+    }
+}
+
+}  // namespace nhwc
+
+// Channels-last tensors (q [B, sH, sW, d], key [B, H, W, d], value [B, H, W, C],
+// attn [B, sH, sW, K*K], out like q with C or K*K channels), f32 / f16 / bf16,
+// K in {3, 5}, s = 2, channel counts multiples of 4 and every tensor aligned to
+// 4 elements; one image's key / value tensor below 2^31 bytes.
+// hipErrorNotSupported otherwise.
+hipError_t sapa_b_nhwc_launch(int mode, const void *q, const void *key, const void *attn_in,
+                              const void *value, void *out, int B, int d, int C, int H, int W,
+                              int K, int s, int dtype, hipStream_t st) {
+    if (s != 2 || (K != 3 && K != 5)) return hipErrorNotSupported;
+    const bool need_qk = mode != TILED_AV, need_av = mode == TILED_AV || mode == TILED_FUSED;
+    if ((need_qk && d % 4 != 0) || (need_av && C % 4 != 0)) return hipErrorNotSupported;
+    const int esize = dtype == 0 ? 4 : 2;
+    const long plane = (long)H * W * esize;
+    if ((need_qk && plane * d >= (1L << 31)) || (need_av && plane * C >= (1L << 31)))
+        return hipErrorNotSupported;
+    const void *vec_ptrs[4] = {need_qk ? q : nullptr, need_qk ? key : nullptr,
+                               need_av ? value : nullptr, need_av ? out : nullptr};
+    for (const void *p : vec_ptrs)
+        if (p && (uintptr_t)p % (4 * esize) != 0) return hipErrorNotSupported;
+    switch (dtype) {
+        case 0: return nhwc::launch_t<float>(mode, q, key, attn_in, value, out, B, d, C, H, W, K, st);
+        case 2: return nhwc::launch_t<f16_t>(mode, q, key, attn_in, value, out, B, d, C, H, W, K, st);
+        case 3: return nhwc::launch_t<bf16_t>(mode, q, key, attn_in, value, out, B, d, C, H, W, K, st);
+        default: return hipErrorNotSupported;
+    }
+}
+
+}  // namespace sapa

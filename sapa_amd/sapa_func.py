@@ -23,6 +23,9 @@ def _wide(*tensors):
 
 
 def _qk_backward(grad_output, query, key, kernel_size, scale_factor, need_q=True, need_k=True):
+    # the gradient kernels take contiguous tensors: operands kept in
+    # channels-last order are copied here (the forward pass is the zero-copy one)
+    query, key = query.contiguous(), key.contiguous()
     if key.dtype in (torch.float16, torch.bfloat16):
         gq, gk = _qk_backward(*_wide(grad_output, query, key), kernel_size, scale_factor,
                               need_q, need_k)
@@ -40,6 +43,7 @@ def _qk_backward(grad_output, query, key, kernel_size, scale_factor, need_q=True
 
 
 def _av_backward(grad_output, attn, value, kernel_size, scale_factor, need_a=True, need_v=True):
+    attn, value = attn.contiguous(), value.contiguous()
     if value.dtype in (torch.float16, torch.bfloat16):
         ga, gv = _av_backward(*_wide(grad_output, attn, value), kernel_size, scale_factor,
                               need_a, need_v)
@@ -72,14 +76,14 @@ class QKFunction(Function):
         ctx.key_size = key.size()
 
         n, c, h, w = key.size()
-        output = _lib.new_out(key, (n, kernel_size ** 2, h * scale_factor, w * scale_factor))
-        if key.is_cuda:
-            _lib.require_cuda_contiguous(key=key, query=query)
-            _lib.call('sapa_qk_forward', key.device, _lib.ptr(query), _lib.ptr(key),
-                      _lib.ptr(output), n, c, h, w, kernel_size, scale_factor,
-                      _lib.dtype_code(key))
-        else:
+        if not key.is_cuda:
             raise NotImplementedError
+        nhwc = _lib.memory_layout(key=key, query=query) == 'channels_last'
+        output = _lib.new_out(key, (n, kernel_size ** 2, h * scale_factor, w * scale_factor), nhwc)
+        (_lib.call_nhwc if nhwc else _lib.call)(
+            'sapa_qk_forward_nhwc' if nhwc else 'sapa_qk_forward', key.device, _lib.ptr(query),
+            _lib.ptr(key), _lib.ptr(output), n, c, h, w, kernel_size, scale_factor,
+            _lib.dtype_code(key))
 
         if query.requires_grad or key.requires_grad:
             ctx.save_for_backward(query, key)
@@ -113,14 +117,14 @@ class AVFunction(Function):
         ctx.value_size = value.size()
 
         n, c, h, w = value.size()
-        output = _lib.new_out(value, (n, c, h * scale_factor, w * scale_factor))
-        if value.is_cuda:
-            _lib.require_cuda_contiguous(value=value, attn=attn)
-            _lib.call('sapa_av_forward', value.device, _lib.ptr(attn), _lib.ptr(value),
-                      _lib.ptr(output), n, c, h, w, kernel_size, scale_factor,
-                      _lib.dtype_code(value))
-        else:
+        if not value.is_cuda:
             raise NotImplementedError
+        nhwc = _lib.memory_layout(value=value, attn=attn) == 'channels_last'
+        output = _lib.new_out(value, (n, c, h * scale_factor, w * scale_factor), nhwc)
+        (_lib.call_nhwc if nhwc else _lib.call)(
+            'sapa_av_forward_nhwc' if nhwc else 'sapa_av_forward', value.device, _lib.ptr(attn),
+            _lib.ptr(value), _lib.ptr(output), n, c, h, w, kernel_size, scale_factor,
+            _lib.dtype_code(value))
 
         if attn.requires_grad or value.requires_grad:
             ctx.save_for_backward(attn, value)
@@ -158,11 +162,13 @@ def softmax_k(logits, dim=1):
     return out
 
 
-def _qk_softmax_forward(query, key, kernel_size, scale_factor):
+def _qk_softmax_forward(query, key, kernel_size, scale_factor, nhwc=False):
     n, c, h, w = key.size()
-    attn = key.new_empty((n, kernel_size ** 2, h * scale_factor, w * scale_factor))
-    _lib.call('sapa_qk_softmax_forward', key.device, _lib.ptr(query), _lib.ptr(key),
-              _lib.ptr(attn), n, c, h, w, kernel_size, scale_factor, _lib.dtype_code(key))
+    attn = _lib.new_out(key, (n, kernel_size ** 2, h * scale_factor, w * scale_factor), nhwc)
+    (_lib.call_nhwc if nhwc else _lib.call)(
+        'sapa_qk_softmax_forward_nhwc' if nhwc else 'sapa_qk_softmax_forward', key.device,
+        _lib.ptr(query), _lib.ptr(key), _lib.ptr(attn), n, c, h, w, kernel_size, scale_factor,
+        _lib.dtype_code(key))
     return attn
 
 
@@ -174,14 +180,15 @@ def qk_softmax(query, key, kernel_size, scale_factor):
     _check_odd_kernel(kernel_size)
     if not key.is_cuda:
         raise NotImplementedError
-    _lib.require_cuda_contiguous(key=key, query=query)
-    return _qk_softmax_forward(query, key, kernel_size, scale_factor)
+    nhwc = _lib.memory_layout(key=key, query=query) == 'channels_last'
+    return _qk_softmax_forward(query, key, kernel_size, scale_factor, nhwc)
 
 
 def _fused_backward(grad_output, query, key, value, K, s, needs=(True, True, True)):
     """Gradients of av(softmax(qk(query, key)), value): the attention weights
     are recomputed (one launch), then the three operators' gradients chain."""
     need_q, need_k, need_v = needs
+    query, key, value = query.contiguous(), key.contiguous(), value.contiguous()
     if value.dtype in (torch.float16, torch.bfloat16):
         # the whole chain in fp32, one rounding at the end
         grads = _fused_backward(*_wide(grad_output, query, key, value), K, s, needs)
@@ -233,14 +240,14 @@ class SAPAFusedFunction(Function):
 
         n, d, h, w = key.size()
         c = value.size(1)
-        output = _lib.new_out(value, (n, c, h * scale_factor, w * scale_factor))
-        if value.is_cuda:
-            _lib.require_cuda_contiguous(value=value, key=key, query=query)
-            _lib.call('sapa_fused_forward', value.device, _lib.ptr(query), _lib.ptr(key),
-                      _lib.ptr(value), _lib.ptr(output), n, d, c, h, w, kernel_size,
-                      scale_factor, _lib.dtype_code(value))
-        else:
+        if not value.is_cuda:
             raise NotImplementedError
+        nhwc = _lib.memory_layout(value=value, key=key, query=query) == 'channels_last'
+        output = _lib.new_out(value, (n, c, h * scale_factor, w * scale_factor), nhwc)
+        (_lib.call_nhwc if nhwc else _lib.call)(
+            'sapa_fused_forward_nhwc' if nhwc else 'sapa_fused_forward', value.device,
+            _lib.ptr(query), _lib.ptr(key), _lib.ptr(value), _lib.ptr(output), n, d, c, h, w,
+            kernel_size, scale_factor, _lib.dtype_code(value))
 
         if query.requires_grad or key.requires_grad or value.requires_grad:
             ctx.save_for_backward(query, key, value)

@@ -1,0 +1,138 @@
+"""GPU parity of the SAPA-B operators on tensors in torch.channels_last order
+(served without a layout copy by the *_nhwc entry points of the C ABI) against
+the CPU oracle and against the library's own contiguous path.
+
+Bars: av bit-exact (the tap sum runs in the reference's order).  The channel
+sums of the logits run in tree order, so qk / fused are compared with the
+float64-accumulated oracle: within 1e-5 rel / 1e-6 abs for short sums (d <= 8);
+for long sums (d = 64 ... 128, logits of magnitude 10 ... 30, whose fp32 spacing
+alone is 1e-6 ... 2e-6) within 1e-5 relative to max(|b|, rms) for the logits
+and within the reference's own check tolerance, allclose(atol=1e-5)
+(sapa/sapa/forward_check.py:37-39), for the fused output -- the reference's
+sequential fp32 sums sit at least as far from the float64 value.  16-bit
+within the usual relative bars.
+"""
+import pytest
+import torch
+import torch.nn.functional as F
+
+import sapa_amd
+from helpers import BF16_REL, F16_REL, assert_f32_close, assert_rel_rms_close, gen, randn
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda:0'
+CL = torch.channels_last
+
+# B, d, C, H, W, K: ragged against the 4x4-parent tiles, one / two / partial
+# 64-channel chunks of key and value
+SHAPES = [(2, 4, 8, 5, 7, 5), (1, 64, 64, 8, 8, 5), (1, 68, 72, 6, 9, 5), (1, 8, 132, 3, 4, 3),
+          (2, 128, 4, 9, 5, 3), (1, 16, 256, 1, 1, 5), (1, 4, 4, 13, 2, 5)]
+IDS = ['-'.join(map(str, s)) for s in SHAPES]
+
+
+def cl(*ts):
+    return [t.to(DEV).contiguous(memory_format=CL) for t in ts]
+
+
+def inputs(g, B, d, C, H, W, K, dtype=torch.float32):
+    q, key, v = (randn(g, *sh).to(dtype) for sh in
+                 ((B, d, 2 * H, 2 * W), (B, d, H, W), (B, C, H, W)))
+    attn = F.softmax(randn(g, B, K * K, 2 * H, 2 * W), 1).to(dtype)
+    return q, key, v, attn
+
+
+@pytest.mark.parametrize('shape', SHAPES, ids=IDS)
+def test_fp32_vs_oracle(coracle, shape):
+    B, d, C, H, W, K = shape
+    q, key, v, attn = inputs(gen(300), *shape)
+    got = sapa_amd.qk(*cl(q, key), K, 2)
+    assert got.is_contiguous(memory_format=CL) and got.shape == (B, K * K, 2 * H, 2 * W)
+    want = coracle.qk(q, key, K, 2, 'f32a64')
+    if d <= 8:
+        assert_f32_close(got, want, 'qk')
+    else:
+        assert_rel_rms_close(got, want, 1e-5, 'qk')
+    got = sapa_amd.qk_softmax(*cl(q, key), K, 2)
+    assert got.is_contiguous(memory_format=CL)
+    torch.testing.assert_close(got.cpu(), coracle.softmax(want.float(), 1, 'f32'), rtol=1e-5,
+                               atol=1e-7 if d <= 8 else 1e-5)
+    got = sapa_amd.av(*cl(attn, v), K, 2)
+    assert got.is_contiguous(memory_format=CL) and got.shape == (B, C, 2 * H, 2 * W)
+    # the sum over the K*K taps runs in the reference's order: same bits
+    assert torch.equal(got.cpu(), coracle.av(attn, v, K, 2, 'f32'))
+    got = sapa_amd.sapa_fused(*cl(q, key, v), K, 2)
+    assert got.is_contiguous(memory_format=CL)
+    want = coracle.sapa_fused(q, key, v, K, 2, 'f32a64')
+    if d <= 8:
+        assert_f32_close(got, want, 'fused')
+    else:
+        torch.testing.assert_close(got.cpu().double(), want, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize('dtype,rel', [(torch.bfloat16, BF16_REL), (torch.float16, F16_REL)])
+@pytest.mark.parametrize('shape', SHAPES[:5], ids=IDS[:5])
+def test_16bit_vs_oracle(coracle, shape, dtype, rel):
+    B, d, C, H, W, K = shape
+    q, key, v, attn = inputs(gen(301), *shape, dtype=dtype)
+    qf, kf, vf, af = (x.float() for x in (q, key, v, attn))
+    got = sapa_amd.qk(*cl(q, key), K, 2)
+    assert got.dtype == dtype and got.is_contiguous(memory_format=CL)
+    assert_rel_rms_close(got.float(), coracle.qk(qf, kf, K, 2, 'f32a64'), rel, 'qk')
+    got = sapa_amd.av(*cl(attn, v), K, 2)
+    assert_rel_rms_close(got.float(), coracle.av(af, vf, K, 2, 'f32a64'), rel, 'av')
+    got = sapa_amd.sapa_fused(*cl(q, key, v), K, 2)
+    assert got.dtype == dtype and got.is_contiguous(memory_format=CL)
+    assert_rel_rms_close(got.float(), coracle.sapa_fused(qf, kf, vf, K, 2, 'f32a64'), rel, 'fused')
+
+
+def test_matches_contiguous_path_at_a_larger_shape():
+    """Several tiles per image and several images: against the library's own
+    NCHW kernels on the same values."""
+    B, d, C, H, W, K = 3, 64, 96, 21, 30, 5
+    q, key, v, attn = inputs(gen(302), B, d, C, H, W, K)
+    qd, kd, vd, ad = (t.to(DEV) for t in (q, key, v, attn))
+    torch.testing.assert_close(sapa_amd.sapa_fused(*cl(q, key, v), K, 2).contiguous(),
+                               sapa_amd.sapa_fused(qd, kd, vd, K, 2), rtol=1e-5, atol=1e-5)
+    assert torch.equal(sapa_amd.av(*cl(attn, v), K, 2).contiguous(), sapa_amd.av(ad, vd, K, 2))
+    assert_rel_rms_close(sapa_amd.qk(*cl(q, key), K, 2), sapa_amd.qk(qd, kd, K, 2), 1e-5, 'qk')
+
+
+def test_zero_query_is_the_box_filter():
+    """q == 0: uniform weights 1/K^2, out-of-range neighbours in the denominator."""
+    B, d, C, H, W, K = 1, 8, 12, 9, 10, 5
+    g = gen(303)
+    key, v = randn(g, B, d, H, W), randn(g, B, C, H, W)
+    q = torch.zeros(B, d, 2 * H, 2 * W)
+    got = sapa_amd.sapa_fused(*cl(q, key, v), K, 2).cpu()
+    want = F.avg_pool2d(v.double(), K, 1, K // 2, count_include_pad=True)
+    want = want.repeat_interleave(2, -2).repeat_interleave(2, -1)
+    assert_f32_close(got, want, 'box filter')
+
+
+def test_layout_errors():
+    B, d, C, H, W, K = 1, 8, 8, 4, 4, 5
+    q, key, v, attn = inputs(gen(304), B, d, C, H, W, K)
+    qc, kc, vc = cl(q, key, v)
+    with pytest.raises(RuntimeError, match='contiguous'):
+        sapa_amd.sapa_fused(qc, key.to(DEV), vc, K, 2)            # mixed orders
+    q7 = randn(gen(305), B, d, 2 * H, 2 * W)
+    with pytest.raises(RuntimeError, match='channels_last'):
+        sapa_amd.qk(*cl(q7, key), 7, 2)                           # no channels-last kernel for K = 7
+    k6 = randn(gen(306), B, 6, H, W)
+    q6 = randn(gen(307), B, 6, 2 * H, 2 * W)
+    with pytest.raises(RuntimeError, match='channels_last'):
+        sapa_amd.qk(*cl(q6, k6), K, 2)                            # channels not a multiple of 4
+
+
+def test_backward_through_channels_last_forward():
+    B, d, C, H, W, K = 2, 8, 12, 6, 7, 5
+    q, key, v, _ = inputs(gen(308), B, d, C, H, W, K)
+    go = randn(gen(309), B, C, 2 * H, 2 * W)
+    grads = []
+    for fmt in (torch.contiguous_format, CL):
+        ts = [t.to(DEV).contiguous(memory_format=fmt).requires_grad_() for t in (q, key, v)]
+        out = sapa_amd.sapa_fused(*ts, K, 2)
+        out.backward(go.to(DEV).contiguous(memory_format=fmt))
+        grads.append([t.grad for t in ts])
+    for a, b, name in zip(grads[0], grads[1], ('query', 'key', 'value')):
+        torch.testing.assert_close(b, a, rtol=1e-4, atol=1e-5, msg=lambda m: f'grad_{name}: {m}')
