@@ -131,6 +131,12 @@ def main():
     ap.add_argument('--pass', dest='direction', default='forward', choices=['forward', 'train'],
                     help="'train' times the fused forward plus its backward (all input "
                          'gradients) through the autograd API instead of the forward alone')
+    ap.add_argument('--layout', default='nchw', choices=['nchw', 'channels_last'],
+                    help="memory order of the SAPA-B tensors: 'nchw' = contiguous, the "
+                         "reference's contract (default); 'channels_last' = torch.channels_last, "
+                         'served by the *_nhwc entry points.  With the default, the forward '
+                         'SAPA-B line also carries the channels_last timing of the same '
+                         "workload under 'channels_last'")
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--calibration-copy', action='store_true',
                     help='after the timed region, run 5 device copies of 1 GiB (a kernel of '
@@ -162,6 +168,12 @@ def main():
         q, key, v = make_inputs(cfg, dtype, dev)
     out = torch.empty(B, C, H * s, W * s, dtype=dtype, device=dev)
     code = _lib.dtype_code(out)
+    nhwc_ok = not deform and K in (3, 5) and s == 2 and d % 4 == 0 and C % 4 == 0
+    if args.layout == 'channels_last':
+        if not nhwc_ok or args.direction == 'train':
+            sys.exit('bench.py: --layout channels_last covers the SAPA-B forward workloads with '
+                     'K in {3, 5}, s = 2')
+        q, key, v, out = (t.contiguous(memory_format=torch.channels_last) for t in (q, key, v, out))
 
     if deform:
         def step():
@@ -169,10 +181,15 @@ def main():
                 q.data_ptr(), key.data_ptr(), v.data_ptr(), off.data_ptr(), out.data_ptr(), B,
                 G * d, C, H, W, P, s, G, code, stream.cuda_stream), 'sapa_deform_fused_forward')
     else:
-        def step():
-            _lib.check(lib.sapa_fused_forward(q.data_ptr(), key.data_ptr(), v.data_ptr(),
-                                              out.data_ptr(), B, d, C, H, W, K, s, code,
-                                              stream.cuda_stream), 'sapa_fused_forward')
+        def fused_step(entry, q, key, v, out):
+            fn = getattr(lib, entry)
+
+            def step():
+                _lib.check(fn(q.data_ptr(), key.data_ptr(), v.data_ptr(), out.data_ptr(), B, d, C,
+                              H, W, K, s, code, stream.cuda_stream), entry)
+            return step
+        step = fused_step('sapa_fused_forward_nhwc' if args.layout == 'channels_last'
+                          else 'sapa_fused_forward', q, key, v, out)
 
     train = args.direction == 'train'
     if train:
@@ -188,19 +205,28 @@ def main():
                 y = sapa_amd.sapa_fused(q, key, v, K, s)
                 torch.autograd.grad(y, leaves, go)
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    # HIP events on the stream the kernel is launched on
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record(stream)
-    for _ in range(args.steps):
-        step()
-    e1.record(stream)
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    ms = e0.elapsed_time(e1) / args.steps
+    def timed(step):
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        # HIP events on the stream the kernel is launched on
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record(stream)
+        for _ in range(args.steps):
+            step()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / args.steps, (time.perf_counter() - t0) * 1e3 / args.steps
+
+    ms, wall_ms = timed(step)
+    ms_cl = None
+    if args.layout == 'nchw' and nhwc_ok and args.direction == 'forward':
+        # the same workload with every tensor in torch.channels_last order
+        cl = [t.contiguous(memory_format=torch.channels_last) for t in (q, key, v, out)]
+        ms_cl, _ = timed(fused_step('sapa_fused_forward_nhwc', *cl))
+        err_cl = (cl[3][:1].float() - out[:1].float()).abs().max().item()
+        del cl
 
     if args.calibration_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
@@ -222,8 +248,11 @@ def main():
         abytes = algorithmic_bytes(B, C, d, H, W, s, esize)
         what = 'fused SAPA-B forward (qk->softmax->av)'
         wl = (f'{args.workload}: SAPA-B FPN-style B={B} C={C} d={d} '
-              f'{H}x{W}->{H * s}x{W * s} K={K} s={s} {args.dtype}, NCHW')
-        if (K, s) != (5, 2):
+              f'{H}x{W}->{H * s}x{W * s} K={K} s={s} {args.dtype}, '
+              + ('channels_last' if args.layout == 'channels_last' else 'NCHW'))
+        if args.layout == 'channels_last':
+            kern = 'sapa_b_nhwc_kernel (fused mode)'
+        elif (K, s) != (5, 2):
             kern = 'sapa_b_mfma_kernel (fused mode)'
         elif esize == 2 and W % 4 == 0 and W >= 32:
             kern = 'sapa_b_dot2_kernel (fused mode)'
@@ -260,11 +289,21 @@ def main():
             'peak': HBM_PEAK_GBS,
             'unit': 'GB/s',
             'frac': achieved / HBM_PEAK_GBS,
-            'traffic': None if train else MEASURED_TRAFFIC_BYTES.get((args.workload, args.dtype)),
+            'traffic': None if train else MEASURED_TRAFFIC_BYTES.get(
+                (args.workload, args.dtype) if args.layout == 'nchw'
+                else (args.workload, args.dtype, args.layout)),
             'algorithmic_bytes': abytes,
             'kernel': kern,
         },
     }
+    if ms_cl is not None:
+        rec['channels_last'] = {
+            'ms_per_step': ms_cl, 'value': pix / (ms_cl * 1e-3) / 1e9, 'unit': 'Gpix/s',
+            'roofline_frac': abytes / (ms_cl * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            'kernel': 'sapa_b_nhwc_kernel (fused mode)',
+            'max_abs_diff_vs_nchw_image0': err_cl,
+            'note': 'same workload and algorithmic bytes, every tensor in torch.channels_last '
+                    'order (python bench.py --layout channels_last makes this the main line)'}
     if not args.no_cpu_baseline and not train:
         if deform:
             from oracle import torch_oracle

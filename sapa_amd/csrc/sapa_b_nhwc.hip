@@ -125,18 +125,23 @@ __device__ __forceinline__ void halve(const float (&in)[N], float (&out)[(N + 1)
     }
 }
 
-template <typename T, int K, int MODE>
-__global__ void __launch_bounds__(256)
+#ifdef SAPA_NHWC_WPE
+#define SAPA_NHWC_OCC __attribute__((amdgpu_waves_per_eu(SAPA_NHWC_WPE, SAPA_NHWC_WPE)))
+#else
+#define SAPA_NHWC_OCC
+#endif
+template <typename T, int K, int QX, int TY, int MODE>
+__global__ void __launch_bounds__(64 * QX * TY) SAPA_NHWC_OCC
 sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
                    const T *__restrict__ attn_in, const T *__restrict__ value,
                    T *__restrict__ out, int d, int C, int H, int W, int tiles_x, int tiles_y,
                    int nblocks, int per_xcd) {
     constexpr int S = 2, NJ = 4, KK = K * K, R = (K - 1) / 2;
-    constexpr int TP = 4;                         // tile: TP x TP parents, one row per wave
-    constexpr int WW = TP + K - 1, NPOS = WW * WW;   // window positions
+    constexpr int TX = 4 * QX;                    // tile: TX x TY parents, QX waves per row
+    constexpr int WW = TX + K - 1, WH = TY + K - 1, NPOS = WW * WH;   // window positions
     constexpr int CHK = 64;                       // channels per chunk: 16 lanes x 4
     constexpr int BUF = NPOS * CHK;               // floats per LDS buffer
-    constexpr int NT = 256, NPASS = (NPOS * 16 + NT - 1) / NT;   // staging passes (16 quads per position)
+    constexpr int NT = 64 * QX * TY, NPASS = (NPOS * 16 + NT - 1) / NT;   // staging passes (16 quads per position)
     constexpr int NV = K * NJ;                    // logits of one window row, index = 4 * kx + child
     constexpr int N1 = (NV + 1) / 2, N2 = (N1 + 1) / 2, N3 = (N2 + 1) / 2;
     constexpr int RPR = (N3 + 1) / 2, NR = K * RPR;   // registers per window row / in all
@@ -156,8 +161,9 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int row = lane >> 4, li = lane & 15;    // parent within the wave, channel quad
-    const int x0 = tx * TP, y0 = ty * TP;
-    const int px = x0 + row, py = y0 + wave;
+    const int x0 = tx * TX, y0 = ty * TY;
+    const int wx = wave % QX, wy = wave / QX;     // this wave's quad of parents in the tile
+    const int px = x0 + 4 * wx + row, py = y0 + wy;
     const bool active = px < W && py < H;
     const int hW = W * S;
     const long lpix = (long)H * W, hpix = lpix * S * S;
@@ -203,9 +209,9 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
         }
     };
 
-    // this row's window origin: tap (ky, kx) of parent (wave, row) sits at
-    // position (wave + ky) * WW + row + kx
-    const float *win = lds + ((wave * WW + row) * CHK + 4 * li);
+    // this row's window origin: tap (ky, kx) of its parent sits at position
+    // (wy + ky) * WW + 4 wx + row + kx
+    const float *win = lds + ((wy * WW + 4 * wx + row) * CHK + 4 * li);
 
     // logits, then weights: w[ky * RPR + m] of lane li is in-row index 16 m + li,
     // i.e. child li & 3 and kx = 4 m + (li >> 2); ok[m]: that index exists
@@ -339,18 +345,21 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
     }
 }
 
-template <typename T, int K>
-static hipError_t launch_k(int mode, const void *q, const void *key, const void *attn_in,
-                           const void *value, void *out, int B, int d, int C, int H, int W,
-                           hipStream_t st) {
-    const int tiles_x = (W + 3) / 4, tiles_y = (H + 3) / 4;
+#ifndef SAPA_NHWC_TILE
+#define SAPA_NHWC_TILE 1, 4
+#endif
+template <typename T, int K, int QX, int TY>
+static hipError_t launch_geom(int mode, const void *q, const void *key, const void *attn_in,
+                              const void *value, void *out, int B, int d, int C, int H, int W,
+                              hipStream_t st) {
+    const int tiles_x = (W + 4 * QX - 1) / (4 * QX), tiles_y = (H + TY - 1) / TY;
     const long nb = (long)tiles_x * tiles_y * B;
     if (nb > (1L << 30)) return hipErrorNotSupported;
     const int per_xcd = (int)((nb + 7) / 8);
-    const dim3 grid(per_xcd * 8), block(256);
+    const dim3 grid(per_xcd * 8), block(64 * QX * TY);
 #define SAPA_NHWC_CASE(M)                                                                      \
     case M:                                                                                    \
-        hipLaunchKernelGGL((sapa_b_nhwc_kernel<T, K, M>), grid, block, 0, st, (const T *)q,    \
+        hipLaunchKernelGGL((sapa_b_nhwc_kernel<T, K, QX, TY, M>), grid, block, 0, st, (const T *)q, \
                            (const T *)key, (const T *)attn_in, (const T *)value, (T *)out, d,  \
                            C, H, W, tiles_x, tiles_y, (int)nb, per_xcd);                       \
         break;
@@ -368,8 +377,8 @@ static hipError_t launch_t(int mode, const void *q, const void *key, const void 
                            const void *value, void *out, int B, int d, int C, int H, int W, int K,
                            hipStream_t st) {
     switch (K) {
-        case 3: return launch_k<T, 3>(mode, q, key, attn_in, value, out, B, d, C, H, W, st);
-        case 5: return launch_k<T, 5>(mode, q, key, attn_in, value, out, B, d, C, H, W, st);
+        case 3: return launch_geom<T, 3, SAPA_NHWC_TILE>(mode, q, key, attn_in, value, out, B, d, C, H, W, st);
+        case 5: return launch_geom<T, 5, SAPA_NHWC_TILE>(mode, q, key, attn_in, value, out, B, d, C, H, W, st);
         default: return hipErrorNotSupported;
     }
 }
