@@ -220,6 +220,23 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
 #pragma unroll
     for (int m = 0; m < RPR; ++m) ok[m] = 16 * m + li < NV;
     const int jl = li & 3, kxl = li >> 2;          // this lane's child and first kx
+    // q of the 4 children, this lane's 4 channels of key chunk j (zeros past d
+    // and for idle rows); the first chunk's is fetched before anything else so
+    // that it arrives while the first window is staged
+    const T *qp = q + ((long)n * hpix + (long)(py * S) * hW + (long)px * S) * d;
+    Raw qraw[NJ];
+    auto load_q = [&](int j) {
+        const int c0 = j * CHK;
+        const bool q_ok = active && c0 + 4 * li < d;
+#pragma unroll
+        for (int jj = 0; jj < NJ; ++jj) {
+            qraw[jj] = Raw{};
+            if (q_ok)
+                qraw[jj] = __builtin_nontemporal_load(
+                    (const Raw *)(qp + ((long)(jj >> 1) * hW + (jj & 1)) * d + c0 + 4 * li));
+        }
+    };
+    if (DO_QK) load_q(0);
     stage_load(0);
     stage_store(0);
     __syncthreads();
@@ -227,21 +244,12 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
     if (DO_QK) {
 #pragma unroll
         for (int i = 0; i < NR; ++i) w[i] = 0.f;
-        const T *qp = q + ((long)n * hpix + (long)(py * S) * hW + (long)px * S) * d;
         for (int j = 0; j < nKc; ++j) {
             if (j + 1 < ntot) stage_load(j + 1);
-            const int c0 = j * CHK;
-            // q of the 4 children, this lane's 4 channels (zeros past d and for idle rows)
             f32x4 qv[NJ];
-            const bool q_ok = active && c0 + 4 * li < d;
 #pragma unroll
-            for (int jj = 0; jj < NJ; ++jj) {
-                Raw raw = {};
-                if (q_ok)
-                    raw = __builtin_nontemporal_load(
-                        (const Raw *)(qp + ((long)(jj >> 1) * hW + (jj & 1)) * d + c0 + 4 * li));
-                qv[jj] = Q4::widen(raw);
-            }
+            for (int jj = 0; jj < NJ; ++jj) qv[jj] = Q4::widen(qraw[jj]);
+            if (j + 1 < nKc) load_q(j + 1);
             const float *wb = win + (j & 1) * BUF;
 #pragma unroll
             for (int ky = 0; ky < K; ++ky) {
@@ -317,21 +325,35 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
             for (int jj = 0; jj < NJ; ++jj)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) o[jj][e] = 0.f;
-            static_for<K>([&](auto iky) {
-                static_for<K>([&](auto ikx) {
-                    constexpr int ky = decltype(iky)::value, kx = decltype(ikx)::value;
-                    const f32x4 vv = *(const f32x4 *)(wb + (ky * WW + kx) * CHK);
-                    static_for<NJ>([&](auto ijj) {
-                        // the weight lives in register ky * RPR + idx / 16 of lane idx % 16
-                        constexpr int jj = decltype(ijj)::value, idx = kx * NJ + jj;
-                        const float wr = w[ky * RPR + idx / 16];
-                        static_for<4>([&](auto ie) {
-                            constexpr int e = decltype(ie)::value;
-                            fma_bcast<idx % 16>(o[jj][e], wr, vv[e]);
-                        });
+            // the window values travel through a ring of AHEAD + 1 registers of
+            // 4 channels: tap t + AHEAD is read while tap t is multiplied (the
+            // FMAs are opaque to the scheduler, so the distance is set here)
+            constexpr int AHEAD = 3;
+            f32x4 ring[AHEAD + 1];
+            static_for<AHEAD>([&](auto it) {
+                constexpr int t = decltype(it)::value;
+                ring[t] = *(const f32x4 *)(wb + ((t / K) * WW + t % K) * CHK);
+            });
+            static_for<KK>([&](auto it) {
+                constexpr int t = decltype(it)::value, ky = t / K, kx = t % K, tn = t + AHEAD;
+                if (tn < KK)
+                    ring[tn % (AHEAD + 1)] = *(const f32x4 *)(wb + ((tn / K) * WW + tn % K) * CHK);
+                const f32x4 vv = ring[t % (AHEAD + 1)];
+                static_for<NJ>([&](auto ijj) {
+                    // the weight lives in register ky * RPR + idx / 16 of lane idx % 16
+                    constexpr int jj = decltype(ijj)::value, idx = kx * NJ + jj;
+                    const float wr = w[ky * RPR + idx / 16];
+                    static_for<4>([&](auto ie) {
+                        constexpr int e = decltype(ie)::value;
+                        fma_bcast<idx % 16>(o[jj][e], wr, vv[e]);
                     });
                 });
             });
+            // The next chunk goes to LDS BEFORE the results are stored: a wait for
+            // a load while stores are in flight is a wait for those stores too
+            // (one counter, no order between the two kinds), so the stores are
+            // issued right after the wait and have a whole chunk to complete.
+            if (j + 1 < ntot) stage_store(j + 1);
             if (active && c0 + 4 * li < C) {
 #pragma unroll
                 for (int jj = 0; jj < NJ; ++jj)
@@ -339,7 +361,6 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
                         Q4::narrow(f32x4{o[jj][0], o[jj][1], o[jj][2], o[jj][3]}),
                         (Raw *)(op + ((long)(jj >> 1) * hW + (jj & 1)) * C + c0 + 4 * li));
             }
-            if (j + 1 < ntot) stage_store(j + 1);
             __syncthreads();
         }
     }
