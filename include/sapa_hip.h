@@ -155,7 +155,7 @@ int sapa_qk_softmax_forward(const void *query, const void *key, void *attn,
  * out [B,sH,sW,C] (qk: [B,sH,sW,K*K]).  The reference requires contiguous
  * NCHW tensors (CHECK_CONTIGUOUS, sapa/sapa/src/qk_cuda.cpp:35-39); these let
  * a channels-last model call the operators without a layout copy.  Covered:
- * SAPA_F32 / F16 / BF16, K in {3, 5}, s = 2, channel counts that are multiples
+ * SAPA_F32 / F16 / BF16, (K, s) in {(3,2), (5,2), (7,2), (5,4), (7,4)}, channel counts that are multiples
  * of 4, tensors aligned to 4 elements; SAPA_ERR_UNSUPPORTED otherwise.  The
  * channel sums run in tree order: results agree with sapa_*_forward to
  * rounding (1e-5 relative in fp32), not bit for bit. */

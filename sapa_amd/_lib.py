@@ -158,7 +158,8 @@ def call_nhwc(name, device, *args):
     if status == UNSUPPORTED:
         raise RuntimeError(
             f'{name}: channels_last tensors are served for float32 / float16 / bfloat16, '
-            'kernel_size 3 or 5, scale_factor 2, channel counts that are multiples of 4; '
+            '(kernel_size, scale_factor) in {(3,2), (5,2), (7,2), (5,4), (7,4)}, channel counts that '
+            'are multiples of 4; '
             'call .contiguous() on the inputs for other configurations')
 
 

@@ -32,7 +32,7 @@ hipError_t sapa_b_tiled_launch(int mode, const void *q, const void *key, const v
                                int K, int s, int dtype, hipStream_t st);
 
 // sapa_b_nhwc.hip: the four forward modes for tensors in channels-last memory
-// order ([B, H, W, channels]); f32 / f16 / bf16, K in {3, 5}, s = 2, channel
+// order ([B, H, W, channels]); f32 / f16 / bf16, (K, s) in {(3,2), (5,2), (7,2), (5,4), (7,4)}, channel
 // counts multiples of 4.  hipErrorNotSupported otherwise.
 hipError_t sapa_b_nhwc_launch(int mode, const void *q, const void *key, const void *attn_in,
                               const void *value, void *out, int B, int d, int C, int H, int W,

@@ -1,20 +1,22 @@
 // SAPA-B for tensors in channels-last memory order (torch.channels_last: the
 // logical [B, C, H, W] tensor stored as [B, H, W, C]): qk, qk+softmax, av and
-// the fused qk -> softmax -> av forward, K in {3, 5}, s = 2.
+// the fused qk -> softmax -> av forward, (K, s) in {(3,2), (5,2), (7,2), (5,4),
+// (7,4)}.
 //
 // With the channels innermost every access of the operation is a long
 // contiguous run -- a pixel's q is one record of d elements, an output pixel
 // one record of C elements -- so the lanes of a wave run along the CHANNELS:
 //
-//   * a row of 16 lanes owns one low-res parent with its 2 x 2 children; lane i
+//   * a row of 16 lanes owns one low-res parent with its s x s children; lane i
 //     of the row holds channels 4i .. 4i+3 of the current 64-channel chunk.  A
 //     wave works on 4 parents that are neighbours in x, a workgroup of 4 waves
 //     on a tile of 4 x 4 parents;
 //   * key and value windows (tile + K-1 halo positions) go through LDS as
 //     [position][64 channels], one chunk at a time, double-buffered; a row of
 //     lanes reads one position as 256 contiguous bytes (no bank conflicts);
-//   * logits, one window row (K taps x 4 children = 20 values for K = 5) at a
-//     time: every lane accumulates its 4 channels' part of the products; the 16
+//   * logits, one window row and one group of 4 children (s = 2: all of them,
+//     s = 4: one child row) at a time, K taps x 4 children = 20 values for
+//     K = 5: every lane accumulates its 4 channels' part of the products; the 16
 //     lanes of a row are then summed with a 4-step butterfly that halves the
 //     number of live values at every step (the lane keeps the sums whose index
 //     bit matches its lane bit and hands the others to its partner: DPP quad
@@ -24,9 +26,9 @@
 //   * softmax per child across the 4 lanes x 10 registers that hold its taps;
 //   * aggregation: the weights stay in those registers; every FMA fetches its
 //     weight from the lane that owns it through a DPP row broadcast
-//     (v_fmac_f32_dpp row_newbcast), so a lane needs 16 accumulators (4 children
-//     x 4 channels) and no copy of the 100 weights.  One 16-byte LDS read feeds
-//     16 FMAs.
+//     (v_fmac_f32_dpp row_newbcast), so a lane needs 4 s^2 accumulators (children
+//     x 4 channels) and no copy of the weights.  One 16-byte LDS read feeds
+//     4 s^2 FMAs.
 //
 // The channel sums run in tree order, not in the reference kernels' sequential
 // order: results agree with them to rounding (1e-5 relative in fp32), not bit
@@ -103,7 +105,10 @@ __device__ __forceinline__ float row_xor(float v, int lane) {
 }
 // acc += v * (w of lane SRC of the own row of 16 lanes): one instruction, the
 // weight is fetched through the DPP row broadcast.  The caller keeps two wait
-// states between the last VALU write of w and the first of these.
+// states between the last VALU write of w and the first of these.  (A DPP
+// operand halves the issue rate of the instruction on this part -- measured 4.4
+// against 2.2 cycles per wave and SIMD -- but fetching the weight with a DPP
+// move and following it with 4 plain FMAs measured slower still.)
 template <int SRC>
 __device__ __forceinline__ void fma_bcast(float &acc, float w, float v) {
     asm("v_fmac_f32_dpp %0, %1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf"
@@ -130,21 +135,24 @@ __device__ __forceinline__ void halve(const float (&in)[N], float (&out)[(N + 1)
 #else
 #define SAPA_NHWC_OCC
 #endif
-template <typename T, int K, int QX, int TY, int MODE>
+template <typename T, int K, int S, int QX, int TY, int MODE>
 __global__ void __launch_bounds__(64 * QX * TY) SAPA_NHWC_OCC
 sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
                    const T *__restrict__ attn_in, const T *__restrict__ value,
                    T *__restrict__ out, int d, int C, int H, int W, int tiles_x, int tiles_y,
                    int nblocks, int per_xcd) {
-    constexpr int S = 2, NJ = 4, KK = K * K, R = (K - 1) / 2;
+    static_assert(S == 2 || S == 4, "children are handled in groups of 4");
+    // children j = cy * S + cx of a parent, in NG groups of 4 (s = 2: all four;
+    // s = 4: one child row per group)
+    constexpr int NJ = S * S, NG = NJ / 4, KK = K * K, R = (K - 1) / 2;
     constexpr int TX = 4 * QX;                    // tile: TX x TY parents, QX waves per row
     constexpr int WW = TX + K - 1, WH = TY + K - 1, NPOS = WW * WH;   // window positions
     constexpr int CHK = 64;                       // channels per chunk: 16 lanes x 4
     constexpr int BUF = NPOS * CHK;               // floats per LDS buffer
     constexpr int NT = 64 * QX * TY, NPASS = (NPOS * 16 + NT - 1) / NT;   // staging passes (16 quads per position)
-    constexpr int NV = K * NJ;                    // logits of one window row, index = 4 * kx + child
+    constexpr int NV = K * 4;                     // logits of one window row and child group, index = 4 * kx + child in group
     constexpr int N1 = (NV + 1) / 2, N2 = (N1 + 1) / 2, N3 = (N2 + 1) / 2;
-    constexpr int RPR = (N3 + 1) / 2, NR = K * RPR;   // registers per window row / in all
+    constexpr int RPR = (N3 + 1) / 2, NR = K * NG * RPR;   // registers per (row, group) / in all
     constexpr bool DO_QK = MODE != TILED_AV;
     constexpr bool DO_SOFTMAX = MODE == TILED_QK_SOFTMAX || MODE == TILED_FUSED;
     constexpr bool DO_AV = MODE == TILED_AV || MODE == TILED_FUSED;
@@ -213,30 +221,35 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
     // (wy + ky) * WW + 4 wx + row + kx
     const float *win = lds + ((wy * WW + 4 * wx + row) * CHK + 4 * li);
 
-    // logits, then weights: w[ky * RPR + m] of lane li is in-row index 16 m + li,
-    // i.e. child li & 3 and kx = 4 m + (li >> 2); ok[m]: that index exists
+    // logits, then weights: w[(ky * NG + g) * RPR + m] of lane li is in-row index
+    // 16 m + li of window row ky and child group g, i.e. child jl = li & 3 of the
+    // group and kx = 4 m + (li >> 2); ok[m]: that index exists
     float w[NR];
     bool ok[RPR];
 #pragma unroll
     for (int m = 0; m < RPR; ++m) ok[m] = 16 * m + li < NV;
-    const int jl = li & 3, kxl = li >> 2;          // this lane's child and first kx
-    // q of the 4 children, this lane's 4 channels of key chunk j (zeros past d
-    // and for idle rows); the first chunk's is fetched before anything else so
-    // that it arrives while the first window is staged
-    const T *qp = q + ((long)n * hpix + (long)(py * S) * hW + (long)px * S) * d;
-    Raw qraw[NJ];
-    auto load_q = [&](int j) {
+    const int jl = li & 3, kxl = li >> 2;          // this lane's child in a group and first kx
+    // this lane's child of group g: its pixel in a [B, sH, sW, n_ch] tensor
+    auto child_pixel = [&](int j) {
+        return (long)n * hpix + (long)(py * S + j / S) * hW + (long)px * S + j % S;
+    };
+    // q of the 4 children of group g, this lane's 4 channels of key chunk j
+    // (zeros past d and for idle rows)
+    Raw qraw[4];
+    auto load_q = [&](int j, int g) {
         const int c0 = j * CHK;
         const bool q_ok = active && c0 + 4 * li < d;
 #pragma unroll
-        for (int jj = 0; jj < NJ; ++jj) {
+        for (int jj = 0; jj < 4; ++jj) {
             qraw[jj] = Raw{};
             if (q_ok)
                 qraw[jj] = __builtin_nontemporal_load(
-                    (const Raw *)(qp + ((long)(jj >> 1) * hW + (jj & 1)) * d + c0 + 4 * li));
+                    (const Raw *)(q + child_pixel(g * 4 + jj) * d + c0 + 4 * li));
         }
     };
-    if (DO_QK) load_q(0);
+    // the first q is fetched before anything else so that it arrives while the
+    // first window is staged
+    if (DO_QK) load_q(0, 0);
     stage_load(0);
     stage_store(0);
     __syncthreads();
@@ -246,76 +259,101 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
         for (int i = 0; i < NR; ++i) w[i] = 0.f;
         for (int j = 0; j < nKc; ++j) {
             if (j + 1 < ntot) stage_load(j + 1);
-            f32x4 qv[NJ];
-#pragma unroll
-            for (int jj = 0; jj < NJ; ++jj) qv[jj] = Q4::widen(qraw[jj]);
-            if (j + 1 < nKc) load_q(j + 1);
             const float *wb = win + (j & 1) * BUF;
 #pragma unroll
-            for (int ky = 0; ky < K; ++ky) {
-                float part[NV];
+            for (int g = 0; g < NG; ++g) {
+                f32x4 qv[4];
 #pragma unroll
-                for (int kx = 0; kx < K; ++kx) {
-                    const f32x4 kv = *(const f32x4 *)(wb + (ky * WW + kx) * CHK);
+                for (int jj = 0; jj < 4; ++jj) qv[jj] = Q4::widen(qraw[jj]);
+                // the next group's (or chunk's) q while this one is used
+                if (g + 1 < NG) load_q(j, g + 1);
+                else if (j + 1 < nKc) load_q(j + 1, 0);
 #pragma unroll
-                    for (int jj = 0; jj < NJ; ++jj) {
-                        float a = kv[0] * qv[jj][0];
+                for (int ky = 0; ky < K; ++ky) {
+                    float part[NV];
 #pragma unroll
-                        for (int e = 1; e < 4; ++e) a = fma_(kv[e], qv[jj][e], a);
-                        part[kx * NJ + jj] = a;
+                    for (int kx = 0; kx < K; ++kx) {
+                        const f32x4 kv = *(const f32x4 *)(wb + (ky * WW + kx) * CHK);
+#pragma unroll
+                        for (int jj = 0; jj < 4; ++jj) {
+                            float a = kv[0] * qv[jj][0];
+#pragma unroll
+                            for (int e = 1; e < 4; ++e) a = fma_(kv[e], qv[jj][e], a);
+                            part[kx * 4 + jj] = a;
+                        }
                     }
-                }
-                // sum over the 16 lanes of the row
-                float p1[N1], p2[N2], p3[N3], p4[RPR];
-                halve<1, NV>(part, p1, lane);
-                halve<2, N1>(p1, p2, lane);
-                halve<4, N2>(p2, p3, lane);
-                halve<8, N3>(p3, p4, lane);
+                    // sum over the 16 lanes of the row
+                    float p1[N1], p2[N2], p3[N3], p4[RPR];
+                    halve<1, NV>(part, p1, lane);
+                    halve<2, N1>(p1, p2, lane);
+                    halve<4, N2>(p2, p3, lane);
+                    halve<8, N3>(p3, p4, lane);
 #pragma unroll
-                for (int m = 0; m < RPR; ++m) w[ky * RPR + m] += p4[m];
+                    for (int m = 0; m < RPR; ++m) w[(ky * NG + g) * RPR + m] += p4[m];
+                }
             }
             if (j + 1 < ntot) stage_store(j + 1);
             __syncthreads();
         }
         if (DO_SOFTMAX) {
-            // a child's taps lie in this lane's registers and in the lanes at
-            // distance 4, 8, 12
-            float mx = w[0];                       // in-row index li < NV always
+            // a child's taps lie in this lane's registers of its group and in the
+            // lanes at distance 4, 8, 12
 #pragma unroll
-            for (int i = 1; i < NR; ++i)
-                if (ok[i % RPR]) mx = max_(mx, w[i]);
-            mx = max_(mx, row_xor<4>(mx, lane));
-            mx = max_(mx, row_xor<8>(mx, lane));
-            float sum = 0.f;
+            for (int g = 0; g < NG; ++g) {
+                float mx = w[g * RPR];             // ky = 0, in-row index li < NV always
 #pragma unroll
-            for (int i = 0; i < NR; ++i) {
-                w[i] = ok[i % RPR] ? exp_(w[i] - mx) : 0.f;
-                sum += w[i];
+                for (int ky = 0; ky < K; ++ky)
+#pragma unroll
+                    for (int m = 0; m < RPR; ++m)
+                        if (ok[m]) mx = max_(mx, w[(ky * NG + g) * RPR + m]);
+                mx = max_(mx, row_xor<4>(mx, lane));
+                mx = max_(mx, row_xor<8>(mx, lane));
+                float sum = 0.f;
+#pragma unroll
+                for (int ky = 0; ky < K; ++ky)
+#pragma unroll
+                    for (int m = 0; m < RPR; ++m) {
+                        float &x = w[(ky * NG + g) * RPR + m];
+                        x = ok[m] ? exp_(x - mx) : 0.f;
+                        sum += x;
+                    }
+                sum += row_xor<4>(sum, lane);
+                sum += row_xor<8>(sum, lane);
+                const float inv = 1.f / sum;
+#pragma unroll
+                for (int ky = 0; ky < K; ++ky)
+#pragma unroll
+                    for (int m = 0; m < RPR; ++m) w[(ky * NG + g) * RPR + m] *= inv;
             }
-            sum += row_xor<4>(sum, lane);
-            sum += row_xor<8>(sum, lane);
-            const float inv = 1.f / sum;
-#pragma unroll
-            for (int i = 0; i < NR; ++i) w[i] *= inv;
         }
         if (!DO_AV && active) {
-            // attn[pixel of child jl][tap]: 4 lanes write 4 consecutive taps
-            T *ap = out + ((long)n * hpix + (long)(py * S + (jl >> 1)) * hW + (long)px * S + (jl & 1)) * KK;
+            // attn[pixel of this lane's child][tap]: 4 lanes write 4 consecutive taps
 #pragma unroll
-            for (int i = 0; i < NR; ++i)
-                if (ok[i % RPR]) ap[(i / RPR) * K + 4 * (i % RPR) + kxl] = (T)w[i];
+            for (int g = 0; g < NG; ++g) {
+                T *ap = out + child_pixel(g * 4 + jl) * KK;
+#pragma unroll
+                for (int ky = 0; ky < K; ++ky)
+#pragma unroll
+                    for (int m = 0; m < RPR; ++m)
+                        if (ok[m]) ap[ky * K + 4 * m + kxl] = (T)w[(ky * NG + g) * RPR + m];
+            }
         }
     } else {
         // av(): the weights come from memory, in the same lane layout
-        const T *ap = attn_in + ((long)n * hpix + (long)(py * S + (jl >> 1)) * hW + (long)px * S + (jl & 1)) * KK;
 #pragma unroll
-        for (int i = 0; i < NR; ++i)
-            w[i] = (active && ok[i % RPR]) ? (float)ap[(i / RPR) * K + 4 * (i % RPR) + kxl] : 0.f;
+        for (int g = 0; g < NG; ++g) {
+            const T *ap = attn_in + child_pixel(g * 4 + jl) * KK;
+#pragma unroll
+            for (int ky = 0; ky < K; ++ky)
+#pragma unroll
+                for (int m = 0; m < RPR; ++m)
+                    w[(ky * NG + g) * RPR + m] =
+                        (active && ok[m]) ? (float)ap[ky * K + 4 * m + kxl] : 0.f;
+        }
     }
 
     if (DO_AV) {
         asm volatile("s_nop 4");                   // w was just written: DPP reads need two wait states
-        T *op = out + ((long)n * hpix + (long)(py * S) * hW + (long)px * S) * C;
         for (int j = nKc; j < ntot; ++j) {
             if (j + 1 < ntot) stage_load(j + 1);
             const int c0 = (j - nKc) * CHK;
@@ -328,7 +366,7 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
             // the window values travel through a ring of AHEAD + 1 registers of
             // 4 channels: tap t + AHEAD is read while tap t is multiplied (the
             // FMAs are opaque to the scheduler, so the distance is set here)
-            constexpr int AHEAD = 3;
+            constexpr int AHEAD = S == 2 ? 3 : 1;
             f32x4 ring[AHEAD + 1];
             static_for<AHEAD>([&](auto it) {
                 constexpr int t = decltype(it)::value;
@@ -340,9 +378,9 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
                     ring[tn % (AHEAD + 1)] = *(const f32x4 *)(wb + ((tn / K) * WW + tn % K) * CHK);
                 const f32x4 vv = ring[t % (AHEAD + 1)];
                 static_for<NJ>([&](auto ijj) {
-                    // the weight lives in register ky * RPR + idx / 16 of lane idx % 16
-                    constexpr int jj = decltype(ijj)::value, idx = kx * NJ + jj;
-                    const float wr = w[ky * RPR + idx / 16];
+                    // the weight lives in register (ky * NG + g) * RPR + idx / 16 of lane idx % 16
+                    constexpr int jj = decltype(ijj)::value, g = jj / 4, idx = kx * 4 + jj % 4;
+                    const float wr = w[(ky * NG + g) * RPR + idx / 16];
                     static_for<4>([&](auto ie) {
                         constexpr int e = decltype(ie)::value;
                         fma_bcast<idx % 16>(o[jj][e], wr, vv[e]);
@@ -359,7 +397,7 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
                 for (int jj = 0; jj < NJ; ++jj)
                     __builtin_nontemporal_store(
                         Q4::narrow(f32x4{o[jj][0], o[jj][1], o[jj][2], o[jj][3]}),
-                        (Raw *)(op + ((long)(jj >> 1) * hW + (jj & 1)) * C + c0 + 4 * li));
+                        (Raw *)(out + child_pixel(jj) * C + c0 + 4 * li));
             }
             __syncthreads();
         }
@@ -369,7 +407,7 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
 #ifndef SAPA_NHWC_TILE
 #define SAPA_NHWC_TILE 1, 4
 #endif
-template <typename T, int K, int QX, int TY>
+template <typename T, int K, int S, int QX, int TY>
 static hipError_t launch_geom(int mode, const void *q, const void *key, const void *attn_in,
                               const void *value, void *out, int B, int d, int C, int H, int W,
                               hipStream_t st) {
@@ -380,7 +418,7 @@ static hipError_t launch_geom(int mode, const void *q, const void *key, const vo
     const dim3 grid(per_xcd * 8), block(64 * QX * TY);
 #define SAPA_NHWC_CASE(M)                                                                      \
     case M:                                                                                    \
-        hipLaunchKernelGGL((sapa_b_nhwc_kernel<T, K, QX, TY, M>), grid, block, 0, st, (const T *)q, \
+        hipLaunchKernelGGL((sapa_b_nhwc_kernel<T, K, S, QX, TY, M>), grid, block, 0, st, (const T *)q, \
                            (const T *)key, (const T *)attn_in, (const T *)value, (T *)out, d,  \
                            C, H, W, tiles_x, tiles_y, (int)nb, per_xcd);                       \
         break;
@@ -396,25 +434,28 @@ static hipError_t launch_geom(int mode, const void *q, const void *key, const vo
 template <typename T>
 static hipError_t launch_t(int mode, const void *q, const void *key, const void *attn_in,
                            const void *value, void *out, int B, int d, int C, int H, int W, int K,
-                           hipStream_t st) {
-    switch (K) {
-        case 3: return launch_geom<T, 3, SAPA_NHWC_TILE>(mode, q, key, attn_in, value, out, B, d, C, H, W, st);
-        case 5: return launch_geom<T, 5, SAPA_NHWC_TILE>(mode, q, key, attn_in, value, out, B, d, C, H, W, st);
-        default: return hipErrorNotSupported;
-    }
+                           int s, hipStream_t st) {
+#define SAPA_NHWC_KS(KV, SV)                                                                  \
+    if (K == KV && s == SV)                                                                   \
+        return launch_geom<T, KV, SV, SAPA_NHWC_TILE>(mode, q, key, attn_in, value, out, B, d, C, \
+                                                      H, W, st);
+    SAPA_NHWC_KS(3, 2) SAPA_NHWC_KS(5, 2) SAPA_NHWC_KS(7, 2) SAPA_NHWC_KS(5, 4) SAPA_NHWC_KS(7, 4)
+#undef SAPA_NHWC_KS
+    return hipErrorNotSupported;
 }
 
 }  // namespace nhwc
 
 // Channels-last tensors (q [B, sH, sW, d], key [B, H, W, d], value [B, H, W, C],
 // attn [B, sH, sW, K*K], out like q with C or K*K channels), f32 / f16 / bf16,
-// K in {3, 5}, s = 2, channel counts multiples of 4 and every tensor aligned to
+// (K, s) in {(3,2), (5,2), (7,2), (5,4), (7,4)}, channel counts multiples of 4 and every tensor aligned to
 // 4 elements; one image's key / value tensor below 2^31 bytes.
 // hipErrorNotSupported otherwise.
 hipError_t sapa_b_nhwc_launch(int mode, const void *q, const void *key, const void *attn_in,
                               const void *value, void *out, int B, int d, int C, int H, int W,
                               int K, int s, int dtype, hipStream_t st) {
-    if (s != 2 || (K != 3 && K != 5)) return hipErrorNotSupported;
+    if (!((s == 2 && (K == 3 || K == 5 || K == 7)) || (s == 4 && (K == 5 || K == 7))))
+        return hipErrorNotSupported;
     const bool need_qk = mode != TILED_AV, need_av = mode == TILED_AV || mode == TILED_FUSED;
     if ((need_qk && d % 4 != 0) || (need_av && C % 4 != 0)) return hipErrorNotSupported;
     const int esize = dtype == 0 ? 4 : 2;
@@ -426,9 +467,9 @@ hipError_t sapa_b_nhwc_launch(int mode, const void *q, const void *key, const vo
     for (const void *p : vec_ptrs)
         if (p && (uintptr_t)p % (4 * esize) != 0) return hipErrorNotSupported;
     switch (dtype) {
-        case 0: return nhwc::launch_t<float>(mode, q, key, attn_in, value, out, B, d, C, H, W, K, st);
-        case 2: return nhwc::launch_t<f16_t>(mode, q, key, attn_in, value, out, B, d, C, H, W, K, st);
-        case 3: return nhwc::launch_t<bf16_t>(mode, q, key, attn_in, value, out, B, d, C, H, W, K, st);
+        case 0: return nhwc::launch_t<float>(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, st);
+        case 2: return nhwc::launch_t<f16_t>(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, st);
+        case 3: return nhwc::launch_t<bf16_t>(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, st);
         default: return hipErrorNotSupported;
     }
 }
