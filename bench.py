@@ -172,11 +172,12 @@ def main():
         q, key, v = make_inputs(cfg, dtype, dev)
     out = torch.empty(B, C, H * s, W * s, dtype=dtype, device=dev)
     code = _lib.dtype_code(out)
-    nhwc_ok = not deform and K in (3, 5) and s == 2 and d % 4 == 0 and C % 4 == 0
+    nhwc_ok = (not deform and (K, s) in ((3, 2), (5, 2), (7, 2), (5, 4), (7, 4))
+               and d % 4 == 0 and C % 4 == 0)
     if args.layout == 'channels_last':
         if not nhwc_ok or args.direction == 'train':
             sys.exit('bench.py: --layout channels_last covers the SAPA-B forward workloads with '
-                     'K in {3, 5}, s = 2')
+                     '(K, s) in {(3,2), (5,2), (7,2), (5,4), (7,4)}')
         q, key, v, out = (t.contiguous(memory_format=torch.channels_last) for t in (q, key, v, out))
 
     if deform:
