@@ -28,6 +28,22 @@ def _hi(t, s):
     return t.shape[2] * s, t.shape[3] * s
 
 
+def _new_out(like, shape, *inputs):
+    """Shape-only result of a SAPA-B forward op: in torch.channels_last order
+    when every input is (the eager kernels serve that order without a copy and
+    answer in it), contiguous otherwise."""
+    cl = (not all(t.is_contiguous() for t in inputs)
+          and all(t.dim() == 4 and t.is_contiguous(memory_format=torch.channels_last)
+                  for t in inputs))
+    return torch.empty(tuple(shape), dtype=like.dtype, device=like.device,
+                       memory_format=torch.channels_last if cl else torch.contiguous_format)
+
+
+def _new_grad(t):
+    # the gradient kernels answer in contiguous order whatever the operand's order
+    return t.new_empty(t.shape)
+
+
 # ------------------------------------------------------------------ SAPA-B
 @custom_op(f'{_NS}::qk', mutates_args=())
 def qk(query: Tensor, key: Tensor, kernel_size: int, scale_factor: int) -> Tensor:
@@ -37,7 +53,7 @@ def qk(query: Tensor, key: Tensor, kernel_size: int, scale_factor: int) -> Tenso
 
 @qk.register_fake
 def _(query, key, kernel_size, scale_factor):
-    return key.new_empty((key.shape[0], kernel_size ** 2) + _hi(key, scale_factor))
+    return _new_out(key, (key.shape[0], kernel_size ** 2) + _hi(key, scale_factor), query, key)
 
 
 @custom_op(f'{_NS}::qk_backward', mutates_args=())
@@ -48,7 +64,7 @@ def qk_backward(grad_output: Tensor, query: Tensor, key: Tensor, kernel_size: in
 
 @qk_backward.register_fake
 def _(grad_output, query, key, kernel_size, scale_factor):
-    return torch.empty_like(query), torch.empty_like(key)
+    return _new_grad(query), _new_grad(key)
 
 
 def _qk_setup(ctx, inputs, output):
@@ -73,7 +89,7 @@ def av(attn: Tensor, value: Tensor, kernel_size: int, scale_factor: int) -> Tens
 
 @av.register_fake
 def _(attn, value, kernel_size, scale_factor):
-    return value.new_empty(value.shape[:2] + _hi(value, scale_factor))
+    return _new_out(value, value.shape[:2] + _hi(value, scale_factor), attn, value)
 
 
 @custom_op(f'{_NS}::av_backward', mutates_args=())
@@ -84,7 +100,7 @@ def av_backward(grad_output: Tensor, attn: Tensor, value: Tensor, kernel_size: i
 
 @av_backward.register_fake
 def _(grad_output, attn, value, kernel_size, scale_factor):
-    return torch.empty_like(attn), torch.empty_like(value)
+    return _new_grad(attn), _new_grad(value)
 
 
 def _av_setup(ctx, inputs, output):
@@ -110,7 +126,7 @@ def sapa_fused(query: Tensor, key: Tensor, value: Tensor, kernel_size: int,
 
 @sapa_fused.register_fake
 def _(query, key, value, kernel_size, scale_factor):
-    return value.new_empty(value.shape[:2] + _hi(value, scale_factor))
+    return _new_out(value, value.shape[:2] + _hi(value, scale_factor), query, key, value)
 
 
 @custom_op(f'{_NS}::sapa_fused_backward', mutates_args=())
@@ -121,7 +137,7 @@ def sapa_fused_backward(grad_output: Tensor, query: Tensor, key: Tensor, value: 
 
 @sapa_fused_backward.register_fake
 def _(grad_output, query, key, value, kernel_size, scale_factor):
-    return torch.empty_like(query), torch.empty_like(key), torch.empty_like(value)
+    return _new_grad(query), _new_grad(key), _new_grad(value)
 
 
 def _fused_setup(ctx, inputs, output):

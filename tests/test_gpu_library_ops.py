@@ -74,6 +74,33 @@ def test_compiled_deform_matches_eager():
         torch.testing.assert_close(a, b, rtol=1e-9, atol=1e-10)   # atomics: order varies
 
 
+def test_channels_last_ops_and_compile():
+    """Channels-last operands: the ops answer in channels-last order, the
+    shape-only implementations agree with that, and a compiled graph matches."""
+    CL = torch.channels_last
+    q, key, v = (t.contiguous(memory_format=CL) for t in _b_inputs())   # channel counts 6, 6, 10
+    q, key, v = (torch.cat([t, t], 1).contiguous(memory_format=CL) for t in (q, key, v))  # 12, 12, 20
+    out = torch.ops.sapa_amd.sapa_fused(q, key, v, 5, 2)
+    assert out.is_contiguous(memory_format=CL)
+    assert torch.equal(out, sapa_amd.sapa_fused(q, key, v, 5, 2))
+    tests = ('test_schema', 'test_faketensor', 'test_autograd_registration')
+    torch.library.opcheck(torch.ops.sapa_amd.sapa_fused.default, (q, key, v, 5, 2), test_utils=tests)
+    torch.library.opcheck(torch.ops.sapa_amd.qk.default, (q, key, 5, 2), test_utils=tests)
+
+    def attention(q, key, v):
+        return torch.ops.sapa_amd.sapa_fused(q, key, v, 5, 2)
+    compiled = torch.compile(attention, backend='aot_eager', fullgraph=True)
+    leaves = [t.clone().requires_grad_() for t in (q, key, v)]
+    ref_leaves = [t.clone().requires_grad_() for t in (q, key, v)]
+    y, y_ref = compiled(*leaves), attention(*ref_leaves)
+    assert torch.equal(y, y_ref)
+    go = torch.randn_like(y_ref)
+    y.backward(go)
+    y_ref.backward(go)
+    for a, b in zip(leaves, ref_leaves):
+        assert torch.equal(a.grad, b.grad)
+
+
 def test_opcheck():
     q, key, v = [t.requires_grad_(True) for t in _b_inputs(torch.float64)]
     tests = ('test_schema', 'test_faketensor', 'test_autograd_registration')
