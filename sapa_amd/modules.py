@@ -105,9 +105,17 @@ class SAPA(nn.Module):
 
     def attention(self, q, k, v):
         K, s = self.up_kernel_size, self.up_factor
+        # the operators take one memory order for all their tensors: the value's
+        # (the caller's feature map) decides, so a channels-last model stays
+        # channels-last end to end; for tensors already in that order these
+        # calls return the tensor itself
+        fmt = (torch.channels_last
+               if not v.is_contiguous() and v.is_contiguous(memory_format=torch.channels_last)
+               else torch.contiguous_format)
+        q, k, v = (t.contiguous(memory_format=fmt) for t in (q, k, v))
         if self.fused:
-            return sapa_fused(q.contiguous(), k.contiguous(), v.contiguous(), K, s)
-        attn = F.softmax(qk(q, k, K, s), dim=1)
+            return sapa_fused(q, k, v, K, s)
+        attn = F.softmax(qk(q, k, K, s), dim=1).contiguous(memory_format=fmt)
         return av(attn, v, K, s)
 
 

@@ -149,3 +149,23 @@ def test_backward_through_channels_last_forward():
         grads.append([t.grad for t in ts])
     for a, b, name in zip(grads[0], grads[1], ('query', 'key', 'value')):
         torch.testing.assert_close(b, a, rtol=1e-4, atol=1e-5, msg=lambda m: f'grad_{name}: {m}')
+
+
+def test_module_in_channels_last_format():
+    """A SAPA module in channels_last memory format: same result as the
+    contiguous run, output in channels_last order, parameters get gradients."""
+    torch.manual_seed(0)
+    m = sapa_amd.SAPA(64, 64, up_factor=2, up_kernel_size=5, embedding_dim=32).to(DEV)
+    g = gen(311)
+    y, x = randn(g, 2, 64, 18, 22).to(DEV), randn(g, 2, 64, 9, 11).to(DEV)
+    want = m(y, x)
+    mc = m.to(memory_format=CL)
+    yc, xc = y.contiguous(memory_format=CL), x.contiguous(memory_format=CL)
+    got = mc(yc, xc)
+    assert got.is_contiguous(memory_format=CL)
+    torch.testing.assert_close(got, want, rtol=1e-4, atol=1e-5)
+    got.sum().backward()
+    assert all(p.grad is not None for p in mc.parameters())
+    unfused = sapa_amd.SAPA(64, 64, embedding_dim=32, fused=False).to(DEV)
+    unfused.load_state_dict(m.state_dict())
+    torch.testing.assert_close(unfused(yc, xc), want, rtol=1e-4, atol=1e-5)
