@@ -172,19 +172,30 @@ def main():
         q, key, v = make_inputs(cfg, dtype, dev)
     out = torch.empty(B, C, H * s, W * s, dtype=dtype, device=dev)
     code = _lib.dtype_code(out)
-    nhwc_ok = (not deform and (K, s) in ((3, 2), (5, 2), (7, 2), (5, 4), (7, 4))
-               and d % 4 == 0 and C % 4 == 0)
+    if deform:
+        nhwc_ok = s in (1, 2, 4) and P <= 32 and d % 4 == 0 and d <= 64 and (C // G) % 4 == 0
+    else:
+        nhwc_ok = ((K, s) in ((3, 2), (5, 2), (7, 2), (5, 4), (7, 4))
+                   and d % 4 == 0 and C % 4 == 0)
     if args.layout == 'channels_last':
         if not nhwc_ok or args.direction == 'train':
-            sys.exit('bench.py: --layout channels_last covers the SAPA-B forward workloads with '
-                     '(K, s) in {(3,2), (5,2), (7,2), (5,4), (7,4)}')
+            sys.exit('bench.py: --layout channels_last covers the forward workloads with '
+                     '(K, s) in {(3,2), (5,2), (7,2), (5,4), (7,4)} (SAPA-B) / P <= 32 (SAPA-D)')
         q, key, v, out = (t.contiguous(memory_format=torch.channels_last) for t in (q, key, v, out))
+        if deform:
+            off = off.contiguous(memory_format=torch.channels_last)
 
     if deform:
-        def step():
-            _lib.check(lib.sapa_deform_fused_forward(
-                q.data_ptr(), key.data_ptr(), v.data_ptr(), off.data_ptr(), out.data_ptr(), B,
-                G * d, C, H, W, P, s, G, code, stream.cuda_stream), 'sapa_deform_fused_forward')
+        def fused_step(entry, q, key, v, out, off):
+            fn = getattr(lib, entry)
+
+            def step():
+                _lib.check(fn(q.data_ptr(), key.data_ptr(), v.data_ptr(), off.data_ptr(),
+                              out.data_ptr(), B, G * d, C, H, W, P, s, G, code,
+                              stream.cuda_stream), entry)
+            return step
+        step = fused_step('sapa_deform_fused_forward_nhwc' if args.layout == 'channels_last'
+                          else 'sapa_deform_fused_forward', q, key, v, out, off)
     else:
         def fused_step(entry, q, key, v, out):
             fn = getattr(lib, entry)
@@ -228,8 +239,10 @@ def main():
     ms_cl = None
     if args.layout == 'nchw' and nhwc_ok and args.direction == 'forward':
         # the same workload with every tensor in torch.channels_last order
-        cl = [t.contiguous(memory_format=torch.channels_last) for t in (q, key, v, out)]
-        ms_cl, _ = timed(fused_step('sapa_fused_forward_nhwc', *cl))
+        cl = [t.contiguous(memory_format=torch.channels_last)
+              for t in ((q, key, v, out, off) if deform else (q, key, v, out))]
+        ms_cl, _ = timed(fused_step('sapa_deform_fused_forward_nhwc' if deform
+                                    else 'sapa_fused_forward_nhwc', *cl))
         err_cl = (cl[3][:1].float() - out[:1].float()).abs().max().item()
         del cl
 
@@ -248,7 +261,9 @@ def main():
         what = 'fused SAPA-D forward (deform_qk->softmax->deform_av)'
         wl = (f'{args.workload}: SAPA-D B={B} C={C} d={d} G={G} P={P} {H}x{W}->{H * s}x{W * s} '
               f's={s} {args.dtype}, NCHW, offsets ~N(0,0.75) clipped to +-4')
-        kern = 'deform_lds_kernel (fused mode)'
+        kern = ('deform_fused_nhwc_kernel' if args.layout == 'channels_last'
+                else 'deform_lds_kernel (fused mode)')
+        wl = wl.replace('NCHW', 'channels_last') if args.layout == 'channels_last' else wl
     else:
         abytes = algorithmic_bytes(B, C, d, H, W, s, esize)
         what = 'fused SAPA-B forward (qk->softmax->av)'
@@ -305,7 +320,7 @@ def main():
         rec['channels_last'] = {
             'ms_per_step': ms_cl, 'value': pix / (ms_cl * 1e-3) / 1e9, 'unit': 'Gpix/s',
             'roofline_frac': abytes / (ms_cl * 1e-3) / 1e9 / HBM_PEAK_GBS,
-            'kernel': 'sapa_b_nhwc_kernel (fused mode)',
+            'kernel': 'deform_fused_nhwc_kernel' if deform else 'sapa_b_nhwc_kernel (fused mode)',
             'max_abs_diff_vs_nchw_image0': err_cl,
             'note': 'same workload and algorithmic bytes, every tensor in torch.channels_last '
                     'order (python bench.py --layout channels_last makes this the main line)'}

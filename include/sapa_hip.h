@@ -235,6 +235,21 @@ int sapa_deform_fused_forward(const void *query, const void *key,
                               int B, int Cq, int C, int H, int W,
                               int P, int s, int G, int dtype, void *stream);
 
+/* sapa_deform_fused_forward for tensors in channels-last memory order:
+ * query [B,sH,sW,Cq], key [B,H,W,Cq], value [B,H,W,C], offset [B,sH,sW,2*G*P]
+ * (channel 2(gP+p) = dx, +1 = dy), out [B,sH,sW,C].  No counterpart in the
+ * reference, which requires contiguous NCHW tensors
+ * (deformsapa/deformsapa/src/deform_qk.cpp, CHECK_CONTIGUOUS); this lets a
+ * channels-last model call SAPADeform.attention (sapa_deform.py:51-53) without
+ * layout copies.  Covered: SAPA_F32 / F16 / BF16, s in {1, 2, 4}, P <= 32,
+ * Cq / G (at most 64) and C / G multiples of 4, tensors aligned to 4 elements;
+ * SAPA_ERR_UNSUPPORTED otherwise.  The logits' channel sums run in tree order
+ * (rounding-level differences from sapa_deform_fused_forward). */
+int sapa_deform_fused_forward_nhwc(const void *query, const void *key,
+                                   const void *value, const void *offset, void *out,
+                                   int B, int Cq, int C, int H, int W,
+                                   int P, int s, int G, int dtype, void *stream);
+
 /* The three sampled forward operators reading the offsets in the layout
  * `offset_layout` (sapa_offset_layout) names; with SAPA_OFFSET_HIRES they are
  * the functions above.  They replace

@@ -37,6 +37,7 @@ SIGNATURES = {
     'sapa_deform_av_forward': [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_deform_av_backward': [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_deform_fused_forward': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
+    'sapa_deform_fused_forward_nhwc': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_deform_qk_forward_from': [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_deform_av_forward_from': [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_deform_fused_forward_from': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
@@ -155,6 +156,12 @@ def call_nhwc(name, device, *args):
     """An *_nhwc entry point; SAPA_ERR_UNSUPPORTED becomes an error that says
     what the channels-last kernels cover (there is no hidden layout copy)."""
     status = call_status(name, device, *args)
+    if status == UNSUPPORTED and 'deform' in name:
+        raise RuntimeError(
+            f'{name}: channels_last tensors are served for float32 / float16 / bfloat16, '
+            'scale_factor 1, 2 or 4, at most 32 points, channels per group that are multiples '
+            'of 4 (at most 64 query / key channels per group); call .contiguous() on the inputs '
+            'for other configurations')
     if status == UNSUPPORTED:
         raise RuntimeError(
             f'{name}: channels_last tensors are served for float32 / float16 / bfloat16, '

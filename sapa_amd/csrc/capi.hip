@@ -377,6 +377,19 @@ int sapa_deform_fused_forward(const void *query, const void *key, const void *va
                                           SAPA_OFFSET_HIRES, dtype, stream);
 }
 
+int sapa_deform_fused_forward_nhwc(const void *query, const void *key, const void *value,
+                                   const void *offset, void *out, int B, int Cq, int C, int H,
+                                   int W, int P, int s, int G, int dtype, void *stream) {
+    const int rc = check_deform_args(B, Cq, C, H, W, P, s, G, dtype);
+    if (rc != SAPA_OK) return rc;
+    if (B == 0) return SAPA_OK;
+    if (!query || !key || !value || !offset || !out) return SAPA_ERR_INVALID_ARGUMENT;
+    const hipError_t e = deform_fused_nhwc_launch(query, key, value, offset, out, B, Cq, C, H, W, P,
+                                                  s, G, dtype, (hipStream_t)stream);
+    if (e == hipErrorNotSupported) return SAPA_ERR_UNSUPPORTED;
+    return finish(e);
+}
+
 int sapa_deform_qk_backward(const void *grad_out, const void *query, const void *key,
                             const void *offset, void *grad_query, void *grad_key,
                             void *grad_offset, int B, int Cq, int H, int W, int P, int s, int G,

@@ -38,6 +38,14 @@ hipError_t sapa_b_nhwc_launch(int mode, const void *q, const void *key, const vo
                               const void *value, void *out, int B, int d, int C, int H, int W,
                               int K, int s, int dtype, hipStream_t st);
 
+// sapa_d_nhwc.hip: fused SAPA-D forward for tensors in channels-last memory
+// order (offsets [B, sH, sW, 2GP]); f32 / f16 / bf16, s in {1, 2, 4}, P <= 32,
+// channels per group multiples of 4, at most 64 query / key channels per group.
+// hipErrorNotSupported otherwise.
+hipError_t deform_fused_nhwc_launch(const void *q, const void *key, const void *value,
+                                    const void *offset, void *out, int B, int Cq, int C, int H,
+                                    int W, int P, int s, int G, int dtype, hipStream_t st);
+
 // sapa_b_dot2.hip: the four forward modes for f16 / bf16 tensors on the
 // two-term dot-product instructions (K = 5, s = 2); hipErrorNotSupported
 // otherwise.

@@ -1,0 +1,489 @@
+// Fused SAPA-D forward (deform_qk -> softmax over the P points -> deform_av)
+// for tensors in channels-last memory order: query [B, sH, sW, G*d], key
+// [B, H, W, G*d], value [B, H, W, C], offset [B, sH, sW, 2*G*P] (channel
+// 2(gP+p) = dx, +1 = dy), out [B, sH, sW, C].
+//
+// The contiguous-layout kernels (sapa_d_lds.hip) gather bilinear corners from
+// an LDS window with one lane per pixel: 64 lanes read 64 unrelated addresses
+// and the LDS bank conflicts of those gathers bound them.  Here the lanes run
+// along the CHANNELS: a row of 16 lanes owns one (pixel, group) pair, lane i
+// holds 4 channels, and a corner is read by the row as 256 contiguous bytes --
+// no bank conflicts whatever the offsets are.
+//
+//   * a wave works on 4 hi-res pixels that are neighbours in x (a quad), a
+//     workgroup of 4 waves on a 4 x 4-pixel tile (larger tiles: one wave takes
+//     several quads in turn), one group at a time: the key window of
+//     the group (the tile's parents + 4 cells of halo and the high corners'
+//     extra cell, [position][64 channels] fp32) goes through LDS, then the value
+//     window(s) of the group; the next chunk's global loads are in flight while
+//     the current one is consumed;
+//   * the sample positions are set up once per point, spread over the lanes:
+//     lane l of a row computes the guard, the four bilinear weights and the
+//     window address of points l and l + 16 of its pixel; the loops over the
+//     points fetch them from that lane with DPP row broadcasts;
+//   * logits: every lane accumulates its 4 channels' part of a point's
+//     sampled-key . query product; 16 points at a time are then summed over the
+//     16 lanes with a butterfly that leaves point 16 m + l in lane l -- the same
+//     lane that holds its setup -- and the softmax runs across the row;
+//   * aggregation: per point one broadcast of the weight, the usual
+//     w1*v1 + w2*v2 + w3*v3 + w4*v4 in the reference's order, one FMA per
+//     channel into 4 accumulators; a row stores 256 contiguous bytes.
+//
+// Index math, the strict guard (a point outside it has logit 0, takes part in
+// the softmax and contributes nothing) and the per-corner zero padding follow
+// deformsapa/deformsapa/src/cuda/deform_qk_cuda_kernel.cu:23-68,187: window
+// cells outside the image hold zeros, a point whose guard fails reads a
+// block of zeros with zero weights.  Points that pass the guard but leave the
+// window (offsets beyond +-4 cells) are sampled from global memory.  The
+// channel sums of the logits run in tree order (rounding-level differences
+// from the reference's sequential sums); the aggregation keeps its order.
+#include <utility>
+
+#include "deform_tap.hpp"
+#include "kernels.hpp"
+
+namespace sapa {
+
+namespace dnhwc {
+
+typedef unsigned u32;
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef u32 u32x2 __attribute__((ext_vector_type(2)));
+typedef u32 u32x4 __attribute__((ext_vector_type(4)));
+
+// 4 consecutive elements <-> 4 floats, 2 consecutive elements -> 2 floats
+template <typename T> struct Quad;
+template <> struct Quad<float> {
+    typedef f32x4 raw;
+    static __device__ __forceinline__ raw buffer_load(__amdgpu_buffer_rsrc_t r, u32 off) {
+        union { u32x4 u; f32x4 f; } x;
+        x.u = __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
+        return x.f;
+    }
+    static __device__ __forceinline__ f32x4 widen(raw v) { return v; }
+    static __device__ __forceinline__ raw narrow(f32x4 v) { return v; }
+    static __device__ __forceinline__ f32x2 load_pair(const float *p) { return *(const f32x2 *)p; }
+};
+template <typename H> struct Quad16 {
+    typedef u32x2 raw;
+    static __device__ __forceinline__ raw buffer_load(__amdgpu_buffer_rsrc_t r, u32 off) {
+        return __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0);
+    }
+    static __device__ __forceinline__ f32x4 widen(raw v) {
+        union { u32x2 u; H h[4]; } x;
+        x.u = v;
+        f32x4 f = {(float)x.h[0], (float)x.h[1], (float)x.h[2], (float)x.h[3]};
+        return f;
+    }
+    static __device__ __forceinline__ raw narrow(f32x4 v) {
+        union { u32x2 u; H h[4]; } x;
+        x.h[0] = (H)v[0];
+        x.h[1] = (H)v[1];
+        x.h[2] = (H)v[2];
+        x.h[3] = (H)v[3];
+        return x.u;
+    }
+    static __device__ __forceinline__ f32x2 load_pair(const H *p) {
+        union { u32 u; H h[2]; } x;
+        x.u = *(const u32 *)p;
+        f32x2 f = {(float)x.h[0], (float)x.h[1]};
+        return f;
+    }
+};
+template <> struct Quad<f16_t> : Quad16<f16_t> {};
+template <> struct Quad<bf16_t> : Quad16<bf16_t> {};
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>)
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+// value of lane (l ^ D) of the same row of 16 lanes
+template <int D>
+__device__ __forceinline__ float row_xor(float v, int lane) {
+    union { float f; int i; } x, y;
+    x.f = v;
+    if (D == 1) y.i = __builtin_amdgcn_mov_dpp(x.i, 0xB1, 0xf, 0xf, true);        // quad_perm [1,0,3,2]
+    else if (D == 2) y.i = __builtin_amdgcn_mov_dpp(x.i, 0x4E, 0xf, 0xf, true);   // quad_perm [2,3,0,1]
+    else y.i = __builtin_amdgcn_ds_bpermute((lane ^ D) << 2, x.i);
+    return y.f;
+}
+// value of lane SRC of the own row of 16 lanes
+template <int SRC>
+__device__ __forceinline__ float row_bcast(float v) {
+    union { float f; int i; } x, y;
+    x.f = v;
+    y.i = __builtin_amdgcn_mov_dpp(x.i, 0x150 + SRC, 0xf, 0xf, true);   // row_newbcast
+    return y.f;
+}
+template <int SRC>
+__device__ __forceinline__ int row_bcast(int v) {
+    return __builtin_amdgcn_mov_dpp(v, 0x150 + SRC, 0xf, 0xf, true);
+}
+
+// One butterfly step over lane distance D: n values per lane -> n / 2; the
+// lane whose bit D is clear keeps the even-indexed sums, its partner the odd.
+template <int D, int N>
+__device__ __forceinline__ void halve(const float (&in)[N], float (&out)[N / 2], int lane) {
+    const bool hi = lane & D;
+#pragma unroll
+    for (int m = 0; m < N / 2; ++m) {
+        const float a = in[2 * m], b = in[2 * m + 1];
+        const float keep = hi ? b : a, send = hi ? a : b;
+        out[m] = keep + row_xor<D>(send, lane);
+    }
+}
+
+constexpr int RCH = 4;          // window reach around the tile's parents, in low-res cells
+constexpr int MAXSETS = 2;      // points are handled 16 at a time: P <= 32
+constexpr u32 FALLBACK = 1u << 30;   // the point passes the guard but leaves the window
+
+template <typename T, int S, int NQX, int NQY>
+__global__ void __launch_bounds__(256)
+deform_fused_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
+                         const T *__restrict__ value, const T *__restrict__ offset,
+                         T *__restrict__ out, int Cq, int C, int H, int W, int P, int G,
+                         int tiles_x, int tiles_y, int nblocks, int per_xcd) {
+    // tile: TPX x TPY hi-res pixels; a wave owns NQY pixel rows of NQX quads
+    // (4 pixels in x) each and works through them one quad at a time
+    constexpr int TPX = 4 * NQX, TPY = 4 * NQY, NQ = NQX * NQY;
+    static_assert(TPX == TPY, "square tiles: one window extent");
+    constexpr int TPL = (TPX + S - 1) / S;       // parents of a tile per axis
+    constexpr int WW = TPL + 2 * RCH + 1, NPOS = WW * WW;   // window cells
+    constexpr int CHK = 64;                      // channels per chunk: 16 lanes x 4
+    constexpr int BUF = NPOS * CHK;              // floats of the window
+    constexpr int ZERO = BUF;                    // then (WW + 2) cells of zeros
+    constexpr int NT = 256, NPASS = (NPOS * 16 + NT - 1) / NT;
+    typedef Quad<T> Q4;
+    typedef typename Q4::raw Raw;
+
+    __shared__ __attribute__((aligned(16))) float lds[BUF + (WW + 2) * CHK];
+
+    const int logical = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
+    if (logical >= nblocks) return;
+    const int tx = logical % tiles_x;
+    const int ty = (logical / tiles_x) % tiles_y;
+    const int n = logical / (tiles_x * tiles_y);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int row = lane >> 4, li = lane & 15;
+    const int hH = H * S, hW = W * S;
+    // the pixel of this row of lanes in the wave's current quad (set_quad)
+    bool active;
+    int ph, pw;
+    long hpixel;
+    auto set_quad = [&](int qi) __attribute__((always_inline)) {
+        const int qh = ty * TPY + wave * NQY + qi / NQX, qw = tx * TPX + 4 * (qi % NQX) + row;
+        active = qh < hH && qw < hW;
+        const int ch = qh < hH ? qh : hH - 1, cw = qw < hW ? qw : hW - 1;   // clamped for loads
+        ph = ch / S;
+        pw = cw / S;
+        hpixel = (long)n * hH * hW + (long)ch * hW + cw;
+    };
+    const int wy0 = (ty * TPY) / S - RCH, wx0 = (tx * TPX) / S - RCH;   // window origin (low-res cell)
+    const long lpix = (long)H * W;
+    const int d = Cq / G, cg = C / G;
+    const int nVc = (cg + CHK - 1) / CHK, nPer = 1 + nVc, ntot = G * nPer;
+    const int nsets = (P + 15) / 16;
+
+    for (int i = tid; i < (WW + 2) * CHK; i += NT) lds[ZERO + i] = 0.f;
+
+    // ---- staging: pass p, thread t moves channel quad t % 16 of window cell
+    // p * 16 + t / 16; -1 marks a cell outside the image (zero fill)
+    int spix[NPASS];
+#pragma unroll
+    for (int p = 0; p < NPASS; ++p) {
+        const int pos = p * (NT / 16) + tid / 16;
+        const int gy = wy0 + pos / WW, gx = wx0 + pos % WW;
+        spix[p] = (pos < NPOS && gy >= 0 && gy < H && gx >= 0 && gx < W) ? gy * W + gx : -1;
+    }
+    const int sq = tid & 15;
+    // chunk j: group j / nPer; its key channels (j % nPer == 0) or value chunk j % nPer - 1
+    auto chunk_of = [&](int j, bool &is_key, int &cbase, int &cvalid, int &nch) __attribute__((always_inline)) {
+        const int g = j / nPer, r = j % nPer;
+        is_key = r == 0;
+        nch = is_key ? Cq : C;
+        cbase = is_key ? g * d : g * cg + (r - 1) * CHK;     // first channel of the chunk
+        const int left = is_key ? d : cg - (r - 1) * CHK;
+        cvalid = left < CHK ? left : CHK;                    // channels of the chunk that exist
+    };
+    Raw st[NPASS];
+    auto stage_load = [&](int j) __attribute__((always_inline)) {
+        bool is_key;
+        int cbase, cvalid, nch;
+        chunk_of(j, is_key, cbase, cvalid, nch);
+        const T *base = (is_key ? key : value) + (long)n * lpix * nch;
+        const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)base, 0, (int)(lpix * nch * (long)sizeof(T)), 0x00020000);
+        const bool c_ok = 4 * sq < cvalid;
+#pragma unroll
+        for (int p = 0; p < NPASS; ++p) {
+            const u32 off = (c_ok && spix[p] >= 0)
+                                ? (u32)(spix[p] * nch + cbase + 4 * sq) * (u32)sizeof(T)
+                                : 0x80000000u;
+            st[p] = Q4::buffer_load(r, off);
+        }
+    };
+    auto stage_store = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int p = 0; p < NPASS; ++p) {
+            const int pos = p * (NT / 16) + tid / 16;
+            if (NPOS % (NT / 16) == 0 || pos < NPOS) *(f32x4 *)(lds + pos * CHK + 4 * sq) = Q4::widen(st[p]);
+        }
+    };
+
+    // per point set m (points 16 m + li of this row's pixel): bilinear weights,
+    // the LDS offset of the low corner (or of the zeros) with the FALLBACK
+    // flag, the sample position for the fallback, the logit / attention weight
+    float tw1[MAXSETS], tw2[MAXSETS], tw3[MAXSETS], tw4[MAXSETS], tkh[MAXSETS], tkw[MAXSETS];
+    int tpk[MAXSETS];
+    // the attention weights of the wave's quads wait in LDS between the key
+    // chunk and the value chunks of a group (per thread: no synchronisation)
+    __shared__ float att_keep[NQ][MAXSETS][NT];
+
+    auto setup_points = [&](int g) __attribute__((always_inline)) {
+        const T *op = offset + hpixel * (2L * G * P) + 2L * g * P;
+#pragma unroll
+        for (int m = 0; m < MAXSETS; ++m) {
+            const int p = 16 * m + li;
+            f32x2 o2 = {0.f, 0.f};
+            if (m < nsets && p < P) o2 = Q4::load_pair(op + 2 * p);
+            const float kw = (float)pw + o2[0], kh = (float)ph + o2[1];
+            const WinTap<float> t = win_tap<float>(kh, kw, H, W, wy0, wx0, WW, WW);
+            const bool live = m < nsets && p < P;
+            const bool in = live && t.inwin;
+            tw1[m] = in ? t.w1 : 0.f;
+            tw2[m] = in ? t.w2 : 0.f;
+            tw3[m] = in ? t.w3 : 0.f;
+            tw4[m] = in ? t.w4 : 0.f;
+            tkh[m] = kh;
+            tkw[m] = kw;
+            tpk[m] = (in ? (t.hl * WW + t.wl) * CHK : ZERO) |
+                     ((live && t.guard && !t.inwin) ? (int)FALLBACK : 0);
+        }
+    };
+
+    // w1*v1 + w2*v2 + w3*v3 + w4*v4 of this lane's 4 channels, left to right with FMAs
+    auto sample_lds = [&](int pk, float w1, float w2, float w3, float w4,
+                          float (&val)[4]) __attribute__((always_inline)) {
+        const float *p0 = lds + (pk & 0xffffff) + 4 * li;
+        const f32x4 v1 = *(const f32x4 *)p0, v2 = *(const f32x4 *)(p0 + CHK);
+        const f32x4 v3 = *(const f32x4 *)(p0 + WW * CHK), v4 = *(const f32x4 *)(p0 + (WW + 1) * CHK);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            float v = w1 * v1[e];
+            v = fma_(w2, v2[e], v);
+            v = fma_(w3, v3[e], v);
+            val[e] = fma_(w4, v4[e], v);
+        }
+    };
+    // the same sample straight from global memory (the point left the window)
+    auto sample_global = [&](const T *src, int nch, int cbase, int cvalid, float kh, float kw,
+                             float (&val)[4]) __attribute__((always_inline)) {
+        Tap<float> t = {};
+        const bool ok = tap_setup(kh, kw, H, W, t) && 4 * li < cvalid;
+        f32x4 v[4];
+        const int idx[4] = {t.i1, t.i2, t.i3, t.i4};
+        const bool msk[4] = {t.m1, t.m2, t.m3, t.m4};
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            Raw raw = Raw{};
+            if (ok && msk[c])
+                raw = *(const Raw *)(src + ((long)n * lpix + idx[c]) * nch + cbase + 4 * li);
+            v[c] = Q4::widen(raw);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            float x = t.w1 * v[0][e];
+            x = fma_(t.w2, v[1][e], x);
+            x = fma_(t.w3, v[2][e], x);
+            val[e] = ok ? fma_(t.w4, v[3][e], x) : 0.f;
+        }
+    };
+
+    // logits of the group's points from the key window in LDS
+    auto qk_group = [&](int cbase, int cvalid, float (&att)[MAXSETS]) __attribute__((always_inline)) {
+        f32x4 qv = {0.f, 0.f, 0.f, 0.f};
+        if (active && 4 * li < cvalid)
+            qv = Q4::widen(__builtin_nontemporal_load((const Raw *)(q + hpixel * Cq + cbase + 4 * li)));
+#pragma unroll
+        for (int m = 0; m < MAXSETS; ++m) {
+            if (m >= nsets) {
+                att[m] = 0.f;
+                continue;
+            }
+            float part[16];
+            static_for<16>([&](auto il) {
+                constexpr int l = decltype(il)::value;
+                part[l] = 0.f;
+                if (16 * m + l < P) {
+                    const int pk = row_bcast<l>(tpk[m]);
+                    float val[4];
+                    sample_lds(pk, row_bcast<l>(tw1[m]), row_bcast<l>(tw2[m]), row_bcast<l>(tw3[m]),
+                               row_bcast<l>(tw4[m]), val);
+                    if (pk & FALLBACK)
+                        sample_global(key, Cq, cbase, cvalid, row_bcast<l>(tkh[m]),
+                                      row_bcast<l>(tkw[m]), val);
+                    float a = val[0] * qv[0];
+#pragma unroll
+                    for (int e = 1; e < 4; ++e) a = fma_(val[e], qv[e], a);
+                    part[l] = a;
+                }
+            });
+            float p1[8], p2[4], p3[2], p4[1];
+            halve<1, 16>(part, p1, lane);
+            halve<2, 8>(p1, p2, lane);
+            halve<4, 4>(p2, p3, lane);
+            halve<8, 2>(p3, p4, lane);
+            att[m] = p4[0];                       // logit of point 16 m + li
+        }
+        // softmax over the P points of the pixel: across the row's lanes and sets
+        bool okp[MAXSETS];
+#pragma unroll
+        for (int m = 0; m < MAXSETS; ++m) okp[m] = m < nsets && 16 * m + li < P;
+        float mx = okp[0] ? att[0] : -__builtin_huge_valf();
+#pragma unroll
+        for (int m = 1; m < MAXSETS; ++m)
+            if (okp[m]) mx = max_(mx, att[m]);
+        mx = max_(mx, row_xor<1>(mx, lane));
+        mx = max_(mx, row_xor<2>(mx, lane));
+        mx = max_(mx, row_xor<4>(mx, lane));
+        mx = max_(mx, row_xor<8>(mx, lane));
+        float sum = 0.f;
+#pragma unroll
+        for (int m = 0; m < MAXSETS; ++m) {
+            att[m] = okp[m] ? exp_(att[m] - mx) : 0.f;
+            sum += att[m];
+        }
+        sum += row_xor<1>(sum, lane);
+        sum += row_xor<2>(sum, lane);
+        sum += row_xor<4>(sum, lane);
+        sum += row_xor<8>(sum, lane);
+        const float inv = 1.f / sum;
+#pragma unroll
+        for (int m = 0; m < MAXSETS; ++m) att[m] *= inv;
+    };
+
+    // one value chunk of the group: 64 output channels of this row's pixel
+    auto av_chunk = [&](int cbase, int cvalid,
+                        const float (&att)[MAXSETS]) __attribute__((always_inline)) {
+        float o[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int m = 0; m < MAXSETS; ++m) {
+            if (m >= nsets) continue;
+            static_for<16>([&](auto il) {
+                constexpr int l = decltype(il)::value;
+                if (16 * m + l < P) {
+                    const int pk = row_bcast<l>(tpk[m]);
+                    const float wa = row_bcast<l>(att[m]);
+                    float val[4];
+                    sample_lds(pk, row_bcast<l>(tw1[m]), row_bcast<l>(tw2[m]), row_bcast<l>(tw3[m]),
+                               row_bcast<l>(tw4[m]), val);
+                    if (pk & FALLBACK)
+                        sample_global(value, C, cbase, cvalid, row_bcast<l>(tkh[m]),
+                                      row_bcast<l>(tkw[m]), val);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) o[e] = fma_(val[e], wa, o[e]);
+                }
+            });
+        }
+        if (active && 4 * li < cvalid)
+            __builtin_nontemporal_store(Q4::narrow(f32x4{o[0], o[1], o[2], o[3]}),
+                                        (Raw *)(out + hpixel * C + cbase + 4 * li));
+    };
+
+    stage_load(0);
+    for (int j = 0; j < ntot; ++j) {
+        stage_store();
+        __syncthreads();
+        if (j + 1 < ntot) stage_load(j + 1);
+        bool is_key;
+        int cbase, cvalid, nch;
+        chunk_of(j, is_key, cbase, cvalid, nch);
+        // the sample positions are set up again for every chunk (two points per
+        // lane: cheap) rather than kept for all the wave's quads
+#pragma unroll 1
+        for (int qi = 0; qi < NQ; ++qi) {
+            set_quad(qi);
+            setup_points(j / nPer);
+            float att[MAXSETS];
+            if (is_key) {
+                qk_group(cbase, cvalid, att);
+#pragma unroll
+                for (int m = 0; m < MAXSETS; ++m) att_keep[qi][m][tid] = att[m];
+            } else {
+#pragma unroll
+                for (int m = 0; m < MAXSETS; ++m) att[m] = att_keep[qi][m][tid];
+                av_chunk(cbase, cvalid, att);
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// quads per tile row / pixel rows per wave: 1, 1 = 4 x 4-pixel tiles.  8 x 8
+// tiles (2, 2) stage 2.9 x fewer window cells per pixel but leave room for two
+// workgroups per CU instead of three and measured 25 % slower.
+#ifndef SAPA_DNHWC_TILE
+#define SAPA_DNHWC_TILE 1, 1
+#endif
+template <typename T, int S, int NQX, int NQY>
+static hipError_t launch_geom(const void *q, const void *key, const void *value, const void *offset,
+                           void *out, int B, int Cq, int C, int H, int W, int P, int G,
+                           hipStream_t st) {
+    const int tiles_x = (W * S + 4 * NQX - 1) / (4 * NQX), tiles_y = (H * S + 4 * NQY - 1) / (4 * NQY);
+    const long nb = (long)tiles_x * tiles_y * B;
+    if (nb > (1L << 30)) return hipErrorNotSupported;
+    const int per_xcd = (int)((nb + 7) / 8);
+    hipLaunchKernelGGL((deform_fused_nhwc_kernel<T, S, NQX, NQY>), dim3(per_xcd * 8), dim3(256), 0, st,
+                       (const T *)q, (const T *)key, (const T *)value, (const T *)offset, (T *)out,
+                       Cq, C, H, W, P, G, tiles_x, tiles_y, (int)nb, per_xcd);
+    return hipGetLastError();
+}
+
+template <typename T>
+static hipError_t launch_t(const void *q, const void *key, const void *value, const void *offset,
+                           void *out, int B, int Cq, int C, int H, int W, int P, int s, int G,
+                           hipStream_t st) {
+    switch (s) {
+        case 1: return launch_geom<T, 1, SAPA_DNHWC_TILE>(q, key, value, offset, out, B, Cq, C, H, W, P, G, st);
+        case 2: return launch_geom<T, 2, SAPA_DNHWC_TILE>(q, key, value, offset, out, B, Cq, C, H, W, P, G, st);
+        case 4: return launch_geom<T, 4, SAPA_DNHWC_TILE>(q, key, value, offset, out, B, Cq, C, H, W, P, G, st);
+        default: return hipErrorNotSupported;
+    }
+}
+
+}  // namespace dnhwc
+
+// Channels-last tensors, f32 / f16 / bf16, s in {1, 2, 4}, P <= 32, channels per
+// group (Cq / G and C / G) multiples of 4, Cq / G <= 64, tensors aligned to 4
+// elements, one image's key / value tensor below 2^31 bytes.
+// hipErrorNotSupported otherwise.
+hipError_t deform_fused_nhwc_launch(const void *q, const void *key, const void *value,
+                                    const void *offset, void *out, int B, int Cq, int C, int H,
+                                    int W, int P, int s, int G, int dtype, hipStream_t st) {
+    // the query / key channels of a group are one LDS chunk
+    if (P > 16 * dnhwc::MAXSETS || (Cq / G) % 4 != 0 || Cq / G > 64 || (C / G) % 4 != 0)
+        return hipErrorNotSupported;
+    const int esize = dtype == 0 ? 4 : 2;
+    const long plane = (long)H * W * esize;
+    if (plane * Cq >= (1L << 31) || plane * C >= (1L << 31)) return hipErrorNotSupported;
+    const void *ptrs[4] = {q, key, value, out};
+    for (const void *p : ptrs)
+        if ((uintptr_t)p % (4 * esize) != 0) return hipErrorNotSupported;
+    if ((uintptr_t)offset % (2 * esize) != 0) return hipErrorNotSupported;
+    switch (dtype) {
+        case 0: return dnhwc::launch_t<float>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);
+        case 2: return dnhwc::launch_t<f16_t>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);
+        case 3: return dnhwc::launch_t<bf16_t>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);
+        default: return hipErrorNotSupported;
+    }
+}
+
+}  // namespace sapa

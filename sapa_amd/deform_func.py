@@ -177,6 +177,10 @@ def _deform_fused_backward(grad_output, query, key, value, offset, P, s, G, offs
     """Gradients of deform_av(softmax(deform_qk(q, k, off), dim=2), v, off)
     with respect to q, k, v and the offset tensor in its own layout."""
     with torch.no_grad():
+        # the gradient kernels take contiguous tensors: operands kept in
+        # channels-last order are copied here
+        query, key, value = query.contiguous(), key.contiguous(), value.contiguous()
+        grad_output = grad_output.contiguous()
         offset = expand_offset(offset, s, offset_layout).contiguous()
         logits = DeformQKFunction.apply(query, key, offset, P, s, G)
         attn = torch.softmax(logits.float(), dim=2).to(logits.dtype)
@@ -226,15 +230,24 @@ class DeformSAPAFusedFunction(Function):
         ctx.offset_layout = offset_layout
 
         n, c, h, w = value.size()
-        output = _lib.new_out(value, (n, c, scale_factor * h, scale_factor * w))
-        if value.is_cuda:
-            _lib.require_cuda_contiguous(query=query, key=key, value=value, offset=offset)
+        if not value.is_cuda:
+            raise NotImplementedError
+        nhwc = _lib.memory_layout(query=query, key=key, value=value,
+                                  offset=offset) == 'channels_last'
+        output = _lib.new_out(value, (n, c, scale_factor * h, scale_factor * w), nhwc)
+        if nhwc:
+            # every tensor in torch.channels_last order: served as it is
+            if offset_layout != 'hires':
+                raise RuntimeError("channels_last tensors take offset_layout='hires'")
+            _lib.call_nhwc('sapa_deform_fused_forward_nhwc', value.device, _lib.ptr(query),
+                           _lib.ptr(key), _lib.ptr(value), _lib.ptr(offset), _lib.ptr(output), n,
+                           key.size(1), c, h, w, num_point, scale_factor, groups,
+                           _lib.dtype_code(value))
+        else:
             _lib.call('sapa_deform_fused_forward_from', value.device, _lib.ptr(query),
                       _lib.ptr(key), _lib.ptr(value), _lib.ptr(offset), _lib.ptr(output), n,
                       key.size(1), c, h, w, num_point, scale_factor, groups,
                       OFFSET_LAYOUTS[offset_layout], _lib.dtype_code(value))
-        else:
-            raise NotImplementedError
 
         if any(t.requires_grad for t in (query, key, value, offset)):
             ctx.save_for_backward(query, key, value, offset)

@@ -1,0 +1,114 @@
+"""GPU parity of the fused SAPA-D forward on tensors in torch.channels_last
+order (sapa_deform_fused_forward_nhwc) against the CPU oracle and against the
+library's contiguous path.
+
+The oracle runs the reference kernels' fp32 arithmetic (same index math, same
+guard).  The logits' channel sums run in tree order here, so the comparison
+uses the reference's own check tolerance, allclose(atol=1e-5)
+(deformsapa/deformsapa/forward_check.py), tightened to 1e-5 rel / 1e-6 abs for
+short sums; 16-bit within the usual relative bars.
+"""
+import pytest
+import torch
+
+import sapa_amd
+from helpers import BF16_REL, F16_REL, assert_f32_close, assert_rel_rms_close, gen, randn
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda:0'
+CL = torch.channels_last
+
+# B, G, d (q/k channels per group), cg (value channels per group), H, W, P, s, offset scale
+SHAPES = [(2, 2, 4, 8, 5, 7, 9, 2, 1.0), (1, 4, 32, 64, 8, 8, 25, 2, 0.75), (1, 1, 64, 72, 6, 5, 4, 2, 1.5),
+          (1, 2, 8, 132, 4, 6, 16, 1, 1.0), (2, 3, 4, 4, 3, 5, 17, 4, 1.0), (1, 2, 8, 8, 9, 9, 32, 2, 1.0),
+          (1, 1, 4, 4, 1, 1, 1, 2, 1.0),
+          # offsets far beyond the +-4 cells of the LDS window: the global-memory path
+          (1, 2, 8, 12, 14, 13, 9, 2, 6.0)]
+IDS = ['-'.join(map(str, s)) for s in SHAPES]
+
+
+def cl(*ts):
+    return [t.to(DEV).contiguous(memory_format=CL) for t in ts]
+
+
+def inputs(g, B, G, d, cg, H, W, P, s, oscale, dtype=torch.float32):
+    q = randn(g, B, G * d, s * H, s * W).to(dtype)
+    key = randn(g, B, G * d, H, W).to(dtype)
+    v = randn(g, B, G * cg, H, W).to(dtype)
+    off = (randn(g, B, 2 * G * P, s * H, s * W) * oscale).to(dtype)
+    return q, key, v, off
+
+
+@pytest.mark.parametrize('shape', SHAPES, ids=IDS)
+def test_fp32_vs_oracle(coracle, shape):
+    B, G, d, cg, H, W, P, s, _ = shape
+    q, key, v, off = inputs(gen(500), *shape)
+    got = sapa_amd.deform_sapa_fused(*cl(q, key, v, off), P, s, G)
+    assert got.is_contiguous(memory_format=CL) and got.shape == (B, G * cg, s * H, s * W)
+    want = coracle.deform_sapa_fused(q, key, v, off, P, s, G, 'f32')
+    if d <= 8:
+        assert_f32_close(got, want, 'fused')
+    else:
+        torch.testing.assert_close(got.cpu(), want, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize('dtype,rel', [(torch.bfloat16, BF16_REL), (torch.float16, F16_REL)])
+@pytest.mark.parametrize('shape', SHAPES[:4] + SHAPES[7:], ids=IDS[:4] + IDS[7:])
+def test_16bit_vs_oracle(coracle, shape, dtype, rel):
+    B, G, d, cg, H, W, P, s, _ = shape
+    q, key, v, off = inputs(gen(501), *shape, dtype=dtype)
+    got = sapa_amd.deform_sapa_fused(*cl(q, key, v, off), P, s, G)
+    assert got.dtype == dtype and got.is_contiguous(memory_format=CL)
+    want = coracle.deform_sapa_fused(q.float(), key.float(), v.float(), off.float(), P, s, G, 'f32')
+    assert_rel_rms_close(got.float(), want, rel, 'fused')
+
+
+def test_matches_contiguous_path_at_a_larger_shape():
+    B, G, d, cg, H, W, P, s = 2, 4, 32, 64, 19, 22, 25, 2
+    q, key, v, off = inputs(gen(502), B, G, d, cg, H, W, P, s, 0.75)
+    off = off.clamp(-4, 4)
+    want = sapa_amd.deform_sapa_fused(*(t.to(DEV) for t in (q, key, v, off)), P, s, G)
+    got = sapa_amd.deform_sapa_fused(*cl(q, key, v, off), P, s, G)
+    torch.testing.assert_close(got.contiguous(), want, rtol=2e-5, atol=2e-5)
+
+
+def test_guard_failures_and_image_border():
+    """Offsets that push most points out of the image: those points keep logit
+    0, take part in the softmax and contribute nothing."""
+    B, G, d, cg, H, W, P, s = 1, 2, 4, 8, 6, 7, 9, 2
+    g = gen(503)
+    q, key, v, off = inputs(g, B, G, d, cg, H, W, P, s, 1.0)
+    off = off + 5.0 * torch.sign(randn(g, *off.shape))      # +-5 cells: in or out of a 6x7 image
+    want_shape = (B, G * cg, s * H, s * W)
+    got = sapa_amd.deform_sapa_fused(*cl(q, key, v, off), P, s, G)
+    assert got.shape == want_shape
+    want = sapa_amd.deform_sapa_fused(*(t.to(DEV) for t in (q, key, v, off)), P, s, G)
+    torch.testing.assert_close(got.contiguous(), want, rtol=1e-5, atol=1e-6)
+    # every point outside: uniform weights over nothing -> exact zeros
+    off_far = torch.full_like(off, 100.0)
+    got = sapa_amd.deform_sapa_fused(*cl(q, key, v, off_far), P, s, G)
+    assert torch.count_nonzero(got) == 0
+
+
+def test_layout_errors_and_backward():
+    B, G, d, cg, H, W, P, s = 1, 2, 4, 8, 5, 6, 9, 2
+    q, key, v, off = inputs(gen(504), B, G, d, cg, H, W, P, s, 1.0)
+    qc, kc, vc, oc = cl(q, key, v, off)
+    with pytest.raises(RuntimeError, match='contiguous'):
+        sapa_amd.deform_sapa_fused(qc, kc, vc, off.to(DEV), P, s, G)          # mixed orders
+    q6 = randn(gen(505), B, G * 3, s * H, s * W)
+    k6 = randn(gen(506), B, G * 3, H, W)
+    with pytest.raises(RuntimeError, match='channels_last'):
+        sapa_amd.deform_sapa_fused(*cl(q6, k6, v, off), P, s, G)              # 3 channels per group
+    q68, k68 = randn(gen(508), B, G * 68, s * H, s * W), randn(gen(509), B, G * 68, H, W)
+    with pytest.raises(RuntimeError, match='channels_last'):
+        sapa_amd.deform_sapa_fused(*cl(q68, k68, v, off), P, s, G)            # 68 channels per group
+    grads = []
+    go = randn(gen(507), B, G * cg, s * H, s * W)
+    for fmt in (torch.contiguous_format, CL):
+        ts = [t.to(DEV).contiguous(memory_format=fmt).requires_grad_() for t in (q, key, v, off)]
+        out = sapa_amd.deform_sapa_fused(*ts, P, s, G)
+        out.backward(go.to(DEV).contiguous(memory_format=fmt))
+        grads.append([t.grad for t in ts])
+    for a, b, name in zip(grads[0], grads[1], ('query', 'key', 'value', 'offset')):
+        torch.testing.assert_close(b, a, rtol=1e-4, atol=1e-5, msg=lambda m: f'grad_{name}: {m}')
