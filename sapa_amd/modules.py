@@ -152,7 +152,8 @@ class SAPADeform(nn.Module):
             if self.norm:
                 y = self.norm_y(y)
             q, k, offset_lo = self.q(y), self.k(x_), self.offset(x_)
-        if self.fused:
+        if self.fused and (x.is_contiguous()
+                           or not x.is_contiguous(memory_format=torch.channels_last)):
             # the kernel reads the offset convolution's output in place
             return deform_sapa_fused(q.contiguous(), k.contiguous(), x.contiguous(),
                                      offset_lo.contiguous(), self.num_point,
@@ -166,9 +167,15 @@ class SAPADeform(nn.Module):
 
     def attention(self, q, k, x, offset):
         P, s, G = self.num_point, self.up_factor, self.groups
-        offset = offset.contiguous()
         if self.fused:
-            return deform_sapa_fused(q.contiguous(), k.contiguous(), x.contiguous(), offset,
-                                     P, s, G)
+            # one memory order for all tensors, the value's: a channels-last
+            # model stays channels-last (the fused kernel serves that order)
+            fmt = (torch.channels_last
+                   if not x.is_contiguous() and x.is_contiguous(memory_format=torch.channels_last)
+                   else torch.contiguous_format)
+            q, k, x, offset = (t.contiguous(memory_format=fmt) for t in (q, k, x, offset))
+            return deform_sapa_fused(q, k, x, offset, P, s, G)
+        # the separate operators take contiguous tensors only
+        q, k, x, offset = (t.contiguous() for t in (q, k, x, offset))
         attn = F.softmax(deform_qk(q, k, offset, P, s, G), dim=2)
         return deform_av(attn, x, offset, P, s, G)

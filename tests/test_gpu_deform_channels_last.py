@@ -112,3 +112,17 @@ def test_layout_errors_and_backward():
         grads.append([t.grad for t in ts])
     for a, b, name in zip(grads[0], grads[1], ('query', 'key', 'value', 'offset')):
         torch.testing.assert_close(b, a, rtol=1e-4, atol=1e-5, msg=lambda m: f'grad_{name}: {m}')
+
+
+def test_module_in_channels_last_format():
+    torch.manual_seed(1)
+    m = sapa_amd.SAPADeform(64, 64, up_factor=2, num_point=9, groups=4, embedding_dim=32).to(DEV)
+    g = gen(510)
+    y, x = randn(g, 2, 64, 18, 22).to(DEV), randn(g, 2, 64, 9, 11).to(DEV)
+    want = m(y, x)
+    mc = m.to(memory_format=CL)
+    got = mc(y.contiguous(memory_format=CL), x.contiguous(memory_format=CL))
+    assert got.is_contiguous(memory_format=CL)
+    torch.testing.assert_close(got, want, rtol=1e-4, atol=1e-5)
+    got.sum().backward()
+    assert all(p.grad is not None for p in mc.parameters())
