@@ -55,6 +55,8 @@ MEASURED_TRAFFIC_BYTES = {
     ('fpn_large', 'fp32', 'channels_last'): 1720616943,
     # profiles/sapa_b_nhwc_fused_fpn_large_bf16.md: (151310.0 * 1.9999 + 537600.0 * 1.0000) KiB
     ('fpn_large', 'bf16', 'channels_last'): 860377478,
+    # profiles/sapa_d_nhwc_fused_deform_p25_fp32.md: (109284.2 * 2.0000 + 131072.0 * 1.0000) KiB
+    ('deform_p25', 'fp32', 'channels_last'): 358026263,
     # profiles/sapa_b_mfma_fused_stress_bf16.md: (39700.2 * 1.9999 + 292841.7 * 1.0000) KiB
     ('stress', 'bf16'): 381173848,
     # profiles/sapa_d_lds_fused_deform_p9_fp32.md: (132709.9 * 1.9999 + 131503.8 * 1.0000) KiB
