@@ -245,7 +245,7 @@ def deform_sapa_fused(query: Tensor, key: Tensor, value: Tensor, offset: Tensor,
 
 @deform_sapa_fused.register_fake
 def _(query, key, value, offset, num_point, scale_factor, groups, offset_layout='hires'):
-    return value.new_empty(value.shape[:2] + _hi(value, scale_factor))
+    return _new_out(value, value.shape[:2] + _hi(value, scale_factor), query, key, value, offset)
 
 
 @custom_op(f'{_NS}::deform_sapa_fused_backward', mutates_args=())
@@ -258,8 +258,7 @@ def deform_sapa_fused_backward(grad_output: Tensor, query: Tensor, key: Tensor, 
 
 @deform_sapa_fused_backward.register_fake
 def _(grad_output, query, key, value, offset, num_point, scale_factor, groups, offset_layout):
-    return (torch.empty_like(query), torch.empty_like(key), torch.empty_like(value),
-            torch.empty_like(offset))
+    return _new_grad(query), _new_grad(key), _new_grad(value), _new_grad(offset)
 
 
 def _dfused_setup(ctx, inputs, output):

@@ -99,6 +99,17 @@ def test_channels_last_ops_and_compile():
     y_ref.backward(go)
     for a, b in zip(leaves, ref_leaves):
         assert torch.equal(a.grad, b.grad)
+    # SAPA-D: 4 channels per group so that the channels-last kernel takes it
+    g = gen(402)
+    B, G, H, W, P, s = 1, 2, 5, 6, 4, 2
+    dq, dk = randn(g, B, G * 4, H * s, W * s).to(DEV), randn(g, B, G * 4, H, W).to(DEV)
+    dv, off = randn(g, B, G * 8, H, W).to(DEV), randn(g, B, 2 * G * P, H * s, W * s).to(DEV)
+    dq, dk, dv, off = (t.contiguous(memory_format=CL) for t in (dq, dk, dv, off))
+    out = torch.ops.sapa_amd.deform_sapa_fused(dq, dk, dv, off, P, s, G)
+    assert out.is_contiguous(memory_format=CL)
+    assert torch.equal(out, sapa_amd.deform_sapa_fused(dq, dk, dv, off, P, s, G))
+    torch.library.opcheck(torch.ops.sapa_amd.deform_sapa_fused.default, (dq, dk, dv, off, P, s, G),
+                          test_utils=tests)
 
 
 def test_opcheck():
