@@ -23,11 +23,15 @@ HIPCC = os.environ.get('HIPCC', '/opt/rocm/bin/hipcc')
 FLAGS = ['-O3', '-std=c++17', '--offload-arch=gfx950', '-fPIC', '-fno-gpu-rdc',
          '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
          '-Wall', '-Wno-unused-function']
+# sapa_b_nhwc keeps its MFMA accumulators in ordinary VGPRs: left to itself the
+# compiler moves them to the accumulation registers on top of an already full
+# VGPR budget, which costs the kernel a wave per SIMD
+SOURCE_FLAGS = {'sapa_b_nhwc.hip': ['-mllvm', '-amdgpu-mfma-vgpr-form']}
 
 
 def _compile(src, extra):
     obj = os.path.join(OBJ, os.path.splitext(src)[0] + '.o')
-    cmd = [HIPCC] + FLAGS + extra + ['-c', os.path.join(CSRC, src), '-o', obj]
+    cmd = [HIPCC] + FLAGS + SOURCE_FLAGS.get(src, []) + extra + ['-c', os.path.join(CSRC, src), '-o', obj]
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     out = '\n'.join(l for l in r.stdout.splitlines()
                     if "is not a recognized feature for this target" not in l)

@@ -24,11 +24,17 @@
 //     Afterwards lane l holds, for window row ky, the logits with in-row index
 //     16 m + l (index = 4 * kx + child): 100 values in 10 registers per lane;
 //   * softmax per child across the 4 lanes x 10 registers that hold its taps;
-//   * aggregation: the weights stay in those registers; every FMA fetches its
-//     weight from the lane that owns it through a DPP row broadcast
-//     (v_fmac_f32_dpp row_newbcast), so a lane needs 4 s^2 accumulators (children
-//     x 4 channels) and no copy of the weights.  One 16-byte LDS read feeds
-//     4 s^2 FMAs.
+//   * aggregation on the matrix pipe: for one tap, out[child][channel] +=
+//     weight[child] * value[channel] is a 4 x 4 outer product per lane quad,
+//     which is what v_mfma_f32_4x4x1 computes for 16 independent blocks of 4
+//     lanes (one FMA per element, so the tap order and the rounding are those
+//     of the scalar loop).  Lanes 4b .. 4b+3 (block b) supply 4 value channels
+//     as B; the weights stay where the butterfly left them -- the 4 children's
+//     weights of tap kx sit in lanes 4 (kx % 4) .. +3 of the row -- and the
+//     instruction's A-broadcast (cbsz = 2: one block feeds its group of 4
+//     blocks, i.e. the row of 16 lanes; abid = kx % 4 picks it) hands them to
+//     the whole row.  One 16-byte LDS read feeds 4 such instructions (one per
+//     channel of the lane), 4 s^2 accumulators per lane, no copy of the weights.
 //
 // The channel sums run in tree order, not in the reference kernels' sequential
 // order: results agree with them to rounding (1e-5 relative in fp32), not bit
@@ -103,19 +109,6 @@ __device__ __forceinline__ float row_xor(float v, int lane) {
     else y.i = __builtin_amdgcn_ds_bpermute((lane ^ D) << 2, x.i);
     return y.f;
 }
-// acc += v * (w of lane SRC of the own row of 16 lanes): one instruction, the
-// weight is fetched through the DPP row broadcast.  The caller keeps two wait
-// states between the last VALU write of w and the first of these.  (A DPP
-// operand halves the issue rate of the instruction on this part -- measured 4.4
-// against 2.2 cycles per wave and SIMD -- but fetching the weight with a DPP
-// move and following it with 4 plain FMAs measured slower still.)
-template <int SRC>
-__device__ __forceinline__ void fma_bcast(float &acc, float w, float v) {
-    asm("v_fmac_f32_dpp %0, %1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf"
-        : "+v"(acc)
-        : "v"(w), "v"(v), "n"(SRC));
-}
-
 // One butterfly step over lane distance D: n values per lane -> (n + 1) / 2.
 // The lane whose bit D is clear keeps the even-indexed sums, its partner the
 // odd-indexed ones; each adds what the other held of them.
@@ -353,19 +346,18 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
     }
 
     if (DO_AV) {
-        asm volatile("s_nop 4");                   // w was just written: DPP reads need two wait states
         for (int j = nKc; j < ntot; ++j) {
             if (j + 1 < ntot) stage_load(j + 1);
             const int c0 = (j - nKc) * CHK;
             const float *wb = win + (j & 1) * BUF;
-            float o[NJ][4];
+            // acc[g][u][i]: child 4g + i, channel c0 + 4 li + u
+            f32x4 acc[NG][4];
 #pragma unroll
-            for (int jj = 0; jj < NJ; ++jj)
+            for (int g = 0; g < NG; ++g)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) o[jj][e] = 0.f;
+                for (int u = 0; u < 4; ++u) acc[g][u] = f32x4{0.f, 0.f, 0.f, 0.f};
             // the window values travel through a ring of AHEAD + 1 registers of
-            // 4 channels: tap t + AHEAD is read while tap t is multiplied (the
-            // FMAs are opaque to the scheduler, so the distance is set here)
+            // 4 channels: tap t + AHEAD is read while tap t is multiplied
             constexpr int AHEAD = S == 2 ? 3 : 1;
             f32x4 ring[AHEAD + 1];
             static_for<AHEAD>([&](auto it) {
@@ -377,13 +369,13 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
                 if (tn < KK)
                     ring[tn % (AHEAD + 1)] = *(const f32x4 *)(wb + ((tn / K) * WW + tn % K) * CHK);
                 const f32x4 vv = ring[t % (AHEAD + 1)];
-                static_for<NJ>([&](auto ijj) {
-                    // the weight lives in register (ky * NG + g) * RPR + idx / 16 of lane idx % 16
-                    constexpr int jj = decltype(ijj)::value, g = jj / 4, idx = kx * 4 + jj % 4;
-                    const float wr = w[(ky * NG + g) * RPR + idx / 16];
-                    static_for<4>([&](auto ie) {
-                        constexpr int e = decltype(ie)::value;
-                        fma_bcast<idx % 16>(o[jj][e], wr, vv[e]);
+                static_for<NG>([&](auto ig) {
+                    // in-row index 4 kx + child: register kx / 4 of (ky, g), lanes 4 (kx % 4) .. +3
+                    constexpr int g = decltype(ig)::value;
+                    const float wr = w[(ky * NG + g) * RPR + kx / 4];
+                    static_for<4>([&](auto iu) {
+                        constexpr int u = decltype(iu)::value;
+                        acc[g][u] = __builtin_amdgcn_mfma_f32_4x4x1f32(wr, vv[u], acc[g][u], 2, kx % 4, 0);
                     });
                 });
             });
@@ -396,7 +388,8 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
 #pragma unroll
                 for (int jj = 0; jj < NJ; ++jj)
                     __builtin_nontemporal_store(
-                        Q4::narrow(f32x4{o[jj][0], o[jj][1], o[jj][2], o[jj][3]}),
+                        Q4::narrow(f32x4{acc[jj / 4][0][jj % 4], acc[jj / 4][1][jj % 4],
+                                         acc[jj / 4][2][jj % 4], acc[jj / 4][3][jj % 4]}),
                         (Raw *)(out + child_pixel(jj) * C + c0 + 4 * li));
             }
             __syncthreads();
