@@ -290,8 +290,12 @@ static int nhwc_common(int mode, const void *query, const void *key, const void 
     const bool need_qk = mode != TILED_AV, need_av = mode == TILED_AV || mode == TILED_FUSED;
     if (!out || (need_qk && (!query || !key)) || (need_av && !value) || (mode == TILED_AV && !attn))
         return SAPA_ERR_INVALID_ARGUMENT;
-    const hipError_t e = sapa_b_nhwc_launch(mode, query, key, attn, value, out, B, d, C, H, W, K, s,
-                                            dtype, (hipStream_t)stream);
+    // 16-bit tensors: the kernel on the 16-bit matrix instructions first
+    hipError_t e = sapa_b_nhwc16_launch(mode, query, key, attn, value, out, B, d, C, H, W, K, s, dtype,
+                                        (hipStream_t)stream);
+    if (e == hipErrorNotSupported)
+        e = sapa_b_nhwc_launch(mode, query, key, attn, value, out, B, d, C, H, W, K, s, dtype,
+                               (hipStream_t)stream);
     if (e == hipErrorNotSupported) return SAPA_ERR_UNSUPPORTED;
     return finish(e);
 }

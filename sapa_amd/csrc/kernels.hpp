@@ -38,6 +38,12 @@ hipError_t sapa_b_nhwc_launch(int mode, const void *q, const void *key, const vo
                               const void *value, void *out, int B, int d, int C, int H, int W,
                               int K, int s, int dtype, hipStream_t st);
 
+// sapa_b_nhwc16.hip: the same four modes for f16 / bf16 channels-last tensors
+// on the 16-bit matrix instructions (hipErrorNotSupported for anything else)
+hipError_t sapa_b_nhwc16_launch(int mode, const void *q, const void *key, const void *attn_in,
+                                const void *value, void *out, int B, int d, int C, int H, int W,
+                                int K, int s, int dtype, hipStream_t st);
+
 // sapa_d_nhwc.hip: fused SAPA-D forward for tensors in channels-last memory
 // order (offsets [B, sH, sW, 2GP]); f32 / f16 / bf16, s in {1, 2, 4}, P <= 32,
 // channels per group multiples of 4, at most 64 query / key channels per group.
