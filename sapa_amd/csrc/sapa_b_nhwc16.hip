@@ -79,12 +79,12 @@ template <> struct Mma<bf16_t> {
     }
 };
 
+// two floats -> two T (round to nearest even) in one dword
 template <typename T>
 __device__ __forceinline__ u32 pack2(float a, float b) {
-    union { u32 u; T h[2]; } x;
-    x.h[0] = (T)a;
-    x.h[1] = (T)b;
-    return x.u;
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef T tx2 __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(u32, __builtin_convertvector(f32x2{a, b}, tx2));
 }
 
 // value of lane (l ^ D) of the same row of 16 lanes, D = 4 or 8
@@ -174,14 +174,28 @@ sapa_b_nhwc16_kernel(const T *__restrict__ q, const T *__restrict__ key,
         const T *base = (is_key ? key : value) + (long)n * lpix * nch;
         const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(
             (void *)base, 0, (int)(lpix * nch * (long)sizeof(T)), 0x00020000);
-        const bool c_ok = c0 + 4 * sq < nch;
+        // bit 31 set = past the descriptor; pure arithmetic (sign bits of "channel
+        // within the tensor" and "position within the image") instead of selects
+        const u32 c_bad = (u32)(nch - 1 - (c0 + 4 * sq));
 #pragma unroll
         for (int p = 0; p < NPASS; ++p) {
-            const u32 off = (c_ok && spix[p] >= 0)
-                                ? (u32)(spix[p] * nch + c0 + 4 * sq) * (u32)sizeof(T)
-                                : 0x80000000u;
+            const u32 off = ((u32)(spix[p] * nch + c0 + 4 * sq) * (u32)sizeof(T)) |
+                            ((c_bad | (u32)spix[p]) & 0x80000000u);
             st[p] = __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0);
         }
+    };
+    // the same for value chunk jv from offsets prepared once (voff0, set up before
+    // the aggregation): two instructions per load instead of the full address
+    u32 voff0[NPASS];
+    auto stage_load_value = [&](int jv) __attribute__((always_inline)) {
+        const T *base = value + (long)n * lpix * C;
+        const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)base, 0, (int)(lpix * C * (long)sizeof(T)), 0x00020000);
+        const u32 c_bad = (u32)(C - 1 - (jv * CHK + 4 * sq)) & 0x80000000u;
+#pragma unroll
+        for (int p = 0; p < NPASS; ++p)
+            st[p] = __builtin_amdgcn_raw_buffer_load_b64(
+                r, (voff0[p] + (u32)(jv * CHK) * (u32)sizeof(T)) | c_bad, 0, 0);
     };
     auto stage_store = [&](int j) __attribute__((always_inline)) {
         u32 *dst = lds + (j & 1) * BUF;
@@ -326,8 +340,11 @@ sapa_b_nhwc16_kernel(const T *__restrict__ q, const T *__restrict__ key,
                 for (int k = 0; k < 4; ++k) x[k] = 4 * gi + k < NTAU ? w[g * NTAU + 4 * gi + k] : 0.f;
                 wpk[g][gi] = u32x2{pack2<T>(x[0], x[1]), pack2<T>(x[2], x[3])};
             }
+#pragma unroll
+        for (int p = 0; p < NPASS; ++p)
+            voff0[p] = ((u32)(spix[p] * C + 4 * sq) * (u32)sizeof(T)) | ((u32)spix[p] & 0x80000000u);
         for (int j = nKc; j < ntot; ++j) {
-            if (j + 1 < ntot) stage_load(j + 1);
+            if (j + 1 < ntot) stage_load_value(j + 1 - nKc);
             const int c0 = (j - nKc) * CHK;
             const u32 *wb = win + (j & 1) * BUF;
             // acc[g][u][i]: child 4g + i, channel c0 + 4 li + u
