@@ -53,8 +53,8 @@ MEASURED_TRAFFIC_BYTES = {
     ('fpn_large', 'bf16'): 966196919,
     # profiles/sapa_b_nhwc_fused_fpn_large_fp32.md: (302512.3 * 2.0000 + 1075280.5 * 1.0000) KiB
     ('fpn_large', 'fp32', 'channels_last'): 1720501948,
-    # profiles/sapa_b_nhwc_fused_fpn_large_bf16.md: (151310.0 * 1.9999 + 537600.0 * 1.0000) KiB
-    ('fpn_large', 'bf16', 'channels_last'): 860344711,
+    # profiles/sapa_b_nhwc_fused_fpn_large_bf16.md: (153483.6 * 2.0000 + 537600.7 * 1.0000) KiB
+    ('fpn_large', 'bf16', 'channels_last'): 864829676,
     # profiles/sapa_d_nhwc_fused_deform_p25_fp32.md: (109284.2 * 2.0000 + 131072.0 * 1.0000) KiB
     ('deform_p25', 'fp32', 'channels_last'): 358026263,
     # profiles/sapa_b_mfma_fused_stress_bf16.md: (39700.2 * 1.9999 + 292841.7 * 1.0000) KiB
@@ -272,8 +272,10 @@ def main():
         wl = (f'{args.workload}: SAPA-B FPN-style B={B} C={C} d={d} '
               f'{H}x{W}->{H * s}x{W * s} K={K} s={s} {args.dtype}, '
               + ('channels_last' if args.layout == 'channels_last' else 'NCHW'))
+        nhwc_kern = ('sapa_b_nhwc16_kernel (fused mode)' if esize == 2 and d % 8 == 0
+                     else 'sapa_b_nhwc_kernel (fused mode)')
         if args.layout == 'channels_last':
-            kern = 'sapa_b_nhwc_kernel (fused mode)'
+            kern = nhwc_kern
         elif (K, s) != (5, 2):
             kern = 'sapa_b_mfma_kernel (fused mode)'
         elif esize == 2 and W % 4 == 0 and W >= 32:
@@ -322,7 +324,7 @@ def main():
         rec['channels_last'] = {
             'ms_per_step': ms_cl, 'value': pix / (ms_cl * 1e-3) / 1e9, 'unit': 'Gpix/s',
             'roofline_frac': abytes / (ms_cl * 1e-3) / 1e9 / HBM_PEAK_GBS,
-            'kernel': 'deform_fused_nhwc_kernel' if deform else 'sapa_b_nhwc_kernel (fused mode)',
+            'kernel': 'deform_fused_nhwc_kernel' if deform else nhwc_kern,
             'max_abs_diff_vs_nchw_image0': err_cl,
             'note': 'same workload and algorithmic bytes, every tensor in torch.channels_last '
                     'order (python bench.py --layout channels_last makes this the main line)'}

@@ -158,7 +158,11 @@ int sapa_qk_softmax_forward(const void *query, const void *key, void *attn,
  * SAPA_F32 / F16 / BF16, (K, s) in {(3,2), (5,2), (7,2), (5,4), (7,4)}, channel counts that are multiples
  * of 4, tensors aligned to 4 elements; SAPA_ERR_UNSUPPORTED otherwise.  The
  * channel sums run in tree order: results agree with sapa_*_forward to
- * rounding (1e-5 relative in fp32), not bit for bit. */
+ * rounding (1e-5 relative in fp32), not bit for bit.  16-bit tensors whose d
+ * is a multiple of 8 run on the 16-bit matrix instructions: fp32 accumulation,
+ * and in the fused operator the softmax weights are rounded to the tensor type
+ * before the aggregation, as they are when qk, softmax and av are called one
+ * after the other on 16-bit tensors. */
 int sapa_qk_forward_nhwc(const void *query, const void *key, void *out,
                          int B, int d, int H, int W, int K, int s,
                          int dtype, void *stream);

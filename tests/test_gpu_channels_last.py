@@ -72,19 +72,43 @@ def test_fp32_vs_oracle(coracle, shape):
 
 
 @pytest.mark.parametrize('dtype,rel', [(torch.bfloat16, BF16_REL), (torch.float16, F16_REL)])
-@pytest.mark.parametrize('shape', SHAPES[:5] + SHAPES[7:10], ids=IDS[:5] + IDS[7:10])
+@pytest.mark.parametrize('shape', SHAPES, ids=IDS)
 def test_16bit_vs_oracle(coracle, shape, dtype, rel):
+    """Shapes with d % 8 == 0 run on the 16-bit matrix-instruction kernel (16-bit
+    windows in LDS, weights rounded to the tensor type before the aggregation),
+    the others on the kernel that widens to fp32 in LDS."""
     B, d, C, H, W, K, s = shape
     q, key, v, attn = inputs(gen(301), *shape, dtype=dtype)
     qf, kf, vf, af = (x.float() for x in (q, key, v, attn))
     got = sapa_amd.qk(*cl(q, key), K, s)
     assert got.dtype == dtype and got.is_contiguous(memory_format=CL)
     assert_rel_rms_close(got.float(), coracle.qk(qf, kf, K, s, 'f32a64'), rel, 'qk')
+    got = sapa_amd.qk_softmax(*cl(q, key), K, s)
+    assert got.dtype == dtype and got.is_contiguous(memory_format=CL)
+    want = coracle.softmax(coracle.qk(qf, kf, K, s, 'f32a64').float(), 1, 'f32')
+    torch.testing.assert_close(got.float().cpu(), want, rtol=rel, atol=rel / 4)
     got = sapa_amd.av(*cl(attn, v), K, s)
     assert_rel_rms_close(got.float(), coracle.av(af, vf, K, s, 'f32a64'), rel, 'av')
     got = sapa_amd.sapa_fused(*cl(q, key, v), K, s)
     assert got.dtype == dtype and got.is_contiguous(memory_format=CL)
     assert_rel_rms_close(got.float(), coracle.sapa_fused(qf, kf, vf, K, s, 'f32a64'), rel, 'fused')
+
+
+@pytest.mark.parametrize('dtype,rel', [(torch.bfloat16, BF16_REL), (torch.float16, F16_REL)])
+@pytest.mark.parametrize('K,s', [(5, 2), (7, 4)])
+def test_16bit_matches_contiguous_path_at_a_larger_shape(dtype, rel, K, s):
+    """Several tiles per image, several images, two key chunks and a ragged
+    value chunk: the 16-bit matrix-instruction kernel against the library's
+    NCHW kernels on the same 16-bit values."""
+    B, d, C, H, W = 3, 72, 100, 11, 14
+    q, key, v, attn = inputs(gen(311), B, d, C, H, W, K, s, dtype=dtype)
+    qd, kd, vd, ad = (t.to(DEV) for t in (q, key, v, attn))
+    assert_rel_rms_close(sapa_amd.sapa_fused(*cl(q, key, v), K, s).float().contiguous(),
+                         sapa_amd.sapa_fused(qd, kd, vd, K, s).float().cpu(), rel, 'fused')
+    assert_rel_rms_close(sapa_amd.av(*cl(attn, v), K, s).float().contiguous(),
+                         sapa_amd.av(ad, vd, K, s).float().cpu(), rel, 'av')
+    assert_rel_rms_close(sapa_amd.qk(*cl(q, key), K, s).float().contiguous(),
+                         sapa_amd.qk(qd, kd, K, s).float().cpu(), rel, 'qk')
 
 
 def test_matches_contiguous_path_at_a_larger_shape():
