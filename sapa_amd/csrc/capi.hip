@@ -291,8 +291,13 @@ static int nhwc_common(int mode, const void *query, const void *key, const void 
     if (!out || (need_qk && (!query || !key)) || (need_av && !value) || (mode == TILED_AV && !attn))
         return SAPA_ERR_INVALID_ARGUMENT;
     // 16-bit tensors: the kernel on the 16-bit matrix instructions first
+    // (SAPA_NHWC16_OFF: a tuning build without it, for comparisons)
+#ifdef SAPA_NHWC16_OFF
+    hipError_t e = hipErrorNotSupported;
+#else
     hipError_t e = sapa_b_nhwc16_launch(mode, query, key, attn, value, out, B, d, C, H, W, K, s, dtype,
                                         (hipStream_t)stream);
+#endif
     if (e == hipErrorNotSupported)
         e = sapa_b_nhwc_launch(mode, query, key, attn, value, out, B, d, C, H, W, K, s, dtype,
                                (hipStream_t)stream);
