@@ -59,6 +59,8 @@ MEASURED_TRAFFIC_BYTES = {
     ('deform_p25', 'fp32', 'channels_last'): 358026263,
     # profiles/sapa_b_mfma_fused_stress_bf16.md: (39700.2 * 1.9999 + 292841.7 * 1.0000) KiB
     ('stress', 'bf16'): 381173848,
+    # profiles/sapa_b_nhwc16_fused_stress_bf16.md
+    ('stress', 'bf16', 'channels_last'): 323034807,
     # profiles/sapa_d_lds_fused_deform_p9_fp32.md: (132709.9 * 1.9999 + 131503.8 * 1.0000) KiB
     ('deform_p9', 'fp32'): 406442924,
     # profiles/sapa_d_lds_fused_deform_p25_fp32.md: (343906.3 * 1.9999 + 131079.0 * 1.0000) KiB
@@ -71,10 +73,17 @@ def algorithmic_bytes(B, C, d, H, W, s, esize):
     return esize * (B * H * s * W * s * (d + C) + B * H * W * (d + C))
 
 
-def make_inputs(cfg, dtype, device, seed=0):
+def make_inputs(cfg, dtype, device, seed=0, heavy_tails=False):
     B, C, d, H, W, K, s = cfg
     g = torch.Generator(device=device).manual_seed(seed)
     q = torch.randn(B, d, H * s, W * s, generator=g, device=device)
+    if heavy_tails:
+        # a random 10 % of the query replaced by Student-t(3) draws (the stress
+        # workload: logits with outliers for the softmax)
+        z = torch.randn(4, *q.shape, generator=g, device=device)
+        t3 = z[0] / (z[1:].pow(2).mean(0)).sqrt()
+        q = torch.where(torch.rand(q.shape, generator=g, device=device) < 0.1, t3, q)
+        del z, t3
     # keys L2-magnitude-varied via a per-channel scale ~U(0.5, 2)
     scale = torch.rand(d, generator=g, device=device) * 1.5 + 0.5
     key = torch.randn(B, d, H, W, generator=g, device=device) * scale.view(1, d, 1, 1)
@@ -171,7 +180,7 @@ def main():
     else:
         cfg = WORKLOADS[args.workload]
         B, C, d, H, W, K, s = cfg
-        q, key, v = make_inputs(cfg, dtype, dev)
+        q, key, v = make_inputs(cfg, dtype, dev, heavy_tails=args.workload == 'stress')
     out = torch.empty(B, C, H * s, W * s, dtype=dtype, device=dev)
     code = _lib.dtype_code(out)
     if deform:
@@ -271,7 +280,8 @@ def main():
         what = 'fused SAPA-B forward (qk->softmax->av)'
         wl = (f'{args.workload}: SAPA-B FPN-style B={B} C={C} d={d} '
               f'{H}x{W}->{H * s}x{W * s} K={K} s={s} {args.dtype}, '
-              + ('channels_last' if args.layout == 'channels_last' else 'NCHW'))
+              + ('channels_last' if args.layout == 'channels_last' else 'NCHW')
+              + (', 10% of q Student-t(3)' if args.workload == 'stress' else ''))
         nhwc_kern = ('sapa_b_nhwc16_kernel (fused mode)' if esize == 2 and d % 8 == 0
                      else 'sapa_b_nhwc_kernel (fused mode)')
         if args.layout == 'channels_last':

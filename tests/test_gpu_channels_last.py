@@ -193,3 +193,24 @@ def test_module_in_channels_last_format():
     unfused = sapa_amd.SAPA(64, 64, embedding_dim=32, fused=False).to(DEV)
     unfused.load_state_dict(m.state_dict())
     torch.testing.assert_close(unfused(yc, xc), want, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize('dtype,rel', [(torch.bfloat16, BF16_REL), (torch.float32, None)])
+def test_heavy_tailed_query_k7_s4(coracle, dtype, rel):
+    """The stress configuration in small: K = 7, s = 4, a tenth of the query
+    drawn from Student-t(3) (logits with outliers), both memory orders against
+    the float64-accumulated oracle on the rounded inputs."""
+    B, d, C, H, W, K, s = 1, 64, 72, 6, 7, 7, 4
+    g = gen(320)
+    q, key, v, _ = inputs(g, B, d, C, H, W, K, s)
+    z = randn(g, 4, *q.shape)
+    t3 = z[0] / z[1:].pow(2).mean(0).sqrt()
+    q = torch.where(torch.rand(q.shape, generator=g) < 0.1, t3, q)
+    q, key, v = (t.to(dtype) for t in (q, key, v))
+    want = coracle.sapa_fused(q.float(), key.float(), v.float(), K, s, 'f32a64')
+    for got in (sapa_amd.sapa_fused(*cl(q, key, v), K, s),
+                sapa_amd.sapa_fused(q.to(DEV), key.to(DEV), v.to(DEV), K, s)):
+        if rel is None:
+            torch.testing.assert_close(got.cpu().double().contiguous(), want, rtol=1e-5, atol=1e-5)
+        else:
+            assert_rel_rms_close(got.float(), want, rel, 'fused')
