@@ -214,3 +214,32 @@ def test_heavy_tailed_query_k7_s4(coracle, dtype, rel):
             torch.testing.assert_close(got.cpu().double().contiguous(), want, rtol=1e-5, atol=1e-5)
         else:
             assert_rel_rms_close(got.float(), want, rel, 'fused')
+
+
+def test_random_configurations_match_contiguous_path():
+    """24 seeded random shapes / window sizes / dtypes: the channels-last entry
+    points (both kernels behind them) against the contiguous-layout ones."""
+    import random
+    rnd = random.Random(7)
+    g = gen(330)
+    for _ in range(24):
+        K, s = rnd.choice([(3, 2), (5, 2), (7, 2), (5, 4), (7, 4)])
+        B, H, W = rnd.randint(1, 2), rnd.randint(1, 13), rnd.randint(1, 14)
+        d, C = 4 * rnd.randint(1, 20), 4 * rnd.randint(1, 36)
+        dtype = rnd.choice([torch.float32, torch.bfloat16, torch.float16])
+        q, key, v, attn = inputs(g, B, d, C, H, W, K, s, dtype=dtype)
+        qd, kd, vd, ad = (t.to(DEV) for t in (q, key, v, attn))
+        what = f'B{B} d{d} C{C} {H}x{W} K{K} s{s} {dtype}'
+        fused_cl = sapa_amd.sapa_fused(*cl(q, key, v), K, s)
+        av_cl = sapa_amd.av(*cl(attn, v), K, s)
+        qk_cl = sapa_amd.qk(*cl(q, key), K, s)
+        fused, av, qk = sapa_amd.sapa_fused(qd, kd, vd, K, s), sapa_amd.av(ad, vd, K, s), sapa_amd.qk(qd, kd, K, s)
+        if dtype == torch.float32:
+            assert torch.equal(av_cl.contiguous(), av), what
+            torch.testing.assert_close(fused_cl.contiguous(), fused, rtol=2e-5, atol=2e-5, msg=what)
+            assert_rel_rms_close(qk_cl, qk, 1e-5, what)
+        else:
+            rel = BF16_REL if dtype == torch.bfloat16 else F16_REL
+            assert_rel_rms_close(av_cl.float(), av.float(), rel, what + ' av')
+            assert_rel_rms_close(fused_cl.float(), fused.float(), rel, what + ' fused')
+            assert_rel_rms_close(qk_cl.float(), qk.float(), rel, what + ' qk')
