@@ -7,7 +7,9 @@ sapa_deform.py:7-62, so its checkpoints load.  `x` is the low-res feature
 `fused=True` (default) runs attention as the single fused launch; False
 runs the reference's three-step composition on the separate operators.
 `fold_norm=True` folds the GroupNorms into the 1x1 projections (one batched
-GEMM per projection straight from the un-normalised feature).
+GEMM per projection straight from the un-normalised feature);
+`SAPA(channels_last=True)` additionally has those GEMMs write q and k in
+channels_last order and runs the operator in that order.
 """
 import torch
 import torch.nn as nn
@@ -17,7 +19,7 @@ from .deform_func import deform_av, deform_qk, deform_sapa_fused
 from .sapa_func import av, qk, sapa_fused
 
 
-def norm_project(x, norm, *convs):
+def norm_project(x, norm, *convs, channels_last=False):
     """conv(norm(x)) for a GroupNorm and one or more 1x1 convolutions fed by
     it (sapa_base.py:26-36: norm_y -> q, norm_x -> k) without materialising
     norm(x): the normalisation is affine per (image, channel), so it folds into
@@ -32,37 +34,62 @@ def norm_project(x, norm, *convs):
     differs from the two-step form by rounding only, with one caveat: the mean
     is subtracted after the GEMM instead of before it, so it loses accuracy if
     |mean| exceeds the standard deviation of a group by many orders of magnitude.
-    Statistics are taken in fp32, like GroupNorm's.  Returns a list, one output
-    per convolution, each [B, out, H, W] contiguous."""
+    Statistics are taken in fp32, like GroupNorm's.  `norm` may be None (plain
+    1x1 convolutions).  x may be contiguous or in channels_last order; either
+    way it is read in place.  Returns a list, one output per convolution, each
+    [B, out, H, W]: contiguous, or -- channels_last=True -- in channels_last
+    order (the GEMM is then written as x[b]^T @ W'[b]^T, whose result is the
+    channels-last tensor: the layout the operators are fastest in costs the
+    projection nothing)."""
     B, C, H, W = x.shape
-    G = norm.num_groups
-    xg = x.reshape(B, G, -1)
-    if x.dtype in (torch.float16, torch.bfloat16):
-        # fp32 accumulation straight from the 16-bit tensor (no fp32 copy)
-        mean = xg.mean(dim=2, dtype=torch.float32)
-        sq = torch.linalg.vector_norm(xg, dim=2, dtype=torch.float32).square() / xg.shape[2]
-        var = (sq - mean * mean).clamp_min(0)
+    x_cl = not x.is_contiguous() and x.is_contiguous(memory_format=torch.channels_last)
+    if norm is not None:
+        G = norm.num_groups
+        per_c = C // G
+        if x_cl:
+            # per-channel moments, then per group: no layout copy of x
+            m1 = x.mean(dim=(2, 3), dtype=torch.float32).reshape(B, G, per_c)
+            m2 = (torch.linalg.vector_norm(x, dim=(2, 3), dtype=torch.float32).square()
+                  / (H * W)).reshape(B, G, per_c)
+            mean = m1.mean(dim=2)
+            var = (m2.mean(dim=2) - mean * mean).clamp_min(0)
+        else:
+            xg = x.reshape(B, G, -1)
+            if x.dtype in (torch.float16, torch.bfloat16):
+                # fp32 accumulation straight from the 16-bit tensor (no fp32 copy)
+                mean = xg.mean(dim=2, dtype=torch.float32)
+                sq = torch.linalg.vector_norm(xg, dim=2, dtype=torch.float32).square() / xg.shape[2]
+                var = (sq - mean * mean).clamp_min(0)
+            else:
+                var, mean = torch.var_mean(xg.float(), dim=2, unbiased=False)
+        rstd = torch.rsqrt(var + norm.eps)
+        rstd_c = rstd.repeat_interleave(per_c, dim=1)                    # [B, C]
+        mean_c = mean.repeat_interleave(per_c, dim=1)
+        gamma = norm.weight.float() if norm.weight is not None else x.new_ones(C, dtype=torch.float32)
+        beta = norm.bias.float() if norm.bias is not None else x.new_zeros(C, dtype=torch.float32)
+        scale = gamma.unsqueeze(0) * rstd_c                              # [B, C]
+        shift = beta.unsqueeze(0) - mean_c * scale                       # [B, C]
     else:
-        var, mean = torch.var_mean(xg.float(), dim=2, unbiased=False)
-    rstd = torch.rsqrt(var + norm.eps)
-    per_c = C // G
-    rstd_c = rstd.repeat_interleave(per_c, dim=1)                    # [B, C]
-    mean_c = mean.repeat_interleave(per_c, dim=1)
-    gamma = norm.weight.float() if norm.weight is not None else x.new_ones(C, dtype=torch.float32)
-    beta = norm.bias.float() if norm.bias is not None else x.new_zeros(C, dtype=torch.float32)
-    scale = gamma.unsqueeze(0) * rstd_c                              # [B, C]
-    shift = beta.unsqueeze(0) - mean_c * scale                       # [B, C]
-    x3 = x.reshape(B, C, H * W)
+        scale = x.new_ones(B, C, dtype=torch.float32)
+        shift = x.new_zeros(B, C, dtype=torch.float32)
+    # [B, C, HW] view of x in either memory order
+    x3 = x.permute(0, 2, 3, 1).reshape(B, H * W, C).transpose(1, 2) if x_cl else x.reshape(B, C, H * W)
     outs = []
     for conv in convs:
         assert conv.kernel_size == (1, 1) and conv.groups == 1
-        w = conv.weight.reshape(conv.out_channels, C).float()
+        O = conv.out_channels
+        w = conv.weight.reshape(O, C).float()
         w_b = (w.unsqueeze(0) * scale.unsqueeze(1)).to(x.dtype)      # [B, O, C]
         b_b = torch.einsum('oc,bc->bo', w, shift)
         if conv.bias is not None:
             b_b = b_b + conv.bias.float().unsqueeze(0)
-        out = torch.baddbmm(b_b.to(x.dtype).unsqueeze(2), w_b, x3)   # [B, O, HW]
-        outs.append(out.view(B, conv.out_channels, H, W))
+        b_b = b_b.to(x.dtype)
+        if channels_last:
+            out = torch.baddbmm(b_b.unsqueeze(1), x3.transpose(1, 2), w_b.transpose(1, 2))   # [B, HW, O]
+            outs.append(out.view(B, H, W, O).permute(0, 3, 1, 2))
+        else:
+            out = torch.baddbmm(b_b.unsqueeze(2), w_b, x3)               # [B, O, HW]
+            outs.append(out.view(B, O, H, W))
     return outs
 
 
@@ -76,11 +103,16 @@ def _init_projection(m):
 
 class SAPA(nn.Module):
     def __init__(self, dim_y, dim_x=None, up_factor=2, up_kernel_size=5, embedding_dim=32,
-                 qkv_bias=True, norm=True, fused=True, fold_norm=False):
+                 qkv_bias=True, norm=True, fused=True, fold_norm=False, channels_last=False):
         super().__init__()
         dim_x = dim_y if dim_x is None else dim_x
         self.up_factor = up_factor
         self.up_kernel_size = up_kernel_size
+        # channels_last: the projections emit q and k in channels_last order
+        # (free: norm_project) and the operator runs in that order, its fastest;
+        # the value is used as it is if it already is channels_last, else copied
+        # once (a low-res tensor); the result is a channels_last tensor
+        self.channels_last = channels_last
         self.embedding_dim = embedding_dim
         self.norm = norm
         self.fused = fused
@@ -95,6 +127,10 @@ class SAPA(nn.Module):
 
     def forward(self, y, x):
         # the value is the un-normalised x; only the key sees norm_x(x)
+        if self.channels_last:
+            (q,) = norm_project(y, self.norm_y if self.norm else None, self.q, channels_last=True)
+            (k,) = norm_project(x, self.norm_x if self.norm else None, self.k, channels_last=True)
+            return self.attention(q, k, x.contiguous(memory_format=torch.channels_last))
         if self.norm and self.fold_norm:
             (q,), (k,) = norm_project(y, self.norm_y, self.q), norm_project(x, self.norm_x, self.k)
             return self.attention(q, k, x)

@@ -243,3 +243,33 @@ def test_random_configurations_match_contiguous_path():
             assert_rel_rms_close(av_cl.float(), av.float(), rel, what + ' av')
             assert_rel_rms_close(fused_cl.float(), fused.float(), rel, what + ' fused')
             assert_rel_rms_close(qk_cl.float(), qk.float(), rel, what + ' qk')
+
+
+@pytest.mark.parametrize('dtype,tol', [(torch.float32, 1e-4), (torch.bfloat16, 6e-2)])
+@pytest.mark.parametrize('norm', [True, False])
+def test_module_emitting_channels_last(dtype, tol, norm):
+    """SAPA(channels_last=True): projections that write q and k in
+    channels_last order, the operator in that order, a channels_last result --
+    same values as the default module on contiguous tensors."""
+    torch.manual_seed(6)
+    m = sapa_amd.SAPA(64, embedding_dim=16, norm=norm).to(DEV)
+    # 16 bits: small projections, i.e. a smooth softmax -- two different 16-bit
+    # pipelines for q and k are compared, and a sharp softmax would turn their
+    # rounding differences into different winners
+    std = 0.2 if dtype == torch.float32 else 0.03
+    torch.nn.init.normal_(m.q.weight, std=std)
+    torch.nn.init.normal_(m.k.weight, std=std)
+    if norm:
+        torch.nn.init.normal_(m.norm_y.weight, 1.0, 0.2)
+        torch.nn.init.normal_(m.norm_x.bias, 0.0, 0.2)
+    m = m.to(dtype)
+    y = (torch.randn(2, 64, 18, 22, device=DEV) + 0.5).to(dtype)
+    x = torch.randn(2, 64, 9, 11, device=DEV).to(dtype)
+    with torch.no_grad():
+        want = m(y, x)
+        m.channels_last = True
+        got = m(y, x)
+        got_cl_in = m(y.contiguous(memory_format=CL), x.contiguous(memory_format=CL))
+    assert got.shape == want.shape and got.is_contiguous(memory_format=CL)
+    torch.testing.assert_close(got.float(), want.float(), rtol=tol, atol=tol)
+    torch.testing.assert_close(got_cl_in.float(), want.float(), rtol=tol, atol=tol)

@@ -41,3 +41,28 @@ def test_norm_project_gradients_match():
         grads.append([x.grad] + [p.grad.clone() for p in list(norm.parameters()) + list(conv.parameters())])
     for a, b in zip(*grads):
         torch.testing.assert_close(a, b, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize('x_order', ['contiguous', 'channels_last'])
+@pytest.mark.parametrize('out_cl', [False, True])
+def test_norm_project_memory_orders(x_order, out_cl):
+    """Either memory order of the feature is read in place, and the
+    projection can be asked for a channels_last result: same values."""
+    torch.manual_seed(3)
+    B, C, H, W = 2, 64, 6, 5
+    x = torch.randn(B, C, H, W) * 1.5 - 0.3
+    if x_order == 'channels_last':
+        x = x.contiguous(memory_format=torch.channels_last)
+    norm = nn.GroupNorm(32, C)
+    nn.init.normal_(norm.weight, 1.0, 0.3)
+    nn.init.normal_(norm.bias, 0.0, 0.3)
+    conv = nn.Conv2d(C, 24, 1)
+    with torch.no_grad():
+        (got,) = norm_project(x, norm, conv, channels_last=out_cl)
+        (plain,) = norm_project(x, None, conv, channels_last=out_cl)
+        want, want_plain = conv(norm(x)), conv(x)
+    for g in (got, plain):
+        assert g.shape == (B, 24, H, W)
+        assert g.is_contiguous(memory_format=torch.channels_last if out_cl else torch.contiguous_format)
+    torch.testing.assert_close(got, want, rtol=2e-5, atol=2e-5)
+    torch.testing.assert_close(plain, want_plain, rtol=2e-5, atol=2e-5)
