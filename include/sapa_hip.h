@@ -272,6 +272,24 @@ int sapa_deform_fused_forward_from(const void *query, const void *key, const voi
                                    int H, int W, int P, int s, int G, int offset_layout,
                                    int dtype, void *stream);
 
+/* ------------------------------------------------------- module front end */
+
+/* Mean and biased variance of every (image, channel) of a feature map, one
+ * pass over it: x [B,C,HW] contiguous (channels_last = 0) or [B,HW,C]
+ * (channels_last = 1) -> mean_var [B,C,2] fp32.  These are the statistics
+ * behind the reference's GroupNorm(32) on y and x ahead of the q / k
+ * projections (sapa/sapa/sapa_base.py:17-19,27-31, an ATen call there); the
+ * caller combines them per group and folds the normalisation into the 1x1
+ * projection weights.  workspace: sapa_channel_moments_workspace(...) bytes of
+ * device memory, contents undefined before and after.  SAPA_F32 / F16 / BF16;
+ * channels_last needs C % 4 == 0, C <= 1024 and x aligned to 4 elements, the
+ * contiguous layout B * C <= 65535; SAPA_ERR_UNSUPPORTED otherwise.  No
+ * atomics: the result does not depend on scheduling. */
+long long sapa_channel_moments_workspace(int B, int C, long long HW, int channels_last);
+int sapa_channel_moments(const void *x, void *workspace, float *mean_var,
+                         int B, int C, long long HW, int channels_last,
+                         int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -20,6 +20,7 @@ DTYPES = {torch.float32: 0, torch.float64: 1, torch.float16: 2, torch.bfloat16: 
 _vp, _i, _ll = ctypes.c_void_p, ctypes.c_int, ctypes.c_longlong
 # name -> argtypes, in the order of include/sapa_hip.h
 SIGNATURES = {
+    'sapa_channel_moments': [_vp, _vp, _vp, _i, _i, _ll, _i, _i, _vp],
     'sapa_qk_forward': [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_qk_backward': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_av_forward': [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
@@ -72,6 +73,8 @@ def lib():
             fn = getattr(handle, name)
             fn.restype = _i
             fn.argtypes = argtypes
+        handle.sapa_channel_moments_workspace.restype = _ll
+        handle.sapa_channel_moments_workspace.argtypes = [_i, _i, _ll, _i]
         _lib = handle
     return _lib
 
@@ -189,3 +192,30 @@ def call(name, device, *args):
     with torch.cuda.device(device):
         stream = torch.cuda.current_stream(device).cuda_stream
         check(getattr(lib(), name)(*args, stream), name)
+
+
+def channel_moments(x):
+    """Mean and biased variance of every (image, channel) of a CUDA feature
+    map x [B, C, H, W] (contiguous or channels_last; f32 / f16 / bf16), one
+    pass over it: two fp32 tensors [B, C].  None if the kernel does not cover
+    the configuration (the caller then uses torch reductions)."""
+    B, C, H, W = x.shape
+    if x.dtype not in (torch.float32, torch.float16, torch.bfloat16) or x.numel() == 0:
+        return None
+    if x.is_contiguous():
+        cl = 0
+    elif x.is_contiguous(memory_format=torch.channels_last):
+        cl = 1
+    else:
+        return None
+    handle = lib()
+    with torch.cuda.device(x.device):
+        ws = torch.empty(max(handle.sapa_channel_moments_workspace(B, C, H * W, cl), 4),
+                         dtype=torch.uint8, device=x.device)
+        mv = torch.empty(B, C, 2, dtype=torch.float32, device=x.device)
+        status = handle.sapa_channel_moments(x.data_ptr(), ws.data_ptr(), mv.data_ptr(), B, C, H * W, cl,
+                                             DTYPES[x.dtype], torch.cuda.current_stream(x.device).cuda_stream)
+    if status == UNSUPPORTED:
+        return None
+    check(status, 'sapa_channel_moments')
+    return mv[..., 0], mv[..., 1]

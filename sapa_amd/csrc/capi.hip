@@ -451,4 +451,22 @@ int sapa_deform_av_backward(const void *grad_out, const void *attn, const void *
     return SAPA_OK;
 }
 
+long long sapa_channel_moments_workspace(int B, int C, long long HW, int channels_last) {
+    if (B <= 0 || C <= 0 || HW <= 0) return 0;
+    return channel_moments_workspace(B, C, (long)HW, channels_last != 0);
+}
+
+int sapa_channel_moments(const void *x, void *workspace, float *mean_var, int B, int C,
+                         long long HW, int channels_last, int dtype, void *stream) {
+    if (!dtype_ok(dtype) || B < 0 || C <= 0 || HW <= 0) return SAPA_ERR_INVALID_ARGUMENT;
+    if (dtype == SAPA_F64) return SAPA_ERR_UNSUPPORTED;
+    if ((long long)B * C * HW >= kMaxElems) return SAPA_ERR_TOO_LARGE;
+    if (B == 0) return SAPA_OK;
+    if (!x || !workspace || !mean_var) return SAPA_ERR_INVALID_ARGUMENT;
+    const hipError_t e = channel_moments_launch(x, workspace, mean_var, B, C, (long)HW,
+                                                channels_last != 0, dtype, (hipStream_t)stream);
+    if (e == hipErrorNotSupported) return SAPA_ERR_UNSUPPORTED;
+    return finish(e);
+}
+
 }  // extern "C"

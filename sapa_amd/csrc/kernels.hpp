@@ -44,6 +44,11 @@ hipError_t sapa_b_nhwc16_launch(int mode, const void *q, const void *key, const 
                                 const void *value, void *out, int B, int d, int C, int H, int W,
                                 int K, int s, int dtype, hipStream_t st);
 
+// sapa_moments.hip: per (image, channel) mean and variance of a feature map
+long channel_moments_workspace(int B, int C, long HW, bool channels_last);
+hipError_t channel_moments_launch(const void *x, void *workspace, float *mean_var, int B, int C,
+                                  long HW, bool channels_last, int dtype, hipStream_t st);
+
 // sapa_d_nhwc.hip: fused SAPA-D forward for tensors in channels-last memory
 // order (offsets [B, sH, sW, 2GP]); f32 / f16 / bf16, s in {1, 2, 4}, P <= 32,
 // channels per group multiples of 4, at most 64 query / key channels per group.
