@@ -8,8 +8,9 @@ sapa_deform.py:7-62, so its checkpoints load.  `x` is the low-res feature
 runs the reference's three-step composition on the separate operators.
 `fold_norm=True` folds the GroupNorms into the 1x1 projections (one batched
 GEMM per projection straight from the un-normalised feature);
-`SAPA(channels_last=True)` additionally has those GEMMs write q and k in
-channels_last order and runs the operator in that order.
+`channels_last=True` (both modules) additionally has those GEMMs write q and
+k (and the offsets) in channels_last order and runs the fused operator in
+that order.
 """
 import torch
 import torch.nn as nn
@@ -169,10 +170,14 @@ class SAPA(nn.Module):
 
 class SAPADeform(nn.Module):
     def __init__(self, dim_y, dim_x=None, up_factor=2, num_point=9, groups=4, embedding_dim=32,
-                 qkv_bias=True, high_offset=True, norm=False, fused=True, fold_norm=False):
+                 qkv_bias=True, high_offset=True, norm=False, fused=True, fold_norm=False,
+                 channels_last=False):
         super().__init__()
         dim_x = dim_y if dim_x is None else dim_x
         self.fold_norm = fold_norm
+        # channels_last: as for SAPA -- q, k and the offsets leave their projections
+        # in channels_last order, the fused operator runs in that order
+        self.channels_last = channels_last
         self.up_factor = up_factor
         self.num_point = num_point
         self.groups = groups
@@ -192,6 +197,15 @@ class SAPADeform(nn.Module):
         self.apply(_init_projection)
 
     def forward(self, y, x):
+        if self.channels_last and self.fused:
+            (q,) = norm_project(y, self.norm_y if self.norm else None, self.q, channels_last=True)
+            k, offset_lo = norm_project(x, self.norm_x if self.norm else None, self.k, self.offset,
+                                        channels_last=True)
+            if self.high_offset:
+                offset = F.pixel_shuffle(offset_lo, upscale_factor=self.up_factor)
+            else:
+                offset = F.interpolate(offset_lo, scale_factor=self.up_factor)
+            return self.attention(q, k, x.contiguous(memory_format=torch.channels_last), offset)
         if self.norm and self.fold_norm:
             (q,) = norm_project(y, self.norm_y, self.q)
             k, offset_lo = norm_project(x, self.norm_x, self.k, self.offset)

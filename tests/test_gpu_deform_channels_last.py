@@ -126,3 +126,27 @@ def test_module_in_channels_last_format():
     torch.testing.assert_close(got, want, rtol=1e-4, atol=1e-5)
     got.sum().backward()
     assert all(p.grad is not None for p in mc.parameters())
+
+
+@pytest.mark.parametrize('norm', [False, True])
+def test_module_emitting_channels_last(norm):
+    """SAPADeform(channels_last=True): projections that write q, k and the
+    offsets in channels_last order, the fused operator in that order -- same
+    values as the default module on contiguous tensors."""
+    import sapa_amd
+    torch.manual_seed(8)
+    m = sapa_amd.SAPADeform(64, embedding_dim=8, norm=norm).to(DEV)
+    torch.nn.init.normal_(m.offset.weight, std=0.1)
+    torch.nn.init.normal_(m.q.weight, std=0.2)
+    torch.nn.init.normal_(m.k.weight, std=0.2)
+    y = torch.randn(2, 64, 18, 22, device=DEV) + 0.5
+    x = torch.randn(2, 64, 9, 11, device=DEV)
+    with torch.no_grad():
+        want = m(y, x)
+        m.channels_last = True
+        got = m(y, x)
+        got_cl_in = m(y.contiguous(memory_format=torch.channels_last),
+                      x.contiguous(memory_format=torch.channels_last))
+    assert got.shape == want.shape and got.is_contiguous(memory_format=torch.channels_last)
+    torch.testing.assert_close(got, want, rtol=2e-4, atol=2e-4)
+    torch.testing.assert_close(got_cl_in, want, rtol=2e-4, atol=2e-4)
