@@ -134,6 +134,58 @@ def cpu_baseline(q, key, v, K, s, budget_s=20.0):
                                     f'query), fp32, median of {runs} runs'), out
 
 
+def module_pass(args, dev, dtype, stream):
+    """The caller of the hot path: SAPA.forward(y, x) = GroupNorm(32) on both
+    features, 1x1 q / k projections, fused operator (sapa_base.py:26-40), timed
+    as the reference composes it and with the projections of this build."""
+    import sapa_amd
+    if args.workload not in WORKLOADS:
+        sys.exit('bench.py: --pass module covers the SAPA-B workloads')
+    B, C, d, H, W, K, s = WORKLOADS[args.workload]
+    g = torch.Generator(device=dev).manual_seed(0)
+    y = torch.randn(B, C, H * s, W * s, generator=g, device=dev).to(dtype)
+    x = torch.randn(B, C, H, W, generator=g, device=dev).to(dtype)
+    m = sapa_amd.SAPA(C, embedding_dim=d, up_factor=s, up_kernel_size=K).to(dev).to(dtype)
+    CL = torch.channels_last
+    ycl, xcl = y.contiguous(memory_format=CL), x.contiguous(memory_format=CL)
+    cases = [('GroupNorm -> Conv2d -> fused operator, contiguous features', {}, (y, x)),
+             ('fold_norm, contiguous features', {'fold_norm': True}, (y, x)),
+             ('channels_last=True, contiguous features', {'channels_last': True}, (y, x)),
+             ('channels_last=True, channels_last features', {'channels_last': True}, (ycl, xcl)),
+             ('GroupNorm -> Conv2d -> fused operator, channels_last features', {}, (ycl, xcl))]
+    res, ref = {}, None
+    with torch.no_grad():
+        for name, kw, feats in cases:
+            m.fold_norm, m.channels_last = kw.get('fold_norm', False), kw.get('channels_last', False)
+            out = m(*feats)
+            if ref is None:
+                ref = out[:1].float()
+            err = (out[:1].float() - ref).abs().max().item()
+            for _ in range(max(args.warmup // 10, 3)):
+                m(*feats)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            n = max(args.steps // 10, 5)
+            e0.record(stream)
+            for _ in range(n):
+                m(*feats)
+            e1.record(stream)
+            torch.cuda.synchronize()
+            res[name] = {'ms': e0.elapsed_time(e1) / n, 'max_abs_diff_vs_first_image0': err}
+    pix = B * H * s * W * s
+    best = min(res, key=lambda k: res[k]['ms'] if 'contiguous features' in k else 1e9)
+    print(json.dumps({
+        'metric': 'upsampled Gpix/s, SAPA module forward (GroupNorm + q/k projections + fused operator), 1 GPU',
+        'value': pix / (res[best]['ms'] * 1e-3) / 1e9, 'unit': 'Gpix/s', 'n_gpus': 1,
+        'steps': max(args.steps // 10, 5), 'warmup': max(args.warmup // 10, 3),
+        'ms_per_step': res[best]['ms'], 'higher_is_better': True, 'scaling': 'weak',
+        'vs_baseline': None, 'dtype': {'fp32': 'f32', 'bf16': 'bf16'}[args.dtype], 'data': 'synthetic',
+        'config': {'workload': f'{args.workload}: SAPA module, features B={B} C={C} {H}x{W} / '
+                               f'{H * s}x{W * s}, embedding_dim={d}, K={K}, s={s}, {args.dtype}; '
+                               f'main line = "{best}"'},
+        'cases': res}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -143,9 +195,11 @@ def main():
     ap.add_argument('--dtype', default='fp32', choices=['fp32', 'bf16'])
     ap.add_argument('--workload', default='fpn_large',
                     choices=sorted(WORKLOADS) + sorted(DEFORM_WORKLOADS))
-    ap.add_argument('--pass', dest='direction', default='forward', choices=['forward', 'train'],
+    ap.add_argument('--pass', dest='direction', default='forward', choices=['forward', 'train', 'module'],
                     help="'train' times the fused forward plus its backward (all input "
-                         'gradients) through the autograd API instead of the forward alone')
+                         'gradients) through the autograd API instead of the forward alone; '
+                         "'module' times the whole SAPA module forward (GroupNorm, q / k "
+                         'projections, fused operator) in its configurations')
     ap.add_argument('--layout', default='nchw', choices=['nchw', 'channels_last'],
                     help="memory order of the SAPA-B tensors: 'nchw' = contiguous, the "
                          "reference's contract (default); 'channels_last' = torch.channels_last, "
@@ -172,6 +226,8 @@ def main():
     torch.cuda.set_device(dev)
     dtype = {'fp32': torch.float32, 'bf16': torch.bfloat16}[args.dtype]
     stream = torch.cuda.current_stream(dev)
+    if args.direction == 'module':
+        return module_pass(args, dev, dtype, stream)
     deform = args.workload in DEFORM_WORKLOADS
     if deform:
         cfg = DEFORM_WORKLOADS[args.workload]
