@@ -71,6 +71,16 @@ def test_argument_validation_returns_codes():
     assert h.sapa_deform_fused_forward(p, p, p, p, p, 1, 8, 8, 8, 8, 65, 2, 4, 0, None) == -2
     assert h.sapa_deform_qk_backward(p, p, p, p, p, p, p, 1, 8, 8, 8, 5, 2, 4, 3, None) == -2
     assert h.sapa_softmax_forward(p, p, 4, 0, 4, 0, None) == -1
+    # channels-last entry points: the same checks in front of the kernels
+    assert h.sapa_fused_forward_nhwc(p, p, p, p, 1, 4, 4, 8, 8, 4, 2, 0, None) == -1
+    assert h.sapa_fused_forward_nhwc(p, p, None, p, 1, 4, 4, 8, 8, 5, 2, 0, None) == -1
+    assert h.sapa_qk_forward_nhwc(None, None, None, 0, 4, 8, 8, 5, 2, 0, None) == 0
+    # channel moments: extents, dtype (no fp64 kernel), null pointers, empty batch
+    assert h.sapa_channel_moments(p, p, p, 1, 0, 64, 0, 0, None) == -1
+    assert h.sapa_channel_moments(p, p, p, 1, 8, 0, 1, 0, None) == -1
+    assert h.sapa_channel_moments(p, p, p, 1, 8, 64, 0, 1, None) == -2
+    assert h.sapa_channel_moments(p, None, p, 1, 8, 64, 0, 0, None) == -1
+    assert h.sapa_channel_moments(None, None, None, 0, 8, 64, 0, 0, None) == 0
 
 
 def test_python_api_surface():
