@@ -290,6 +290,19 @@ int sapa_channel_moments(const void *x, void *workspace, float *mean_var,
                          int B, int C, long long HW, int channels_last,
                          int dtype, void *stream);
 
+/* GroupNorm folded into a 1x1 projection, per image: from mean_var (above),
+ * the norm's gamma / beta [C] (NULL: 1 / 0), `groups` and eps, and the
+ * projection's weight [O,C] and bias [O] (NULL: none), all of type `dtype`:
+ *   weight_out[b,o,c] = weight[o,c] * gamma[c] * rstd[b,g(c)]
+ *   bias_out[b,o]     = bias[o] + sum_c weight[o,c] * (beta[c] - mean[b,g(c)] * gamma[c] * rstd[b,g(c)])
+ * so that conv(groupnorm(x))[b] = weight_out[b] x[b] + bias_out[b]: the
+ * reference's norm_y -> q and norm_x -> k (sapa/sapa/sapa_base.py:26-36) become
+ * one GEMM each on the un-normalised feature.  SAPA_F32 / F16 / BF16,
+ * C <= 8192. */
+int sapa_groupnorm_fold(const float *mean_var, const void *gamma, const void *beta,
+                        const void *weight, const void *bias, void *weight_out, void *bias_out,
+                        int B, int C, int O, int groups, float eps, int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

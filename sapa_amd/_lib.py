@@ -21,6 +21,7 @@ _vp, _i, _ll = ctypes.c_void_p, ctypes.c_int, ctypes.c_longlong
 # name -> argtypes, in the order of include/sapa_hip.h
 SIGNATURES = {
     'sapa_channel_moments': [_vp, _vp, _vp, _i, _i, _ll, _i, _i, _vp],
+    'sapa_groupnorm_fold': [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, ctypes.c_float, _i, _vp],
     'sapa_qk_forward': [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_qk_backward': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_av_forward': [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
@@ -197,7 +198,7 @@ def call(name, device, *args):
 def channel_moments(x):
     """Mean and biased variance of every (image, channel) of a CUDA feature
     map x [B, C, H, W] (contiguous or channels_last; f32 / f16 / bf16), one
-    pass over it: two fp32 tensors [B, C].  None if the kernel does not cover
+    pass over it: an fp32 tensor [B, C, 2].  None if the kernel does not cover
     the configuration (the caller then uses torch reductions)."""
     B, C, H, W = x.shape
     if x.dtype not in (torch.float32, torch.float16, torch.bfloat16) or x.numel() == 0:
@@ -218,4 +219,27 @@ def channel_moments(x):
     if status == UNSUPPORTED:
         return None
     check(status, 'sapa_channel_moments')
-    return mv[..., 0], mv[..., 1]
+    return mv
+
+
+def groupnorm_fold(mean_var, norm, conv, dtype):
+    """Per-image projection weights [B, O, C] and bias [B, O] (type `dtype`) of
+    conv(norm(x)) from channel_moments' [B, C, 2] tensor; None if the kernel
+    does not cover the configuration."""
+    B, C, _ = mean_var.shape
+    O = conv.out_channels
+    params = [norm.weight, norm.bias, conv.weight, conv.bias]
+    if C > 8192 or any(p is not None and (p.dtype != dtype or not p.is_contiguous()) for p in params):
+        return None
+    ptr = lambda t: None if t is None else t.data_ptr()
+    with torch.cuda.device(mean_var.device):
+        w_out = torch.empty(B, O, C, dtype=dtype, device=mean_var.device)
+        b_out = torch.empty(B, O, dtype=dtype, device=mean_var.device)
+        status = lib().sapa_groupnorm_fold(
+            mean_var.data_ptr(), ptr(norm.weight), ptr(norm.bias), conv.weight.data_ptr(), ptr(conv.bias),
+            w_out.data_ptr(), b_out.data_ptr(), B, C, O, norm.num_groups, float(norm.eps), DTYPES[dtype],
+            torch.cuda.current_stream(mean_var.device).cuda_stream)
+    if status == UNSUPPORTED:
+        return None
+    check(status, 'sapa_groupnorm_fold')
+    return w_out, b_out

@@ -469,4 +469,18 @@ int sapa_channel_moments(const void *x, void *workspace, float *mean_var, int B,
     return finish(e);
 }
 
+int sapa_groupnorm_fold(const float *mean_var, const void *gamma, const void *beta, const void *weight,
+                        const void *bias, void *weight_out, void *bias_out, int B, int C, int O,
+                        int groups, float eps, int dtype, void *stream) {
+    if (!dtype_ok(dtype) || B < 0 || C <= 0 || O <= 0 || groups < 1 || C % groups != 0 || !(eps >= 0.f))
+        return SAPA_ERR_INVALID_ARGUMENT;
+    if (dtype == SAPA_F64) return SAPA_ERR_UNSUPPORTED;
+    if (B == 0) return SAPA_OK;
+    if (!mean_var || !weight || !weight_out || !bias_out) return SAPA_ERR_INVALID_ARGUMENT;
+    const hipError_t e = groupnorm_fold_launch(mean_var, gamma, beta, weight, bias, weight_out, bias_out,
+                                               B, C, O, groups, eps, dtype, (hipStream_t)stream);
+    if (e == hipErrorNotSupported) return SAPA_ERR_UNSUPPORTED;
+    return finish(e);
+}
+
 }  // extern "C"

@@ -237,6 +237,65 @@ static hipError_t launch_t(const T *x, float *ws, float *mean_var, int B, int C,
     return hipGetLastError();
 }
 
+// GroupNorm folded into a 1x1 projection, per image: from the (image, channel)
+// moments, gamma / beta and the projection's weight W [O, C] and bias,
+//   rstd_g   = 1 / sqrt(var_g + eps),  group moments from the channel moments
+//   W'[b,o,c] = W[o,c] * gamma[c] * rstd_g(c)
+//   b'[b,o]   = bias[o] + sum_c W[o,c] * (beta[c] - mean_g(c) * gamma[c] * rstd_g(c))
+// so that  conv(groupnorm(x))[b] = W'[b] x[b] + b'[b].  One block per image;
+// scale and shift of every channel go through LDS, then one wave per output row.
+template <typename T>
+__global__ void __launch_bounds__(256)
+fold_kernel(const float *__restrict__ mean_var, const T *__restrict__ gamma,
+            const T *__restrict__ beta, const T *__restrict__ w, const T *__restrict__ bias,
+            T *__restrict__ w_out, T *__restrict__ b_out, int C, int O, int G, float eps) {
+    extern __shared__ float sh[];                  // scale[C], shift[C]
+    float *scale = sh, *shift = sh + C;
+    const int b = blockIdx.x, per = C / G;
+    const float *mv = mean_var + (long)b * C * 2;
+    for (int g = threadIdx.x; g < G; g += 256) {
+        float m = 0.f;
+        for (int c = g * per; c < (g + 1) * per; ++c) m += mv[2 * c];
+        m /= (float)per;
+        float v = 0.f;
+        for (int c = g * per; c < (g + 1) * per; ++c) {
+            const float dm = mv[2 * c] - m;
+            v += mv[2 * c + 1] + dm * dm;
+        }
+        const float rstd = 1.f / __builtin_sqrtf(v / (float)per + eps);
+        for (int c = g * per; c < (g + 1) * per; ++c) {
+            const float ga = gamma ? (float)gamma[c] : 1.f, be = beta ? (float)beta[c] : 0.f;
+            scale[c] = ga * rstd;
+            shift[c] = be - m * ga * rstd;
+        }
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int o = wave; o < O; o += 4) {
+        const T *wr = w + (long)o * C;
+        T *wo = w_out + ((long)b * O + o) * C;
+        float acc = 0.f;
+        for (int c = lane; c < C; c += 64) {
+            const float x = (float)wr[c];
+            wo[c] = (T)(x * scale[c]);
+            acc = fma_(x, shift[c], acc);
+        }
+#pragma unroll
+        for (int d = 32; d > 0; d >>= 1) acc += __shfl_xor(acc, d);
+        if (lane == 0) b_out[(long)b * O + o] = (T)(acc + (bias ? (float)bias[o] : 0.f));
+    }
+}
+
+template <typename T>
+static hipError_t fold_t(const float *mean_var, const void *gamma, const void *beta, const void *w,
+                         const void *bias, void *w_out, void *b_out, int B, int C, int O, int G,
+                         float eps, hipStream_t st) {
+    hipLaunchKernelGGL((fold_kernel<T>), dim3(B), dim3(256), 2 * C * sizeof(float), st, mean_var,
+                       (const T *)gamma, (const T *)beta, (const T *)w, (const T *)bias, (T *)w_out,
+                       (T *)b_out, C, O, G, eps);
+    return hipGetLastError();
+}
+
 }  // namespace moments
 
 // bytes of workspace channel_moments_launch needs for these extents
@@ -265,6 +324,21 @@ hipError_t channel_moments_launch(const void *x, void *workspace, float *mean_va
         case 0: return moments::launch_t((const float *)x, ws, mean_var, B, C, HW, channels_last, st);
         case 2: return moments::launch_t((const f16_t *)x, ws, mean_var, B, C, HW, channels_last, st);
         case 3: return moments::launch_t((const bf16_t *)x, ws, mean_var, B, C, HW, channels_last, st);
+        default: return hipErrorNotSupported;
+    }
+}
+
+// mean_var [B, C, 2] fp32 (channel_moments_launch); gamma, beta [C] or null, w
+// [O, C], bias [O] or null, all of type `dtype` (f32 / f16 / bf16); w_out
+// [B, O, C] and b_out [B, O] of the same type.  C % G == 0, C <= 8192.
+hipError_t groupnorm_fold_launch(const float *mean_var, const void *gamma, const void *beta,
+                                 const void *w, const void *bias, void *w_out, void *b_out, int B,
+                                 int C, int O, int G, float eps, int dtype, hipStream_t st) {
+    if (G < 1 || C % G != 0 || C > 8192) return hipErrorNotSupported;
+    switch (dtype) {
+        case 0: return moments::fold_t<float>(mean_var, gamma, beta, w, bias, w_out, b_out, B, C, O, G, eps, st);
+        case 2: return moments::fold_t<f16_t>(mean_var, gamma, beta, w, bias, w_out, b_out, B, C, O, G, eps, st);
+        case 3: return moments::fold_t<bf16_t>(mean_var, gamma, beta, w, bias, w_out, b_out, B, C, O, G, eps, st);
         default: return hipErrorNotSupported;
     }
 }

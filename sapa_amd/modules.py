@@ -54,7 +54,7 @@ def norm_project(x, norm, *convs, channels_last=False):
         if x.is_cuda and not (torch.is_grad_enabled() and x.requires_grad):
             mom = _lib.channel_moments(x)
         if mom is not None:
-            mean_ch, var_ch = (t.reshape(B, G, per_c) for t in mom)
+            mean_ch, var_ch = (mom[..., i].reshape(B, G, per_c) for i in (0, 1))
             mean = mean_ch.mean(dim=2)
             var = (var_ch + (mean_ch - mean.unsqueeze(2)).square()).mean(dim=2)
         elif x_cl:
@@ -81,6 +81,7 @@ def norm_project(x, norm, *convs, channels_last=False):
         scale = gamma.unsqueeze(0) * rstd_c                              # [B, C]
         shift = beta.unsqueeze(0) - mean_c * scale                       # [B, C]
     else:
+        mom = None
         scale = x.new_ones(B, C, dtype=torch.float32)
         shift = x.new_zeros(B, C, dtype=torch.float32)
     # [B, C, HW] view of x in either memory order
@@ -89,12 +90,19 @@ def norm_project(x, norm, *convs, channels_last=False):
     for conv in convs:
         assert conv.kernel_size == (1, 1) and conv.groups == 1
         O = conv.out_channels
-        w = conv.weight.reshape(O, C).float()
-        w_b = (w.unsqueeze(0) * scale.unsqueeze(1)).to(x.dtype)      # [B, O, C]
-        b_b = torch.einsum('oc,bc->bo', w, shift)
-        if conv.bias is not None:
-            b_b = b_b + conv.bias.float().unsqueeze(0)
-        b_b = b_b.to(x.dtype)
+        folded = None
+        if norm is not None and mom is not None:
+            # the per-image weights and bias in one small kernel launch
+            folded = _lib.groupnorm_fold(mom, norm, conv, x.dtype)
+        if folded is not None:
+            w_b, b_b = folded
+        else:
+            w = conv.weight.reshape(O, C).float()
+            w_b = (w.unsqueeze(0) * scale.unsqueeze(1)).to(x.dtype)      # [B, O, C]
+            b_b = torch.einsum('oc,bc->bo', w, shift)
+            if conv.bias is not None:
+                b_b = b_b + conv.bias.float().unsqueeze(0)
+            b_b = b_b.to(x.dtype)
         # GEMM, then the bias in place: measurably faster than baddbmm here, which
         # first spreads the bias over the whole output
         if channels_last:

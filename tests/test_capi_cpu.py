@@ -81,6 +81,10 @@ def test_argument_validation_returns_codes():
     assert h.sapa_channel_moments(p, p, p, 1, 8, 64, 0, 1, None) == -2
     assert h.sapa_channel_moments(p, None, p, 1, 8, 64, 0, 0, None) == -1
     assert h.sapa_channel_moments(None, None, None, 0, 8, 64, 0, 0, None) == 0
+    # GroupNorm fold: channels not divisible by the groups, null weight, empty batch
+    assert h.sapa_groupnorm_fold(p, p, p, p, p, p, p, 1, 10, 4, 4, 1e-5, 0, None) == -1
+    assert h.sapa_groupnorm_fold(p, p, p, None, p, p, p, 1, 8, 4, 4, 1e-5, 0, None) == -1
+    assert h.sapa_groupnorm_fold(None, None, None, None, None, None, None, 0, 8, 4, 4, 1e-5, 0, None) == 0
 
 
 def test_python_api_surface():

@@ -292,7 +292,36 @@ def test_channel_moments_kernel(dtype, shape):
         if C % 4 != 0 and not t.is_contiguous():
             assert got is None                      # channels-last needs whole channel quads
             continue
-        mean, var = got
-        assert mean.shape == (B, C) and mean.dtype == torch.float32
+        assert got.shape == (B, C, 2) and got.dtype == torch.float32
+        mean, var = got[..., 0], got[..., 1]
         torch.testing.assert_close(mean.cpu().double(), want_mean, rtol=1e-6, atol=1e-6)
         torch.testing.assert_close(var.cpu().double(), want_var, rtol=2e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize('dtype,tol', [(torch.float32, 2e-5), (torch.bfloat16, 2e-2), (torch.float16, 3e-3)])
+def test_groupnorm_fold_kernel(dtype, tol):
+    """Per-image folded projection weights / bias from the moments, against
+    float64 arithmetic on the same parameters."""
+    from sapa_amd import _lib
+    torch.manual_seed(9)
+    B, C, O, G = 3, 64, 24, 32
+    x = (torch.randn(B, C, 7, 9) * 1.3 + 0.4).to(dtype).to(DEV)
+    norm = torch.nn.GroupNorm(G, C).to(DEV)
+    torch.nn.init.normal_(norm.weight, 1.0, 0.3)
+    torch.nn.init.normal_(norm.bias, 0.0, 0.3)
+    conv = torch.nn.Conv2d(C, O, 1).to(DEV)
+    norm, conv = norm.to(dtype), conv.to(dtype)
+    mom = _lib.channel_moments(x)
+    w_b, b_b = _lib.groupnorm_fold(mom, norm, conv, dtype)
+    assert w_b.shape == (B, O, C) and b_b.shape == (B, O) and w_b.dtype == dtype
+    xd = x.double().cpu().reshape(B, G, -1)
+    mean, var = xd.mean(2), xd.var(2, unbiased=False)
+    rstd = (var + norm.eps).rsqrt().repeat_interleave(C // G, 1)
+    mean_c = mean.repeat_interleave(C // G, 1)
+    gamma, beta = norm.weight.double().cpu(), norm.bias.double().cpu()
+    w = conv.weight.double().cpu().reshape(O, C)
+    scale = gamma * rstd
+    want_w = w.unsqueeze(0) * scale.unsqueeze(1)
+    want_b = conv.bias.double().cpu() + torch.einsum('oc,bc->bo', w, beta - mean_c * scale)
+    torch.testing.assert_close(w_b.double().cpu(), want_w, rtol=tol, atol=tol * 0.1)
+    torch.testing.assert_close(b_b.double().cpu(), want_b, rtol=tol, atol=tol)
