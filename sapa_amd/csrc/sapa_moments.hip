@@ -242,8 +242,9 @@ static hipError_t launch_t(const T *x, float *ws, float *mean_var, int B, int C,
 //   rstd_g   = 1 / sqrt(var_g + eps),  group moments from the channel moments
 //   W'[b,o,c] = W[o,c] * gamma[c] * rstd_g(c)
 //   b'[b,o]   = bias[o] + sum_c W[o,c] * (beta[c] - mean_g(c) * gamma[c] * rstd_g(c))
-// so that  conv(groupnorm(x))[b] = W'[b] x[b] + b'[b].  One block per image;
-// scale and shift of every channel go through LDS, then one wave per output row.
+// so that  conv(groupnorm(x))[b] = W'[b] x[b] + b'[b].  Block = (image, 4 output
+// rows): scale and shift of every channel go through LDS (recomputed per block:
+// a few hundred operations), then one wave per output row.
 template <typename T>
 __global__ void __launch_bounds__(256)
 fold_kernel(const float *__restrict__ mean_var, const T *__restrict__ gamma,
@@ -271,7 +272,7 @@ fold_kernel(const float *__restrict__ mean_var, const T *__restrict__ gamma,
     }
     __syncthreads();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (int o = wave; o < O; o += 4) {
+    for (int o = blockIdx.y * 4 + wave; o < O; o += 4 * gridDim.y) {
         const T *wr = w + (long)o * C;
         T *wo = w_out + ((long)b * O + o) * C;
         float acc = 0.f;
@@ -290,7 +291,7 @@ template <typename T>
 static hipError_t fold_t(const float *mean_var, const void *gamma, const void *beta, const void *w,
                          const void *bias, void *w_out, void *b_out, int B, int C, int O, int G,
                          float eps, hipStream_t st) {
-    hipLaunchKernelGGL((fold_kernel<T>), dim3(B), dim3(256), 2 * C * sizeof(float), st, mean_var,
+    hipLaunchKernelGGL((fold_kernel<T>), dim3(B, (O + 3) / 4), dim3(256), 2 * C * sizeof(float), st, mean_var,
                        (const T *)gamma, (const T *)beta, (const T *)w, (const T *)bias, (T *)w_out,
                        (T *)b_out, C, O, G, eps);
     return hipGetLastError();
