@@ -176,6 +176,16 @@ int sapa_fused_forward_nhwc(const void *query, const void *key, const void *valu
                             void *out, int B, int d, int C, int H, int W,
                             int K, int s, int dtype, void *stream);
 
+/* sapa_fused_forward_nhwc on query + q_bias: q_bias [B,d] (may be NULL) is the
+ * per-image bias of the query projection, added to every query vector inside
+ * the kernel.  With the GroupNorm-folded projections of the module front end
+ * (below) this replaces the bias pass over the hi-res query tensor that the
+ * reference's Conv2d does as part of self.q (sapa/sapa/sapa_base.py:32).
+ * q_bias aligned like the tensors (16 bytes for 16-bit tensors). */
+int sapa_fused_forward_nhwc_qbias(const void *query, const void *key, const void *value,
+                                  const void *q_bias, void *out, int B, int d, int C,
+                                  int H, int W, int K, int s, int dtype, void *stream);
+
 /* ------------------------------------------------------------------ SAPA-D */
 
 /* Offset-sampled query-key similarity.

@@ -20,6 +20,7 @@ DTYPES = {torch.float32: 0, torch.float64: 1, torch.float16: 2, torch.bfloat16: 
 _vp, _i, _ll = ctypes.c_void_p, ctypes.c_int, ctypes.c_longlong
 # name -> argtypes, in the order of include/sapa_hip.h
 SIGNATURES = {
+    'sapa_fused_forward_nhwc_qbias': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_channel_moments': [_vp, _vp, _vp, _i, _i, _ll, _i, _i, _vp],
     'sapa_groupnorm_fold': [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, ctypes.c_float, _i, _vp],
     'sapa_qk_forward': [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],

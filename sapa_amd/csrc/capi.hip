@@ -283,7 +283,7 @@ int sapa_qk_softmax_forward(const void *query, const void *key, void *attn, int 
 // Channels-last memory order: only the kernel of sapa_b_nhwc.hip serves it.
 static int nhwc_common(int mode, const void *query, const void *key, const void *attn,
                        const void *value, void *out, int B, int d, int C, int H, int W, int K,
-                       int s, int dtype, void *stream) {
+                       int s, int dtype, void *stream, const void *q_bias = nullptr) {
     const int rc = check_window_args(B, d, C, H, W, K, s, dtype);
     if (rc != SAPA_OK) return rc;
     if (B == 0) return SAPA_OK;
@@ -295,11 +295,11 @@ static int nhwc_common(int mode, const void *query, const void *key, const void 
 #ifdef SAPA_NHWC16_OFF
     hipError_t e = hipErrorNotSupported;
 #else
-    hipError_t e = sapa_b_nhwc16_launch(mode, query, key, attn, value, out, B, d, C, H, W, K, s, dtype,
-                                        (hipStream_t)stream);
+    hipError_t e = sapa_b_nhwc16_launch(mode, query, key, attn, value, q_bias, out, B, d, C, H, W, K, s,
+                                        dtype, (hipStream_t)stream);
 #endif
     if (e == hipErrorNotSupported)
-        e = sapa_b_nhwc_launch(mode, query, key, attn, value, out, B, d, C, H, W, K, s, dtype,
+        e = sapa_b_nhwc_launch(mode, query, key, attn, value, q_bias, out, B, d, C, H, W, K, s, dtype,
                                (hipStream_t)stream);
     if (e == hipErrorNotSupported) return SAPA_ERR_UNSUPPORTED;
     return finish(e);
@@ -325,6 +325,13 @@ int sapa_fused_forward_nhwc(const void *query, const void *key, const void *valu
                             int B, int d, int C, int H, int W, int K, int s, int dtype,
                             void *stream) {
     return nhwc_common(TILED_FUSED, query, key, nullptr, value, out, B, d, C, H, W, K, s, dtype, stream);
+}
+
+int sapa_fused_forward_nhwc_qbias(const void *query, const void *key, const void *value,
+                                  const void *q_bias, void *out, int B, int d, int C, int H, int W,
+                                  int K, int s, int dtype, void *stream) {
+    return nhwc_common(TILED_FUSED, query, key, nullptr, value, out, B, d, C, H, W, K, s, dtype, stream,
+                       q_bias);
 }
 
 int sapa_deform_qk_forward_from(const void *query, const void *key, const void *offset,

@@ -35,14 +35,14 @@ hipError_t sapa_b_tiled_launch(int mode, const void *q, const void *key, const v
 // order ([B, H, W, channels]); f32 / f16 / bf16, (K, s) in {(3,2), (5,2), (7,2), (5,4), (7,4)}, channel
 // counts multiples of 4.  hipErrorNotSupported otherwise.
 hipError_t sapa_b_nhwc_launch(int mode, const void *q, const void *key, const void *attn_in,
-                              const void *value, void *out, int B, int d, int C, int H, int W,
-                              int K, int s, int dtype, hipStream_t st);
+                              const void *value, const void *qbias, void *out, int B, int d, int C,
+                              int H, int W, int K, int s, int dtype, hipStream_t st);
 
 // sapa_b_nhwc16.hip: the same four modes for f16 / bf16 channels-last tensors
 // on the 16-bit matrix instructions (hipErrorNotSupported for anything else)
 hipError_t sapa_b_nhwc16_launch(int mode, const void *q, const void *key, const void *attn_in,
-                                const void *value, void *out, int B, int d, int C, int H, int W,
-                                int K, int s, int dtype, hipStream_t st);
+                                const void *value, const void *qbias, void *out, int B, int d,
+                                int C, int H, int W, int K, int s, int dtype, hipStream_t st);
 
 // sapa_moments.hip: per (image, channel) mean and variance of a feature map
 long channel_moments_workspace(int B, int C, long HW, bool channels_last);

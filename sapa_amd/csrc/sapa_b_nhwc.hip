@@ -132,8 +132,8 @@ template <typename T, int K, int S, int QX, int TY, int MODE>
 __global__ void __launch_bounds__(64 * QX * TY) SAPA_NHWC_OCC
 sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
                    const T *__restrict__ attn_in, const T *__restrict__ value,
-                   T *__restrict__ out, int d, int C, int H, int W, int tiles_x, int tiles_y,
-                   int nblocks, int per_xcd) {
+                   const T *__restrict__ qbias, T *__restrict__ out, int d, int C, int H, int W,
+                   int tiles_x, int tiles_y, int nblocks, int per_xcd) {
     static_assert(S == 2 || S == 4, "children are handled in groups of 4");
     // children j = cy * S + cx of a parent, in NG groups of 4 (s = 2: all four;
     // s = 4: one child row per group)
@@ -258,6 +258,13 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
                 f32x4 qv[4];
 #pragma unroll
                 for (int jj = 0; jj < 4; ++jj) qv[jj] = Q4::widen(qraw[jj]);
+                // optional per-image bias of the query projection [B, d], added here
+                // instead of in a pass of its own over the query tensor
+                if (qbias && j * CHK + 4 * li < d) {
+                    const f32x4 qb = Q4::widen(*(const Raw *)(qbias + (long)n * d + j * CHK + 4 * li));
+#pragma unroll
+                    for (int jj = 0; jj < 4; ++jj) qv[jj] += qb;
+                }
                 // the next group's (or chunk's) q while this one is used
                 if (g + 1 < NG) load_q(j, g + 1);
                 else if (j + 1 < nKc) load_q(j + 1, 0);
@@ -402,8 +409,8 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
 #endif
 template <typename T, int K, int S, int QX, int TY>
 static hipError_t launch_geom(int mode, const void *q, const void *key, const void *attn_in,
-                              const void *value, void *out, int B, int d, int C, int H, int W,
-                              hipStream_t st) {
+                              const void *value, const void *qbias, void *out, int B, int d, int C,
+                              int H, int W, hipStream_t st) {
     const int tiles_x = (W + 4 * QX - 1) / (4 * QX), tiles_y = (H + TY - 1) / TY;
     const long nb = (long)tiles_x * tiles_y * B;
     if (nb > (1L << 30)) return hipErrorNotSupported;
@@ -412,8 +419,9 @@ static hipError_t launch_geom(int mode, const void *q, const void *key, const vo
 #define SAPA_NHWC_CASE(M)                                                                      \
     case M:                                                                                    \
         hipLaunchKernelGGL((sapa_b_nhwc_kernel<T, K, S, QX, TY, M>), grid, block, 0, st, (const T *)q, \
-                           (const T *)key, (const T *)attn_in, (const T *)value, (T *)out, d,  \
-                           C, H, W, tiles_x, tiles_y, (int)nb, per_xcd);                       \
+                           (const T *)key, (const T *)attn_in, (const T *)value,               \
+                           (const T *)qbias, (T *)out, d, C, H, W, tiles_x, tiles_y, (int)nb,  \
+                           per_xcd);                                                           \
         break;
     switch (mode) {
         SAPA_NHWC_CASE(TILED_QK) SAPA_NHWC_CASE(TILED_QK_SOFTMAX) SAPA_NHWC_CASE(TILED_AV)
@@ -426,12 +434,12 @@ static hipError_t launch_geom(int mode, const void *q, const void *key, const vo
 
 template <typename T>
 static hipError_t launch_t(int mode, const void *q, const void *key, const void *attn_in,
-                           const void *value, void *out, int B, int d, int C, int H, int W, int K,
-                           int s, hipStream_t st) {
+                           const void *value, const void *qbias, void *out, int B, int d, int C,
+                           int H, int W, int K, int s, hipStream_t st) {
 #define SAPA_NHWC_KS(KV, SV)                                                                  \
     if (K == KV && s == SV)                                                                   \
-        return launch_geom<T, KV, SV, SAPA_NHWC_TILE>(mode, q, key, attn_in, value, out, B, d, C, \
-                                                      H, W, st);
+        return launch_geom<T, KV, SV, SAPA_NHWC_TILE>(mode, q, key, attn_in, value, qbias, out, B, \
+                                                      d, C, H, W, st);
     SAPA_NHWC_KS(3, 2) SAPA_NHWC_KS(5, 2) SAPA_NHWC_KS(7, 2) SAPA_NHWC_KS(5, 4) SAPA_NHWC_KS(7, 4)
 #undef SAPA_NHWC_KS
     return hipErrorNotSupported;
@@ -442,11 +450,12 @@ static hipError_t launch_t(int mode, const void *q, const void *key, const void 
 // Channels-last tensors (q [B, sH, sW, d], key [B, H, W, d], value [B, H, W, C],
 // attn [B, sH, sW, K*K], out like q with C or K*K channels), f32 / f16 / bf16,
 // (K, s) in {(3,2), (5,2), (7,2), (5,4), (7,4)}, channel counts multiples of 4 and every tensor aligned to
-// 4 elements; one image's key / value tensor below 2^31 bytes.
+// 4 elements; one image's key / value tensor below 2^31 bytes.  qbias: optional
+// [B, d] added to every query vector (the modes that read the query).
 // hipErrorNotSupported otherwise.
 hipError_t sapa_b_nhwc_launch(int mode, const void *q, const void *key, const void *attn_in,
-                              const void *value, void *out, int B, int d, int C, int H, int W,
-                              int K, int s, int dtype, hipStream_t st) {
+                              const void *value, const void *qbias, void *out, int B, int d, int C,
+                              int H, int W, int K, int s, int dtype, hipStream_t st) {
     if (!((s == 2 && (K == 3 || K == 5 || K == 7)) || (s == 4 && (K == 5 || K == 7))))
         return hipErrorNotSupported;
     const bool need_qk = mode != TILED_AV, need_av = mode == TILED_AV || mode == TILED_FUSED;
@@ -455,14 +464,15 @@ hipError_t sapa_b_nhwc_launch(int mode, const void *q, const void *key, const vo
     const long plane = (long)H * W * esize;
     if ((need_qk && plane * d >= (1L << 31)) || (need_av && plane * C >= (1L << 31)))
         return hipErrorNotSupported;
-    const void *vec_ptrs[4] = {need_qk ? q : nullptr, need_qk ? key : nullptr,
-                               need_av ? value : nullptr, need_av ? out : nullptr};
+    const void *vec_ptrs[5] = {need_qk ? q : nullptr, need_qk ? key : nullptr,
+                               need_av ? value : nullptr, need_av ? out : nullptr,
+                               need_qk ? qbias : nullptr};
     for (const void *p : vec_ptrs)
         if (p && (uintptr_t)p % (4 * esize) != 0) return hipErrorNotSupported;
     switch (dtype) {
-        case 0: return nhwc::launch_t<float>(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, st);
-        case 2: return nhwc::launch_t<f16_t>(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, st);
-        case 3: return nhwc::launch_t<bf16_t>(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, st);
+        case 0: return nhwc::launch_t<float>(mode, q, key, attn_in, value, qbias, out, B, d, C, H, W, K, s, st);
+        case 2: return nhwc::launch_t<f16_t>(mode, q, key, attn_in, value, qbias, out, B, d, C, H, W, K, s, st);
+        case 3: return nhwc::launch_t<bf16_t>(mode, q, key, attn_in, value, qbias, out, B, d, C, H, W, K, s, st);
         default: return hipErrorNotSupported;
     }
 }

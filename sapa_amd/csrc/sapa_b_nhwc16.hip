@@ -109,12 +109,13 @@ __device__ __forceinline__ void halve(const float (&in)[N], float (&out)[N / 2],
     }
 }
 
-template <typename T, int K, int S, int QX, int TY, int MODE>
+// QB: the query bias is given (its own instantiation: the bias costs 8 registers)
+template <typename T, int K, int S, int QX, int TY, int MODE, bool QB>
 __global__ void __launch_bounds__(64 * QX * TY)
 sapa_b_nhwc16_kernel(const T *__restrict__ q, const T *__restrict__ key,
                      const T *__restrict__ attn_in, const T *__restrict__ value,
-                     T *__restrict__ out, int d, int C, int H, int W, int tiles_x, int tiles_y,
-                     int nblocks, int per_xcd) {
+                     const T *__restrict__ qbias, T *__restrict__ out, int d, int C, int H, int W,
+                     int tiles_x, int tiles_y, int nblocks, int per_xcd) {
     static_assert(S == 2 || S == 4, "children are handled in groups of 4");
     // children j = cy * S + cx of a parent, in NG groups of 4 (s = 2: all four;
     // s = 4: one child row per group)
@@ -253,6 +254,15 @@ sapa_b_nhwc16_kernel(const T *__restrict__ q, const T *__restrict__ key,
         for (int j = 0; j < nKc; ++j) {
             if (j + 1 < ntot) stage_load(j + 1);
             const u32 *kb = kwin + (j & 1) * BUF;
+            // optional per-image bias of the query projection [B, d]: key . (q + b) =
+            // key . q + key . b, the second product as four more instructions per tap
+            // group with the bias as the B operand (same for the four children)
+            u32x4 qb0 = {0u, 0u, 0u, 0u}, qb1 = {0u, 0u, 0u, 0u};
+            if (QB) {
+                const T *bp = qbias + (long)n * d + j * CHK + 8 * bq;
+                if (j * CHK + 8 * bq < d) qb0 = *(const u32x4 *)bp;
+                if (j * CHK + 8 * bq + 32 < d) qb1 = *(const u32x4 *)(bp + 32);
+            }
 #pragma unroll
             for (int g = 0; g < NG; ++g) {
                 const u32x4 q0 = qraw[0], q1 = qraw[1];
@@ -268,6 +278,12 @@ sapa_b_nhwc16_kernel(const T *__restrict__ q, const T *__restrict__ key,
                     a = M::template run<0, 0>(u32x2{k0[2], k0[3]}, u32x2{q0[2], q0[3]}, a);
                     a = M::template run<0, 0>(u32x2{k1[0], k1[1]}, u32x2{q1[0], q1[1]}, a);
                     a = M::template run<0, 0>(u32x2{k1[2], k1[3]}, u32x2{q1[2], q1[3]}, a);
+                    if (QB) {
+                        a = M::template run<0, 0>(u32x2{k0[0], k0[1]}, u32x2{qb0[0], qb0[1]}, a);
+                        a = M::template run<0, 0>(u32x2{k0[2], k0[3]}, u32x2{qb0[2], qb0[3]}, a);
+                        a = M::template run<0, 0>(u32x2{k1[0], k1[1]}, u32x2{qb1[0], qb1[1]}, a);
+                        a = M::template run<0, 0>(u32x2{k1[2], k1[3]}, u32x2{qb1[2], qb1[3]}, a);
+                    }
                     // a[i]: tap 4 tau + i times child jl over the 16 channels of quad bq;
                     // summed over the 4 quads, tap 4 tau + bq stays in this lane
                     const float flat[4] = {a[0], a[1], a[2], a[3]};
@@ -399,25 +415,34 @@ sapa_b_nhwc16_kernel(const T *__restrict__ q, const T *__restrict__ key,
 
 template <typename T, int K, int S, int QX, int TY>
 static hipError_t launch_geom(int mode, const void *q, const void *key, const void *attn_in,
-                              const void *value, void *out, int B, int d, int C, int H, int W,
-                              hipStream_t st) {
+                              const void *value, const void *qbias, void *out, int B, int d, int C,
+                              int H, int W, hipStream_t st) {
     const int tiles_x = (W + 4 * QX - 1) / (4 * QX), tiles_y = (H + TY - 1) / TY;
     const long nb = (long)tiles_x * tiles_y * B;
     if (nb > (1L << 30)) return hipErrorNotSupported;
     const int per_xcd = (int)((nb + 7) / 8);
     const dim3 grid(per_xcd * 8), block(64 * QX * TY);
+#define SAPA_NHWC16_LAUNCH(M, QB)                                                               \
+    hipLaunchKernelGGL((sapa_b_nhwc16_kernel<T, K, S, QX, TY, M, QB>), grid, block, 0, st,      \
+                       (const T *)q, (const T *)key, (const T *)attn_in, (const T *)value,      \
+                       (const T *)qbias, (T *)out, d, C, H, W, tiles_x, tiles_y, (int)nb, per_xcd)
 #define SAPA_NHWC16_CASE(M)                                                                     \
     case M:                                                                                     \
-        hipLaunchKernelGGL((sapa_b_nhwc16_kernel<T, K, S, QX, TY, M>), grid, block, 0, st,      \
-                           (const T *)q, (const T *)key, (const T *)attn_in, (const T *)value,  \
-                           (T *)out, d, C, H, W, tiles_x, tiles_y, (int)nb, per_xcd);           \
+        SAPA_NHWC16_LAUNCH(M, false);                                                           \
         break;
+    if (qbias) {
+        // the bias is carried by the fused mode only
+        if (mode != TILED_FUSED) return hipErrorNotSupported;
+        SAPA_NHWC16_LAUNCH(TILED_FUSED, true);
+        return hipGetLastError();
+    }
     switch (mode) {
         SAPA_NHWC16_CASE(TILED_QK) SAPA_NHWC16_CASE(TILED_QK_SOFTMAX) SAPA_NHWC16_CASE(TILED_AV)
         SAPA_NHWC16_CASE(TILED_FUSED)
         default: return hipErrorNotSupported;
     }
 #undef SAPA_NHWC16_CASE
+#undef SAPA_NHWC16_LAUNCH
     return hipGetLastError();
 }
 
@@ -426,12 +451,12 @@ static hipError_t launch_geom(int mode, const void *q, const void *key, const vo
 #endif
 template <typename T>
 static hipError_t launch_t(int mode, const void *q, const void *key, const void *attn_in,
-                           const void *value, void *out, int B, int d, int C, int H, int W, int K,
-                           int s, hipStream_t st) {
+                           const void *value, const void *qbias, void *out, int B, int d, int C,
+                           int H, int W, int K, int s, hipStream_t st) {
 #define SAPA_NHWC16_KS(KV, SV)                                                                  \
     if (K == KV && s == SV)                                                                     \
-        return launch_geom<T, KV, SV, SAPA_NHWC16_TILE>(mode, q, key, attn_in, value, out, B, d, \
-                                                        C, H, W, st);
+        return launch_geom<T, KV, SV, SAPA_NHWC16_TILE>(mode, q, key, attn_in, value, qbias, out, \
+                                                        B, d, C, H, W, st);
     SAPA_NHWC16_KS(3, 2) SAPA_NHWC16_KS(5, 2) SAPA_NHWC16_KS(7, 2) SAPA_NHWC16_KS(5, 4)
     SAPA_NHWC16_KS(7, 4)
 #undef SAPA_NHWC16_KS
@@ -443,10 +468,11 @@ static hipError_t launch_t(int mode, const void *q, const void *key, const void 
 // Channels-last f16 / bf16 tensors (layouts as for sapa_b_nhwc_launch), (K, s) in
 // {(3,2), (5,2), (7,2), (5,4), (7,4)}, d a multiple of 8, C of 4, q aligned to 16
 // bytes and key / value / out to 8; one image's key / value tensor below 2^31
-// bytes.  hipErrorNotSupported otherwise (fp32 tensors included).
+// bytes; qbias: optional [B, d] added to every query vector, aligned to 16 bytes.
+// hipErrorNotSupported otherwise (fp32 tensors included).
 hipError_t sapa_b_nhwc16_launch(int mode, const void *q, const void *key, const void *attn_in,
-                                const void *value, void *out, int B, int d, int C, int H, int W,
-                                int K, int s, int dtype, hipStream_t st) {
+                                const void *value, const void *qbias, void *out, int B, int d,
+                                int C, int H, int W, int K, int s, int dtype, hipStream_t st) {
     if (dtype != 2 && dtype != 3) return hipErrorNotSupported;
     if (!((s == 2 && (K == 3 || K == 5 || K == 7)) || (s == 4 && (K == 5 || K == 7))))
         return hipErrorNotSupported;
@@ -455,11 +481,12 @@ hipError_t sapa_b_nhwc16_launch(int mode, const void *q, const void *key, const 
     const long plane = (long)H * W * 2;
     if ((need_qk && plane * d >= (1L << 31)) || (need_av && plane * C >= (1L << 31)))
         return hipErrorNotSupported;
-    if (need_qk && ((uintptr_t)q % 16 != 0 || (uintptr_t)key % 8 != 0)) return hipErrorNotSupported;
+    if (need_qk && ((uintptr_t)q % 16 != 0 || (uintptr_t)key % 8 != 0 || (uintptr_t)qbias % 16 != 0))
+        return hipErrorNotSupported;
     if (need_av && ((uintptr_t)value % 8 != 0 || (uintptr_t)out % 8 != 0)) return hipErrorNotSupported;
     if (dtype == 2)
-        return nhwc16::launch_t<f16_t>(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, st);
-    return nhwc16::launch_t<bf16_t>(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, st);
+        return nhwc16::launch_t<f16_t>(mode, q, key, attn_in, value, qbias, out, B, d, C, H, W, K, s, st);
+    return nhwc16::launch_t<bf16_t>(mode, q, key, attn_in, value, qbias, out, B, d, C, H, W, K, s, st);
 }
 
 }  // namespace sapa

@@ -21,7 +21,7 @@ from .deform_func import deform_av, deform_qk, deform_sapa_fused
 from .sapa_func import av, qk, sapa_fused
 
 
-def norm_project(x, norm, *convs, channels_last=False):
+def norm_project(x, norm, *convs, channels_last=False, defer_bias=False):
     """conv(norm(x)) for a GroupNorm and one or more 1x1 convolutions fed by
     it (sapa_base.py:26-36: norm_y -> q, norm_x -> k) without materialising
     norm(x): the normalisation is affine per (image, channel), so it folds into
@@ -42,7 +42,9 @@ def norm_project(x, norm, *convs, channels_last=False):
     [B, out, H, W]: contiguous, or -- channels_last=True -- in channels_last
     order (the GEMM is then written as x[b]^T @ W'[b]^T, whose result is the
     channels-last tensor: the layout the operators are fastest in costs the
-    projection nothing)."""
+    projection nothing).  defer_bias=True: the per-image biases [B, out] are not
+    added; the list holds (output without bias, bias) pairs (for an operator
+    that adds the bias itself)."""
     B, C, H, W = x.shape
     x_cl = not x.is_contiguous() and x.is_contiguous(memory_format=torch.channels_last)
     if norm is not None:
@@ -106,11 +108,16 @@ def norm_project(x, norm, *convs, channels_last=False):
         # GEMM, then the bias in place: measurably faster than baddbmm here, which
         # first spreads the bias over the whole output
         if channels_last:
-            out = torch.bmm(x3.transpose(1, 2), w_b.transpose(1, 2)).add_(b_b.unsqueeze(1))   # [B, HW, O]
-            outs.append(out.view(B, H, W, O).permute(0, 3, 1, 2))
+            out = torch.bmm(x3.transpose(1, 2), w_b.transpose(1, 2))      # [B, HW, O]
+            if not defer_bias:
+                out.add_(b_b.unsqueeze(1))
+            out = out.view(B, H, W, O).permute(0, 3, 1, 2)
         else:
-            out = torch.bmm(w_b, x3).add_(b_b.unsqueeze(2))              # [B, O, HW]
-            outs.append(out.view(B, O, H, W))
+            out = torch.bmm(w_b, x3)                                     # [B, O, HW]
+            if not defer_bias:
+                out.add_(b_b.unsqueeze(2))
+            out = out.view(B, O, H, W)
+        outs.append((out, b_b) if defer_bias else out)
     return outs
 
 
@@ -149,9 +156,14 @@ class SAPA(nn.Module):
     def forward(self, y, x):
         # the value is the un-normalised x; only the key sees norm_x(x)
         if self.channels_last:
-            (q,) = norm_project(y, self.norm_y if self.norm else None, self.q, channels_last=True)
-            (k,) = norm_project(x, self.norm_x if self.norm else None, self.k, channels_last=True)
-            return self.attention(q, k, x.contiguous(memory_format=torch.channels_last))
+            ny, nx = (self.norm_y, self.norm_x) if self.norm else (None, None)
+            # the query's bias goes into the fused operator instead of a pass of its
+            # own over the hi-res query tensor
+            ((q, q_bias),) = norm_project(y, ny, self.q, channels_last=True, defer_bias=True)
+            if not self.fused:
+                q, q_bias = q.add_(q_bias[:, :, None, None]), None
+            (k,) = norm_project(x, nx, self.k, channels_last=True)
+            return self.attention(q, k, x.contiguous(memory_format=torch.channels_last), q_bias)
         if self.norm and self.fold_norm:
             (q,), (k,) = norm_project(y, self.norm_y, self.q), norm_project(x, self.norm_x, self.k)
             return self.attention(q, k, x)
@@ -160,7 +172,7 @@ class SAPA(nn.Module):
             y = self.norm_y(y)
         return self.attention(self.q(y), self.k(x_), x)
 
-    def attention(self, q, k, v):
+    def attention(self, q, k, v, q_bias=None):
         K, s = self.up_kernel_size, self.up_factor
         # the operators take one memory order for all their tensors: the value's
         # (the caller's feature map) decides, so a channels-last model stays
@@ -171,7 +183,8 @@ class SAPA(nn.Module):
                else torch.contiguous_format)
         q, k, v = (t.contiguous(memory_format=fmt) for t in (q, k, v))
         if self.fused:
-            return sapa_fused(q, k, v, K, s)
+            return sapa_fused(q, k, v, K, s, q_bias)
+        assert q_bias is None
         attn = F.softmax(qk(q, k, K, s), dim=1).contiguous(memory_format=fmt)
         return av(attn, v, K, s)
 

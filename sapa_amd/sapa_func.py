@@ -224,10 +224,16 @@ class SAPAFusedFunction(Function):
     """av(softmax(qk(query, key), dim=1), value) -- SAPA.attention
     (sapa_base.py:38-40) -- as one launch in the forward pass.  The backward
     pass recomputes the attention weights (one launch) instead of keeping the
-    [B,K*K,sH,sW] tensor alive, then chains the three operators' gradients."""
+    [B,K*K,sH,sW] tensor alive, then chains the three operators' gradients.
+
+    query_bias [B, d] (optional): a per-image bias added to every query vector,
+    i.e. the result for query + query_bias[:, :, None, None] -- what a 1x1
+    projection with a (per-image) bias produces -- without that sum being
+    written first.  The channels_last kernels add it on the fly; other layouts
+    form the sum."""
 
     @staticmethod
-    def forward(ctx, query, key, value, kernel_size, scale_factor):
+    def forward(ctx, query, key, value, kernel_size, scale_factor, query_bias=None):
         assert scale_factor >= 1
         assert query.size(0) == key.size(0) == value.size(0)
         assert query.size(1) == key.size(1)
@@ -243,24 +249,43 @@ class SAPAFusedFunction(Function):
         if not value.is_cuda:
             raise NotImplementedError
         nhwc = _lib.memory_layout(value=value, key=key, query=query) == 'channels_last'
+        if query_bias is not None:
+            assert query_bias.shape == (n, d) and query_bias.dtype == query.dtype
+        ctx.has_bias = query_bias is not None
+        if query.requires_grad or key.requires_grad or value.requires_grad or \
+                (query_bias is not None and query_bias.requires_grad):
+            ctx.save_for_backward(*((query, key, value) + ((query_bias,) if ctx.has_bias else ())))
+        if query_bias is not None and not nhwc:
+            query = query + query_bias[:, :, None, None]
+            query_bias = None
         output = _lib.new_out(value, (n, c, h * scale_factor, w * scale_factor), nhwc)
-        (_lib.call_nhwc if nhwc else _lib.call)(
-            'sapa_fused_forward_nhwc' if nhwc else 'sapa_fused_forward', value.device,
-            _lib.ptr(query), _lib.ptr(key), _lib.ptr(value), _lib.ptr(output), n, d, c, h, w,
-            kernel_size, scale_factor, _lib.dtype_code(value))
-
-        if query.requires_grad or key.requires_grad or value.requires_grad:
-            ctx.save_for_backward(query, key, value)
+        if query_bias is not None:
+            query_bias = query_bias.contiguous()
+            _lib.call_nhwc('sapa_fused_forward_nhwc_qbias', value.device, _lib.ptr(query), _lib.ptr(key),
+                           _lib.ptr(value), _lib.ptr(query_bias), _lib.ptr(output), n, d, c, h, w,
+                           kernel_size, scale_factor, _lib.dtype_code(value))
+        else:
+            (_lib.call_nhwc if nhwc else _lib.call)(
+                'sapa_fused_forward_nhwc' if nhwc else 'sapa_fused_forward', value.device,
+                _lib.ptr(query), _lib.ptr(key), _lib.ptr(value), _lib.ptr(output), n, d, c, h, w,
+                kernel_size, scale_factor, _lib.dtype_code(value))
         return output
 
     @staticmethod
     def backward(ctx, grad_output):
         assert grad_output.is_cuda
-        query, key, value = ctx.saved_tensors
+        query, key, value = ctx.saved_tensors[:3]
+        needs = ctx.needs_input_grad
+        grad_bias = None
+        if ctx.has_bias:
+            query = query + ctx.saved_tensors[3][:, :, None, None]
         grad_query, grad_key, grad_value = _fused_backward(
             grad_output, query, key, value, ctx.kernel_size, ctx.scale_factor,
-            ctx.needs_input_grad[:3])
-        return grad_query, grad_key, grad_value, None, None
+            (needs[0] or (ctx.has_bias and needs[5]), needs[1], needs[2]))
+        if ctx.has_bias and needs[5]:
+            grad_bias = grad_query.sum(dim=(2, 3), dtype=torch.float32).to(grad_query.dtype)
+        return (grad_query if needs[0] else None), grad_key, grad_value, None, None, grad_bias
 
 
-sapa_fused = SAPAFusedFunction.apply
+def sapa_fused(query, key, value, kernel_size, scale_factor, query_bias=None):
+    return SAPAFusedFunction.apply(query, key, value, kernel_size, scale_factor, query_bias)

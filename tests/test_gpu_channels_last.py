@@ -325,3 +325,48 @@ def test_groupnorm_fold_kernel(dtype, tol):
     want_b = conv.bias.double().cpu() + torch.einsum('oc,bc->bo', w, beta - mean_c * scale)
     torch.testing.assert_close(w_b.double().cpu(), want_w, rtol=tol, atol=tol * 0.1)
     torch.testing.assert_close(b_b.double().cpu(), want_b, rtol=tol, atol=tol)
+
+
+@pytest.mark.parametrize('dtype,rel', [(torch.float32, None), (torch.bfloat16, BF16_REL), (torch.float16, F16_REL)])
+@pytest.mark.parametrize('shape', [(2, 64, 40, 9, 11, 5, 2), (1, 72, 36, 5, 6, 7, 4), (2, 12, 8, 6, 7, 3, 2)],
+                         ids=['d64', 'd72-k7s4', 'd12'])
+def test_fused_with_query_bias(coracle, dtype, rel, shape):
+    """sapa_fused(q, k, v, K, s, query_bias) = sapa_fused(q + bias, k, v, K, s): the
+    channels-last kernels add the per-image bias on the fly (16-bit: as four more
+    matrix instructions per tap group), the contiguous path forms the sum."""
+    B, d, C, H, W, K, s = shape
+    g = gen(350)
+    q, key, v, _ = inputs(g, B, d, C, H, W, K, s, dtype=dtype)
+    bias = (randn(g, B, d) * 0.7).to(dtype)
+    qb = q.float() + bias.float()[:, :, None, None]
+    want = coracle.sapa_fused(qb, key.float(), v.float(), K, s, 'f32a64')
+    # the contiguous path writes the sum in the tensors' type first: one more rounding
+    want_rounded = coracle.sapa_fused(qb.to(dtype).float(), key.float(), v.float(), K, s, 'f32a64')
+    got_cl = sapa_amd.sapa_fused(*cl(q, key, v), K, s, bias.to(DEV))
+    got = sapa_amd.sapa_fused(q.to(DEV), key.to(DEV), v.to(DEV), K, s, bias.to(DEV))
+    assert got_cl.is_contiguous(memory_format=CL)
+    for out, want in ((got_cl, want), (got, want_rounded)):
+        if rel is None:
+            torch.testing.assert_close(out.cpu().double().contiguous(), want, rtol=1e-5, atol=1e-5)
+        else:
+            assert_rel_rms_close(out.float(), want, rel, 'fused with bias')
+
+
+def test_fused_with_query_bias_gradients():
+    """Gradients through the biased call equal those of the explicit sum."""
+    g = gen(351)
+    B, d, C, H, W, K, s = 2, 8, 12, 5, 6, 5, 2
+    q, key, v, _ = inputs(g, B, d, C, H, W, K, s)
+    bias = randn(g, B, d) * 0.5
+    go = randn(g, B, C, s * H, s * W).to(DEV)
+    grads = []
+    for biased in (True, False):
+        leaves = [t.to(DEV).contiguous(memory_format=CL).requires_grad_() for t in (q, key, v)]
+        bl = bias.to(DEV).requires_grad_()
+        if biased:
+            out = sapa_amd.sapa_fused(*leaves, K, s, bl)
+        else:
+            out = sapa_amd.sapa_fused(leaves[0] + bl[:, :, None, None], leaves[1], leaves[2], K, s)
+        grads.append(torch.autograd.grad(out, leaves + [bl], go))
+    for a, b in zip(*grads):
+        torch.testing.assert_close(a, b, rtol=1e-4, atol=1e-5)
