@@ -313,6 +313,17 @@ int sapa_groupnorm_fold(const float *mean_var, const void *gamma, const void *be
                         const void *weight, const void *bias, void *weight_out, void *bias_out,
                         int B, int C, int O, int groups, float eps, int dtype, void *stream);
 
+/* 1x1 projection with per-image weights on a channels-last feature:
+ *   out[b,p,o] = sum_c x[b,p,c] * weight[b,o,c] (+ bias[b,o]),
+ * x [B,HW,C], weight [B,O,C] (sapa_groupnorm_fold's output), bias [B,O] or NULL,
+ * out [B,HW,O] -- self.q(norm_y(y)) / self.k(norm_x(x)) of the reference
+ * (sapa/sapa/sapa_base.py:32-35; Conv2d and GroupNorm, ATen calls there) as one
+ * stream over the feature.  SAPA_F16 / SAPA_BF16, C in {64,128,256,512}, O in
+ * {32,64,128} (not every pair), pointers aligned to 16 bytes;
+ * SAPA_ERR_UNSUPPORTED otherwise. */
+int sapa_project_nhwc(const void *x, const void *weight, const void *bias, void *out,
+                      int B, int C, int O, long long HW, int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -490,4 +490,16 @@ int sapa_groupnorm_fold(const float *mean_var, const void *gamma, const void *be
     return finish(e);
 }
 
+int sapa_project_nhwc(const void *x, const void *weight, const void *bias, void *out, int B, int C,
+                      int O, long long HW, int dtype, void *stream) {
+    if (!dtype_ok(dtype) || B < 0 || C <= 0 || O <= 0 || HW <= 0) return SAPA_ERR_INVALID_ARGUMENT;
+    if ((long long)B * HW * (C > O ? C : O) >= kMaxElems) return SAPA_ERR_TOO_LARGE;
+    if (B == 0) return SAPA_OK;
+    if (!x || !weight || !out) return SAPA_ERR_INVALID_ARGUMENT;
+    const hipError_t e = project_nhwc_launch(x, weight, bias, out, B, C, O, (long)HW, dtype,
+                                             (hipStream_t)stream);
+    if (e == hipErrorNotSupported) return SAPA_ERR_UNSUPPORTED;
+    return finish(e);
+}
+
 }  // extern "C"

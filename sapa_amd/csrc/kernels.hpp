@@ -52,6 +52,10 @@ hipError_t groupnorm_fold_launch(const float *mean_var, const void *gamma, const
                                  const void *w, const void *bias, void *w_out, void *b_out, int B,
                                  int C, int O, int G, float eps, int dtype, hipStream_t st);
 
+// sapa_project.hip: 1x1 projection of a channels-last 16-bit feature with per-image weights
+hipError_t project_nhwc_launch(const void *x, const void *w, const void *bias, void *out, int B,
+                               int C, int O, long HW, int dtype, hipStream_t st);
+
 // sapa_d_nhwc.hip: fused SAPA-D forward for tensors in channels-last memory
 // order (offsets [B, sH, sW, 2GP]); f32 / f16 / bf16, s in {1, 2, 4}, P <= 32,
 // channels per group multiples of 4, at most 64 query / key channels per group.

@@ -108,10 +108,16 @@ def norm_project(x, norm, *convs, channels_last=False, defer_bias=False):
         # GEMM, then the bias in place: measurably faster than baddbmm here, which
         # first spreads the bias over the whole output
         if channels_last:
-            out = torch.bmm(x3.transpose(1, 2), w_b.transpose(1, 2))      # [B, HW, O]
-            if not defer_bias:
-                out.add_(b_b.unsqueeze(1))
-            out = out.view(B, H, W, O).permute(0, 3, 1, 2)
+            # a 16-bit channels_last feature that needs no gradient: the library's
+            # streaming projection kernel (bias in its epilogue); else a library GEMM
+            out = None
+            if x_cl and x.is_cuda and not torch.is_grad_enabled():
+                out = _lib.project_nhwc(x, w_b, None if defer_bias else b_b)
+            if out is None:
+                out = torch.bmm(x3.transpose(1, 2), w_b.transpose(1, 2))      # [B, HW, O]
+                if not defer_bias:
+                    out.add_(b_b.unsqueeze(1))
+                out = out.view(B, H, W, O).permute(0, 3, 1, 2)
         else:
             out = torch.bmm(w_b, x3)                                     # [B, O, HW]
             if not defer_bias:

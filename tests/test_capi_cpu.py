@@ -81,6 +81,11 @@ def test_argument_validation_returns_codes():
     assert h.sapa_channel_moments(p, p, p, 1, 8, 64, 0, 1, None) == -2
     assert h.sapa_channel_moments(p, None, p, 1, 8, 64, 0, 0, None) == -1
     assert h.sapa_channel_moments(None, None, None, 0, 8, 64, 0, 0, None) == 0
+    # projection: extents, null pointers, fp32 (no kernel), empty batch
+    assert h.sapa_project_nhwc(p, p, p, p, 1, 0, 64, 100, 3, None) == -1
+    assert h.sapa_project_nhwc(p, None, p, p, 1, 256, 64, 100, 3, None) == -1
+    assert h.sapa_project_nhwc(p, p, None, p, 1, 256, 64, 100, 0, None) == -2
+    assert h.sapa_project_nhwc(None, None, None, None, 0, 256, 64, 100, 3, None) == 0
     # GroupNorm fold: channels not divisible by the groups, null weight, empty batch
     assert h.sapa_groupnorm_fold(p, p, p, p, p, p, p, 1, 10, 4, 4, 1e-5, 0, None) == -1
     assert h.sapa_groupnorm_fold(p, p, p, None, p, p, p, 1, 8, 4, 4, 1e-5, 0, None) == -1

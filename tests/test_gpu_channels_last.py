@@ -370,3 +370,26 @@ def test_fused_with_query_bias_gradients():
         grads.append(torch.autograd.grad(out, leaves + [bl], go))
     for a, b in zip(*grads):
         torch.testing.assert_close(a, b, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize('dtype,tol', [(torch.bfloat16, 2e-2), (torch.float16, 3e-3)])
+@pytest.mark.parametrize('shape', [(2, 256, 64, 9, 11), (1, 128, 32, 40, 33), (3, 64, 64, 5, 7),
+                                   (1, 512, 64, 4, 4), (2, 256, 128, 1, 1), (1, 256, 64, 130, 129)])
+def test_projection_kernel(dtype, tol, shape):
+    """The streaming 1x1 projection with per-image weights on a channels_last
+    16-bit feature (ragged last pixel tile, one pixel, several images) against
+    float64 arithmetic on the same values; None for shapes it is not built for."""
+    from sapa_amd import _lib
+    B, C, O, H, W = shape
+    g = gen(360)
+    x = randn(g, B, C, H, W).to(dtype).to(DEV).contiguous(memory_format=CL)
+    w = (randn(g, B, O, C) * 0.1).to(dtype).to(DEV)
+    b = randn(g, B, O).to(dtype).to(DEV)
+    want = torch.einsum('boc,bchw->bohw', w.double().cpu(), x.double().cpu())
+    for bias in (None, b):
+        out = _lib.project_nhwc(x, w, bias)
+        assert out is not None and out.shape == (B, O, H, W) and out.is_contiguous(memory_format=CL)
+        ref = want if bias is None else want + bias.double().cpu()[:, :, None, None]
+        torch.testing.assert_close(out.double().cpu(), ref, rtol=tol, atol=tol)
+    assert _lib.project_nhwc(x[:, :48].contiguous(memory_format=CL), w[:, :, :48].contiguous()) is None
+    assert _lib.project_nhwc(x.float(), w.float()) is None
