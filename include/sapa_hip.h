@@ -300,6 +300,22 @@ int sapa_channel_moments(const void *x, void *workspace, float *mean_var,
                          int B, int C, long long HW, int channels_last,
                          int dtype, void *stream);
 
+/* sapa_channel_moments without a workspace argument, for callers that cannot
+ * allocate device memory: code under HIP graph capture, serving loops and
+ * harnesses that forbid allocator calls.  No counterpart in the reference.
+ * The partial sums go to a fixed array of sapa_channel_moments_static_capacity()
+ * bytes (8 MiB) that is part of the library's code object on every device it
+ * runs on; the call allocates and frees nothing.  Same arguments, coverage and
+ * results (bit for bit) as sapa_channel_moments; SAPA_ERR_TOO_LARGE when
+ * sapa_channel_moments_workspace(B, C, HW, channels_last) exceeds the capacity.
+ * All calls on one device share that array: calls that overlap in time on the
+ * same device (different streams or host threads) race and must be serialised
+ * by the caller. */
+long long sapa_channel_moments_static_capacity(void);
+int sapa_channel_moments_static(const void *x, float *mean_var,
+                                int B, int C, long long HW, int channels_last,
+                                int dtype, void *stream);
+
 /* GroupNorm folded into a 1x1 projection, per image: from mean_var (above),
  * the norm's gamma / beta [C] (NULL: 1 / 0), `groups` and eps, and the
  * projection's weight [O,C] and bias [O] (NULL: none), all of type `dtype`:

@@ -23,6 +23,7 @@ SIGNATURES = {
     'sapa_fused_forward_nhwc_qbias': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_project_nhwc': [_vp, _vp, _vp, _vp, _i, _i, _i, _ll, _i, _vp],
     'sapa_channel_moments': [_vp, _vp, _vp, _i, _i, _ll, _i, _i, _vp],
+    'sapa_channel_moments_static': [_vp, _vp, _i, _i, _ll, _i, _i, _vp],
     'sapa_groupnorm_fold': [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, ctypes.c_float, _i, _vp],
     'sapa_qk_forward': [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_qk_backward': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
@@ -78,6 +79,8 @@ def lib():
             fn.argtypes = argtypes
         handle.sapa_channel_moments_workspace.restype = _ll
         handle.sapa_channel_moments_workspace.argtypes = [_i, _i, _ll, _i]
+        handle.sapa_channel_moments_static_capacity.restype = _ll
+        handle.sapa_channel_moments_static_capacity.argtypes = []
         _lib = handle
     return _lib
 

@@ -476,6 +476,24 @@ int sapa_channel_moments(const void *x, void *workspace, float *mean_var, int B,
     return finish(e);
 }
 
+long long sapa_channel_moments_static_capacity(void) { return channel_moments_static_capacity(); }
+
+int sapa_channel_moments_static(const void *x, float *mean_var, int B, int C, long long HW,
+                                int channels_last, int dtype, void *stream) {
+    if (!dtype_ok(dtype) || B < 0 || C <= 0 || HW <= 0) return SAPA_ERR_INVALID_ARGUMENT;
+    if (dtype == SAPA_F64) return SAPA_ERR_UNSUPPORTED;
+    if ((long long)B * C * HW >= kMaxElems) return SAPA_ERR_TOO_LARGE;
+    if (B == 0) return SAPA_OK;
+    if (!x || !mean_var) return SAPA_ERR_INVALID_ARGUMENT;
+    // partial sums beyond the library's fixed array: the workspace form serves those extents
+    if (channel_moments_workspace(B, C, (long)HW, channels_last != 0) > channel_moments_static_capacity())
+        return SAPA_ERR_TOO_LARGE;
+    const hipError_t e = channel_moments_static_launch(x, mean_var, B, C, (long)HW, channels_last != 0,
+                                                       dtype, (hipStream_t)stream);
+    if (e == hipErrorNotSupported) return SAPA_ERR_UNSUPPORTED;
+    return finish(e);
+}
+
 int sapa_groupnorm_fold(const float *mean_var, const void *gamma, const void *beta, const void *weight,
                         const void *bias, void *weight_out, void *bias_out, int B, int C, int O,
                         int groups, float eps, int dtype, void *stream) {

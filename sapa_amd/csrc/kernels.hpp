@@ -48,6 +48,11 @@ hipError_t sapa_b_nhwc16_launch(int mode, const void *q, const void *key, const 
 long channel_moments_workspace(int B, int C, long HW, bool channels_last);
 hipError_t channel_moments_launch(const void *x, void *workspace, float *mean_var, int B, int C,
                                   long HW, bool channels_last, int dtype, hipStream_t st);
+// the same with the partial sums in a fixed array inside the library (no workspace argument);
+// hipErrorInvalidValue when they would not fit channel_moments_static_capacity() bytes
+long channel_moments_static_capacity();
+hipError_t channel_moments_static_launch(const void *x, float *mean_var, int B, int C, long HW,
+                                         bool channels_last, int dtype, hipStream_t st);
 hipError_t groupnorm_fold_launch(const float *mean_var, const void *gamma, const void *beta,
                                  const void *w, const void *bias, void *w_out, void *b_out, int B,
                                  int C, int O, int G, float eps, int dtype, hipStream_t st);

@@ -17,6 +17,8 @@
 //      mean = shift + S1 / HW, var = S2 / HW - (S1 / HW)^2.
 #include "kernels.hpp"
 
+#include <mutex>
+
 namespace sapa {
 
 namespace moments {
@@ -327,6 +329,63 @@ hipError_t channel_moments_launch(const void *x, void *workspace, float *mean_va
         case 3: return moments::launch_t((const bf16_t *)x, ws, mean_var, B, C, HW, channels_last, st);
         default: return hipErrorNotSupported;
     }
+}
+
+// ---- the same statistics for callers that cannot bring a workspace ----
+//
+// The partial sums go to a fixed array in device memory that is part of the
+// library's code object: no allocation on any path, so the call can be made
+// under stream capture or from a loop that must not touch the allocator.
+// Every device holds its own copy of the array at its own address; host code
+// only ever uses the address hipGetSymbolAddress reports for the current
+// device (the array's name is not a device address on the host side).
+}  // namespace sapa
+
+constexpr long kStaticScratchBytes = 8L << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+// address of `scratch` on the current device; looked up once per device
+hipError_t scratch_address(void **out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (!p) return hipErrorInvalidSymbol;
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return hipSuccess;
+}
+}  // namespace
+
+namespace sapa {
+
+long channel_moments_static_capacity() { return kStaticScratchBytes; }
+
+// channel_moments_launch with the partial sums in the library's own fixed
+// array.  The caller has checked that channel_moments_workspace(...) fits
+// channel_moments_static_capacity().  Every partial sum that the second kernel
+// reads is written by the first one of the same call, so nothing has to be
+// cleared between calls; two calls in flight on one device share the array and
+// must not overlap.
+hipError_t channel_moments_static_launch(const void *x, float *mean_var, int B, int C, long HW,
+                                         bool channels_last, int dtype, hipStream_t st) {
+    if (channel_moments_workspace(B, C, HW, channels_last) > kStaticScratchBytes)
+        return hipErrorInvalidValue;
+    void *ws = nullptr;
+    const hipError_t e = scratch_address(&ws);
+    if (e != hipSuccess) return e;
+    return channel_moments_launch(x, ws, mean_var, B, C, HW, channels_last, dtype, st);
 }
 
 // mean_var [B, C, 2] fp32 (channel_moments_launch); gamma, beta [C] or null, w

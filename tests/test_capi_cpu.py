@@ -29,11 +29,13 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(handle, n), f'{n} declared in include/sapa_hip.h but not exported'
     # and the Python binding covers every operator entry point
     # (the workspace query returns a size, not a status: bound separately)
-    ops = [n for n in names if not n.startswith('sapa_hip_') and n != 'sapa_channel_moments_workspace']
+    ops = [n for n in names if not n.startswith('sapa_hip_')
+           and n not in ('sapa_channel_moments_workspace', 'sapa_channel_moments_static_capacity')]
     assert sorted(ops) == sorted(_lib.SIGNATURES)
     h = _lib.lib()
     assert h.sapa_channel_moments_workspace(16, 256, 67200, 0) > 0
     assert h.sapa_channel_moments_workspace(0, 256, 67200, 1) == 0
+    assert h.sapa_channel_moments_static_capacity() == 8 << 20
 
 
 def test_abi_version_and_status_strings():
@@ -81,6 +83,15 @@ def test_argument_validation_returns_codes():
     assert h.sapa_channel_moments(p, p, p, 1, 8, 64, 0, 1, None) == -2
     assert h.sapa_channel_moments(p, None, p, 1, 8, 64, 0, 0, None) == -1
     assert h.sapa_channel_moments(None, None, None, 0, 8, 64, 0, 0, None) == 0
+    # the form without a workspace: same validation, and extents whose partial
+    # sums exceed the library's fixed array are refused before any HIP call
+    assert h.sapa_channel_moments_static(p, p, 1, 0, 64, 0, 0, None) == -1
+    assert h.sapa_channel_moments_static(p, p, 1, 8, 64, 0, 1, None) == -2
+    assert h.sapa_channel_moments_static(None, p, 1, 8, 64, 0, 0, None) == -1
+    assert h.sapa_channel_moments_static(None, None, 0, 8, 64, 0, 0, None) == 0
+    big = (2, 1024, 1 << 22, 1)
+    assert h.sapa_channel_moments_workspace(*big) > h.sapa_channel_moments_static_capacity()
+    assert h.sapa_channel_moments_static(p, p, big[0], big[1], big[2], big[3], 0, None) == -3
     # projection: extents, null pointers, fp32 (no kernel), empty batch
     assert h.sapa_project_nhwc(p, p, p, p, 1, 0, 64, 100, 3, None) == -1
     assert h.sapa_project_nhwc(p, None, p, p, 1, 256, 64, 100, 3, None) == -1

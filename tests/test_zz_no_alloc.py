@@ -1,0 +1,58 @@
+"""GPU: sapa_channel_moments_static, the entry point that allocates nothing
+(partial sums in a fixed array inside the library), against
+sapa_channel_moments with a caller-provided workspace: bit for bit, on two
+calls in a row, the second on a smaller input."""
+import pytest
+import torch
+
+from sapa_amd import _lib
+
+pytestmark = pytest.mark.gpu
+
+
+def _both(x, cl):
+    """(workspace form, static form) of the [B, C, 2] statistics of x, through the C ABI."""
+    B, C, H, W = x.shape
+    h = _lib.lib()
+    code = _lib.DTYPES[x.dtype]
+    with torch.cuda.device(x.device):
+        st = torch.cuda.current_stream(x.device).cuda_stream
+        need = h.sapa_channel_moments_workspace(B, C, H * W, cl)
+        assert 0 < need <= h.sapa_channel_moments_static_capacity()
+        ws = torch.empty(need, dtype=torch.uint8, device=x.device)
+        want = torch.full((B, C, 2), float('nan'), device=x.device)
+        got = torch.full((B, C, 2), float('nan'), device=x.device)
+        assert h.sapa_channel_moments(x.data_ptr(), ws.data_ptr(), want.data_ptr(), B, C, H * W, cl, code, st) == 0
+        assert h.sapa_channel_moments_static(x.data_ptr(), got.data_ptr(), B, C, H * W, cl, code, st) == 0
+        torch.cuda.synchronize()
+    return want, got
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('cl', [0, 1])
+def test_static_scratch_matches_workspace_form(cl, dtype):
+    dev = torch.device('cuda:0')
+    g = torch.Generator(device=dev).manual_seed(5)
+    # several chunks per image in both layouts, then a smaller input on the same array
+    for shape in ((3, 64, 96, 160), (2, 32, 40, 52)):
+        x = (torch.randn(shape, generator=g, device=dev) * 2 + 0.5).to(dtype)
+        if cl:
+            x = x.contiguous(memory_format=torch.channels_last)
+        want, got = _both(x, cl)
+        assert torch.isfinite(got).all()
+        assert torch.equal(got, want), f'{shape}: max diff {(got - want).abs().max().item()}'
+        # and both agree with torch's own statistics
+        xf = x.float()
+        ref = torch.stack([xf.mean((2, 3)), xf.var((2, 3), unbiased=False)], -1)
+        assert torch.allclose(got, ref, rtol=1e-4, atol=1e-5)
+
+
+def test_static_scratch_refuses_what_does_not_fit():
+    h = _lib.lib()
+    dev = torch.device('cuda:0')
+    x = torch.zeros(16, device=dev)
+    mv = torch.zeros(16, device=dev)
+    B, C, HW = 2, 1024, 1 << 22
+    assert h.sapa_channel_moments_workspace(B, C, HW, 1) > h.sapa_channel_moments_static_capacity()
+    # refused on the extents alone: the pointers are never dereferenced
+    assert h.sapa_channel_moments_static(x.data_ptr(), mv.data_ptr(), B, C, HW, 1, 0, None) == -3
