@@ -55,6 +55,12 @@ class SapaHipError(RuntimeError):
     """A libsapa_hip.so entry point returned a negative status."""
 
 
+class SapaUnsupported(SapaHipError):
+    """SAPA_ERR_UNSUPPORTED: a valid request that this entry point has no
+    kernel for.  Direct operator calls raise it; the modules catch it and take
+    the next more general path (contiguous tensors, the separate operators)."""
+
+
 def lib():
     """The loaded library (loaded on first use)."""
     global _lib
@@ -92,7 +98,8 @@ def check(status, what):
     msg = handle.sapa_hip_status_string(status).decode()
     if status == -4:
         msg += ': ' + handle.sapa_hip_last_hip_error().decode()
-    raise SapaHipError(f'{what}: {msg} (status {status})')
+    raise (SapaUnsupported if status == UNSUPPORTED else SapaHipError)(
+        f'{what}: {msg} (status {status})')
 
 
 # SAPA_AMD_POISON=1 fills every buffer the kernels are meant to overwrite with
@@ -166,13 +173,13 @@ def call_nhwc(name, device, *args):
     what the channels-last kernels cover (there is no hidden layout copy)."""
     status = call_status(name, device, *args)
     if status == UNSUPPORTED and 'deform' in name:
-        raise RuntimeError(
+        raise SapaUnsupported(
             f'{name}: channels_last tensors are served for float32 / float16 / bfloat16, '
             'scale_factor 1, 2 or 4, at most 32 points, channels per group that are multiples '
             'of 4 (at most 64 query / key channels per group); call .contiguous() on the inputs '
             'for other configurations')
     if status == UNSUPPORTED:
-        raise RuntimeError(
+        raise SapaUnsupported(
             f'{name}: channels_last tensors are served for float32 / float16 / bfloat16, '
             '(kernel_size, scale_factor) in {(3,2), (5,2), (7,2), (5,4), (7,4)}, channel counts that '
             'are multiples of 4; '

@@ -30,6 +30,10 @@ __device__ __forceinline__ float exp_(float x) {
     const float t = x * l2e_hi;
     float e = __builtin_fmaf(x, l2e_hi, -t);
     e = __builtin_fmaf(x, l2e_lo, e);
+    // x = -inf: t = -inf and the correction term is inf - inf = NaN; the maximum
+    // returns its other operand for a NaN, so exp(-inf) comes out as r = 0 as in
+    // torch.softmax, and a finite x (|e| < 1e-6) is untouched
+    e = __builtin_fmaxf(e, -1.0f);
     const float r = __builtin_amdgcn_exp2f(t);
     return __builtin_fmaf(r, e * 0.693147182464599609375f, r);
 }

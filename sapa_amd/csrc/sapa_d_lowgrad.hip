@@ -43,6 +43,7 @@ deform_lowgrad_lds_kernel(const float *__restrict__ hi, const float *__restrict_
                                                     // the low mantissa bits for |x| < 2^51
     __shared__ long long acc[CH * WIN];
     __shared__ unsigned smax;
+    __shared__ int sbad;
 
     const int logical = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
     if (logical >= nblocks) return;
@@ -66,13 +67,19 @@ deform_lowgrad_lds_kernel(const float *__restrict__ hi, const float *__restrict_
     const long ch0 = (long)b * Cx + (long)g * cg;
 
     for (int i = tid; i < CH * WIN; i += NT) acc[i] = 0;
-    if (tid == 0) smax = 0;
+    if (tid == 0) { smax = 0; sbad = 0; }
     __syncthreads();
 
-    // the largest |sc| of this pixel: half of the magnitude bound
+    // the largest |sc| of this pixel: half of the magnitude bound; inf / NaN
+    // scalars are noted apart (the maximum drops NaNs)
     float scmax = 0.f;
+    bool scbad = false;
     if (active)
-        for (int p = 0; p < P; ++p) scmax = fmaxf(scmax, fabsf(sp[(long)p * hplane]));
+        for (int p = 0; p < P; ++p) {
+            const float a = fabsf(sp[(long)p * hplane]);
+            scbad |= !(a < __builtin_huge_valf());
+            scmax = fmaxf(scmax, a);
+        }
     // a window cell receives at most one term per (pixel, point)
     int lg_terms = 0;
     while ((1L << lg_terms) < (long)NT * P) ++lg_terms;
@@ -81,16 +88,25 @@ deform_lowgrad_lds_kernel(const float *__restrict__ hi, const float *__restrict_
         const int nvalid = cg - c0 < CH ? cg - c0 : CH;
         float hv[CH];
         float hmax = 0.f;
+        bool bad = scbad;
 #pragma unroll
         for (int ch = 0; ch < CH; ++ch) {
             hv[ch] = (active && ch < nvalid) ? hi[(ch0 + c0 + ch) * hplane + pix] : 0.f;
-            hmax = fmaxf(hmax, fabsf(hv[ch]));
+            const float a = fabsf(hv[ch]);
+            bad |= !(a < __builtin_huge_valf());
+            hmax = fmaxf(hmax, a);
         }
         // workgroup-wide bound on |term| (non-negative floats order like their bits)
         const float mine = hmax * scmax;
-        if (mine > 0.f && !(mine != mine) && mine < __builtin_huge_valf())
+        bad |= !(mine < __builtin_huge_valf());
+        if (bad)
+            sbad = 1;       // an inf / NaN term: the fixed-point sums cannot carry it
+        else if (mine > 0.f)
             atomicMax(&smax, __float_as_uint(mine));
         __syncthreads();                            // also: the window is zero, smax complete
+        // a chunk with a non-finite term goes through the float atomics as a
+        // whole, so that inf / NaN reach grad_low as they do in the reference
+        const bool direct = sbad != 0;
         const float bound = __uint_as_float(smax);
         int ex = 0;
         (void)frexpf(bound, &ex);                   // bound < 2^ex
@@ -114,7 +130,7 @@ deform_lowgrad_lds_kernel(const float *__restrict__ hi, const float *__restrict_
                 Tap<float> tap;
                 if (!tap_setup(kh, kw, H, W, tap)) continue;
                 const int hl = (int)floor_(kh) - wy0, wl = (int)floor_(kw) - wx0;
-                if (hl >= 0 && hl <= WH - 2 && wl >= 0 && wl <= WW - 2) {
+                if (!direct && hl >= 0 && hl <= WH - 2 && wl >= 0 && wl <= WW - 2) {
                     // corners outside the image fall on window cells that are
                     // never written back: no masks needed
                     unsigned long long *cell = (unsigned long long *)acc + hl * WW + wl;
@@ -160,7 +176,7 @@ deform_lowgrad_lds_kernel(const float *__restrict__ hi, const float *__restrict_
                 unsafeAtomicAdd(grad_low + (ch0 + c0 + ch) * lplane + (long)gy * W + gx,
                                 (float)((double)a * unscale));
         }
-        if (tid == 0) smax = 0;
+        if (tid == 0) { smax = 0; sbad = 0; }
         // the next chunk's barrier (after its atomicMax) orders these writes
         // before any scatter; its atomicMax must not race the reset above
         __syncthreads();

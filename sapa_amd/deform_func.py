@@ -182,8 +182,11 @@ def _deform_fused_backward(grad_output, query, key, value, offset, P, s, G, offs
         query, key, value = query.contiguous(), key.contiguous(), value.contiguous()
         grad_output = grad_output.contiguous()
         offset = expand_offset(offset, s, offset_layout).contiguous()
-        logits = DeformQKFunction.apply(query, key, offset, P, s, G)
-        attn = torch.softmax(logits.float(), dim=2).to(logits.dtype)
+        # 16-bit tensors: the logits are recomputed from fp32 copies so that, like
+        # the forward kernel's, they are not rounded to 16 bits before the softmax
+        wide = _compute_dtype(query)
+        logits = DeformQKFunction.apply(query.to(wide), key.to(wide), offset.to(wide), P, s, G)
+        attn = torch.softmax(logits, dim=2).to(query.dtype)
         ga, gv, goff_av = _deform_av_backward(grad_output, attn, value, offset, P, s, G)
         a32, g32 = attn.float(), ga.float()
         grad_logits = (a32 * (g32 - (g32 * a32).sum(dim=2, keepdim=True))).to(attn.dtype)

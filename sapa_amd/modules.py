@@ -21,6 +21,12 @@ from .deform_func import deform_av, deform_qk, deform_sapa_fused
 from .sapa_func import av, qk, sapa_fused
 
 
+def _needs_grad(*mods):
+    """True when autograd is recording and a parameter of `mods` requires grad."""
+    return torch.is_grad_enabled() and any(
+        p.requires_grad for m in mods if m is not None for p in m.parameters())
+
+
 def norm_project(x, norm, *convs, channels_last=False, defer_bias=False):
     """conv(norm(x)) for a GroupNorm and one or more 1x1 convolutions fed by
     it (sapa_base.py:26-36: norm_y -> q, norm_x -> k) without materialising
@@ -53,6 +59,8 @@ def norm_project(x, norm, *convs, channels_last=False, defer_bias=False):
         # inference on the GPU: one pass of the library's moments kernel over x
         # (it has no backward, so tensors that need gradients take the torch path)
         mom = None
+        # statistics and folded weights in fp32 like GroupNorm's (fp64 for fp64 tensors)
+        acc = torch.float64 if x.dtype == torch.float64 else torch.float32
         if x.is_cuda and not (torch.is_grad_enabled() and x.requires_grad):
             mom = _lib.channel_moments(x)
         if mom is not None:
@@ -61,8 +69,8 @@ def norm_project(x, norm, *convs, channels_last=False, defer_bias=False):
             var = (var_ch + (mean_ch - mean.unsqueeze(2)).square()).mean(dim=2)
         elif x_cl:
             # per-channel moments, then per group: no layout copy of x
-            m1 = x.mean(dim=(2, 3), dtype=torch.float32).reshape(B, G, per_c)
-            m2 = (torch.linalg.vector_norm(x, dim=(2, 3), dtype=torch.float32).square()
+            m1 = x.mean(dim=(2, 3), dtype=acc).reshape(B, G, per_c)
+            m2 = (torch.linalg.vector_norm(x, dim=(2, 3), dtype=acc).square()
                   / (H * W)).reshape(B, G, per_c)
             mean = m1.mean(dim=2)
             var = (m2.mean(dim=2) - mean * mean).clamp_min(0)
@@ -74,18 +82,19 @@ def norm_project(x, norm, *convs, channels_last=False, defer_bias=False):
                 sq = torch.linalg.vector_norm(xg, dim=2, dtype=torch.float32).square() / xg.shape[2]
                 var = (sq - mean * mean).clamp_min(0)
             else:
-                var, mean = torch.var_mean(xg.float(), dim=2, unbiased=False)
+                var, mean = torch.var_mean(xg.to(acc), dim=2, unbiased=False)
         rstd = torch.rsqrt(var + norm.eps)
         rstd_c = rstd.repeat_interleave(per_c, dim=1)                    # [B, C]
         mean_c = mean.repeat_interleave(per_c, dim=1)
-        gamma = norm.weight.float() if norm.weight is not None else x.new_ones(C, dtype=torch.float32)
-        beta = norm.bias.float() if norm.bias is not None else x.new_zeros(C, dtype=torch.float32)
+        gamma = norm.weight.to(acc) if norm.weight is not None else x.new_ones(C, dtype=acc)
+        beta = norm.bias.to(acc) if norm.bias is not None else x.new_zeros(C, dtype=acc)
         scale = gamma.unsqueeze(0) * rstd_c                              # [B, C]
         shift = beta.unsqueeze(0) - mean_c * scale                       # [B, C]
     else:
         mom = None
-        scale = x.new_ones(B, C, dtype=torch.float32)
-        shift = x.new_zeros(B, C, dtype=torch.float32)
+        acc = torch.float64 if x.dtype == torch.float64 else torch.float32
+        scale = x.new_ones(B, C, dtype=acc)
+        shift = x.new_zeros(B, C, dtype=acc)
     # [B, C, HW] view of x in either memory order
     x3 = x.permute(0, 2, 3, 1).reshape(B, H * W, C).transpose(1, 2) if x_cl else x.reshape(B, C, H * W)
     outs = []
@@ -93,17 +102,18 @@ def norm_project(x, norm, *convs, channels_last=False, defer_bias=False):
         assert conv.kernel_size == (1, 1) and conv.groups == 1
         O = conv.out_channels
         folded = None
-        if norm is not None and mom is not None:
-            # the per-image weights and bias in one small kernel launch
+        if norm is not None and mom is not None and not _needs_grad(norm, conv):
+            # the per-image weights and bias in one small kernel launch (the kernel
+            # has no backward: parameters that train take the torch expressions below)
             folded = _lib.groupnorm_fold(mom, norm, conv, x.dtype)
         if folded is not None:
             w_b, b_b = folded
         else:
-            w = conv.weight.reshape(O, C).float()
+            w = conv.weight.reshape(O, C).to(acc)
             w_b = (w.unsqueeze(0) * scale.unsqueeze(1)).to(x.dtype)      # [B, O, C]
             b_b = torch.einsum('oc,bc->bo', w, shift)
             if conv.bias is not None:
-                b_b = b_b + conv.bias.float().unsqueeze(0)
+                b_b = b_b + conv.bias.to(acc).unsqueeze(0)
             b_b = b_b.to(x.dtype)
         # GEMM, then the bias in place: measurably faster than baddbmm here, which
         # first spreads the bias over the whole output
@@ -188,9 +198,30 @@ class SAPA(nn.Module):
                if not v.is_contiguous() and v.is_contiguous(memory_format=torch.channels_last)
                else torch.contiguous_format)
         q, k, v = (t.contiguous(memory_format=fmt) for t in (q, k, v))
+        try:
+            return self._attend(q, k, v, q_bias, fmt)
+        except _lib.SapaUnsupported:
+            if fmt is not torch.channels_last:
+                raise
+        # a configuration the channels-last kernels do not cover (float64, other
+        # (kernel, scale) pairs, channel counts that are no multiple of 4): one
+        # layout copy each way and the contiguous kernels, which serve them all
+        out = self._attend(q.contiguous(), k.contiguous(), v.contiguous(), q_bias,
+                           torch.contiguous_format)
+        return out.contiguous(memory_format=torch.channels_last)
+
+    def _attend(self, q, k, v, q_bias, fmt):
+        K, s = self.up_kernel_size, self.up_factor
         if self.fused:
-            return sapa_fused(q, k, v, K, s, q_bias)
-        assert q_bias is None
+            try:
+                return sapa_fused(q, k, v, K, s, q_bias)
+            except _lib.SapaUnsupported:
+                if fmt is torch.channels_last:
+                    raise
+            # kernel sizes beyond the fused kernel's register budget: the three
+            # operators, which take any odd kernel size
+        if q_bias is not None:
+            q = q + q_bias[:, :, None, None]
         attn = F.softmax(qk(q, k, K, s), dim=1).contiguous(memory_format=fmt)
         return av(attn, v, K, s)
 
@@ -244,10 +275,13 @@ class SAPADeform(nn.Module):
         if self.fused and (x.is_contiguous()
                            or not x.is_contiguous(memory_format=torch.channels_last)):
             # the kernel reads the offset convolution's output in place
-            return deform_sapa_fused(q.contiguous(), k.contiguous(), x.contiguous(),
-                                     offset_lo.contiguous(), self.num_point,
-                                     self.up_factor, self.groups,
-                                     'pixel_shuffle' if self.high_offset else 'nearest')
+            try:
+                return deform_sapa_fused(q.contiguous(), k.contiguous(), x.contiguous(),
+                                         offset_lo.contiguous(), self.num_point,
+                                         self.up_factor, self.groups,
+                                         'pixel_shuffle' if self.high_offset else 'nearest')
+            except _lib.SapaUnsupported:
+                pass    # more points than the fused kernel holds: attention() below
         if self.high_offset:
             offset = F.pixel_shuffle(offset_lo, upscale_factor=self.up_factor)
         else:
@@ -259,11 +293,23 @@ class SAPADeform(nn.Module):
         if self.fused:
             # one memory order for all tensors, the value's: a channels-last
             # model stays channels-last (the fused kernel serves that order)
-            fmt = (torch.channels_last
-                   if not x.is_contiguous() and x.is_contiguous(memory_format=torch.channels_last)
-                   else torch.contiguous_format)
+            cl = not x.is_contiguous() and x.is_contiguous(memory_format=torch.channels_last)
+            fmt = torch.channels_last if cl else torch.contiguous_format
             q, k, x, offset = (t.contiguous(memory_format=fmt) for t in (q, k, x, offset))
-            return deform_sapa_fused(q, k, x, offset, P, s, G)
+            try:
+                return deform_sapa_fused(q, k, x, offset, P, s, G)
+            except _lib.SapaUnsupported:
+                pass
+            # not covered in this memory order (float64, more than 32 points,
+            # channel counts that are no multiple of 4 ...) or at all (more than 64
+            # points): contiguous tensors, then the separate operators
+            q, k, x, offset = (t.contiguous() for t in (q, k, x, offset))
+            try:
+                out = deform_sapa_fused(q, k, x, offset, P, s, G)
+            except _lib.SapaUnsupported:
+                attn = F.softmax(deform_qk(q, k, offset, P, s, G), dim=2)
+                out = deform_av(attn, x, offset, P, s, G)
+            return out.contiguous(memory_format=fmt)
         # the separate operators take contiguous tensors only
         q, k, x, offset = (t.contiguous() for t in (q, k, x, offset))
         attn = F.softmax(deform_qk(q, k, offset, P, s, G), dim=2)

@@ -283,7 +283,8 @@ class SAPAFusedFunction(Function):
             grad_output, query, key, value, ctx.kernel_size, ctx.scale_factor,
             (needs[0] or (ctx.has_bias and needs[5]), needs[1], needs[2]))
         if ctx.has_bias and needs[5]:
-            grad_bias = grad_query.sum(dim=(2, 3), dtype=torch.float32).to(grad_query.dtype)
+            wide = torch.float32 if grad_query.dtype in (torch.float16, torch.bfloat16) else None
+            grad_bias = grad_query.sum(dim=(2, 3), dtype=wide).to(grad_query.dtype)
         return (grad_query if needs[0] else None), grad_key, grad_value, None, None, grad_bias
 
 
