@@ -4,7 +4,8 @@ one MI355X; the default workload is the largest FPN level (B=16, C=256, d=64,
 K=5, 100x168 -> 200x336, fp32).
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype fp32|bf16]
-                    [--workload fpn_large|fpn_mid|fpn_small|stress|deform_p25|deform_p9|deform_p5]
+                    [--workload fpn_large|fpn_mid|fpn_small|segformer_16|segformer_32|segformer_64|
+                                stress|deform_p25|deform_p9|deform_p5]
                     [--pass forward|train] [--no-cpu-baseline] [--calibration-copy]
 
 A step is one fused forward over the whole synthetic batch, inputs already
@@ -34,6 +35,12 @@ WORKLOADS = {
     'fpn_mid': (16, 256, 64, 50, 84, 5, 2),
     'fpn_small': (16, 256, 64, 25, 42, 5, 2),
     'stress': (4, 512, 64, 64, 64, 7, 4),
+    # SegFormer-style decoder chain 16^2 -> 32^2 -> 64^2 -> 128^2 (B=8, C=256, d=32): one
+    # workload per stage; query / key come from 1x1 projections ~N(0, .02) of
+    # random features (sapa_base.py:21-22,42-46)
+    'segformer_16': (8, 256, 32, 16, 16, 5, 2),
+    'segformer_32': (8, 256, 32, 32, 32, 5, 2),
+    'segformer_64': (8, 256, 32, 64, 64, 5, 2),
 }
 # SAPA-D (fused deform_qk -> softmax -> deform_av), BASELINE config 4:
 # name -> (B, C, d, G, H, W, P, s); offsets ~N(0, 0.75) clipped to +-4 cells
@@ -44,28 +51,40 @@ DEFORM_WORKLOADS = {
 }
 
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE + WRITE_SIZE,
-# scaled by what the same counters read for a plain copy of known size); see
-# the summaries under profiles/.  None = not measured for that case.
-MEASURED_TRAFFIC_BYTES = {
-    # profiles/sapa_b_fused_fpn_large_fp32.md: (324281.2 * 1.9999 + 1106514.0 * 1.0000) KiB
-    ('fpn_large', 'fp32'): 1797181513,
-    # profiles/sapa_b_fused_fpn_large_bf16.md: (174519.2 * 2.0000 + 594522.0 * 1.0000) KiB
-    ('fpn_large', 'bf16'): 966196919,
-    # profiles/sapa_b_nhwc_fused_fpn_large_fp32.md: (302512.3 * 2.0000 + 1075280.5 * 1.0000) KiB
-    ('fpn_large', 'fp32', 'channels_last'): 1720501948,
-    # profiles/sapa_b_nhwc_fused_fpn_large_bf16.md: (153483.6 * 2.0000 + 537600.7 * 1.0000) KiB
-    ('fpn_large', 'bf16', 'channels_last'): 864829676,
-    # profiles/sapa_d_nhwc_fused_deform_p25_fp32.md: (109284.2 * 2.0000 + 131072.0 * 1.0000) KiB
-    ('deform_p25', 'fp32', 'channels_last'): 358026263,
-    # profiles/sapa_b_mfma_fused_stress_bf16.md: (39700.2 * 1.9999 + 292841.7 * 1.0000) KiB
-    ('stress', 'bf16'): 381173848,
-    # profiles/sapa_b_nhwc16_fused_stress_bf16.md
-    ('stress', 'bf16', 'channels_last'): 323034807,
-    # profiles/sapa_d_lds_fused_deform_p9_fp32.md: (132709.9 * 1.9999 + 131503.8 * 1.0000) KiB
-    ('deform_p9', 'fp32'): 406442924,
-    # profiles/sapa_d_lds_fused_deform_p25_fp32.md: (343906.3 * 1.9999 + 131079.0 * 1.0000) KiB
-    ('deform_p25', 'fp32'): 838527266,
+# scaled by what the same counters read for a plain copy of known size), per
+# (workload, dtype, layout): bytes, the summary under profiles/ they come from
+# and the kernel they were measured on.  A run whose dispatched kernel is not
+# that kernel stops with an error instead of printing a stale figure.
+MEASURED_TRAFFIC = {
+    ('fpn_large', 'fp32', 'nchw'): (1797181513, 'profiles/sapa_b_fused_fpn_large_fp32.md', 'sapa_b_tiled_kernel'),
+    ('fpn_large', 'bf16', 'nchw'): (966196919, 'profiles/sapa_b_fused_fpn_large_bf16.md', 'sapa_b_dot2_kernel'),
+    ('fpn_large', 'fp32', 'channels_last'): (1720501948, 'profiles/sapa_b_nhwc_fused_fpn_large_fp32.md',
+                                             'sapa_b_nhwc_kernel'),
+    ('fpn_large', 'bf16', 'channels_last'): (864829676, 'profiles/sapa_b_nhwc_fused_fpn_large_bf16.md',
+                                             'sapa_b_nhwc16_kernel'),
+    ('stress', 'bf16', 'nchw'): (381173848, 'profiles/sapa_b_mfma_fused_stress_bf16.md', 'sapa_b_mfma_kernel'),
+    ('stress', 'bf16', 'channels_last'): (323034807, 'profiles/sapa_b_nhwc16_fused_stress_bf16.md',
+                                          'sapa_b_nhwc16_kernel'),
+    ('deform_p25', 'fp32', 'nchw'): (838527266, 'profiles/sapa_d_lds_fused_deform_p25_fp32.md', 'deform_lds_kernel'),
+    ('deform_p9', 'fp32', 'nchw'): (406442924, 'profiles/sapa_d_lds_fused_deform_p9_fp32.md', 'deform_lds_kernel'),
+    ('deform_p25', 'fp32', 'channels_last'): (358026263, 'profiles/sapa_d_nhwc_fused_deform_p25_fp32.md',
+                                              'deform_fused_nhwc_kernel'),
 }
+
+
+def measured_traffic(workload, dtype, layout, kernel):
+    """(bytes, {'file', 'kernel'}) for the run's configuration, (None, None) if
+    it was never measured; exits if it was measured on another kernel than the
+    one this run dispatched to."""
+    hit = MEASURED_TRAFFIC.get((workload, dtype, layout))
+    if hit is None:
+        return None, None
+    nbytes, source, measured_on = hit
+    if measured_on != kernel:
+        sys.exit(f'bench.py: the traffic figure for {workload}/{dtype}/{layout} in {source} was measured on '
+                 f'{measured_on}, this run dispatched to {kernel}: re-measure it (rocprofv3 --pmc FETCH_SIZE / '
+                 'WRITE_SIZE) and update MEASURED_TRAFFIC')
+    return nbytes, {'file': source, 'kernel': measured_on}
 
 
 def algorithmic_bytes(B, C, d, H, W, s, esize):
@@ -73,9 +92,20 @@ def algorithmic_bytes(B, C, d, H, W, s, esize):
     return esize * (B * H * s * W * s * (d + C) + B * H * W * (d + C))
 
 
-def make_inputs(cfg, dtype, device, seed=0, heavy_tails=False):
+def make_inputs(cfg, dtype, device, seed=0, heavy_tails=False, projected=False):
     B, C, d, H, W, K, s = cfg
     g = torch.Generator(device=device).manual_seed(seed)
+    if projected:
+        # q, key = 1x1 projections ~N(0, .02) (zero bias) of GroupNorm(32)-normalised
+        # random features; the value is the un-normalised low-res feature
+        y = torch.randn(B, C, H * s, W * s, generator=g, device=device)
+        x = torch.randn(B, C, H, W, generator=g, device=device)
+        wq = torch.randn(d, C, 1, 1, generator=g, device=device) * 0.02
+        wk = torch.randn(d, C, 1, 1, generator=g, device=device) * 0.02
+        gn = torch.nn.functional.group_norm
+        q = torch.nn.functional.conv2d(gn(y, 32), wq)
+        key = torch.nn.functional.conv2d(gn(x, 32), wk)
+        return q.to(dtype).contiguous(), key.to(dtype).contiguous(), x.to(dtype).contiguous()
     q = torch.randn(B, d, H * s, W * s, generator=g, device=device)
     if heavy_tails:
         # a random 10 % of the query replaced by Student-t(3) draws (the stress
@@ -122,16 +152,28 @@ def timed_median(fn, budget_s):
     return times[len(times) // 2], len(times), out
 
 
-def cpu_baseline(q, key, v, K, s, budget_s=20.0):
-    """Time the unfold-based CPU math on image 0 of the batch (repeated while
-    the budget lasts); returns (Gpix/s, cores, description, output)."""
-    from oracle import torch_oracle
-    q0, k0, v0 = (t[:1].float().cpu() for t in (q, key, v))
+def cpu_baseline(fn, tensors, pix_per_image, median_budget_s=8.0, batch_budget_s=60.0):
+    """CPU time of fn(image tensors...) on this host's cores: the median over
+    repeated runs on image 0, then the whole batch once, image by image (the
+    unfold formulation needs several GB per image, so the batch is chunked),
+    summed -- or as many images as fit batch_budget_s, and the count says so.
+    Returns the record for the JSON line and image 0's output."""
+    imgs = [[t[i:i + 1].float().cpu() for t in tensors] for i in range(tensors[0].shape[0])]
     cores = torch.get_num_threads()
-    med, runs, out = timed_median(lambda: torch_oracle.sapa_fused(q0, k0, v0, K, s), budget_s)
-    pix = q0.shape[2] * q0.shape[3]
-    return pix / med / 1e9, cores, (f'image 0 of the batch (1x{q0.shape[1]}x{q0.shape[2]}x{q0.shape[3]} '
-                                    f'query), fp32, median of {runs} runs'), out
+    med, runs, out = timed_median(lambda: fn(*imgs[0]), median_budget_s)
+    total, done = 0.0, 0
+    for im in imgs:
+        t0 = time.perf_counter()
+        fn(*im)
+        total += time.perf_counter() - t0
+        done += 1
+        if total > batch_budget_s:
+            break
+    rec = {'value': pix_per_image * done / total / 1e9, 'unit': 'Gpix/s', 'cores': cores, 'kind': 'port',
+           'sample': f'{done} of {len(imgs)} images of the batch, one at a time, fp32, {total:.1f} s in all '
+                     f'(torch CPU, {cores} threads)',
+           'image0_median': {'value': pix_per_image / med / 1e9, 'unit': 'Gpix/s', 'runs': runs}}
+    return rec, out
 
 
 def module_pass(args, dev, dtype, stream):
@@ -242,7 +284,8 @@ def main():
     else:
         cfg = WORKLOADS[args.workload]
         B, C, d, H, W, K, s = cfg
-        q, key, v = make_inputs(cfg, dtype, dev, heavy_tails=args.workload == 'stress')
+        q, key, v = make_inputs(cfg, dtype, dev, heavy_tails=args.workload == 'stress',
+                                projected=args.workload.startswith('segformer'))
     out = torch.empty(B, C, H * s, W * s, dtype=dtype, device=dev)
     code = _lib.dtype_code(out)
     if deform:
@@ -309,6 +352,7 @@ def main():
         return e0.elapsed_time(e1) / args.steps, (time.perf_counter() - t0) * 1e3 / args.steps
 
     ms, wall_ms = timed(step)
+    main_kernel = _lib.last_kernel()
     ms_cl = None
     if args.layout == 'nchw' and nhwc_ok and args.direction == 'forward':
         # the same workload with every tensor in torch.channels_last order
@@ -316,6 +360,7 @@ def main():
               for t in ((q, key, v, out, off) if deform else (q, key, v, out))]
         ms_cl, _ = timed(fused_step('sapa_deform_fused_forward_nhwc' if deform
                                     else 'sapa_fused_forward_nhwc', *cl))
+        cl_kernel = _lib.last_kernel()
         err_cl = (cl[3][:1].float() - out[:1].float()).abs().max().item()
         del cl
 
@@ -334,26 +379,18 @@ def main():
         what = 'fused SAPA-D forward (deform_qk->softmax->deform_av)'
         wl = (f'{args.workload}: SAPA-D B={B} C={C} d={d} G={G} P={P} {H}x{W}->{H * s}x{W * s} '
               f's={s} {args.dtype}, NCHW, offsets ~N(0,0.75) clipped to +-4')
-        kern = ('deform_fused_nhwc_kernel' if args.layout == 'channels_last'
-                else 'deform_lds_kernel (fused mode)')
         wl = wl.replace('NCHW', 'channels_last') if args.layout == 'channels_last' else wl
     else:
         abytes = algorithmic_bytes(B, C, d, H, W, s, esize)
         what = 'fused SAPA-B forward (qk->softmax->av)'
-        wl = (f'{args.workload}: SAPA-B FPN-style B={B} C={C} d={d} '
+        style = ('SegFormer-style stage, q / k from 1x1 projections ~N(0,.02) of GroupNorm-ed features'
+                 if args.workload.startswith('segformer') else 'FPN-style')
+        wl = (f'{args.workload}: SAPA-B {style} B={B} C={C} d={d} '
               f'{H}x{W}->{H * s}x{W * s} K={K} s={s} {args.dtype}, '
               + ('channels_last' if args.layout == 'channels_last' else 'NCHW')
               + (', 10% of q Student-t(3)' if args.workload == 'stress' else ''))
-        nhwc_kern = ('sapa_b_nhwc16_kernel (fused mode)' if esize == 2 and d % 8 == 0
-                     else 'sapa_b_nhwc_kernel (fused mode)')
-        if args.layout == 'channels_last':
-            kern = nhwc_kern
-        elif (K, s) != (5, 2):
-            kern = 'sapa_b_mfma_kernel (fused mode)'
-        elif esize == 2 and W % 4 == 0 and W >= 32:
-            kern = 'sapa_b_dot2_kernel (fused mode)'
-        else:
-            kern = 'sapa_b_tiled_kernel (fused mode)'
+    # the kernel the library dispatched this workload to
+    kern = main_kernel + ' (fused mode)'
     if train:
         # backward: read grad_out, q, key, value (offset); write every input gradient
         hi_px, lo_px = B * H * s * W * s, B * H * W
@@ -363,6 +400,9 @@ def main():
             abytes += esize * hi_px * 2 * (2 * G * P)
         what = what.replace('forward', 'forward + backward')
         kern = 'several (see profiles/)'
+    traffic = traffic_source = None
+    if not train:
+        traffic, traffic_source = measured_traffic(args.workload, args.dtype, args.layout, main_kernel)
     achieved = abytes / (ms * 1e-3) / 1e9
     rec = {
         'metric': f'upsampled Gpix/s, {what}, 1 GPU',
@@ -385,33 +425,34 @@ def main():
             'peak': HBM_PEAK_GBS,
             'unit': 'GB/s',
             'frac': achieved / HBM_PEAK_GBS,
-            'traffic': None if train else MEASURED_TRAFFIC_BYTES.get(
-                (args.workload, args.dtype) if args.layout == 'nchw'
-                else (args.workload, args.dtype, args.layout)),
+            'traffic': traffic,
+            'traffic_source': traffic_source,
             'algorithmic_bytes': abytes,
             'kernel': kern,
+            # a working set below the 256 MB Infinity Cache stays cache-resident
+            # when the same buffers are iterated: the rate is then no HBM rate
+            'cache_resident': abytes < 256e6,
         },
     }
     if ms_cl is not None:
         rec['channels_last'] = {
             'ms_per_step': ms_cl, 'value': pix / (ms_cl * 1e-3) / 1e9, 'unit': 'Gpix/s',
             'roofline_frac': abytes / (ms_cl * 1e-3) / 1e9 / HBM_PEAK_GBS,
-            'kernel': 'deform_fused_nhwc_kernel' if deform else nhwc_kern,
+            'kernel': cl_kernel + ' (fused mode)',
             'max_abs_diff_vs_nchw_image0': err_cl,
             'note': 'same workload and algorithmic bytes, every tensor in torch.channels_last '
                     'order (python bench.py --layout channels_last makes this the main line)'}
     if not args.no_cpu_baseline and not train:
+        from oracle import torch_oracle
         if deform:
-            from oracle import torch_oracle
-            q0, k0, v0, o0 = (t[:1].float().cpu() for t in (q, key, v, off))
-            med, runs, ref = timed_median(
-                lambda: torch_oracle.deform_sapa_fused(q0, k0, v0, o0, P, s, G), 20.0)
-            gpix, cores = q0.shape[2] * q0.shape[3] / med / 1e9, torch.get_num_threads()
-            sample = (f'image 0 of the batch (grid_sample formulation, fp32), median of {runs} runs')
+            # grid_sample formulation of deformsapa/deformsapa/forward_check.py:6-40
+            rec['cpu_baseline'], ref = cpu_baseline(
+                lambda a, b, c, o: torch_oracle.deform_sapa_fused(a, b, c, o, P, s, G), (q, key, v, off),
+                H * s * W * s)
         else:
-            gpix, cores, sample, ref = cpu_baseline(q, key, v, K, s)
-        rec['cpu_baseline'] = {'value': gpix, 'unit': 'Gpix/s', 'cores': cores, 'kind': 'port',
-                               'sample': sample}
+            # unfold + einsum formulation of sapa/sapa/forward_check.py:9-24
+            rec['cpu_baseline'], ref = cpu_baseline(
+                lambda a, b, c: torch_oracle.sapa_fused(a, b, c, K, s), (q, key, v), H * s * W * s)
         # the timed GPU output for the same image, against the CPU result
         got = out[:1].float().cpu()
         err = (got - ref).abs()

@@ -66,6 +66,11 @@ const char *sapa_hip_status_string(int status);
 /* Text of the HIP error behind the calling thread's most recent
  * SAPA_ERR_LAUNCH ("" if none). */
 const char *sapa_hip_last_hip_error(void);
+/* Name of the kernel that served the calling thread's most recent forward
+ * entry-point call ("" before the first): several kernels stand behind one
+ * entry point and the choice depends on dtype, extents and alignment, so a
+ * profile or a benchmark line can say which one it measured. */
+const char *sapa_hip_last_kernel(void);
 
 /* ------------------------------------------------------------------ SAPA-B */
 

@@ -79,6 +79,8 @@ def lib():
         handle.sapa_hip_status_string.argtypes = [_i]
         handle.sapa_hip_last_hip_error.restype = ctypes.c_char_p
         handle.sapa_hip_last_hip_error.argtypes = []
+        handle.sapa_hip_last_kernel.restype = ctypes.c_char_p
+        handle.sapa_hip_last_kernel.argtypes = []
         for name, argtypes in SIGNATURES.items():
             fn = getattr(handle, name)
             fn.restype = _i
@@ -89,6 +91,11 @@ def lib():
         handle.sapa_channel_moments_static_capacity.argtypes = []
         _lib = handle
     return _lib
+
+
+def last_kernel():
+    """Name of the kernel behind this thread's most recent forward call."""
+    return lib().sapa_hip_last_kernel().decode()
 
 
 def check(status, what):

@@ -12,6 +12,15 @@ using namespace sapa;
 namespace {
 
 thread_local char g_hip_error[256] = "";
+// kernel that took the calling thread's last forward request (sapa_hip_last_kernel)
+thread_local const char *g_last_kernel = "";
+
+// runs one candidate launcher; when it takes the request (anything but
+// hipErrorNotSupported) its kernel's name is recorded
+hipError_t took(const char *kernel, hipError_t e) {
+    if (e != hipErrorNotSupported) g_last_kernel = kernel;
+    return e;
+}
 
 int fail_hip(hipError_t e) {
     strncpy(g_hip_error, hipGetErrorString(e), sizeof(g_hip_error) - 1);
@@ -33,12 +42,14 @@ const long long kMaxElems = 1LL << 40;
 hipError_t tiled_launch(int mode, const void *q, const void *key, const void *attn_in,
                         const void *value, void *out, int B, int d, int C, int H, int W, int K,
                         int s, int dtype, hipStream_t st) {
-    hipError_t e = sapa_b_dot2_launch(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s,
-                                      dtype, st);
+    hipError_t e = took("sapa_b_dot2_kernel", sapa_b_dot2_launch(mode, q, key, attn_in, value, out, B,
+                                                                  d, C, H, W, K, s, dtype, st));
     if (e == hipErrorNotSupported)
-        e = sapa_b_tiled_launch(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, dtype, st);
+        e = took("sapa_b_tiled_kernel",
+                 sapa_b_tiled_launch(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, dtype, st));
     if (e == hipErrorNotSupported)
-        e = sapa_b_mfma_launch(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, dtype, st);
+        e = took("sapa_b_mfma_kernel",
+                 sapa_b_mfma_launch(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, dtype, st));
     return e;
 }
 
@@ -80,33 +91,34 @@ hipError_t lowres_grad_any(const void *hi, const void *w, void *out, int B, int 
 hipError_t deform_qk_any(const void *q, const void *key, const void *offset, void *out, int B,
                          int Cq, int H, int W, int P, int s, int G, int olayout, int dtype,
                          hipStream_t st) {
-    hipError_t e = deform_lds_launch(0, q, key, nullptr, nullptr, offset, out, B, Cq, Cq, H, W, P,
-                                     s, G, olayout, dtype, st);
+    hipError_t e = took("deform_lds_kernel", deform_lds_launch(0, q, key, nullptr, nullptr, offset, out, B,
+                                                                Cq, Cq, H, W, P, s, G, olayout, dtype, st));
     if (e == hipErrorNotSupported)
-        e = deform_qk_forward_launch(q, key, offset, out, B, Cq, H, W, P, s, G, olayout, dtype,
-                                     st);
+        e = took("deform_qk_forward_kernel",
+                 deform_qk_forward_launch(q, key, offset, out, B, Cq, H, W, P, s, G, olayout, dtype, st));
     return e;
 }
 
 hipError_t deform_av_any(const void *attn, const void *value, const void *offset, void *out, int B,
                          int C, int H, int W, int P, int s, int G, int olayout, int dtype,
                          hipStream_t st) {
-    hipError_t e = deform_lds_launch(1, nullptr, nullptr, attn, value, offset, out, B, C, C, H, W,
-                                     P, s, G, olayout, dtype, st);
+    hipError_t e = took("deform_lds_kernel", deform_lds_launch(1, nullptr, nullptr, attn, value, offset, out,
+                                                                B, C, C, H, W, P, s, G, olayout, dtype, st));
     if (e == hipErrorNotSupported)
-        e = deform_av_forward_launch(attn, value, offset, out, B, C, H, W, P, s, G, olayout,
-                                     dtype, st);
+        e = took("deform_av_forward_kernel",
+                 deform_av_forward_launch(attn, value, offset, out, B, C, H, W, P, s, G, olayout, dtype, st));
     return e;
 }
 
 hipError_t deform_fused_any(const void *q, const void *key, const void *value, const void *offset,
                             void *out, int B, int Cq, int C, int H, int W, int P, int s, int G,
                             int olayout, int dtype, hipStream_t st) {
-    hipError_t e = deform_lds_launch(2, q, key, nullptr, value, offset, out, B, Cq, C, H, W, P, s,
-                                     G, olayout, dtype, st);
+    hipError_t e = took("deform_lds_kernel", deform_lds_launch(2, q, key, nullptr, value, offset, out, B, Cq,
+                                                                C, H, W, P, s, G, olayout, dtype, st));
     if (e == hipErrorNotSupported)
-        e = deform_fused_forward_launch(q, key, value, offset, out, B, Cq, C, H, W, P, s, G,
-                                        olayout, dtype, st);
+        e = took("deform_fused_forward_kernel",
+                 deform_fused_forward_launch(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, olayout,
+                                             dtype, st));
     return e;
 }
 
@@ -156,6 +168,8 @@ const char *sapa_hip_status_string(int status) {
 
 const char *sapa_hip_last_hip_error(void) { return g_hip_error; }
 
+const char *sapa_hip_last_kernel(void) { return g_last_kernel; }
+
 int sapa_qk_forward(const void *query, const void *key, void *out, int B, int d, int H, int W,
                     int K, int s, int dtype, void *stream) {
     const int rc = check_window_args(B, d, d, H, W, K, s, dtype);
@@ -166,7 +180,8 @@ int sapa_qk_forward(const void *query, const void *key, void *out, int B, int d,
     hipError_t e = tiled_launch(TILED_QK, query, key, nullptr, nullptr, out, B, d, 0, H, W,
                                        K, s, dtype, st);
     if (e == hipErrorNotSupported)
-        e = qk_forward_generic_launch(query, key, out, B, d, H, W, K, s, dtype, st);
+        e = took("qk_forward_generic_kernel",
+                 qk_forward_generic_launch(query, key, out, B, d, H, W, K, s, dtype, st));
     return finish(e);
 }
 
@@ -180,7 +195,8 @@ int sapa_av_forward(const void *attn, const void *value, void *out, int B, int C
     hipError_t e = tiled_launch(TILED_AV, nullptr, nullptr, attn, value, out, B, 0, C, H, W,
                                        K, s, dtype, st);
     if (e == hipErrorNotSupported)
-        e = av_forward_generic_launch(attn, value, out, B, C, H, W, K, s, dtype, st);
+        e = took("av_forward_generic_kernel",
+                 av_forward_generic_launch(attn, value, out, B, C, H, W, K, s, dtype, st));
     return finish(e);
 }
 
@@ -265,7 +281,8 @@ static int fused_common(int attn_only, const void *query, const void *key, const
                                        nullptr, value, out, B, d, attn_only ? 0 : C, H, W, K, s,
                                        dtype, st);
     if (e == hipErrorNotSupported)
-        e = fused_pixel_launch(query, key, value, out, B, d, C, H, W, K, s, attn_only, dtype, st);
+        e = took("fused_pixel_kernel",
+                 fused_pixel_launch(query, key, value, out, B, d, C, H, W, K, s, attn_only, dtype, st));
     if (e == hipErrorNotSupported) return SAPA_ERR_UNSUPPORTED;
     return finish(e);
 }
@@ -295,12 +312,13 @@ static int nhwc_common(int mode, const void *query, const void *key, const void 
 #ifdef SAPA_NHWC16_OFF
     hipError_t e = hipErrorNotSupported;
 #else
-    hipError_t e = sapa_b_nhwc16_launch(mode, query, key, attn, value, q_bias, out, B, d, C, H, W, K, s,
-                                        dtype, (hipStream_t)stream);
+    hipError_t e = took("sapa_b_nhwc16_kernel",
+                        sapa_b_nhwc16_launch(mode, query, key, attn, value, q_bias, out, B, d, C, H, W, K, s,
+                                             dtype, (hipStream_t)stream));
 #endif
     if (e == hipErrorNotSupported)
-        e = sapa_b_nhwc_launch(mode, query, key, attn, value, q_bias, out, B, d, C, H, W, K, s, dtype,
-                               (hipStream_t)stream);
+        e = took("sapa_b_nhwc_kernel", sapa_b_nhwc_launch(mode, query, key, attn, value, q_bias, out, B, d, C,
+                                                          H, W, K, s, dtype, (hipStream_t)stream));
     if (e == hipErrorNotSupported) return SAPA_ERR_UNSUPPORTED;
     return finish(e);
 }
@@ -400,8 +418,9 @@ int sapa_deform_fused_forward_nhwc(const void *query, const void *key, const voi
     if (rc != SAPA_OK) return rc;
     if (B == 0) return SAPA_OK;
     if (!query || !key || !value || !offset || !out) return SAPA_ERR_INVALID_ARGUMENT;
-    const hipError_t e = deform_fused_nhwc_launch(query, key, value, offset, out, B, Cq, C, H, W, P,
-                                                  s, G, dtype, (hipStream_t)stream);
+    const hipError_t e =
+        took("deform_fused_nhwc_kernel", deform_fused_nhwc_launch(query, key, value, offset, out, B, Cq, C, H, W,
+                                                                  P, s, G, dtype, (hipStream_t)stream));
     if (e == hipErrorNotSupported) return SAPA_ERR_UNSUPPORTED;
     return finish(e);
 }

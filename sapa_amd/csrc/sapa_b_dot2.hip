@@ -3,19 +3,18 @@
 // the fused qk -> softmax -> av forward.
 //
 // With 16-bit operands one dot2 instruction does two multiply-adds into an fp32
-// accumulator:
-//   logits:  over a PAIR OF CHANNELS   a[j][k] += key[c][k]*q[c][j] + key[c+1][k]*q[c+1][j]
-//   output:  over a PAIR OF NEIGHBOURS o[j] += v[k]*w[j][k] + v[k+1]*w[j][k+1]
-// (k, k+1 adjacent in a window row; a row of K = 5 neighbours is 3 pairs, one
-// of them padded with a zero weight), i.e. 50 + 60 instructions per channel
-// and parent instead of the 100 + 100 fp32 FMAs of sapa_b_tiled.hip, and half
-// the LDS words.  On gfx950 a dot2 issues at half the rate of an fp32 FMA
-// (measured: 4 against 2 cycles per wave and SIMD with enough waves), so the
-// multiplier time of the logits halves and that of the aggregation does not
-// shrink; what the aggregation gains is LDS traffic and instruction issue
-// slots.  Products of 16-bit values are exact in fp32 and the sums stay in
-// fp32; the softmax weights are rounded to the tensors' 16-bit type before the
-// aggregation.
+// accumulator; the logits run on it over a PAIR OF CHANNELS
+//   a[j][k] += key[c][k]*q[c][j] + key[c+1][k]*q[c+1][j]
+// i.e. 50 instructions per channel and parent instead of the 100 fp32 FMAs of
+// sapa_b_tiled.hip, and half the LDS words.  On gfx950 a dot2 issues at half
+// the rate of an fp32 FMA (measured: 4 against 2 cycles per wave and SIMD with
+// enough waves), so the multiplier time of the logits halves.  The aggregation
+// keeps the softmax weights in fp32: each 16-bit value is widened (one byte
+// permute) and multiplied with fp32 FMAs, 25 + 100 instructions per channel
+// and parent at full rate -- the same issue time as 60 half-rate dot2 on
+// weight pairs rounded to 16 bits, without that rounding.  Products of a
+// 16-bit value and an fp32 weight and all sums are fp32; only the inputs and
+// the result are 16-bit.
 //
 // Work decomposition as in sapa_b_tiled.hip: a thread owns one low-res parent
 // with its 2 x 2 children, a wave 32 x 2 parents, a workgroup NWX x NWY waves.
@@ -25,8 +24,8 @@
 //   value chunk: CHV = 16 channels, each window row as it lies in memory, one
 //                word = (v[2i], v[2i+1]).  A parent whose first tap falls on an
 //                even window column reads the words (t0,t1) (t2,t3) (t4,-);
-//                one on an odd column reads (-,t0) (t1,t2) (t3,t4) and pairs
-//                its weights the other way, so neither needs a shifted copy.
+//                one on an odd column reads (-,t0) (t1,t2) (t3,t4); a per-lane
+//                byte selector picks the taps, so neither needs a shifted copy.
 // Window positions outside the image and channels past the last one are
 // fetched through a buffer descriptor sized to the remaining channels of the
 // chunk: the hardware returns zeros for them, which is the zero padding the
@@ -308,22 +307,25 @@ sapa_b_dot2_kernel(const T *__restrict__ q, const T *__restrict__ key,
     }
 
     if (DO_AV) {
-        // weights as 16-bit pairs of row neighbours, matched to the words this
-        // parent reads: first tap on an even window column -> (t0,t1) (t2,t3)
-        // (t4,-); on an odd one -> (-,t0) (t1,t2) (t3,t4)
+        // The weights stay fp32 (only the tensors are 16-bit): every tap's value is
+        // widened to fp32 and multiplied with plain FMAs.  The words this parent
+        // reads hold its row of taps as (t0,t1) (t2,t3) (t4,-) when its first tap
+        // falls on an even window column and as (-,t0) (t1,t2) (t3,t4) on an odd
+        // one; one byte permute with a per-lane selector picks tap k out of the
+        // word pair (k / 2, (k + 1) / 2) either way and, for bf16, already is the
+        // widening (the 16 bits land in the upper half of a zero word).
         const bool odd = wcol & 1;
-        u32 wp[NJ][NPK];
-#pragma unroll
-        for (int jj = 0; jj < NJ; ++jj)
-#pragma unroll
-            for (int ky = 0; ky < K; ++ky)
-#pragma unroll
-                for (int p = 0; p < KP; ++p) {
-                    const float *w = a[jj] + ky * K;
-                    const float e0 = w[2 * p], e1 = 2 * p + 1 < K ? w[2 * p + 1] : 0.f;
-                    const float o0 = p > 0 ? w[2 * p - 1] : 0.f, o1 = 2 * p < K ? w[2 * p] : 0.f;
-                    wp[jj][ky * KP + p] = pack2<T>(odd ? o0 : e0, odd ? o1 : e1);
-                }
+        constexpr bool BF = sizeof(T) == 2 && !__is_same(T, f16_t);
+        // bytes 0-3 = first word, 4-7 = second word, 0x0c = zero
+        constexpr u32 LO1 = BF ? 0x01000c0cu : 0x0c0c0100u, HI1 = BF ? 0x03020c0cu : 0x0c0c0302u,
+                      LO2 = BF ? 0x05040c0cu : 0x0c0c0504u;
+        const u32 sel_even = odd ? HI1 : LO1;      // taps 0, 2, 4: one word, either half
+        const u32 sel_odd = odd ? LO2 : HI1;       // taps 1, 3: end of one word or start of the next
+        auto tap_value = [&](u32 w_first, u32 w_second, u32 sel) {
+            const u32 r = __builtin_amdgcn_perm(w_second, w_first, sel);
+            if (BF) return __builtin_bit_cast(float, r);
+            return (float)__builtin_bit_cast(_Float16, (unsigned short)r);
+        };
         const u32 *vbase = lds + ly * RSV + wcol / 2;
         T *op = out + (long)n * C * hplane + hpix;
         auto load_v = [&](const u32 *wc, u32 (&dst)[NPK]) {
@@ -337,9 +339,14 @@ sapa_b_dot2_kernel(const T *__restrict__ q, const T *__restrict__ key,
 #pragma unroll
             for (int jj = 0; jj < NJ; ++jj) o[jj] = 0;
 #pragma unroll
-            for (int t = 0; t < NPK; ++t)
+            for (int ky = 0; ky < K; ++ky)
 #pragma unroll
-                for (int jj = 0; jj < NJ; ++jj) o[jj] = Dot<T>::run(vv[t], wp[jj][t], o[jj]);
+                for (int kx = 0; kx < K; ++kx) {
+                    const float v = tap_value(vv[ky * KP + kx / 2], vv[ky * KP + (kx + 1) / 2],
+                                              kx % 2 ? sel_odd : sel_even);
+#pragma unroll
+                    for (int jj = 0; jj < NJ; ++jj) o[jj] = fma_(v, a[jj][ky * K + kx], o[jj]);
+                }
             if (active && c < cend) {
 #pragma unroll
                 for (int cy = 0; cy < S; ++cy)

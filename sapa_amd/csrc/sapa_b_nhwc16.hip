@@ -33,9 +33,10 @@
 // quads 4 channel blocks) then fall on disjoint banks.
 //
 // Numerics: products of 16-bit values are exact in fp32; the sums run in the
-// matrix pipe's order and, in the fused mode, the softmax weights are rounded
-// to the 16-bit type before the aggregation -- as they are when qk, softmax
-// and av run as separate operators on 16-bit tensors.
+// matrix pipe's order.  In the fused mode the softmax weights enter the
+// aggregation as hi + lo pairs of 16-bit numbers (two instructions per B
+// operand), i.e. with fp32-like precision: only the inputs and the result are
+// 16-bit.  av() on its own takes the 16-bit weights it is given.
 #include <utility>
 
 #include "kernels.hpp"
@@ -345,8 +346,13 @@ sapa_b_nhwc16_kernel(const T *__restrict__ q, const T *__restrict__ key,
     }
 
     if (DO_AV) {
-        // the weights of taps 4 (4 gi + k) + bq, k = 0..3, as one A operand
-        u32x2 wpk[NG][NGRP];
+        // the weights of taps 4 (4 gi + k) + bq, k = 0..3, as one A operand.  Fused
+        // mode: the fp32 softmax weights go in as a sum of two 16-bit numbers,
+        // w = hi + lo with hi = T(w), lo = T(w - hi) (relative error 2^-16 for
+        // bf16, 2^-22 for fp16), each with its own matrix instruction on the same
+        // B operand, so the aggregation sees weights of fp32 quality.
+        constexpr bool SPLIT = MODE == TILED_FUSED;
+        u32x2 wpk[NG][NGRP], wlo[SPLIT ? NG : 1][SPLIT ? NGRP : 1];
 #pragma unroll
         for (int g = 0; g < NG; ++g)
 #pragma unroll
@@ -355,6 +361,13 @@ sapa_b_nhwc16_kernel(const T *__restrict__ q, const T *__restrict__ key,
 #pragma unroll
                 for (int k = 0; k < 4; ++k) x[k] = 4 * gi + k < NTAU ? w[g * NTAU + 4 * gi + k] : 0.f;
                 wpk[g][gi] = u32x2{pack2<T>(x[0], x[1]), pack2<T>(x[2], x[3])};
+                if constexpr (SPLIT) {
+                    typedef T tx4 __attribute__((ext_vector_type(4)));
+                    const tx4 hi = __builtin_bit_cast(tx4, wpk[g][gi]);
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) x[k] -= (float)hi[k];
+                    wlo[g][gi] = u32x2{pack2<T>(x[0], x[1]), pack2<T>(x[2], x[3])};
+                }
             }
 #pragma unroll
         for (int p = 0; p < NPASS; ++p)
@@ -391,8 +404,11 @@ sapa_b_nhwc16_kernel(const T *__restrict__ q, const T *__restrict__ key,
 #pragma unroll
                     for (int g = 0; g < NG; ++g)
 #pragma unroll
-                        for (int u = 0; u < 4; ++u)
+                        for (int u = 0; u < 4; ++u) {
                             acc[g][u] = M::template run<2, bsel>(wpk[g][gi], bop[u], acc[g][u]);
+                            if constexpr (SPLIT)
+                                acc[g][u] = M::template run<2, bsel>(wlo[g][gi], bop[u], acc[g][u]);
+                        }
                 }
             });
             // The next chunk goes to LDS BEFORE the results are stored: a wait for

@@ -46,6 +46,7 @@ def test_abi_version_and_status_strings():
         assert h.sapa_hip_status_string(code) not in (b'ok', b'unknown status')
     assert h.sapa_hip_status_string(-99) == b'unknown status'
     assert h.sapa_hip_last_hip_error() == b''
+    assert h.sapa_hip_last_kernel() == b''
 
 
 def test_argument_validation_returns_codes():

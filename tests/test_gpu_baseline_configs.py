@@ -1,0 +1,332 @@
+"""GPU: every benchmark configuration at its own parameters.
+
+  c2  SegFormer-style chain  B8  C256 d32  K5 s2  16^2 -> 32^2 -> 64^2 -> 128^2,
+      query / key from the module's 1x1 projections (normal_(std=.02))
+  c3  FPN levels             B16 C256 d64  K5 s2  25x42, 50x84, 100x168 -> x2,
+      keys scaled per channel ~U(0.5, 2); fp32 and bf16
+  c4  SAPA-D                 B8  C256 d32 G4  64^2 -> 128^2, P in {25, 9, 5},
+      offsets clamp(0.75 randn, +-4); with a sigmoid gate on the logits
+  c5  stress                 B4  C512 d64  K7 s4  64^2 -> 256^2, bf16, 10 % of
+      the query elements Student-t(3)
+
+One or two full-resolution images are compared with the C oracle (the
+reference kernels' arithmetic, qk_cuda_kernel.cu:39-67, av_cuda_kernel.cu:37-74,
+deform_*_cuda_kernel.cu:139-197, composed as sapa_base.py:38-40 /
+sapa_deform.py:51-53); the full batch goes through properties a wrong tile,
+channel slice or batch stride breaks: the batch result equals the per-image
+results bit for bit, a zero query gives the box filter, integer-valued inputs
+give exact logits and sums.  Contiguous and channels_last tensors both.
+
+Bars: fp32 |a-b| <= 1e-6 + 1e-5 |b| against the reference-order ('f32')
+oracle; bf16 |a-b| <= 1e-2 max(|b|, rms(b)) against the oracle with double
+sums on the bf16-rounded inputs.  The channels_last fp32 kernel sums the
+channels of a logit in tree order, not the reference's sequential order: its
+bar is that it is no further from the exact (double) result than the
+reference order is: RMS error, number of elements outside the fp32 bar and
+largest error (assert_no_worse_than_reference_order).
+"""
+from concurrent.futures import ThreadPoolExecutor
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import sapa_amd
+from helpers import BF16_REL, F32_ATOL, F32_RTOL, assert_f32_close, assert_rel_rms_close, gen, randn
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda:0'
+CL = torch.channels_last
+
+
+def dev(*ts):
+    return [t.to(DEV) for t in ts]
+
+
+def as_cl(*ts):
+    return [t.contiguous(memory_format=CL) for t in ts]
+
+
+def per_image(fn, tensors, *args, images=None):
+    """fn on single images in host threads (the C oracle is single-threaded and
+    ctypes releases the GIL), concatenated."""
+    idx = list(range(tensors[0].shape[0])) if images is None else list(images)
+    with ThreadPoolExecutor(max_workers=min(8, len(idx))) as ex:
+        outs = list(ex.map(lambda i: fn(*[t[i:i + 1].contiguous() for t in tensors], *args), idx))
+    return torch.cat(outs)
+
+
+def assert_batch_equals_images(fn, tensors, what, images=None):
+    """fn(batch)[i] == fn(image i), bit for bit."""
+    full = fn(*tensors)
+    B = tensors[0].shape[0]
+    for i in (range(B) if images is None else images):
+        one = fn(*[t[i:i + 1] for t in tensors])
+        assert torch.equal(full[i:i + 1], one), f'{what}: image {i} differs between batch and single call'
+    return full
+
+
+def assert_no_worse_than_reference_order(got, ref32, exact, what):
+    """`got` (fp32 sums in another order) against the exact (double) result,
+    next to the reference-order fp32 result `ref32` against the same: its RMS
+    error is not larger, no more of its elements lie outside the fp32 bar
+    1e-6 + 1e-5 |b|, and its largest error is not larger (the maximum over 1e7
+    elements of two independent rounding errors is a noisy statistic: 25 %
+    slack on that one)."""
+    got, ref32, exact = got.double().cpu(), ref32.double().cpu(), exact.double().cpu()
+    e_got, e_ref = (got - exact).abs(), (ref32 - exact).abs()
+    bar = F32_ATOL + F32_RTOL * exact.abs()
+    st = dict(rms=e_got.square().mean().sqrt().item(), rms_ref=e_ref.square().mean().sqrt().item(),
+              max=e_got.max().item(), max_ref=e_ref.max().item(),
+              outside=int((e_got > bar).sum()), outside_ref=int((e_ref > bar).sum()), n=exact.numel())
+    print(what, ' '.join(f'{k}={v:.3e}' if isinstance(v, float) else f'{k}={v}' for k, v in st.items()))
+    assert st['rms'] <= st['rms_ref'], f"{what}: rms error {st['rms']:.3e} > reference order {st['rms_ref']:.3e}"
+    assert st['outside'] <= st['outside_ref'], \
+        f"{what}: {st['outside']} elements outside the fp32 bar, reference order {st['outside_ref']}"
+    assert st['max'] <= 1.25 * st['max_ref'], \
+        f"{what}: max error {st['max']:.3e} > 1.25 x reference order {st['max_ref']:.3e}"
+    return st
+
+
+# ---------------------------------------------------------------- c3: FPN levels
+
+C3_LEVELS = [(25, 42), (50, 84), (100, 168)]
+
+
+def c3_inputs(B, H, W, seed):
+    g = gen(seed)
+    scale = torch.rand(64, generator=g) * 1.5 + 0.5
+    q = randn(g, B, 64, 2 * H, 2 * W)
+    key = randn(g, B, 64, H, W) * scale[None, :, None, None]
+    v = randn(g, B, 256, H, W)
+    return q, key, v
+
+
+@pytest.mark.parametrize('H,W', C3_LEVELS)
+def test_c3_fpn_fp32_against_oracle(coracle, H, W):
+    q, key, v = c3_inputs(2, H, W, 300 + H)
+    ref32 = per_image(coracle.sapa_fused, (q, key, v), 5, 2, 'f32')
+    exact = per_image(coracle.sapa_fused, (q, key, v), 5, 2, 'f32a64')
+    got = sapa_amd.sapa_fused(*dev(q, key, v), 5, 2).cpu()
+    assert_f32_close(got, ref32, f'c3 {H}x{W} fp32 contiguous')
+    got_cl = sapa_amd.sapa_fused(*as_cl(*dev(q, key, v)), 5, 2)
+    assert got_cl.is_contiguous(memory_format=CL)
+    assert_no_worse_than_reference_order(got_cl, ref32, exact, f'c3 {H}x{W} fp32 channels_last')
+    # the separate operators at this shape: reference arithmetic bit for bit
+    logits = sapa_amd.qk(*dev(q[:1], key[:1]), 5, 2)
+    assert torch.equal(logits.cpu(), coracle.qk(q[:1], key[:1], 5, 2, 'f32'))
+    attn = torch.softmax(logits, 1)
+    assert torch.equal(sapa_amd.av(attn, v[:1].to(DEV), 5, 2).cpu(), coracle.av(attn.cpu(), v[:1], 5, 2, 'f32'))
+
+
+@pytest.mark.parametrize('dtype,rel', [(torch.bfloat16, BF16_REL), (torch.float16, 2e-3)])
+@pytest.mark.parametrize('H,W', C3_LEVELS)
+def test_c3_fpn_16bit_against_oracle(coracle, H, W, dtype, rel):
+    """Inputs rounded to the 16-bit type, the oracle with double sums on those
+    values: the kernels keep every intermediate in fp32, so only the rounding of
+    the result (at most 2^-8 relative for bf16) is left of the bar."""
+    q, key, v = (t.to(dtype) for t in c3_inputs(2, H, W, 300 + H))
+    exact = per_image(coracle.sapa_fused, (q.float(), key.float(), v.float()), 5, 2, 'f32a64')
+    got = sapa_amd.sapa_fused(*dev(q, key, v), 5, 2)
+    assert got.dtype == dtype
+    assert_rel_rms_close(got.float(), exact, rel, f'c3 {H}x{W} {dtype} contiguous')
+    got_cl = sapa_amd.sapa_fused(*as_cl(*dev(q, key, v)), 5, 2)
+    assert got_cl.is_contiguous(memory_format=CL)
+    assert_rel_rms_close(got_cl.float(), exact, rel, f'c3 {H}x{W} {dtype} channels_last')
+    # the rounding of the result is all that is left: at most half the 16-bit
+    # spacing at the exact value (2^-8 resp. 2^-11 of it) plus fp32 noise
+    half_ulp = 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
+    for name, o in (('contiguous', got), ('channels_last', got_cl)):
+        err = (o.float().cpu().double() - exact).abs()
+        rms = exact.square().mean().sqrt()
+        worst = (err / torch.maximum(exact.abs(), rms)).max().item()
+        assert worst <= 1.05 * half_ulp, f'c3 {H}x{W} {dtype} {name}: {worst / half_ulp:.2f} half-ulps'
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('layout', ['contiguous', 'channels_last'])
+def test_c3_full_batch_properties(layout, dtype):
+    """B = 16 at the largest level."""
+    H, W = 100, 168
+    q, key, v = (t.to(dtype) for t in c3_inputs(16, H, W, 333))
+    conv = (lambda *ts: as_cl(*dev(*ts))) if layout == 'channels_last' else dev
+    qd, kd, vd = conv(q, key, v)
+    fused = lambda a, b, c: sapa_amd.sapa_fused(a, b, c, 5, 2)
+    out = assert_batch_equals_images(fused, (qd, kd, vd), f'c3 fused {layout} {dtype}', images=(0, 7, 15))
+    assert torch.isfinite(out).all()
+    # zero query: uniform weights, the result is the 5x5 box filter of the value
+    # (zero padding counted in the mean), nearest-upsampled
+    box = F.interpolate(F.avg_pool2d(vd.float().contiguous(), 5, 1, 2, count_include_pad=True), scale_factor=2)
+    got0 = fused(torch.zeros_like(qd), kd, vd).float()
+    if dtype == torch.float32:
+        assert_f32_close(got0, box, f'c3 box filter {layout}')
+    else:
+        assert_rel_rms_close(got0, box, BF16_REL, f'c3 box filter {layout} bf16')
+
+
+@pytest.mark.parametrize('layout', ['contiguous', 'channels_last'])
+def test_c3_full_batch_integer_inputs_exact(layout):
+    """Integer-valued tensors make every product and sum exact in fp32 whatever
+    the order: qk and av over the whole batch equal the unfold + einsum
+    restatement (sapa/sapa/forward_check.py:9-24) bit for bit."""
+    B, H, W, K, s = 16, 100, 168, 5, 2
+    g = gen(334)
+    ri = lambda *shape: torch.randint(-3, 4, shape, generator=g).float()
+    q, key, v = ri(B, 64, s * H, s * W), ri(B, 64, H, W), ri(B, 256, H, W)
+    attn = torch.randint(0, 3, (B, K * K, s * H, s * W), generator=g).float()
+    conv = (lambda *ts: as_cl(*dev(*ts))) if layout == 'channels_last' else dev
+    qd, kd, vd, ad = conv(q, key, v, attn)
+    logits = sapa_amd.qk(qd, kd, K, s)
+    out = sapa_amd.av(ad, vd, K, s)
+    for i in range(0, B, 4):    # the restatement in slices of 4 images (unfold of v: 1.7 GB each)
+        sl = slice(i, i + 4)
+        ku = F.unfold(kd[sl].contiguous(), K, padding=K // 2).view(4, 64, K * K, H, W)
+        want = torch.einsum('bckhw,bchiwj->bkhiwj', ku, qd[sl].contiguous().view(4, 64, H, s, W, s))
+        assert torch.equal(logits[sl].contiguous(), want.reshape(4, K * K, s * H, s * W))
+        vu = F.unfold(vd[sl].contiguous(), K, padding=K // 2).view(4, 256, K * K, H, W)
+        want = torch.einsum('bckhw,bkhiwj->bchiwj', vu, ad[sl].contiguous().view(4, K * K, H, s, W, s))
+        assert torch.equal(out[sl].contiguous(), want.reshape(4, 256, s * H, s * W))
+
+
+# ---------------------------------------------------------------- c2: SegFormer-style chain
+
+def test_c2_segformer_chain_module_and_operators(coracle):
+    """Three stages 16^2 -> 32^2 -> 64^2 -> 128^2; each stage's output is the next
+    stage's low-res feature; SAPA(256, embedding_dim=32) with GroupNorm(32) and
+    1x1 projections ~N(0, .02) (sapa_base.py:17-22,42-46)."""
+    B = 8
+    torch.manual_seed(2)
+    g = gen(200)
+    stages = [sapa_amd.SAPA(256, embedding_dim=32).to(DEV) for _ in range(3)]
+    x = randn(g, B, 256, 16, 16).to(DEV)
+    with torch.no_grad():
+        for m, h in zip(stages, (16, 32, 64)):
+            y = randn(g, B, 256, 2 * h, 2 * h).to(DEV)
+            out = m(y, x)
+            assert out.shape == (B, 256, 2 * h, 2 * h)
+            q, k = m.q(m.norm_y(y)), m.k(m.norm_x(x))
+            # raw operators, fused and the reference's three steps (sapa_base.py:38-40)
+            fused = lambda a, b, c: sapa_amd.sapa_fused(a, b, c, 5, 2)
+            raw = assert_batch_equals_images(fused, (q, k, x), f'c2 {h} fused')
+            assert torch.equal(raw, out)
+            three = sapa_amd.av(F.softmax(sapa_amd.qk(q, k, 5, 2), dim=1), x, 5, 2)
+            want = per_image(coracle.sapa_fused, (q.cpu(), k.cpu(), x.cpu()), 5, 2, 'f32', images=(0, B - 1))
+            for got, name in ((out, 'module'), (three, 'three-step')):
+                assert_f32_close(got[[0, B - 1]].cpu(), want, f'c2 {h}->{2 * h} {name}')
+            # the module's other forward routes on the same features
+            m.fold_norm = True
+            torch.testing.assert_close(m(y, x), out, rtol=1e-4, atol=1e-5)
+            m.fold_norm, m.channels_last = False, True
+            out_cl = m(*as_cl(y, x))
+            assert out_cl.is_contiguous(memory_format=CL)
+            torch.testing.assert_close(out_cl.contiguous(), out, rtol=1e-4, atol=1e-5)
+            m.channels_last = False
+            # channels_last operator on the same projections: within the fp32 bar of the oracle
+            got_cl = sapa_amd.sapa_fused(*as_cl(q, k, x), 5, 2)
+            assert_f32_close(got_cl[[0, B - 1]].cpu(), want, f'c2 {h}->{2 * h} channels_last')
+            x = out
+
+
+# ---------------------------------------------------------------- c4: SAPA-D
+
+def c4_inputs(B, P, seed, G=4):
+    g = gen(seed)
+    q = randn(g, B, 128, 128, 128)
+    key = randn(g, B, 128, 64, 64)
+    v = randn(g, B, 256, 64, 64)
+    off = (0.75 * randn(g, B, 2 * G * P, 128, 128)).clamp(-4, 4)
+    gate = torch.sigmoid(randn(g, B, 1, 1, 128, 128))
+    return q, key, v, off, gate
+
+
+@pytest.mark.parametrize('P', [25, 9, 5])
+def test_c4_deform_against_oracle(coracle, P):
+    """B = 8, G = 4, d = 32 per group, C = 256, 64^2 -> 128^2.  The sigmoid gate
+    of the benchmark description has no counterpart in sapa_deform.py: it is
+    input conditioning, applied to the logits in the same way on both sides
+    (separate operators); the fused operator is compared without it."""
+    B, s, G = 8, 2, 4
+    q, key, v, off, gate = c4_inputs(B, P, 400 + P)
+    qd, kd, vd, od, gd = dev(q, key, v, off, gate)
+    imgs = (0, B - 1)
+    sub = lambda *ts: [t[list(imgs)] for t in ts]
+    # separate operators: bit for bit the reference arithmetic
+    logits = sapa_amd.deform_qk(qd, kd, od, P, s, G)
+    want_logits = per_image(coracle.deform_qk, sub(q, key, off), P, s, G, 'f32')
+    assert torch.equal(logits[list(imgs)].cpu(), want_logits)
+    attn = torch.softmax(logits * gd, dim=2)
+    want_attn = torch.softmax(want_logits * gate[list(imgs)], dim=2)
+    torch.testing.assert_close(attn[list(imgs)].cpu(), want_attn, rtol=1e-5, atol=1e-7)
+    out = sapa_amd.deform_av(attn, vd, od, P, s, G)
+    want = per_image(coracle.deform_av, [attn[list(imgs)].cpu()] + sub(v, off), P, s, G, 'f32')
+    assert torch.equal(out[list(imgs)].cpu(), want)
+    # fused, both memory orders
+    fused = lambda a, b, c, o: sapa_amd.deform_sapa_fused(a, b, c, o, P, s, G)
+    got = assert_batch_equals_images(fused, (qd, kd, vd, od), f'c4 P={P} fused', images=(0, 3, B - 1))
+    want_f = per_image(coracle.deform_sapa_fused, sub(q, key, v, off), P, s, G, 'f32')
+    assert_f32_close(got[list(imgs)].cpu(), want_f, f'c4 P={P} fused')
+    got_cl = assert_batch_equals_images(fused, as_cl(qd, kd, vd, od), f'c4 P={P} fused channels_last',
+                                        images=(0, 3, B - 1))
+    exact = per_image(coracle.deform_sapa_fused, [t.double() for t in sub(q, key, v, off)], P, s, G, 'f64')
+    assert_no_worse_than_reference_order(got_cl[list(imgs)], want_f, exact, f'c4 P={P} fused channels_last')
+    # 16-bit tensors, contiguous and channels_last
+    hq, hk, hv, ho = (t.to(torch.bfloat16) for t in (qd, kd, vd, od))
+    exact16 = per_image(coracle.deform_sapa_fused, [t[list(imgs)].double().cpu() for t in (hq, hk, hv, ho)],
+                        P, s, G, 'f64')
+    assert_rel_rms_close(fused(hq, hk, hv, ho)[list(imgs)].float(), exact16, BF16_REL, f'c4 P={P} bf16')
+    assert_rel_rms_close(fused(*as_cl(hq, hk, hv, ho))[list(imgs)].float(), exact16, BF16_REL,
+                         f'c4 P={P} bf16 channels_last')
+
+
+def test_c4_regular_grid_offsets_reduce_to_sapa_b():
+    """P = 25 regular-grid integer offsets, G = 1: SAPA-D is SAPA-B with K = 5,
+    at the full c4 extent (cross-check between the two operator families)."""
+    B, d, C, H, W, K, s = 8, 32, 256, 64, 64, 5, 2
+    g = gen(440)
+    q, key, v = randn(g, B, d, s * H, s * W), randn(g, B, d, H, W), randn(g, B, C, H, W)
+    off = torch.empty(B, 2 * K * K, s * H, s * W)
+    for ky in range(K):
+        for kx in range(K):
+            off[:, 2 * (ky * K + kx)] = kx - K // 2         # width offset first
+            off[:, 2 * (ky * K + kx) + 1] = ky - K // 2
+    qd, kd, vd, od = dev(q, key, v, off)
+    assert torch.equal(sapa_amd.deform_qk(qd, kd, od, K * K, s, 1).squeeze(1), sapa_amd.qk(qd, kd, K, s))
+    want = sapa_amd.sapa_fused(qd, kd, vd, K, s)
+    assert_f32_close(sapa_amd.deform_sapa_fused(qd, kd, vd, od, K * K, s, 1), want, 'regular grid, contiguous')
+    exact = sapa_amd.sapa_fused(qd.double(), kd.double(), vd.double(), K, s)
+    assert_no_worse_than_reference_order(sapa_amd.deform_sapa_fused(*as_cl(qd, kd, vd, od), K * K, s, 1), want,
+                                         exact, 'regular grid, channels_last')
+
+
+# ---------------------------------------------------------------- c5: stress
+
+def c5_inputs(B, seed):
+    g = gen(seed)
+    q = randn(g, B, 64, 256, 256)
+    heavy = torch.rand(q.shape, generator=g) < 0.1
+    # Student-t(3) = normal / sqrt(chi2_3 / 3), drawn from the seeded generator
+    t3 = randn(g, *q.shape) / (randn(g, 3, *q.shape).square().sum(0) / 3).sqrt()
+    q = torch.where(heavy, t3, q)
+    key = randn(g, B, 64, 64, 64)
+    v = randn(g, B, 512, 64, 64)
+    return q, key, v
+
+
+def test_c5_stress_bf16_against_oracle(coracle):
+    """B = 4, C = 512, d = 64, K = 7, s = 4, 64^2 -> 256^2, bf16, heavy-tailed query."""
+    B, K, s = 4, 7, 4
+    q, key, v = (t.to(torch.bfloat16) for t in c5_inputs(B, 500))
+    qd, kd, vd = dev(q, key, v)
+    fused = lambda a, b, c: sapa_amd.sapa_fused(a, b, c, K, s)
+    got = assert_batch_equals_images(fused, (qd, kd, vd), 'c5 contiguous')
+    got_cl = assert_batch_equals_images(fused, as_cl(qd, kd, vd), 'c5 channels_last')
+    exact = per_image(coracle.sapa_fused, (q.float(), key.float(), v.float()), K, s, 'f32a64', images=(0, B - 1))
+    assert_rel_rms_close(got[[0, B - 1]].float(), exact, BF16_REL, 'c5 bf16 contiguous')
+    assert_rel_rms_close(got_cl[[0, B - 1]].float(), exact, BF16_REL, 'c5 bf16 channels_last')
+    # fp32 at the same extent, one image: the reference-order bar
+    q32, k32, v32 = q[:1].float(), key[:1].float(), v[:1].float()
+    want = coracle.sapa_fused(q32, k32, v32, K, s, 'f32')
+    assert_f32_close(sapa_amd.sapa_fused(*dev(q32, k32, v32), K, s).cpu(), want, 'c5 fp32 contiguous')
+    exact1 = exact[:1]
+    assert_no_worse_than_reference_order(sapa_amd.sapa_fused(*as_cl(*dev(q32, k32, v32)), K, s), want, exact1,
+                                         'c5 fp32 channels_last')
