@@ -23,11 +23,12 @@ HIPCC = os.environ.get('HIPCC', '/opt/rocm/bin/hipcc')
 FLAGS = ['-O3', '-std=c++17', '--offload-arch=gfx950', '-fPIC', '-fno-gpu-rdc',
          '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
          '-Wall', '-Wno-unused-function']
-# sapa_b_nhwc / sapa_b_nhwc16 keep their MFMA accumulators in ordinary VGPRs: left to itself the
+# sapa_b_nhwc / sapa_b_nhwc16 / sapa_d_nhwc keep their MFMA accumulators in ordinary VGPRs: left to itself the
 # compiler moves them to the accumulation registers on top of an already full
 # VGPR budget, which costs the kernels a wave per SIMD
 SOURCE_FLAGS = {'sapa_b_nhwc.hip': ['-mllvm', '-amdgpu-mfma-vgpr-form'],
-                'sapa_b_nhwc16.hip': ['-mllvm', '-amdgpu-mfma-vgpr-form']}
+                'sapa_b_nhwc16.hip': ['-mllvm', '-amdgpu-mfma-vgpr-form'],
+                'sapa_d_nhwc.hip': ['-mllvm', '-amdgpu-mfma-vgpr-form']}
 
 
 def _compile(src, extra):

@@ -74,6 +74,21 @@ __device__ __forceinline__ void store_stream(T *p, const Vec<T, N> &v) {
     __builtin_nontemporal_store(u.b, (B *)p);
 }
 
+// The same streaming store through a buffer descriptor: byte offset `off`
+// from the descriptor's base, dropped by the hardware when off + size exceeds
+// the descriptor's extent.
+template <typename T, int N>
+__device__ __forceinline__ void store_buffer(__amdgpu_buffer_rsrc_t r, unsigned off, const Vec<T, N> &v) {
+    typedef typename Bits<sizeof(T) * N>::type B;
+    union { B b; Vec<T, N> v; } u;
+    u.v = v;
+    constexpr int NT_HINT = 2;      // non-temporal
+    if constexpr (sizeof(B) == 2) __builtin_amdgcn_raw_buffer_store_b16(u.b, r, off, 0, NT_HINT);
+    else if constexpr (sizeof(B) == 4) __builtin_amdgcn_raw_buffer_store_b32(u.b, r, off, 0, NT_HINT);
+    else if constexpr (sizeof(B) == 8) __builtin_amdgcn_raw_buffer_store_b64(u.b, r, off, 0, NT_HINT);
+    else __builtin_amdgcn_raw_buffer_store_b128(u.b, r, off, 0, NT_HINT);
+}
+
 #ifndef SAPA_TILED_WPE
 #define SAPA_TILED_WPE 3
 #endif
@@ -351,38 +366,48 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
     }
 
     if (DO_AV) {
-        T *op = out + (long)n * C * hplane + hpix;
+        // The results leave through buffer stores whose descriptor covers exactly
+        // the channels of the chunk that exist: idle lanes (offset 2^31) and
+        // channels past the slice fall outside it and the hardware drops them.
+        // That keeps the channel loop free of branches, so it can be unrolled with
+        // a known number of stores behind the next chunk's staging loads: the wait
+        // for those loads then leaves this chunk's stores in flight (the counter
+        // retires in issue order) instead of draining them at every chunk.
+        const unsigned ooff = active ? (unsigned)(hpix * (long)sizeof(T)) : 0x80000000u;
+        const unsigned plane_bytes = (unsigned)(hplane * (long)sizeof(T));
         for (int j = nKc; j < ntot; ++j) {
             if (j + 1 < ntot) stage_load(j + 1);
             const int c0 = cbeg + (j - nKc) * CH;
             const A *wb = win + (j & 1) * BUF;
-#pragma unroll 1
+            const int nleft = cend - c0 < CH ? cend - c0 : CH;
+            const __amdgpu_buffer_rsrc_t orsrc = __builtin_amdgcn_make_buffer_rsrc(
+                (void *)(out + ((long)n * C + c0) * hplane), 0, (int)((unsigned)nleft * plane_bytes), 0x00020000);
+#pragma unroll
             for (int ch = 0; ch < CH; ++ch) {
-                {
-                    const int c = c0 + ch;
-                    const A *wc = wb + (ch >> 1) * WH * STRIDE + (ch & 1) * HALF;
-                    A o[NJ];
+                const A *wc = wb + (ch >> 1) * WH * STRIDE + (ch & 1) * HALF;
+                A o[NJ];
 #pragma unroll
-                    for (int jj = 0; jj < NJ; ++jj) o[jj] = 0;
+                for (int jj = 0; jj < NJ; ++jj) o[jj] = 0;
 #pragma unroll
-                    for (int ky = 0; ky < K; ++ky)
+                for (int ky = 0; ky < K; ++ky)
 #pragma unroll
-                        for (int kx = 0; kx < K; ++kx) {
-                            const A vv = wc[ky * STRIDE + kx];
+                    for (int kx = 0; kx < K; ++kx) {
+                        const A vv = wc[ky * STRIDE + kx];
 #pragma unroll
-                            for (int jj = 0; jj < NJ; ++jj)
-                                o[jj] = fma_(vv, a[jj][ky * K + kx], o[jj]);
-                        }
-                    if (active && c < cend) {
-#pragma unroll
-                        for (int cy = 0; cy < CY; ++cy) {
-                            VecS v;
-#pragma unroll
-                            for (int cx = 0; cx < S; ++cx) v.v[cx] = (T)o[cy * S + cx];
-                            store_stream<T, S>(op + (long)c * hplane + (long)cy * hW, v);
-                        }
+                        for (int jj = 0; jj < NJ; ++jj)
+                            o[jj] = fma_(vv, a[jj][ky * K + kx], o[jj]);
                     }
+#pragma unroll
+                for (int cy = 0; cy < CY; ++cy) {
+                    VecS v;
+#pragma unroll
+                    for (int cx = 0; cx < S; ++cx) v.v[cx] = (T)o[cy * S + cx];
+                    store_buffer<T, S>(orsrc, ooff + (unsigned)ch * plane_bytes +
+                                                  (unsigned)(cy * hW) * (unsigned)sizeof(T), v);
                 }
+                // one channel at a time: keeps the next channel's window reads from
+                // being hoisted over this channel's FMAs (register pressure)
+                __builtin_amdgcn_sched_barrier(0);
             }
             if (j + 1 < ntot) stage_store(j + 1);
             __syncthreads();
@@ -416,6 +441,8 @@ static hipError_t launch_mode(int mode, const void *q, const void *key, const vo
     const int cper = ((C + cgroups - 1) / cgroups + CH - 1) / CH * CH;
     const long nb = (long)tiles_x * tiles_y * B * cgroups;
     if (nb > (1L << 30)) return hipErrorNotSupported;
+    // the output leaves through 32-bit byte offsets inside one chunk of CH planes
+    if ((long)CH * H * S * W * S * (long)sizeof(T) > (1L << 31)) return hipErrorNotSupported;
     const int per_xcd = (int)((nb + 7) / 8);
     const dim3 grid(per_xcd * 8), block(NT);
 #define SAPA_TM_CASE(M)                                                                       \

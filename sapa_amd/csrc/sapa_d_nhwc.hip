@@ -56,9 +56,9 @@ typedef u32 u32x4 __attribute__((ext_vector_type(4)));
 template <typename T> struct Quad;
 template <> struct Quad<float> {
     typedef f32x4 raw;
-    static __device__ __forceinline__ raw buffer_load(__amdgpu_buffer_rsrc_t r, u32 off) {
+    static __device__ __forceinline__ raw buffer_load(__amdgpu_buffer_rsrc_t r, u32 off, u32 soff = 0) {
         union { u32x4 u; f32x4 f; } x;
-        x.u = __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
+        x.u = __builtin_amdgcn_raw_buffer_load_b128(r, off, soff, 0);
         return x.f;
     }
     static __device__ __forceinline__ f32x4 widen(raw v) { return v; }
@@ -67,8 +67,8 @@ template <> struct Quad<float> {
 };
 template <typename H> struct Quad16 {
     typedef u32x2 raw;
-    static __device__ __forceinline__ raw buffer_load(__amdgpu_buffer_rsrc_t r, u32 off) {
-        return __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0);
+    static __device__ __forceinline__ raw buffer_load(__amdgpu_buffer_rsrc_t r, u32 off, u32 soff = 0) {
+        return __builtin_amdgcn_raw_buffer_load_b64(r, off, soff, 0);
     }
     static __device__ __forceinline__ f32x4 widen(raw v) {
         union { u32x2 u; H h[4]; } x;
@@ -459,6 +459,389 @@ static hipError_t launch_t(const void *q, const void *key, const void *value, co
     }
 }
 
+
+// ---------------------------------------------------------------------------
+// The same operator as two small matrix products per (tile, group).
+//
+// Every sample of a pixel lies within RCH cells of the pixel's parent (the
+// few that do not are handled apart), so all 4 P corners of a pixel fall on the
+// WW x WW window cells of its tile.  Writing the bilinear corner weights of a
+// pixel as a row over those cells turns both sampled products into dense ones
+// whose big operand -- the window -- is shared by all 16 pixels of the tile:
+//
+//   similarity  Sim[pixel][cell] = q[pixel] . key[cell]              (16 x KP x d)
+//   logits      l[pixel][p]      = sum_corners w_c * Sim[pixel][cell_c]   (gather)
+//   softmax over the P points of the pixel
+//   weights     Wm[pixel][cell] += att_p * w_c                            (scatter)
+//   output      out[pixel][ch]   = sum_cells Wm[pixel][cell] * value[cell][ch]
+//                                                                    (16 x KP x 64)
+//
+// Both products run on v_mfma_f32_16x16x4f32.  A window cell is read from LDS
+// once per 16-channel block and tile instead of once per sample and pixel,
+// which takes the LDS traffic of the gather formulation above -- what bounds
+// it -- down by more than an order of magnitude.  The sums run in another
+// order than the reference's (per cell instead of per point): results agree to
+// fp32 rounding.  All contributions to a row of Wm come from one wave, in
+// program order, so the result does not depend on scheduling.
+//
+// Thread views of the 256 threads: a row of 16 lanes per pixel for staging q
+// and storing the output (lane = 4 channels); the matrix instruction's
+// (lane % 16, lane / 16) operand layout; half a wave per pixel, one lane per
+// point, for the per-sample work.
+constexpr int TPW = 4;          // tile edge, hi-res pixels
+#ifndef SAPA_WMAT_SKIP
+#define SAPA_WMAT_SKIP 0
+#endif
+
+// max / sum of a value over the aligned group of N = 16 or 32 lanes a lane is in
+template <bool MAX, int N>
+__device__ __forceinline__ float reduce_lanes(float v) {
+    union { float f; int i; } x, y;
+    auto step = [&](int other) __attribute__((always_inline)) {
+        y.i = other;
+        x.f = MAX ? max_(x.f, y.f) : x.f + y.f;
+    };
+    x.f = v;
+    step(__builtin_amdgcn_mov_dpp(x.i, 0xB1, 0xf, 0xf, true));     // lane ^ 1 (quad_perm [1,0,3,2])
+    step(__builtin_amdgcn_mov_dpp(x.i, 0x4E, 0xf, 0xf, true));     // lane ^ 2 (quad_perm [2,3,0,1])
+    step(__builtin_amdgcn_mov_dpp(x.i, 0x141, 0xf, 0xf, true));    // the other quad of 8 (row_half_mirror)
+    step(__builtin_amdgcn_mov_dpp(x.i, 0x140, 0xf, 0xf, true));    // the other 8 of the row (row_mirror)
+    if (N == 32) step(__builtin_amdgcn_ds_swizzle(x.i, 0x401F));   // lane ^ 16
+    return x.f;
+}
+
+template <typename T, int S, int DP>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3)))
+deform_fused_wmat_kernel(const T *__restrict__ q, const T *__restrict__ key,
+                         const T *__restrict__ value, const T *__restrict__ offset,
+                         T *__restrict__ out, int Cq, int C, int H, int W, int P, int G,
+                         int tiles_x, int tiles_y, int nblocks, int per_xcd) {
+    constexpr int TPL = (TPW + S - 1) / S;                   // parents of a tile per axis
+    constexpr int WW = TPL + 2 * RCH + 1, NPOS = WW * WW;    // window cells
+    constexpr int KP = (NPOS + 15) / 16 * 16, NKB = KP / 16; // cells padded to blocks of 16
+    constexpr int CHK = 64;                                  // value channels per chunk
+    constexpr int VS = CHK + 4;     // row strides in floats: 4 mod 16, so that the four
+    constexpr int KS = DP + 4;      // k-quarters of a matrix operand read disjoint banks
+    constexpr int WS = KP + 4;
+    constexpr int NPX = TPW * TPW;                           // pixels of a tile
+    constexpr int NT = 256, NPASS = (NPOS * 16 + NT - 1) / NT;
+    constexpr float WSCALE = 1073741824.f;                   // 2^30: fixed-point scale of Wm
+    static_assert(NPX == 16 && WS >= VS && KS <= VS, "one block of 16 matrix rows; shared buffers");
+    typedef Quad<T> Q4;
+    typedef typename Q4::raw Raw;
+
+    // the key window [cell][KS] (similarity), then the value window [cell][VS]
+    __shared__ __attribute__((aligned(16))) float Xl[KP * VS];
+    __shared__ __attribute__((aligned(16))) float Sl[NPX * WS];    // Sim [pixel][cell]; later the output tile [pixel][VS]
+    __shared__ __attribute__((aligned(16))) float Wl[NPX * WS];    // Wm [pixel][cell], 2^30-scaled integers
+
+    const int logical = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
+    if (logical >= nblocks) return;
+    const int tx = logical % tiles_x;
+    const int ty = (logical / tiles_x) % tiles_y;
+    const int n = logical / (tiles_x * tiles_y);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int hH = H * S, hW = W * S;
+    const int y0 = ty * TPW, x0 = tx * TPW;                          // tile origin, hi-res
+    const int wy0 = y0 / S - RCH, wx0 = x0 / S - RCH;                // window origin, low-res cell
+    const long lpix = (long)H * W;
+    const int d = Cq / G, cg = C / G;
+    const int nVc = (cg + CHK - 1) / CHK;
+
+    // pixel i of the tile (row-major 4 x 4): inside the image?  its flat hi-res
+    // index, clamped for loads, and its parent
+    struct Pix { bool active; long hp; int ph, pw; };
+    auto pixel = [&](int i) __attribute__((always_inline)) {
+        const int qh = y0 + i / TPW, qw = x0 + i % TPW;
+        Pix r;
+        r.active = qh < hH && qw < hW;
+        const int ch = qh < hH ? qh : hH - 1, cw = qw < hW ? qw : hW - 1;
+        r.hp = (long)n * hH * hW + (long)ch * hW + cw;
+        r.ph = ch / S;
+        r.pw = cw / S;
+        return r;
+    };
+    // view 1: a row of 16 lanes per pixel (output stores, window staging)
+    const int srow = tid >> 4, sq = tid & 15;
+    const Pix spx = pixel(srow);
+    // view 2: matrix operands
+    const int mi = lane & 15, mk = lane >> 4;
+    const Pix mpx = pixel(mi);
+    // view 3: half a wave per pixel (two passes over the tile), a lane per point
+    const int half = tid >> 5, pl = tid & 31;
+    const Pix bpx[2] = {pixel(half), pixel(8 + half)};
+
+    // ---- window staging: pass p, thread t moves channel quad t % 16 of window
+    // cell p * 16 + t / 16.  Per-thread byte offsets of the key and the value
+    // tensor, fixed for the whole kernel; 2^31 = beyond every descriptor, i.e.
+    // zero fill: cells outside the image, the padding cells NPOS .. KP, channel
+    // quads past the group's channels.  A chunk's first channel travels as the
+    // instruction's scalar offset, so a load costs no address arithmetic.
+    static_assert(NPASS * (NT / 16) == KP, "the staging passes cover the padded window exactly");
+    const int cv0 = cg < CHK ? cg : CHK;                             // channels of a full value chunk
+    u32 koff[NPASS], voff[NPASS];
+#pragma unroll
+    for (int p = 0; p < NPASS; ++p) {
+        const int pos = p * (NT / 16) + tid / 16;
+        const int gy = wy0 + pos / WW, gx = wx0 + pos % WW;
+        const bool ok = pos < NPOS && gy >= 0 && gy < H && gx >= 0 && gx < W;
+        const int pix = gy * W + gx;
+        koff[p] = (ok && 4 * sq < d) ? (u32)(pix * Cq + 4 * sq) * (u32)sizeof(T) : 0x80000000u;
+        voff[p] = (ok && 4 * sq < cv0) ? (u32)(pix * C + 4 * sq) * (u32)sizeof(T) : 0x80000000u;
+    }
+    const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(key + (long)n * lpix * Cq), 0, (int)(lpix * Cq * (long)sizeof(T)), 0x00020000);
+    const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(value + (long)n * lpix * C), 0, (int)(lpix * C * (long)sizeof(T)), 0x00020000);
+    Raw st[NPASS];
+    auto stage_load = [&](bool is_key, int cbase, int cvalid) __attribute__((always_inline)) {
+        const u32 soff = (u32)cbase * (u32)sizeof(T);
+        if (is_key) {
+#pragma unroll
+            for (int p = 0; p < NPASS; ++p) st[p] = Q4::buffer_load(krsrc, koff[p], soff);
+        } else if (cvalid == cv0) {
+#pragma unroll
+            for (int p = 0; p < NPASS; ++p) st[p] = Q4::buffer_load(vrsrc, voff[p], soff);
+        } else {
+            // the ragged last chunk of a group
+#pragma unroll
+            for (int p = 0; p < NPASS; ++p)
+                st[p] = Q4::buffer_load(vrsrc, 4 * sq < cvalid ? voff[p] : 0x80000000u, soff);
+        }
+    };
+    // rows of `stride` floats; quads past `nquads` have no place in them
+    float *const xrow = Xl + 4 * sq;
+    auto stage_store = [&](int stride, int nquads) __attribute__((always_inline)) {
+        if (sq < nquads) {
+            float *dst = xrow + (tid / 16) * stride;
+#pragma unroll
+            for (int p = 0; p < NPASS; ++p) *(f32x4 *)(dst + p * (NT / 16) * stride) = Q4::widen(st[p]);
+        }
+    };
+    // q of pixel mi as the A operand: channels 16 s + 4 mk .. + 3 of the group, s < DP / 16
+    Raw qa[DP / 16];
+    auto load_q = [&](int g) __attribute__((always_inline)) {
+#pragma unroll
+        for (int s16 = 0; s16 < DP / 16; ++s16) {
+            qa[s16] = Raw{};
+            if (mpx.active && 16 * s16 + 4 * mk < d)
+                qa[s16] = *(const Raw *)(q + mpx.hp * Cq + g * d + 16 * s16 + 4 * mk);
+        }
+    };
+
+    stage_load(true, 0, d);
+    load_q(0);
+    for (int g = 0; g < G; ++g) {
+        // ---- (a) key window and an empty weight matrix
+        stage_store(KS, DP / 4);
+        for (int i = tid; i < NPX * WS / 4; i += NT) ((f32x4 *)Wl)[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        __syncthreads();
+        // the group's first value chunk and the offsets travel during the similarity
+        stage_load(false, g * cg, cg < CHK ? cg : CHK);
+        // per-sample work: P <= 16 -> a row of 16 lanes per pixel, one pass over
+        // the tile; else half a wave per pixel, two passes
+        const bool narrow = P <= 16;
+        f32x2 off2[2] = {f32x2{0.f, 0.f}, f32x2{0.f, 0.f}};
+        if (narrow) {
+            if (spx.active && sq < P)
+                off2[0] = Q4::load_pair(offset + spx.hp * (2L * G * P) + 2L * ((long)g * P + sq));
+        } else {
+#pragma unroll
+            for (int ps = 0; ps < 2; ++ps)
+                if (bpx[ps].active && pl < P)
+                    off2[ps] = Q4::load_pair(offset + bpx[ps].hp * (2L * G * P) + 2L * ((long)g * P + pl));
+        }
+
+        // ---- (b) Sim = q . key over the window: this wave's blocks of 16 cells
+        {
+            f32x4 a4[DP / 16];
+#pragma unroll
+            for (int s16 = 0; s16 < DP / 16; ++s16) a4[s16] = Q4::widen(qa[s16]);
+            for (int nb = wave; nb < NKB; nb += 4) {
+                if (SAPA_WMAT_SKIP & 2) break;
+                f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int s16 = 0; s16 < DP / 16; ++s16) {
+                    const f32x4 b4 = *(const f32x4 *)(Xl + (16 * nb + mi) * KS + 16 * s16 + 4 * mk);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[s16][r], b4[r], acc, 0, 0, 0);
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r) Sl[(4 * mk + r) * WS + 16 * nb + mi] = acc[r];
+            }
+        }
+        __syncthreads();
+
+        // ---- (c) per (pixel, point): logit from Sim, softmax over the points,
+        // attention-weighted corner weights into Wm
+        bool fb[2] = {false, false};        // the point passes the guard but leaves the window
+        float fatt[2], fkh[2], fkw[2];
+        // sample `pt` of pixel `pi` of the tile (its Pix record px); NL lanes per pixel
+        auto sample = [&](auto nl, int ps, int pi, const Pix &px, int pt) __attribute__((always_inline)) {
+            constexpr int NL = decltype(nl)::value;
+            const bool live = px.active && pt < P;
+            const float kw = (float)px.pw + off2[ps][0], kh = (float)px.ph + off2[ps][1];
+            const WinTap<float> t = win_tap<float>(kh, kw, H, W, wy0, wx0, WW, WW);
+            const bool in = live && t.inwin;
+            fb[ps] = live && t.guard && !t.inwin;
+            fkh[ps] = kh;
+            fkw[ps] = kw;
+            const int cell = in ? t.hl * WW + t.wl : 0;
+            float lg = 0.f;
+            if (in) {
+                const float *sp = Sl + pi * WS + cell;
+                lg = t.w1 * sp[0];
+                lg = fma_(t.w2, sp[1], lg);
+                lg = fma_(t.w3, sp[WW], lg);
+                lg = fma_(t.w4, sp[WW + 1], lg);
+            }
+            if (fb[ps]) {
+                // sampled straight from global memory (rare)
+                Tap<float> tp = {};
+                tap_setup(kh, kw, H, W, tp);
+                const T *kp = key + (long)n * lpix * Cq + g * d;
+                const T *qp = q + px.hp * Cq + g * d;
+                for (int c = 0; c < d; ++c) {
+                    const float v1 = tp.m1 ? (float)kp[(long)tp.i1 * Cq + c] : 0.f;
+                    const float v2 = tp.m2 ? (float)kp[(long)tp.i2 * Cq + c] : 0.f;
+                    const float v3 = tp.m3 ? (float)kp[(long)tp.i3 * Cq + c] : 0.f;
+                    const float v4 = tp.m4 ? (float)kp[(long)tp.i4 * Cq + c] : 0.f;
+                    float v = tp.w1 * v1;
+                    v = fma_(tp.w2, v2, v);
+                    v = fma_(tp.w3, v3, v);
+                    v = fma_(tp.w4, v4, v);
+                    lg = fma_(v, (float)qp[c], lg);
+                }
+            }
+            // softmax over the pixel's points = the lanes pt < P of its group of NL lanes
+            const float mx = reduce_lanes<true, NL>(pt < P ? lg : -__builtin_huge_valf());
+            const float e = pt < P ? exp_(lg - mx) : 0.f;
+            const float att = e * (1.f / reduce_lanes<false, NL>(e));
+            fatt[ps] = att;
+            if (in) {
+                // Wm holds 2^30-scaled integers: every entry and every row sum is at
+                // most 1, integer adds are exact in any order (the result does not
+                // depend on which lane the LDS serves first) and run at the rate of
+                // plain LDS writes, which float atomics do not; the rounding of a
+                // contribution, 2^-31, is below that of an fp32 weight near 1
+                u32 *wp = (u32 *)Wl + pi * WS + cell;
+                const float sc = att * WSCALE;
+                __hip_atomic_fetch_add(wp, (u32)__float2uint_rn(sc * t.w1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                __hip_atomic_fetch_add(wp + 1, (u32)__float2uint_rn(sc * t.w2), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                __hip_atomic_fetch_add(wp + WW, (u32)__float2uint_rn(sc * t.w3), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                __hip_atomic_fetch_add(wp + WW + 1, (u32)__float2uint_rn(sc * t.w4), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+        };
+        if (!(SAPA_WMAT_SKIP & 1)) {
+            if (narrow) {
+                sample(std::integral_constant<int, 16>{}, 0, srow, spx, sq);
+            } else {
+                sample(std::integral_constant<int, 32>{}, 0, half, bpx[0], pl);
+                sample(std::integral_constant<int, 32>{}, 1, 8 + half, bpx[1], pl);
+            }
+        }
+        // ---- (d) value chunks: out tile = Wm . value window (the key window is done with)
+        stage_store(VS, 16);
+        const bool any_fb = __syncthreads_or(fb[0] || fb[1]);
+        for (int vc = 0; vc < nVc; ++vc) {
+            const int cbase = g * cg + vc * CHK;
+            const int cvalid = cg - vc * CHK < CHK ? cg - vc * CHK : CHK;
+            // next in line: the group's next value chunk, or the next group's key and q
+            if (vc + 1 < nVc) {
+                const int left = cg - (vc + 1) * CHK;
+                stage_load(false, cbase + CHK, left < CHK ? left : CHK);
+            } else if (g + 1 < G) {
+                stage_load(true, (g + 1) * d, d);
+                load_q(g + 1);
+            }
+            if (16 * wave < cvalid && !(SAPA_WMAT_SKIP & 2)) {
+                // two accumulators: consecutive instructions do not wait for each other
+                f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int s16 = 0; s16 < NKB; ++s16) {
+                    const u32x4 ai = *(const u32x4 *)(Wl + mi * WS + 16 * s16 + 4 * mk);
+                    const f32x4 a4 = {(float)ai[0] * (1.f / WSCALE), (float)ai[1] * (1.f / WSCALE),
+                                      (float)ai[2] * (1.f / WSCALE), (float)ai[3] * (1.f / WSCALE)};
+                    const float *vp = Xl + (16 * s16 + 4 * mk) * VS + 16 * wave + mi;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        if (r % 2 == 0) acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[r], vp[r * VS], acc0, 0, 0, 0);
+                        else acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[r], vp[r * VS], acc1, 0, 0, 0);
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r) Sl[(4 * mk + r) * VS + 16 * wave + mi] = acc0[r] + acc1[r];
+            }
+            __syncthreads();
+            if (any_fb) {
+                // points outside the window add their sample to the tile (rare)
+#pragma unroll
+                for (int ps = 0; ps < 2; ++ps) {
+                    if (!fb[ps]) continue;
+                    const int pi = narrow ? srow : ps * 8 + half;
+                    Tap<float> tp = {};
+                    tap_setup(fkh[ps], fkw[ps], H, W, tp);
+                    const T *vp = value + (long)n * lpix * C + cbase;
+                    for (int c = 0; c < cvalid; ++c) {
+                        const float v1 = tp.m1 ? (float)vp[(long)tp.i1 * C + c] : 0.f;
+                        const float v2 = tp.m2 ? (float)vp[(long)tp.i2 * C + c] : 0.f;
+                        const float v3 = tp.m3 ? (float)vp[(long)tp.i3 * C + c] : 0.f;
+                        const float v4 = tp.m4 ? (float)vp[(long)tp.i4 * C + c] : 0.f;
+                        float v = tp.w1 * v1;
+                        v = fma_(tp.w2, v2, v);
+                        v = fma_(tp.w3, v3, v);
+                        v = fma_(tp.w4, v4, v);
+                        __hip_atomic_fetch_add(Sl + pi * VS + c, fatt[ps] * v, __ATOMIC_RELAXED,
+                                               __HIP_MEMORY_SCOPE_WORKGROUP);
+                    }
+                }
+                __syncthreads();
+            }
+            // a row of 16 lanes stores its pixel's 64 channels: 256 contiguous bytes
+            if (spx.active && 4 * sq < cvalid && !(SAPA_WMAT_SKIP & 8))
+                __builtin_nontemporal_store(Q4::narrow(*(const f32x4 *)(Sl + srow * VS + 4 * sq)),
+                                            (Raw *)(out + spx.hp * C + cbase + 4 * sq));
+            if (vc + 1 < nVc) {
+                __syncthreads();        // everyone is done with this chunk's window and tile
+                stage_store(VS, 16);
+                __syncthreads();
+            }
+        }
+    }
+}
+
+template <typename T, int S, int DP>
+static hipError_t launch_wmat(const void *q, const void *key, const void *value, const void *offset,
+                              void *out, int B, int Cq, int C, int H, int W, int P, int G,
+                              hipStream_t st) {
+    const int tiles_x = (W * S + TPW - 1) / TPW, tiles_y = (H * S + TPW - 1) / TPW;
+    const long nb = (long)tiles_x * tiles_y * B;
+    if (nb > (1L << 30)) return hipErrorNotSupported;
+    const int per_xcd = (int)((nb + 7) / 8);
+    hipLaunchKernelGGL((deform_fused_wmat_kernel<T, S, DP>), dim3(per_xcd * 8), dim3(256), 0, st,
+                       (const T *)q, (const T *)key, (const T *)value, (const T *)offset, (T *)out,
+                       Cq, C, H, W, P, G, tiles_x, tiles_y, (int)nb, per_xcd);
+    return hipGetLastError();
+}
+
+template <typename T>
+static hipError_t launch_wmat_t(const void *q, const void *key, const void *value, const void *offset,
+                                void *out, int B, int Cq, int C, int H, int W, int P, int s, int G,
+                                hipStream_t st) {
+    const int d = Cq / G;
+#define SAPA_WMAT(SV)                                                                               \
+    case SV:                                                                                        \
+        return d <= 32 ? launch_wmat<T, SV, 32>(q, key, value, offset, out, B, Cq, C, H, W, P, G, st) \
+                       : launch_wmat<T, SV, 64>(q, key, value, offset, out, B, Cq, C, H, W, P, G, st);
+    switch (s) {
+        SAPA_WMAT(1) SAPA_WMAT(2) SAPA_WMAT(4)
+        default: return hipErrorNotSupported;
+    }
+#undef SAPA_WMAT
+}
+
 }  // namespace dnhwc
 
 // Channels-last tensors, f32 / f16 / bf16, s in {1, 2, 4}, P <= 32, channels per
@@ -478,12 +861,22 @@ hipError_t deform_fused_nhwc_launch(const void *q, const void *key, const void *
     for (const void *p : ptrs)
         if ((uintptr_t)p % (4 * esize) != 0) return hipErrorNotSupported;
     if ((uintptr_t)offset % (2 * esize) != 0) return hipErrorNotSupported;
+#ifdef SAPA_DNHWC_GATHER
+    // tuning build: the gather formulation (one row of lanes per pixel and group)
     switch (dtype) {
         case 0: return dnhwc::launch_t<float>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);
         case 2: return dnhwc::launch_t<f16_t>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);
         case 3: return dnhwc::launch_t<bf16_t>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);
         default: return hipErrorNotSupported;
     }
+#else
+    switch (dtype) {
+        case 0: return dnhwc::launch_wmat_t<float>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);
+        case 2: return dnhwc::launch_wmat_t<f16_t>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);
+        case 3: return dnhwc::launch_wmat_t<bf16_t>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);
+        default: return hipErrorNotSupported;
+    }
+#endif
 }
 
 }  // namespace sapa

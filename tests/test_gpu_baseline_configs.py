@@ -72,7 +72,7 @@ def assert_no_worse_than_reference_order(got, ref32, exact, what):
     error is not larger, no more of its elements lie outside the fp32 bar
     1e-6 + 1e-5 |b|, and its largest error is not larger (the maximum over 1e7
     elements of two independent rounding errors is a noisy statistic: 25 %
-    slack on that one)."""
+    slack on that one, 1 % on the other two)."""
     got, ref32, exact = got.double().cpu(), ref32.double().cpu(), exact.double().cpu()
     e_got, e_ref = (got - exact).abs(), (ref32 - exact).abs()
     bar = F32_ATOL + F32_RTOL * exact.abs()
@@ -80,8 +80,11 @@ def assert_no_worse_than_reference_order(got, ref32, exact, what):
               max=e_got.max().item(), max_ref=e_ref.max().item(),
               outside=int((e_got > bar).sum()), outside_ref=int((e_ref > bar).sum()), n=exact.numel())
     print(what, ' '.join(f'{k}={v:.3e}' if isinstance(v, float) else f'{k}={v}' for k, v in st.items()))
-    assert st['rms'] <= st['rms_ref'], f"{what}: rms error {st['rms']:.3e} > reference order {st['rms_ref']:.3e}"
-    assert st['outside'] <= st['outside_ref'], \
+    # (1 % slack on the two averages: where both orders are equally good -- SAPA-D,
+    # whose error is the fp32 rounding of the sample coordinates in either order --
+    # they differ by sampling noise only)
+    assert st['rms'] <= 1.01 * st['rms_ref'], f"{what}: rms error {st['rms']:.3e} > reference order {st['rms_ref']:.3e}"
+    assert st['outside'] <= 1.01 * st['outside_ref'] + 10, \
         f"{what}: {st['outside']} elements outside the fp32 bar, reference order {st['outside_ref']}"
     assert st['max'] <= 1.25 * st['max_ref'], \
         f"{what}: max error {st['max']:.3e} > 1.25 x reference order {st['max_ref']:.3e}"
