@@ -129,6 +129,26 @@ int sapa_av_backward_logits(const void *grad_out, const void *attn, const void *
                             void *grad_logits, int B, int C, int H, int W,
                             int K, int s, int dtype, void *stream);
 
+/* Backward of sapa_fused_forward in one call: the attention weights are
+ * recomputed (they are not kept by the forward pass), then
+ *   grad_value  = the aggregation's gradient for its low-res operand,
+ *   grad_logits = softmax backward of the aggregation's gradient for the weights,
+ *   grad_query, grad_key = the similarity's gradients for grad_logits,
+ * i.e. what autograd derives from SAPA.attention (sapa_base.py:38-40) through
+ * AVFunction.backward and QKFunction.backward (sapa/sapa/sapa_func.py:34-48,
+ * 79-93).  The two [B,K*K,sH,sW] intermediates live in `workspace` as fp32
+ * whatever `dtype` is (sapa_fused_backward_workspace bytes), so 16-bit tensors
+ * are read and written as they are while nothing between them is rounded to 16
+ * bits.  grad_query / grad_key / grad_value may each be NULL (not wanted); the
+ * others are fully overwritten.  SAPA_ERR_UNSUPPORTED when the LDS-tiled
+ * kernels do not cover the call (K other than 5, s other than 2, f64, unaligned
+ * tensors): compose the gradient from sapa_av_backward / sapa_qk_backward then. */
+long long sapa_fused_backward_workspace(int B, int H, int W, int K, int s);
+int sapa_fused_backward(const void *grad_out, const void *query, const void *key,
+                        const void *value, void *workspace, void *grad_query,
+                        void *grad_key, void *grad_value, int B, int d, int C,
+                        int H, int W, int K, int s, int dtype, void *stream);
+
 /* Softmax over the middle axis of x [N,R,M] -> y [N,R,M] (max-subtracted,
  * fp32 arithmetic for 16-bit types).  Covers the reference's
  * F.softmax(logits, dim=1) on [B,K*K,sH,sW] (sapa_base.py:39: N=B, R=K*K,

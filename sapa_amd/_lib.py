@@ -33,6 +33,7 @@ SIGNATURES = {
     'sapa_fused_forward': [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_qk_softmax_forward': [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_av_backward_logits': [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
+    'sapa_fused_backward': [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_qk_forward_nhwc': [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_qk_softmax_forward_nhwc': [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_av_forward_nhwc': [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
@@ -87,6 +88,8 @@ def lib():
             fn.argtypes = argtypes
         handle.sapa_channel_moments_workspace.restype = _ll
         handle.sapa_channel_moments_workspace.argtypes = [_i, _i, _ll, _i]
+        handle.sapa_fused_backward_workspace.restype = _ll
+        handle.sapa_fused_backward_workspace.argtypes = [_i, _i, _i, _i, _i]
         handle.sapa_channel_moments_static_capacity.restype = _ll
         handle.sapa_channel_moments_static_capacity.argtypes = []
         _lib = handle

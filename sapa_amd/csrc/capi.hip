@@ -259,6 +259,56 @@ int sapa_av_backward_logits(const void *grad_out, const void *attn, const void *
     return finish(e);
 }
 
+long long sapa_fused_backward_workspace(int B, int H, int W, int K, int s) {
+    if (B < 0 || H <= 0 || W <= 0 || K < 1 || s < 1) return 0;
+    return 2LL * B * K * K * H * s * W * s * (long long)sizeof(float);
+}
+
+int sapa_fused_backward(const void *grad_out, const void *query, const void *key, const void *value,
+                        void *workspace, void *grad_query, void *grad_key, void *grad_value, int B,
+                        int d, int C, int H, int W, int K, int s, int dtype, void *stream) {
+    const int rc = check_window_args(B, d, C, H, W, K, s, dtype);
+    if (rc != SAPA_OK) return rc;
+    if (dtype == SAPA_F64 || K != 5 || s != 2) return SAPA_ERR_UNSUPPORTED;
+    if (B == 0) return SAPA_OK;
+    if (!grad_out || !query || !key || !value || !workspace) return SAPA_ERR_INVALID_ARGUMENT;
+    hipStream_t st = (hipStream_t)stream;
+    float *attn = (float *)workspace;
+    float *grad_logits = attn + (long long)B * K * K * H * s * W * s;
+    // every stage on the LDS-tiled kernels with fp32 K*K tensors; a stage they do
+    // not cover ends the call before anything the caller keeps has been written
+    // by a later stage (the caller recomputes everything on its own path)
+#define SAPA_STAGE(call)                                                       \
+    do {                                                                       \
+        const hipError_t e_ = (call);                                          \
+        if (e_ == hipErrorNotSupported) return SAPA_ERR_UNSUPPORTED;           \
+        if (e_ != hipSuccess) return fail_hip(e_);                             \
+    } while (0)
+    // the similarity stages: the dot-product kernel where it applies (16-bit
+    // tensors), else the fp32-arithmetic one
+    auto similarity = [&](int mode, const void *qq, const void *kk, const void *attn_in, void *res, int ch) {
+        hipError_t e = sapa_b_dot2_launch(mode, qq, kk, attn_in, nullptr, res, B, ch, 0, H, W, K, s, dtype, st,
+                                          true);
+        if (e == hipErrorNotSupported)
+            e = sapa_b_tiled_launch(mode, qq, kk, attn_in, nullptr, res, B, ch, 0, H, W, K, s, dtype, st, true);
+        return e;
+    };
+    SAPA_STAGE(similarity(TILED_QK_SOFTMAX, query, key, nullptr, attn, d));
+    if (grad_value)
+        SAPA_STAGE(lowres_grad_tiled_launch(grad_out, attn, grad_value, B, C, H, W, K, s, dtype, st, true));
+    if (grad_query || grad_key) {
+        SAPA_STAGE(similarity(TILED_QK_SOFTMAX_BWD, grad_out, value, attn, grad_logits, C));
+        if (grad_query)
+            SAPA_STAGE(sapa_b_tiled_launch(TILED_AV, nullptr, nullptr, grad_logits, key, grad_query, B, 0,
+                                           d, H, W, K, s, dtype, st, true));
+        if (grad_key)
+            SAPA_STAGE(lowres_grad_tiled_launch(query, grad_logits, grad_key, B, d, H, W, K, s, dtype, st,
+                                                true));
+    }
+#undef SAPA_STAGE
+    return SAPA_OK;
+}
+
 int sapa_softmax_forward(const void *x, void *y, long long N, int R, long long M, int dtype,
                          void *stream) {
     if (!dtype_ok(dtype) || N < 0 || R < 1 || M < 0) return SAPA_ERR_INVALID_ARGUMENT;

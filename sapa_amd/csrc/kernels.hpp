@@ -26,10 +26,12 @@ hipError_t fused_pixel_launch(const void *q, const void *key, const void *value,
 enum TiledMode { TILED_QK = 0, TILED_QK_SOFTMAX = 1, TILED_AV = 2, TILED_FUSED = 3,
                  TILED_QK_SOFTMAX_BWD = 4 };
 // Returns hipErrorNotSupported when no tiled kernel covers (K, s, dtype, shape);
-// the caller then takes the generic path.
+// the caller then takes the generic path.  wide: the K*K-channel tensors of the
+// call (attn_in; the result of the modes without aggregation) are fp32 whatever
+// dtype is (modes TILED_QK_SOFTMAX, TILED_AV, TILED_QK_SOFTMAX_BWD only).
 hipError_t sapa_b_tiled_launch(int mode, const void *q, const void *key, const void *attn_in,
                                const void *value, void *out, int B, int d, int C, int H, int W,
-                               int K, int s, int dtype, hipStream_t st);
+                               int K, int s, int dtype, hipStream_t st, bool wide = false);
 
 // sapa_b_nhwc.hip: the four forward modes for tensors in channels-last memory
 // order ([B, H, W, channels]); f32 / f16 / bf16, (K, s) in {(3,2), (5,2), (7,2), (5,4), (7,4)}, channel
@@ -69,12 +71,13 @@ hipError_t deform_fused_nhwc_launch(const void *q, const void *key, const void *
                                     const void *offset, void *out, int B, int Cq, int C, int H,
                                     int W, int P, int s, int G, int dtype, hipStream_t st);
 
-// sapa_b_dot2.hip: the four forward modes for f16 / bf16 tensors on the
+// sapa_b_dot2.hip: qk, qk+softmax and fused for f16 / bf16 tensors on the
 // two-term dot-product instructions (K = 5, s = 2); hipErrorNotSupported
-// otherwise.
+// otherwise.  wide: fp32 K*K-channel tensors next to the 16-bit features
+// (TILED_QK_SOFTMAX, and TILED_QK_SOFTMAX_BWD, which exists in this form only).
 hipError_t sapa_b_dot2_launch(int mode, const void *q, const void *key, const void *attn_in,
                               const void *value, void *out, int B, int d, int C, int H, int W,
-                              int K, int s, int dtype, hipStream_t st);
+                              int K, int s, int dtype, hipStream_t st, bool wide = false);
 
 // sapa_b_mfma.hip: the same four modes on the matrix pipe (4x4x1 MFMA, one
 // block per parent); hipErrorNotSupported when (K, s, dtype) has no instance.
@@ -83,10 +86,11 @@ hipError_t sapa_b_mfma_launch(int mode, const void *q, const void *key, const vo
                               int K, int s, int dtype, hipStream_t st);
 
 // sapa_b_lowgrad.hip: grad_key / grad_value as an LDS-tiled gather (no
-// atomics, `out` fully overwritten).  hipErrorNotSupported unless fp32,
-// s = 2, K in {3, 5}.
+// atomics, `out` fully overwritten).  hipErrorNotSupported unless f32 / f16 /
+// bf16, s = 2, K in {3, 5}.  wide: the weight tensor w is fp32 whatever dtype is.
 hipError_t lowres_grad_tiled_launch(const void *hi, const void *w, void *out, int B, int C, int H,
-                                    int W, int K, int s, int dtype, hipStream_t st);
+                                    int W, int K, int s, int dtype, hipStream_t st,
+                                    bool wide = false);
 
 // sapa_d_lds.hip: the SAPA-D forward ops gathering from an LDS-resident
 // window; mode 0 = deform_qk (out = logits), 1 = deform_av (attn_in given),

@@ -84,7 +84,9 @@ __device__ __forceinline__ float hi_f(u32 w) {
     return (float)x.t[1];
 }
 
-template <typename T, int K, int NWX, int NWY, int MODE>
+// WIDE: the K*K-channel tensors of the call (the result of qk+softmax; attn_in
+// and the result of TILED_QK_SOFTMAX_BWD) are fp32 next to the 16-bit features
+template <typename T, int K, int NWX, int NWY, int MODE, bool WIDE = false>
 __global__ void __launch_bounds__(64 * NWX *NWY) __attribute__((amdgpu_waves_per_eu(3, 3)))
 sapa_b_dot2_kernel(const T *__restrict__ q, const T *__restrict__ key,
                    const T *__restrict__ attn_in, const T *__restrict__ value,
@@ -295,14 +297,52 @@ sapa_b_dot2_kernel(const T *__restrict__ q, const T *__restrict__ key,
 #pragma unroll
             for (int jj = 0; jj < NJ; ++jj) softmax_inplace<float, KK>(a[jj]);
         }
-        if (!DO_AV && active) {
-            T *op = out + (long)n * KK * hplane + hpix;
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        if (MODE == TILED_QK_SOFTMAX_BWD && active) {
+            // a[][] holds g = d(loss)/d(attn); with the fp32 weights in attn_in it
+            // becomes d(loss)/d(logits) = attn * (g - sum_k g * attn).  The weights
+            // are read twice (the second time from cache) rather than kept.
+            static_assert(MODE != TILED_QK_SOFTMAX_BWD || WIDE, "the weights of this mode are fp32");
+            const float *ap = reinterpret_cast<const float *>(attn_in) + (long)n * KK * hplane + hpix;
+            float dot[NJ];
+#pragma unroll
+            for (int jj = 0; jj < NJ; ++jj) dot[jj] = 0;
 #pragma unroll
             for (int k = 0; k < KK; ++k)
 #pragma unroll
-                for (int cy = 0; cy < S; ++cy)
-                    *(u32 *)(op + (long)k * hplane + (long)cy * hW) =
-                        pack2<T>(a[cy * S][k], a[cy * S + 1][k]);
+                for (int cy = 0; cy < S; ++cy) {
+                    const f32x2 v = *(const f32x2 *)(ap + (long)k * hplane + (long)cy * hW);
+#pragma unroll
+                    for (int cx = 0; cx < S; ++cx)
+                        dot[cy * S + cx] = fma_(a[cy * S + cx][k], v[cx], dot[cy * S + cx]);
+                }
+#pragma unroll
+            for (int k = 0; k < KK; ++k)
+#pragma unroll
+                for (int cy = 0; cy < S; ++cy) {
+                    const f32x2 v = *(const f32x2 *)(ap + (long)k * hplane + (long)cy * hW);
+#pragma unroll
+                    for (int cx = 0; cx < S; ++cx)
+                        a[cy * S + cx][k] = v[cx] * (a[cy * S + cx][k] - dot[cy * S + cx]);
+                }
+        }
+        if (!DO_AV && active) {
+            if (WIDE) {
+                float *op = reinterpret_cast<float *>(out) + (long)n * KK * hplane + hpix;
+#pragma unroll
+                for (int k = 0; k < KK; ++k)
+#pragma unroll
+                    for (int cy = 0; cy < S; ++cy)
+                        *(f32x2 *)(op + (long)k * hplane + (long)cy * hW) = f32x2{a[cy * S][k], a[cy * S + 1][k]};
+            } else {
+                T *op = out + (long)n * KK * hplane + hpix;
+#pragma unroll
+                for (int k = 0; k < KK; ++k)
+#pragma unroll
+                    for (int cy = 0; cy < S; ++cy)
+                        *(u32 *)(op + (long)k * hplane + (long)cy * hW) =
+                            pack2<T>(a[cy * S][k], a[cy * S + 1][k]);
+            }
         }
     }
 
@@ -378,7 +418,7 @@ sapa_b_dot2_kernel(const T *__restrict__ q, const T *__restrict__ key,
 }
 
 template <typename T, int K, int NWX, int NWY>
-static hipError_t launch_mode(int mode, const void *q, const void *key, const void *attn_in,
+static hipError_t launch_mode(int mode, bool wide, const void *q, const void *key, const void *attn_in,
                               const void *value, void *out, int B, int d, int C, int H, int W,
                               hipStream_t st) {
     constexpr int TW = 32 * NWX, TH = 2 * NWY, NT = 64 * NWX * NWY, CHV = 16;
@@ -394,18 +434,28 @@ static hipError_t launch_mode(int mode, const void *q, const void *key, const vo
     if (nb > (1L << 30)) return hipErrorNotSupported;
     const int per_xcd = (int)((nb + 7) / 8);
     const dim3 grid(per_xcd * 8), block(NT);
+#define SAPA_D2_LAUNCH(M, WD)                                                                  \
+    hipLaunchKernelGGL((sapa_b_dot2_kernel<T, K, NWX, NWY, M, WD>), grid, block, 0, st,        \
+                       (const T *)q, (const T *)key, (const T *)attn_in, (const T *)value,     \
+                       (T *)out, d, C, H, W, tiles_x, tiles_y, (int)nb, per_xcd, cgroups, cper)
 #define SAPA_D2_CASE(M)                                                                        \
     case M:                                                                                    \
-        hipLaunchKernelGGL((sapa_b_dot2_kernel<T, K, NWX, NWY, M>), grid, block, 0, st,        \
-                           (const T *)q, (const T *)key, (const T *)attn_in, (const T *)value, \
-                           (T *)out, d, C, H, W, tiles_x, tiles_y, (int)nb, per_xcd, cgroups,  \
-                           cper);                                                              \
+        SAPA_D2_LAUNCH(M, false);                                                              \
         break;
+    if (wide) {
+        switch (mode) {
+            case TILED_QK_SOFTMAX: SAPA_D2_LAUNCH(TILED_QK_SOFTMAX, true); break;
+            case TILED_QK_SOFTMAX_BWD: SAPA_D2_LAUNCH(TILED_QK_SOFTMAX_BWD, true); break;
+            default: return hipErrorNotSupported;
+        }
+        return hipGetLastError();
+    }
     switch (mode) {
         SAPA_D2_CASE(TILED_QK) SAPA_D2_CASE(TILED_QK_SOFTMAX) SAPA_D2_CASE(TILED_FUSED)
         default: return hipErrorNotSupported;
     }
 #undef SAPA_D2_CASE
+#undef SAPA_D2_LAUNCH
     return hipGetLastError();
 }
 
@@ -419,8 +469,9 @@ static hipError_t launch_mode(int mode, const void *q, const void *key, const vo
 // while the channel pairs of the logits have no such padding.
 hipError_t sapa_b_dot2_launch(int mode, const void *q, const void *key, const void *attn_in,
                               const void *value, void *out, int B, int d, int C, int H, int W,
-                              int K, int s, int dtype, hipStream_t st) {
+                              int K, int s, int dtype, hipStream_t st, bool wide) {
     if (mode == TILED_AV || K != 5 || s != 2 || W % 4 != 0 || W < 32) return hipErrorNotSupported;
+    if (mode == TILED_QK_SOFTMAX_BWD && !wide) return hipErrorNotSupported;
     // staging offsets are 32-bit byte offsets below 2^31 inside one image
     const long plane_bytes = (long)H * W * 2;
     if ((long)(d > C ? d : C) * plane_bytes >= (1L << 30)) return hipErrorNotSupported;
@@ -429,9 +480,11 @@ hipError_t sapa_b_dot2_launch(int mode, const void *q, const void *key, const vo
         if (p && (uintptr_t)p % 8 != 0) return hipErrorNotSupported;
     for (const void *p : hi_ptrs)
         if (p && (uintptr_t)p % 4 != 0) return hipErrorNotSupported;
+    // fp32 K*K tensors are accessed as pairs of floats
+    if (wide && (((uintptr_t)attn_in | (uintptr_t)out) % 8 != 0)) return hipErrorNotSupported;
     switch (dtype) {
-        case 2: return dot2::launch_mode<f16_t, 5, 1, 4>(mode, q, key, attn_in, value, out, B, d, C, H, W, st);
-        case 3: return dot2::launch_mode<bf16_t, 5, 1, 4>(mode, q, key, attn_in, value, out, B, d, C, H, W, st);
+        case 2: return dot2::launch_mode<f16_t, 5, 1, 4>(mode, wide, q, key, attn_in, value, out, B, d, C, H, W, st);
+        case 3: return dot2::launch_mode<bf16_t, 5, 1, 4>(mode, wide, q, key, attn_in, value, out, B, d, C, H, W, st);
         default: return hipErrorNotSupported;
     }
 }

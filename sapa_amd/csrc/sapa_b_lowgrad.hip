@@ -34,10 +34,24 @@ template <int N> struct FVec;
 template <> struct FVec<2> { typedef float type __attribute__((ext_vector_type(2))); };
 template <> struct FVec<4> { typedef float type __attribute__((ext_vector_type(4))); };
 
-template <int K, int S, int NWX, int NWY, int CH, int VEC>
+// N consecutive tensor elements as one load, widened to floats
+template <typename T, int N>
+__device__ __forceinline__ typename FVec<N>::type load_wide(const T *p) {
+    typedef T tvec __attribute__((ext_vector_type(N)));
+    const tvec v = *(const tvec *)p;
+    typename FVec<N>::type f;
+#pragma unroll
+    for (int i = 0; i < N; ++i) f[i] = (float)v[i];
+    return f;
+}
+
+// T = float, f16_t or bf16_t: the type of hi and out; WT: that of the weight
+// tensor (T, or float next to 16-bit features); the window in LDS, the weights
+// in registers and the sums are fp32 whatever they are
+template <typename T, typename WT, int K, int S, int NWX, int NWY, int CH, int VEC>
 __global__ void __launch_bounds__(64 * NWX *NWY) __attribute__((amdgpu_waves_per_eu(3, 3)))
-lowgrad_gather_kernel(const float *__restrict__ hi, const float *__restrict__ w,
-                      float *__restrict__ out, int C, int H, int W, int tiles_x, int tiles_y,
+lowgrad_gather_kernel(const T *__restrict__ hi, const WT *__restrict__ w,
+                      T *__restrict__ out, int C, int H, int W, int tiles_x, int tiles_y,
                       int nblocks, int per_xcd, int cgroups, int cper) {
     static_assert(S == 2, "children are read as 2-wide vectors");
     constexpr int TW = 16 * NWX, TH = 4 * NWY, NT = 64 * NWX * NWY;
@@ -73,7 +87,7 @@ lowgrad_gather_kernel(const float *__restrict__ hi, const float *__restrict__ w,
     // image contribute nothing
     float wr[KK][NJ];
     {
-        const float *wp = w + (long)n * KK * hplane;
+        const WT *wp = w + (long)n * KK * hplane;
 #pragma unroll
         for (int k = 0; k < KK; ++k) {
             const int py = y + R - k / K, px = x + R - k % K;
@@ -81,7 +95,7 @@ lowgrad_gather_kernel(const float *__restrict__ hi, const float *__restrict__ w,
             const long base = (long)k * hplane + (long)((ok ? py : 0) * S) * hW + (ok ? px : 0) * S;
 #pragma unroll
             for (int cy = 0; cy < S; ++cy) {
-                const V2 v = *(const V2 *)(wp + base + (long)cy * hW);
+                const V2 v = load_wide<WT, S>(wp + base + (long)cy * hW);
 #pragma unroll
                 for (int cx = 0; cx < S; ++cx) wr[k][cy * S + cx] = ok ? v[cx] : 0.f;
             }
@@ -90,7 +104,7 @@ lowgrad_gather_kernel(const float *__restrict__ hi, const float *__restrict__ w,
 
     // staging: element e of a chunk = (channel, window row, vector in the row)
     const int wy0 = (ty * TH - R) * S, wx0 = (tx * TW - R) * S;   // window origin, high-res
-    const float *hp = hi + (long)n * C * hplane;
+    const T *hp = hi + (long)n * C * hplane;
     V stage[NLD];
     unsigned okmask = 0;
     auto issue = [&](int c0) {
@@ -106,7 +120,7 @@ lowgrad_gather_kernel(const float *__restrict__ hi, const float *__restrict__ w,
             const bool ok =
                 e < CH * NV && c0 + ch < cend && gy >= 0 && gy < hH && gx >= 0 && gx < hW;
             const long off = ok ? (long)(c0 + ch) * hplane + (long)gy * hW + gx : 0;
-            stage[i] = *(const V *)(hp + off);
+            stage[i] = load_wide<T, VEC>(hp + off);
             okmask |= (unsigned)ok << i;
         }
     };
@@ -132,7 +146,7 @@ lowgrad_gather_kernel(const float *__restrict__ hi, const float *__restrict__ w,
     const float *base = win + (ly + 2 * R) * S * RS + (lx + 2 * R) * S;
     const bool live = x < W && y < H;
     const long lplane = (long)H * W;
-    float *op = out + (long)n * C * lplane + (long)(y < H ? y : 0) * W + (x < W ? x : 0);
+    T *op = out + (long)n * C * lplane + (long)(y < H ? y : 0) * W + (x < W ? x : 0);
     int parity = 0;
     for (int c0 = cbeg; c0 < cend; c0 += CH, parity ^= 1) {
         const bool more = c0 + CH < cend;
@@ -152,14 +166,14 @@ lowgrad_gather_kernel(const float *__restrict__ hi, const float *__restrict__ w,
                     acc[cy] = __builtin_fmaf(wr[k][cy * S], h[0], acc[cy]);
                     acc[cy] = __builtin_fmaf(wr[k][cy * S + 1], h[1], acc[cy]);
                 }
-            if (live && c0 + ch < cend) op[(long)(c0 + ch) * lplane] = acc[0] + acc[1];
+            if (live && c0 + ch < cend) op[(long)(c0 + ch) * lplane] = (T)(acc[0] + acc[1]);
         }
         if (more) commit(win + (parity ^ 1) * CH * PS);
         __syncthreads();
     }
 }
 
-template <int K, int S, int NWX, int NWY, int CH, int VEC>
+template <typename T, typename WT, int K, int S, int NWX, int NWY, int CH, int VEC>
 static hipError_t lowgrad_launch_geom(const void *hi, const void *w, void *out, int B, int C, int H, int W,
                        hipStream_t st) {
     constexpr int TW = 16 * NWX, TH = 4 * NWY, NT = 64 * NWX * NWY;
@@ -174,33 +188,49 @@ static hipError_t lowgrad_launch_geom(const void *hi, const void *w, void *out, 
     const long nb = tiles * cgroups;
     if (nb > (1L << 30)) return hipErrorNotSupported;
     const int per_xcd = (int)((nb + 7) / 8);
-    hipLaunchKernelGGL((lowgrad_gather_kernel<K, S, NWX, NWY, CH, VEC>), dim3(per_xcd * 8),
-                       dim3(NT), 0, st, (const float *)hi, (const float *)w, (float *)out, C, H, W,
+    hipLaunchKernelGGL((lowgrad_gather_kernel<T, WT, K, S, NWX, NWY, CH, VEC>), dim3(per_xcd * 8),
+                       dim3(NT), 0, st, (const T *)hi, (const WT *)w, (T *)out, C, H, W,
                        tiles_x, tiles_y, (int)nb, per_xcd, cgroups, cper);
     return hipGetLastError();
 }
 
-template <int K, int VEC>
+template <typename T, typename WT, int K, int VEC>
 static hipError_t lowgrad_launch_k(const void *hi, const void *w, void *out, int B, int C, int H, int W,
                     hipStream_t st) {
     const bool wide = (W + 31) / 32 * 32 * 0.9 <= (W + 15) / 16 * 16;
-    return wide ? lowgrad_launch_geom<K, 2, 2, 2, 2, VEC>(hi, w, out, B, C, H, W, st)
-                : lowgrad_launch_geom<K, 2, 1, 2, 2, VEC>(hi, w, out, B, C, H, W, st);
+    return wide ? lowgrad_launch_geom<T, WT, K, 2, 2, 2, 2, VEC>(hi, w, out, B, C, H, W, st)
+                : lowgrad_launch_geom<T, WT, K, 2, 1, 2, 2, VEC>(hi, w, out, B, C, H, W, st);
 }
 
-// fp32, (K, s) in {(3, 2), (5, 2)}, hi / w aligned to s elements;
+template <typename T, typename WT>
+static hipError_t lowgrad_launch_t(const void *hi, const void *w, void *out, int B, int C, int H, int W,
+                                   int K, hipStream_t st) {
+    // vector loads of s = 2 elements
+    if ((uintptr_t)hi % (2 * sizeof(T)) || (uintptr_t)w % (2 * sizeof(WT))) return hipErrorNotSupported;
+    if (K == 3) return lowgrad_launch_k<T, WT, 3, 2>(hi, w, out, B, C, H, W, st);
+    // 4-element staging loads when the rows of hi allow it (the window starts
+    // r * s = 4 pixels left of a tile, which keeps them aligned)
+    const bool v4 = (uintptr_t)hi % (4 * sizeof(T)) == 0 && W % 2 == 0;
+    return v4 ? lowgrad_launch_k<T, WT, 5, 4>(hi, w, out, B, C, H, W, st)
+              : lowgrad_launch_k<T, WT, 5, 2>(hi, w, out, B, C, H, W, st);
+}
+
+// f32 / f16 / bf16, (K, s) in {(3, 2), (5, 2)}, hi / w aligned to s elements;
 // hipErrorNotSupported otherwise (the caller then takes the generic kernel).
 // `out` is fully overwritten.
 hipError_t lowres_grad_tiled_launch(const void *hi, const void *w, void *out, int B, int C, int H,
-                                    int W, int K, int s, int dtype, hipStream_t st) {
-    if (dtype != 0 || s != 2 || (K != 3 && K != 5)) return hipErrorNotSupported;
-    if ((uintptr_t)hi % 8 || (uintptr_t)w % 8) return hipErrorNotSupported;
-    if (K == 3) return lowgrad_launch_k<3, 2>(hi, w, out, B, C, H, W, st);
-    // 16-byte staging loads when the rows of hi allow it (the window starts
-    // r * s = 4 pixels left of a tile, which keeps them aligned)
-    const bool v4 = (uintptr_t)hi % 16 == 0 && W % 2 == 0;
-    return v4 ? lowgrad_launch_k<5, 4>(hi, w, out, B, C, H, W, st)
-              : lowgrad_launch_k<5, 2>(hi, w, out, B, C, H, W, st);
+                                    int W, int K, int s, int dtype, hipStream_t st, bool wide) {
+    if (s != 2 || (K != 3 && K != 5)) return hipErrorNotSupported;
+    switch (dtype) {
+        case 0: return lowgrad_launch_t<float, float>(hi, w, out, B, C, H, W, K, st);
+        case 2:
+            return wide ? lowgrad_launch_t<f16_t, float>(hi, w, out, B, C, H, W, K, st)
+                        : lowgrad_launch_t<f16_t, f16_t>(hi, w, out, B, C, H, W, K, st);
+        case 3:
+            return wide ? lowgrad_launch_t<bf16_t, float>(hi, w, out, B, C, H, W, K, st)
+                        : lowgrad_launch_t<bf16_t, bf16_t>(hi, w, out, B, C, H, W, K, st);
+        default: return hipErrorNotSupported;
+    }
 }
 
 }  // namespace sapa

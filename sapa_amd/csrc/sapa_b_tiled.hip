@@ -32,6 +32,8 @@
 // leave a logit at exactly 0 (and that 0 takes part in the softmax) and add
 // exactly 0 to the aggregation, which is what the reference's `continue`
 // does.  16-bit tensors are widened to fp32 on the way into LDS/registers.
+#include <type_traits>
+
 #include "kernels.hpp"
 
 namespace sapa {
@@ -92,7 +94,10 @@ __device__ __forceinline__ void store_buffer(__amdgpu_buffer_rsrc_t r, unsigned 
 #ifndef SAPA_TILED_WPE
 #define SAPA_TILED_WPE 3
 #endif
-template <typename T, int K, int S, int CY, int NWX, int NWY, int CH, int VEC, int WLX, int MODE>
+// WIDE: the K*K-channel tensors of the call (attn_in; the result of the modes
+// without aggregation) are fp32 while the feature tensors are T -- the form the
+// backward pass of 16-bit tensors keeps its intermediates in
+template <typename T, int K, int S, int CY, int NWX, int NWY, int CH, int VEC, int WLX, int MODE, bool WIDE = false>
 __global__ void __launch_bounds__(64 * NWX * NWY * (S / CY)) __attribute__((amdgpu_waves_per_eu(SAPA_TILED_WPE, SAPA_TILED_WPE)))
 sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
                     const T *__restrict__ attn_in, const T *__restrict__ value,
@@ -133,6 +138,11 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
     static_assert(CH % 2 == 0, "channels are staged in pairs");
     static_assert(S % CY == 0, "CY must divide S");
     typedef Vec<T, S> VecS;
+    static_assert(!WIDE || MODE == TILED_AV || MODE == TILED_QK_SOFTMAX || MODE == TILED_QK_SOFTMAX_BWD,
+                  "fp32 K*K tensors: the modes the backward pass uses");
+    typedef typename std::conditional<WIDE, float, T>::type TA;   // type of the K*K-channel tensors
+    typedef Vec<TA, S> VecA;
+    const TA *attn_w = reinterpret_cast<const TA *>(attn_in);
 
     __shared__ __attribute__((aligned(16))) A lds[2 * BUF];
 
@@ -247,12 +257,12 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
 
     stage_load(0);
     if (MODE == TILED_AV && active) {
-        const T *ap = attn_in + (long)n * KK * hplane + hpix;
+        const TA *ap = attn_w + (long)n * KK * hplane + hpix;
 #pragma unroll
         for (int k = 0; k < KK; ++k)
 #pragma unroll
             for (int cy = 0; cy < CY; ++cy) {
-                const VecS v = *(const VecS *)(ap + (long)k * hplane + (long)cy * hW);
+                const VecA v = *(const VecA *)(ap + (long)k * hplane + (long)cy * hW);
 #pragma unroll
                 for (int cx = 0; cx < S; ++cx) a[cy * S + cx][k] = (A)v.v[cx];
             }
@@ -328,7 +338,7 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
             // a[][] holds g = d(loss)/d(attn); turn it into d(loss)/d(logits).
             // The weights are read twice (the second time from cache) rather
             // than kept in another K*K registers per child.
-            const T *ap = attn_in + (long)n * KK * hplane + hpix;
+            const TA *ap = attn_w + (long)n * KK * hplane + hpix;
             A dot[NJ];
 #pragma unroll
             for (int jj = 0; jj < NJ; ++jj) dot[jj] = 0;
@@ -336,7 +346,7 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
             for (int k = 0; k < KK; ++k)
 #pragma unroll
                 for (int cy = 0; cy < CY; ++cy) {
-                    const VecS v = *(const VecS *)(ap + (long)k * hplane + (long)cy * hW);
+                    const VecA v = *(const VecA *)(ap + (long)k * hplane + (long)cy * hW);
 #pragma unroll
                     for (int cx = 0; cx < S; ++cx)
                         dot[cy * S + cx] = fma_(a[cy * S + cx][k], (A)v.v[cx], dot[cy * S + cx]);
@@ -345,22 +355,22 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
             for (int k = 0; k < KK; ++k)
 #pragma unroll
                 for (int cy = 0; cy < CY; ++cy) {
-                    const VecS v = *(const VecS *)(ap + (long)k * hplane + (long)cy * hW);
+                    const VecA v = *(const VecA *)(ap + (long)k * hplane + (long)cy * hW);
 #pragma unroll
                     for (int cx = 0; cx < S; ++cx)
                         a[cy * S + cx][k] = (A)v.v[cx] * (a[cy * S + cx][k] - dot[cy * S + cx]);
                 }
         }
         if (!DO_AV && active) {
-            T *op = out + (long)n * KK * hplane + hpix;
+            TA *op = reinterpret_cast<TA *>(out) + (long)n * KK * hplane + hpix;
 #pragma unroll
             for (int k = 0; k < KK; ++k)
 #pragma unroll
                 for (int cy = 0; cy < CY; ++cy) {
-                    VecS v;
+                    VecA v;
 #pragma unroll
-                    for (int cx = 0; cx < S; ++cx) v.v[cx] = (T)a[cy * S + cx][k];
-                    *(VecS *)(op + (long)k * hplane + (long)cy * hW) = v;
+                    for (int cx = 0; cx < S; ++cx) v.v[cx] = (TA)a[cy * S + cx][k];
+                    *(VecA *)(op + (long)k * hplane + (long)cy * hW) = v;
                 }
         }
     }
@@ -417,7 +427,7 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
 
 // ------------------------------------------------------------------ launcher
 template <typename T, int K, int S, int CY, int NWX, int NWY, int CH, int VEC, int WLX>
-static hipError_t launch_mode(int mode, const void *q, const void *key, const void *attn_in,
+static hipError_t launch_mode(int mode, bool wide, const void *q, const void *key, const void *attn_in,
                               const void *value, void *out, int B, int d, int C, int H, int W,
                               hipStream_t st) {
     constexpr int TW = WLX * NWX, TH = (64 / WLX) * NWY, NT = 64 * NWX * NWY * (S / CY);
@@ -445,34 +455,50 @@ static hipError_t launch_mode(int mode, const void *q, const void *key, const vo
     if ((long)CH * H * S * W * S * (long)sizeof(T) > (1L << 31)) return hipErrorNotSupported;
     const int per_xcd = (int)((nb + 7) / 8);
     const dim3 grid(per_xcd * 8), block(NT);
+#define SAPA_TM_LAUNCH(M, WD)                                                                 \
+    hipLaunchKernelGGL((sapa_b_tiled_kernel<T, K, S, CY, NWX, NWY, CH, VEC, WLX, M, WD>), grid, block, 0, st, \
+                       (const T *)q, (const T *)key, (const T *)attn_in, (const T *)value,    \
+                       (T *)out, d, C, H, W, tiles_x, tiles_y, (int)nb, per_xcd, cgroups, cper)
 #define SAPA_TM_CASE(M)                                                                       \
     case M:                                                                                   \
-        hipLaunchKernelGGL((sapa_b_tiled_kernel<T, K, S, CY, NWX, NWY, CH, VEC, WLX, M>), grid, block, 0, st,    \
-                           (const T *)q, (const T *)key, (const T *)attn_in,                  \
-                           (const T *)value, (T *)out, d, C, H, W, tiles_x, tiles_y, (int)nb, \
-                           per_xcd, cgroups, cper);                                                          \
+        SAPA_TM_LAUNCH(M, false);                                                             \
         break;
+    if (wide) {
+        // fp32 K*K tensors next to 16-bit features (for fp32 features that is the plain form)
+        if constexpr (sizeof(T) == 2) {
+            switch (mode) {
+                case TILED_QK_SOFTMAX: SAPA_TM_LAUNCH(TILED_QK_SOFTMAX, true); break;
+                case TILED_AV: SAPA_TM_LAUNCH(TILED_AV, true); break;
+                case TILED_QK_SOFTMAX_BWD: SAPA_TM_LAUNCH(TILED_QK_SOFTMAX_BWD, true); break;
+                default: return hipErrorNotSupported;
+            }
+            return hipGetLastError();
+        }
+    }
     switch (mode) {
         SAPA_TM_CASE(TILED_QK) SAPA_TM_CASE(TILED_QK_SOFTMAX) SAPA_TM_CASE(TILED_AV)
         SAPA_TM_CASE(TILED_FUSED) SAPA_TM_CASE(TILED_QK_SOFTMAX_BWD)
         default: return hipErrorInvalidValue;
     }
+#undef SAPA_TM_LAUNCH
 #undef SAPA_TM_CASE
     return hipGetLastError();
 }
 
 template <typename T>
-static hipError_t launch_t(int mode, const void *q, const void *key, const void *attn_in,
+static hipError_t launch_t(int mode, bool wide, const void *q, const void *key, const void *attn_in,
                            const void *value, void *out, int B, int d, int C, int H, int W, int K,
                            int s, hipStream_t st) {
     // vector accesses of s elements on the high-res tensors
-    const uintptr_t align = (uintptr_t)(sizeof(T) * s);
+    const uintptr_t align = (uintptr_t)(sizeof(T) * s), walign = wide ? (uintptr_t)(4 * s) : align;
+    const bool out_is_kk = mode != TILED_AV && mode != TILED_FUSED;
     const void *hi_ptrs[3] = {q, attn_in, out};
+    const uintptr_t hi_align[3] = {align, walign, out_is_kk ? walign : align};
     for (int i = 0; i < 3; ++i)
-        if (hi_ptrs[i] && ((uintptr_t)hi_ptrs[i] % align) != 0) return hipErrorNotSupported;
+        if (hi_ptrs[i] && ((uintptr_t)hi_ptrs[i] % hi_align[i]) != 0) return hipErrorNotSupported;
     if (K == 5 && s == 2) {
 #ifdef SAPA_TUNE_GEOM
-        return launch_mode<T, 5, 2, SAPA_TUNE_GEOM>(mode, q, key, attn_in, value, out, B, d, C, H, W, st);
+        return launch_mode<T, 5, 2, SAPA_TUNE_GEOM>(mode, wide, q, key, attn_in, value, out, B, d, C, H, W, st);
 #else
         // Tile geometry: padded parent count times the relative cost per
         // parent measured at the FPN shapes on MI355X (wider tiles fetch
@@ -492,7 +518,7 @@ static hipError_t launch_t(int mode, const void *q, const void *key, const void 
                    (!value || (uintptr_t)value % a == 0);
         };
 #define SAPA_GEOM(NWX, NWY, VEC, WLX)                                                            \
-    launch_mode<T, 5, 2, 2, NWX, NWY, 8, VEC, WLX>(mode, q, key, attn_in, value, out, B, d, C, H, \
+    launch_mode<T, 5, 2, 2, NWX, NWY, 8, VEC, WLX>(mode, wide, q, key, attn_in, value, out, B, d, C, H, \
                                                    W, st)
         if (c22 <= c12 && c22 <= c14)
             return aligned(4) ? SAPA_GEOM(1, 4, 4, 32) : SAPA_GEOM(1, 4, 1, 32);
@@ -506,12 +532,12 @@ static hipError_t launch_t(int mode, const void *q, const void *key, const void 
 
 hipError_t sapa_b_tiled_launch(int mode, const void *q, const void *key, const void *attn_in,
                                const void *value, void *out, int B, int d, int C, int H, int W,
-                               int K, int s, int dtype, hipStream_t st) {
+                               int K, int s, int dtype, hipStream_t st, bool wide) {
     switch (dtype) {
-        case 0: return launch_t<float>(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, st);
+        case 0: return launch_t<float>(mode, wide, q, key, attn_in, value, out, B, d, C, H, W, K, s, st);
 #if !defined(SAPA_TUNE_GEOM) || defined(SAPA_TUNE_ALLTYPES)
-        case 2: return launch_t<f16_t>(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, st);
-        case 3: return launch_t<bf16_t>(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, st);
+        case 2: return launch_t<f16_t>(mode, wide, q, key, attn_in, value, out, B, d, C, H, W, K, s, st);
+        case 3: return launch_t<bf16_t>(mode, wide, q, key, attn_in, value, out, B, d, C, H, W, K, s, st);
 #endif
         default: return hipErrorNotSupported;
     }

@@ -16,21 +16,12 @@ def _check_odd_kernel(kernel_size):
     assert (kernel_size - 1) % 2 == 0 and kernel_size >= 1
 
 
-def _wide(*tensors):
-    # the tiled gradient kernels are fp32; 16-bit tensors take them and the
-    # gradients are rounded back
-    return [t.float() if t.dtype in (torch.float16, torch.bfloat16) else t for t in tensors]
-
-
 def _qk_backward(grad_output, query, key, kernel_size, scale_factor, need_q=True, need_k=True):
     # the gradient kernels take contiguous tensors: operands kept in
     # channels-last order are copied here (the forward pass is the zero-copy one)
+    # 16-bit tensors are read and written as they are (fp32 sums inside the
+    # kernels), as the reference's half dispatch does (qk_cuda_kernel.cu:139-171)
     query, key = query.contiguous(), key.contiguous()
-    if key.dtype in (torch.float16, torch.bfloat16):
-        gq, gk = _qk_backward(*_wide(grad_output, query, key), kernel_size, scale_factor,
-                              need_q, need_k)
-        return (None if gq is None else gq.to(query.dtype),
-                None if gk is None else gk.to(key.dtype))
     grad_output = grad_output.contiguous()
     grad_query = _lib.new_out(query) if need_q else None
     grad_key = _lib.new_out(key) if need_k else None
@@ -44,11 +35,6 @@ def _qk_backward(grad_output, query, key, kernel_size, scale_factor, need_q=True
 
 def _av_backward(grad_output, attn, value, kernel_size, scale_factor, need_a=True, need_v=True):
     attn, value = attn.contiguous(), value.contiguous()
-    if value.dtype in (torch.float16, torch.bfloat16):
-        ga, gv = _av_backward(*_wide(grad_output, attn, value), kernel_size, scale_factor,
-                              need_a, need_v)
-        return (None if ga is None else ga.to(attn.dtype),
-                None if gv is None else gv.to(value.dtype))
     grad_output = grad_output.contiguous()
     grad_attn = _lib.new_out(attn) if need_a else None
     grad_value = _lib.new_out(value) if need_v else None
@@ -189,11 +175,23 @@ def _fused_backward(grad_output, query, key, value, K, s, needs=(True, True, Tru
     are recomputed (one launch), then the three operators' gradients chain."""
     need_q, need_k, need_v = needs
     query, key, value = query.contiguous(), key.contiguous(), value.contiguous()
-    if value.dtype in (torch.float16, torch.bfloat16):
-        # the whole chain in fp32, one rounding at the end
-        grads = _fused_backward(*_wide(grad_output, query, key, value), K, s, needs)
-        return tuple(None if g is None else g.to(t.dtype)
-                     for g, t in zip(grads, (query, key, value)))
+    grad_output = grad_output.contiguous()
+    _lib.require_cuda_contiguous(grad_output=grad_output, query=query, key=key, value=value)
+    # the whole chain in one library call where the tiled kernels cover it: 16-bit
+    # tensors go in and out as they are, the [B,K*K,sH,sW] intermediates stay fp32
+    n, c, h, w = value.size()
+    d = key.size(1)
+    nbytes = _lib.lib().sapa_fused_backward_workspace(n, h, w, K, s)
+    ws = torch.empty(max(nbytes // 4, 1), dtype=torch.float32, device=value.device)
+    grads = [_lib.new_out(t) if need else None
+             for t, need in ((query, need_q), (key, need_k), (value, need_v))]
+    status = _lib.call_status('sapa_fused_backward', value.device, _lib.ptr(grad_output), _lib.ptr(query),
+                              _lib.ptr(key), _lib.ptr(value), _lib.ptr(ws), _lib.ptr(grads[0]),
+                              _lib.ptr(grads[1]), _lib.ptr(grads[2]), n, d, c, h, w, K, s,
+                              _lib.dtype_code(value))
+    if status != _lib.UNSUPPORTED:
+        return tuple(grads)
+    del ws, grads
     attn = _qk_softmax_forward(query, key, K, s)
     grad_query = grad_key = grad_logits = None
     if need_q or need_k:

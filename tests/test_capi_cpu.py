@@ -30,12 +30,14 @@ def test_library_exports_every_declared_symbol():
     # and the Python binding covers every operator entry point
     # (the workspace query returns a size, not a status: bound separately)
     ops = [n for n in names if not n.startswith('sapa_hip_')
-           and n not in ('sapa_channel_moments_workspace', 'sapa_channel_moments_static_capacity')]
+           and n not in ('sapa_channel_moments_workspace', 'sapa_channel_moments_static_capacity',
+                         'sapa_fused_backward_workspace')]
     assert sorted(ops) == sorted(_lib.SIGNATURES)
     h = _lib.lib()
     assert h.sapa_channel_moments_workspace(16, 256, 67200, 0) > 0
     assert h.sapa_channel_moments_workspace(0, 256, 67200, 1) == 0
     assert h.sapa_channel_moments_static_capacity() == 8 << 20
+    assert h.sapa_fused_backward_workspace(2, 10, 12, 5, 2) == 2 * 2 * 25 * 20 * 24 * 4
 
 
 def test_abi_version_and_status_strings():

@@ -310,6 +310,60 @@ def test_backward_16bit_tensors():
             assert_rel_rms_close(a.grad.float().cpu(), b.grad.cpu(), rel, str(dt))
 
 
+def _fused_backward_oracle(coracle, go, q, key, v, K, s):
+    """float64 chain of the reference's backward (sapa/sapa/sapa_func.py:34-48,79-93
+    under sapa_base.py:38-40): av backward, softmax backward, qk backward."""
+    q, key, v, go = (t.double() for t in (q, key, v, go))
+    attn = torch.softmax(coracle.qk(q, key, K, s, 'f64'), dim=1)
+    ga, gv = coracle.av_backward(go, attn, v, K, s, 'f64')
+    gl = attn * (ga - (ga * attn).sum(dim=1, keepdim=True))
+    gq, gk = coracle.qk_backward(gl, q, key, K, s, 'f64')
+    return gq, gk, gv
+
+
+@pytest.mark.parametrize('dtype,tol', [(torch.float32, dict(rtol=1e-4, atol=1e-5)),
+                                        (torch.bfloat16, 1.5e-2), (torch.float16, 2e-3)])
+def test_fused_backward_entry_point(coracle, dtype, tol):
+    """sapa_fused_backward through the C ABI: all three gradients against the
+    float64 oracle chain on the same (rounded) inputs, fp32 intermediates for
+    16-bit tensors (only the gradients themselves are rounded to 16 bits);
+    outputs that are not wanted are not touched; K = 3 is left to the caller."""
+    from sapa_amd import _lib
+    g = gen(170)
+    B, d, C, H, W, K, s = 2, 16, 24, 21, 36, 5, 2      # W % 4 == 0, W >= 32: the dot-product stages for 16-bit
+    q, key, v = (randn(g, *sh).to(dtype) for sh in ((B, d, H * s, W * s), (B, d, H, W), (B, C, H, W)))
+    go = randn(g, B, C, H * s, W * s).to(dtype)
+    qd, kd, vd, god = dev(q, key, v, go)
+    h = _lib.lib()
+    ws = torch.empty(h.sapa_fused_backward_workspace(B, H, W, K, s) // 4, device=DEV)
+    gq, gk, gv = (torch.full_like(t, float('nan')) for t in (qd, kd, vd))
+    args = (B, d, C, H, W, K, s, _lib.DTYPES[dtype])
+    assert _lib.call_status('sapa_fused_backward', DEV, _lib.ptr(god), _lib.ptr(qd), _lib.ptr(kd), _lib.ptr(vd),
+                            _lib.ptr(ws), _lib.ptr(gq), _lib.ptr(gk), _lib.ptr(gv), *args) == 0
+    want = _fused_backward_oracle(coracle, go.float(), q.float(), key.float(), v.float(), K, s)
+    for got, w, name in zip((gq, gk, gv), want, ('grad_query', 'grad_key', 'grad_value')):
+        assert torch.isfinite(got).all(), name
+        if dtype == torch.float32:
+            torch.testing.assert_close(got.cpu().double(), w, msg=lambda m: f'{name}: {m}', **tol)
+        else:
+            assert_rel_rms_close(got.float().cpu(), w, tol, f'{name} {dtype}')
+    # only grad_key wanted: the other buffers stay as they are
+    gq2, gv2 = torch.full_like(qd, 7.0), torch.full_like(vd, 7.0)
+    gk2 = torch.full_like(kd, float('nan'))
+    assert _lib.call_status('sapa_fused_backward', DEV, _lib.ptr(god), _lib.ptr(qd), _lib.ptr(kd), _lib.ptr(vd),
+                            _lib.ptr(ws), None, _lib.ptr(gk2), None, *args) == 0
+    assert torch.equal(gk2, gk) and (gq2 == 7).all() and (gv2 == 7).all()
+    # the autograd route takes the same entry point
+    leaves = [t.clone().requires_grad_() for t in (qd, kd, vd)]
+    sapa_amd.sapa_fused(*leaves, K, s).backward(god)
+    for leaf, got in zip(leaves, (gq, gk, gv)):
+        assert torch.equal(leaf.grad, got)
+    # K = 3: no tiled kernels behind this call
+    assert _lib.call_status('sapa_fused_backward', DEV, _lib.ptr(god), _lib.ptr(qd), _lib.ptr(kd), _lib.ptr(vd),
+                            _lib.ptr(ws), _lib.ptr(gq), _lib.ptr(gk), _lib.ptr(gv), B, d, C, H, W, 3, s,
+                            _lib.DTYPES[dtype]) == _lib.UNSUPPORTED
+
+
 def test_gradcheck_reference_shapes():
     """sapa/sapa/grad_check.py:8-33: float64 gradcheck at its shapes."""
     from torch.autograd import gradcheck
