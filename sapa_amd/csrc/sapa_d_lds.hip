@@ -33,19 +33,26 @@ deform_lds_kernel(const T *__restrict__ q, const T *__restrict__ key,
                   const T *__restrict__ offset, T *__restrict__ out, int Cq, int C, int H, int W,
                   int P, int G, int olayout, int tiles_x, int tiles_y, int nblocks, int per_xcd) {
     typedef float A;
+    typedef float F4 __attribute__((ext_vector_type(4)));
     constexpr int HR = 4;                           // window reach in low-res cells
     constexpr int NT = TPW * TPH * S * S;
     constexpr int WW = TPW + 2 * HR + 1, WH = TPH + 2 * HR + 1;
-    constexpr int RS = WW | 1;                      // odd row stride
-    constexpr int CS = WH * RS;
     constexpr int WIN = WH * WW;
+    // LDS window: [cell][CH channels], cells CST floats apart.  A thread reads the
+    // CH channels of a corner as 16-byte vectors; with CST = 4 mod 16 the cells
+    // that the lanes of a wave pick -- anywhere in the window -- spread over all
+    // 16 four-bank groups instead of colliding on the one bank that a
+    // [channel][cell] layout gives each channel.
+    constexpr int CST = CH + 4;
+    constexpr int RS = WW * CST;                    // floats between window rows
+    static_assert(CH % 4 == 0, "channels are read four at a time");
     constexpr int TXP = TPW * S;                    // tile width in pixels
     constexpr bool DO_QK = MODE == DEFORM_QK || MODE == DEFORM_FUSED;
     constexpr bool DO_AV = MODE == DEFORM_AV || MODE == DEFORM_FUSED;
 
-    extern __shared__ float smem[];
-    A *win = smem;                                  // [CH][WH][RS]
-    A *lg = smem + CH * CS;                         // [P][NT]
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    A *win = smem;                                  // [WH][WW][CST]
+    A *lg = smem + WIN * CST;                       // [P][NT]
 
     const int logical = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
     if (logical >= nblocks) return;
@@ -77,7 +84,7 @@ deform_lds_kernel(const T *__restrict__ q, const T *__restrict__ key,
             A v = 0;
             if (ch < nvalid && gy >= 0 && gy < H && gx >= 0 && gx < W)
                 v = (A)src[(long)ch * lplane + (long)gy * W + gx];
-            win[ch * CS + row * RS + col] = v;
+            win[row * RS + col * CST + ch] = v;
         }
     };
 
@@ -115,16 +122,20 @@ deform_lds_kernel(const T *__restrict__ q, const T *__restrict__ key,
                 if (tap_setup(kh, kw, H, W, tap)) {
                     const int hl = (int)floor_(kh) - wy0, wl = (int)floor_(kw) - wx0;
                     if (hl >= 0 && hl <= WH - 2 && wl >= 0 && wl <= WW - 2) {
-                        const A *wp = win + hl * RS + wl;
+                        const A *wp = win + hl * RS + wl * CST;
 #pragma unroll
-                        for (int ch = 0; ch < CH; ++ch) {
-                            const A tv = qv[ch] * scv;
-                            const A v1 = wp[ch * CS], v2 = wp[ch * CS + 1];
-                            const A v3 = wp[ch * CS + RS], v4 = wp[ch * CS + RS + 1];
-                            const A ghc = -tap.hw * v1 - tap.lw * v2 + tap.hw * v3 + tap.lw * v4;
-                            const A gwc = -tap.hh * v1 + tap.hh * v2 - tap.lh * v3 + tap.lh * v4;
-                            gh = fma_(ghc, tv, gh);
-                            gw = fma_(gwc, tv, gw);
+                        for (int c4 = 0; c4 < CH; c4 += 4) {
+                            const F4 a1 = *(const F4 *)(wp + c4), a2 = *(const F4 *)(wp + CST + c4);
+                            const F4 a3 = *(const F4 *)(wp + RS + c4), a4 = *(const F4 *)(wp + RS + CST + c4);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                const A tv = qv[c4 + e] * scv;
+                                const A v1 = a1[e], v2 = a2[e], v3 = a3[e], v4 = a4[e];
+                                const A ghc = -tap.hw * v1 - tap.lw * v2 + tap.hw * v3 + tap.lw * v4;
+                                const A gwc = -tap.hh * v1 + tap.hh * v2 - tap.lh * v3 + tap.lh * v4;
+                                gh = fma_(ghc, tv, gh);
+                                gw = fma_(gwc, tv, gw);
+                            }
                         }
                     } else {
                         const T *kp = key + (ch0 + c0) * lplane;
@@ -180,14 +191,19 @@ deform_lds_kernel(const T *__restrict__ q, const T *__restrict__ key,
                 if (tap_setup(kh, kw, H, W, tap)) {
                     const int hl = (int)floor_(kh) - wy0, wl = (int)floor_(kw) - wx0;
                     if (hl >= 0 && hl <= WH - 2 && wl >= 0 && wl <= WW - 2) {
-                        const A *wp = win + hl * RS + wl;
+                        const A *wp = win + hl * RS + wl * CST;
 #pragma unroll
-                        for (int ch = 0; ch < CH; ++ch) {
-                            A val = tap.w1 * wp[ch * CS];
-                            val = fma_(tap.w2, wp[ch * CS + 1], val);
-                            val = fma_(tap.w3, wp[ch * CS + RS], val);
-                            val = fma_(tap.w4, wp[ch * CS + RS + 1], val);
-                            acc = fma_(val, qv[ch], acc);
+                        for (int c4 = 0; c4 < CH; c4 += 4) {
+                            const F4 a1 = *(const F4 *)(wp + c4), a2 = *(const F4 *)(wp + CST + c4);
+                            const F4 a3 = *(const F4 *)(wp + RS + c4), a4 = *(const F4 *)(wp + RS + CST + c4);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                A val = tap.w1 * a1[e];
+                                val = fma_(tap.w2, a2[e], val);
+                                val = fma_(tap.w3, a3[e], val);
+                                val = fma_(tap.w4, a4[e], val);
+                                acc = fma_(val, qv[c4 + e], acc);
+                            }
                         }
                     } else {
                         const T *kp = key + (ch0 + c0) * lplane;
@@ -245,15 +261,20 @@ deform_lds_kernel(const T *__restrict__ q, const T *__restrict__ key,
                 // where the guard holds, so that consecutive points can be
                 // interleaved by the scheduler.
                 const WinTap<A> wt = win_tap(kh, kw, H, W, wy0, wx0, WH, WW);
-                const A *wp = win + (wt.inwin ? wt.hl * RS + wt.wl : 0);
+                const A *wp = win + (wt.inwin ? wt.hl * RS + wt.wl * CST : 0);
 #pragma unroll
-                for (int ch = 0; ch < CH; ++ch) {
-                    A val = wt.w1 * wp[ch * CS];
-                    val = fma_(wt.w2, wp[ch * CS + 1], val);
-                    val = fma_(wt.w3, wp[ch * CS + RS], val);
-                    val = fma_(wt.w4, wp[ch * CS + RS + 1], val);
-                    const A on = fma_(val, wa, o[ch]);
-                    o[ch] = wt.inwin ? on : o[ch];
+                for (int c4 = 0; c4 < CH; c4 += 4) {
+                    const F4 a1 = *(const F4 *)(wp + c4), a2 = *(const F4 *)(wp + CST + c4);
+                    const F4 a3 = *(const F4 *)(wp + RS + c4), a4 = *(const F4 *)(wp + RS + CST + c4);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        A val = wt.w1 * a1[e];
+                        val = fma_(wt.w2, a2[e], val);
+                        val = fma_(wt.w3, a3[e], val);
+                        val = fma_(wt.w4, a4[e], val);
+                        const A on = fma_(val, wa, o[c4 + e]);
+                        o[c4 + e] = wt.inwin ? on : o[c4 + e];
+                    }
                 }
                 if (wt.guard && !wt.inwin) {       // rare: the tap left the window
                     Tap<A> tap;
@@ -281,9 +302,9 @@ static hipError_t launch_geom(int mode, const void *q, const void *key, const vo
                               const void *value, const void *offset, void *out, int B, int Cq,
                               int C, int H, int W, int P, int G, int olayout, hipStream_t st) {
     constexpr int HR = 4, NT = TPW * TPH * S * S;
-    constexpr int WW = TPW + 2 * HR + 1, WH = TPH + 2 * HR + 1, RS = WW | 1, CS = WH * RS;
+    constexpr int WW = TPW + 2 * HR + 1, WH = TPH + 2 * HR + 1, CST = CH + 4;
     const size_t smem =
-        ((size_t)CH * CS + (size_t)(mode == DEFORM_OFFGRAD ? 2 : 1) * P * NT) * sizeof(float);
+        ((size_t)WH * WW * CST + (size_t)(mode == DEFORM_OFFGRAD ? 2 : 1) * P * NT) * sizeof(float);
     if (smem > 160 * 1024) return hipErrorNotSupported;  // LDS of one CU
     const bool big = smem > 64 * 1024;                   // beyond the default dynamic-LDS limit
     const int tiles_x = (W + TPW - 1) / TPW, tiles_y = (H + TPH - 1) / TPH;
@@ -323,7 +344,13 @@ static hipError_t launch_t(int mode, const void *q, const void *key, const void 
 #else
     switch (s) {
         case 1: return launch_geom<T, 1, 16, 16, 8>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, G, olayout, st);
-        case 2: return launch_geom<T, 2, 8, 8, 16>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, G, olayout, st);
+        case 2:
+            // few points leave LDS room for a 16 x 8-parent tile (512 threads): a
+            // smaller share of halo cells per staged window (measured at P = 9: 12 % faster;
+            // at P = 25 the [P][thread] logits of 512 threads cost a workgroup per CU)
+            if (P <= 12 && W > 8)
+                return launch_geom<T, 2, 16, 8, 16>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, G, olayout, st);
+            return launch_geom<T, 2, 8, 8, 16>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, G, olayout, st);
         case 4: return launch_geom<T, 4, 4, 4, 16>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, G, olayout, st);
         default: return hipErrorNotSupported;
     }
