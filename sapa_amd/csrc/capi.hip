@@ -469,7 +469,13 @@ int sapa_deform_fused_forward_nhwc(const void *query, const void *key, const voi
     if (B == 0) return SAPA_OK;
     if (!query || !key || !value || !offset || !out) return SAPA_ERR_INVALID_ARGUMENT;
     const hipError_t e =
-        took("deform_fused_nhwc_kernel", deform_fused_nhwc_launch(query, key, value, offset, out, B, Cq, C, H, W,
+        took(
+#ifdef SAPA_DNHWC_GATHER
+            "deform_fused_nhwc_kernel",
+#else
+            "deform_fused_wmat_kernel",
+#endif
+            deform_fused_nhwc_launch(query, key, value, offset, out, B, Cq, C, H, W,
                                                                   P, s, G, dtype, (hipStream_t)stream));
     if (e == hipErrorNotSupported) return SAPA_ERR_UNSUPPORTED;
     return finish(e);
