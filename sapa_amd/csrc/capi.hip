@@ -473,7 +473,8 @@ int sapa_deform_fused_forward_nhwc(const void *query, const void *key, const voi
 #ifdef SAPA_DNHWC_GATHER
             "deform_fused_nhwc_kernel",
 #else
-            "deform_fused_wmat_kernel",
+            // the launcher's own rule: gathers for few points, the matrix formulation else
+            P <= 12 ? "deform_fused_nhwc_kernel" : "deform_fused_wmat_kernel",
 #endif
             deform_fused_nhwc_launch(query, key, value, offset, out, B, Cq, C, H, W,
                                                                   P, s, G, dtype, (hipStream_t)stream));

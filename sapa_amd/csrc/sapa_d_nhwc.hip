@@ -861,15 +861,21 @@ hipError_t deform_fused_nhwc_launch(const void *q, const void *key, const void *
     for (const void *p : ptrs)
         if ((uintptr_t)p % (4 * esize) != 0) return hipErrorNotSupported;
     if ((uintptr_t)offset % (2 * esize) != 0) return hipErrorNotSupported;
-#ifdef SAPA_DNHWC_GATHER
-    // tuning build: the gather formulation (one row of lanes per pixel and group)
+    // Few points: the matrix formulation's fixed work per tile (two products over the
+    // whole window whatever P is) outweighs the gathers it saves; measured at
+    // B=8, C=256, G=4, d=32, 64x64 -> 128x128: P = 9 259 against 248 us, P = 5 257
+    // against 225 us, P = 25 292 against 450 us.
+    // (SAPA_DNHWC_GATHER: a tuning build with the gather formulation throughout.)
+#ifndef SAPA_DNHWC_GATHER
+    if (P <= 12)
+#endif
     switch (dtype) {
         case 0: return dnhwc::launch_t<float>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);
         case 2: return dnhwc::launch_t<f16_t>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);
         case 3: return dnhwc::launch_t<bf16_t>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);
         default: return hipErrorNotSupported;
     }
-#else
+#ifndef SAPA_DNHWC_GATHER
     switch (dtype) {
         case 0: return dnhwc::launch_wmat_t<float>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);
         case 2: return dnhwc::launch_wmat_t<f16_t>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);
