@@ -23,7 +23,13 @@ SHAPES = [(2, 2, 4, 8, 5, 7, 9, 2, 1.0), (1, 4, 32, 64, 8, 8, 25, 2, 0.75), (1, 
           (1, 2, 8, 132, 4, 6, 16, 1, 1.0), (2, 3, 4, 4, 3, 5, 17, 4, 1.0), (1, 2, 8, 8, 9, 9, 32, 2, 1.0),
           (1, 1, 4, 4, 1, 1, 1, 2, 1.0),
           # offsets far beyond the +-4 cells of the LDS window: the global-memory path
-          (1, 2, 8, 12, 14, 13, 9, 2, 6.0)]
+          (1, 2, 8, 12, 14, 13, 9, 2, 6.0),
+          # more than 12 points take the matrix formulation: the same far offsets; 64 and 48
+          # query / key channels per group (the padded instance), a ragged second value
+          # chunk (72 = 64 + 8) and a short single one (20); s = 4 and s = 1 with part of
+          # the samples outside the window; odd extents
+          (1, 2, 8, 12, 14, 13, 16, 2, 6.0), (1, 1, 64, 72, 6, 5, 20, 2, 1.5), (1, 2, 48, 20, 7, 9, 13, 4, 2.5),
+          (2, 1, 12, 36, 11, 6, 29, 1, 3.0)]
 IDS = ['-'.join(map(str, s)) for s in SHAPES]
 
 
@@ -53,7 +59,7 @@ def test_fp32_vs_oracle(coracle, shape):
 
 
 @pytest.mark.parametrize('dtype,rel', [(torch.bfloat16, BF16_REL), (torch.float16, F16_REL)])
-@pytest.mark.parametrize('shape', SHAPES[:4] + SHAPES[7:], ids=IDS[:4] + IDS[7:])
+@pytest.mark.parametrize('shape', SHAPES[:4] + SHAPES[7:], ids=IDS[:4] + IDS[7:])  # incl. the matrix-formulation shapes
 def test_16bit_vs_oracle(coracle, shape, dtype, rel):
     B, G, d, cg, H, W, P, s, _ = shape
     q, key, v, off = inputs(gen(501), *shape, dtype=dtype)
@@ -72,10 +78,11 @@ def test_matches_contiguous_path_at_a_larger_shape():
     torch.testing.assert_close(got.contiguous(), want, rtol=2e-5, atol=2e-5)
 
 
-def test_guard_failures_and_image_border():
+@pytest.mark.parametrize('P', [9, 17])      # the gather kernel / the matrix formulation
+def test_guard_failures_and_image_border(P):
     """Offsets that push most points out of the image: those points keep logit
     0, take part in the softmax and contribute nothing."""
-    B, G, d, cg, H, W, P, s = 1, 2, 4, 8, 6, 7, 9, 2
+    B, G, d, cg, H, W, s = 1, 2, 4, 8, 6, 7, 2
     g = gen(503)
     q, key, v, off = inputs(g, B, G, d, cg, H, W, P, s, 1.0)
     off = off + 5.0 * torch.sign(randn(g, *off.shape))      # +-5 cells: in or out of a 6x7 image
