@@ -468,16 +468,10 @@ int sapa_deform_fused_forward_nhwc(const void *query, const void *key, const voi
     if (rc != SAPA_OK) return rc;
     if (B == 0) return SAPA_OK;
     if (!query || !key || !value || !offset || !out) return SAPA_ERR_INVALID_ARGUMENT;
-    const hipError_t e =
-        took(
-#ifdef SAPA_DNHWC_GATHER
-            "deform_fused_nhwc_kernel",
-#else
-            // the launcher's own rule: gathers for few points, the matrix formulation else
-            P <= 12 ? "deform_fused_nhwc_kernel" : "deform_fused_wmat_kernel",
-#endif
-            deform_fused_nhwc_launch(query, key, value, offset, out, B, Cq, C, H, W,
-                                                                  P, s, G, dtype, (hipStream_t)stream));
+    const char *name = "";
+    const hipError_t e0 = deform_fused_nhwc_launch(query, key, value, offset, out, B, Cq, C, H, W, P,
+                                                   s, G, dtype, (hipStream_t)stream, &name);
+    const hipError_t e = took(name, e0);
     if (e == hipErrorNotSupported) return SAPA_ERR_UNSUPPORTED;
     return finish(e);
 }

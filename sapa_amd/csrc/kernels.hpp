@@ -67,9 +67,18 @@ hipError_t project_nhwc_launch(const void *x, const void *w, const void *bias, v
 // order (offsets [B, sH, sW, 2GP]); f32 / f16 / bf16, s in {1, 2, 4}, P <= 32,
 // channels per group multiples of 4, at most 64 query / key channels per group.
 // hipErrorNotSupported otherwise.
+// *kernel (if given): the name of the kernel the call went to.
 hipError_t deform_fused_nhwc_launch(const void *q, const void *key, const void *value,
                                     const void *offset, void *out, int B, int Cq, int C, int H,
-                                    int W, int P, int s, int G, int dtype, hipStream_t st);
+                                    int W, int P, int s, int G, int dtype, hipStream_t st,
+                                    const char **kernel = nullptr);
+
+// sapa_d_wmat16.hip: the same operator for f16 / bf16 on the 16-bit matrix
+// instructions; channels per group multiples of 8, tensors aligned to 16 bytes,
+// P <= 32.  hipErrorNotSupported otherwise.
+hipError_t deform_fused_wmat16_launch(const void *q, const void *key, const void *value,
+                                      const void *offset, void *out, int B, int Cq, int C, int H,
+                                      int W, int P, int s, int G, int dtype, hipStream_t st);
 
 // sapa_b_dot2.hip: qk, qk+softmax and fused for f16 / bf16 tensors on the
 // two-term dot-product instructions (K = 5, s = 2); hipErrorNotSupported

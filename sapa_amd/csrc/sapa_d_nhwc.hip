@@ -489,26 +489,6 @@ static hipError_t launch_t(const void *q, const void *key, const void *value, co
 // (lane % 16, lane / 16) operand layout; half a wave per pixel, one lane per
 // point, for the per-sample work.
 constexpr int TPW = 4;          // tile edge, hi-res pixels
-#ifndef SAPA_WMAT_SKIP
-#define SAPA_WMAT_SKIP 0
-#endif
-
-// max / sum of a value over the aligned group of N = 16 or 32 lanes a lane is in
-template <bool MAX, int N>
-__device__ __forceinline__ float reduce_lanes(float v) {
-    union { float f; int i; } x, y;
-    auto step = [&](int other) __attribute__((always_inline)) {
-        y.i = other;
-        x.f = MAX ? max_(x.f, y.f) : x.f + y.f;
-    };
-    x.f = v;
-    step(__builtin_amdgcn_mov_dpp(x.i, 0xB1, 0xf, 0xf, true));     // lane ^ 1 (quad_perm [1,0,3,2])
-    step(__builtin_amdgcn_mov_dpp(x.i, 0x4E, 0xf, 0xf, true));     // lane ^ 2 (quad_perm [2,3,0,1])
-    step(__builtin_amdgcn_mov_dpp(x.i, 0x141, 0xf, 0xf, true));    // the other quad of 8 (row_half_mirror)
-    step(__builtin_amdgcn_mov_dpp(x.i, 0x140, 0xf, 0xf, true));    // the other 8 of the row (row_mirror)
-    if (N == 32) step(__builtin_amdgcn_ds_swizzle(x.i, 0x401F));   // lane ^ 16
-    return x.f;
-}
 
 template <typename T, int S, int DP>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3)))
@@ -659,7 +639,6 @@ deform_fused_wmat_kernel(const T *__restrict__ q, const T *__restrict__ key,
 #pragma unroll
             for (int s16 = 0; s16 < DP / 16; ++s16) a4[s16] = Q4::widen(qa[s16]);
             for (int nb = wave; nb < NKB; nb += 4) {
-                if (SAPA_WMAT_SKIP & 2) break;
                 f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int s16 = 0; s16 < DP / 16; ++s16) {
@@ -734,13 +713,11 @@ deform_fused_wmat_kernel(const T *__restrict__ q, const T *__restrict__ key,
                 __hip_atomic_fetch_add(wp + WW + 1, (u32)__float2uint_rn(sc * t.w4), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             }
         };
-        if (!(SAPA_WMAT_SKIP & 1)) {
-            if (narrow) {
-                sample(std::integral_constant<int, 16>{}, 0, srow, spx, sq);
-            } else {
-                sample(std::integral_constant<int, 32>{}, 0, half, bpx[0], pl);
-                sample(std::integral_constant<int, 32>{}, 1, 8 + half, bpx[1], pl);
-            }
+        if (narrow) {
+            sample(std::integral_constant<int, 16>{}, 0, srow, spx, sq);
+        } else {
+            sample(std::integral_constant<int, 32>{}, 0, half, bpx[0], pl);
+            sample(std::integral_constant<int, 32>{}, 1, 8 + half, bpx[1], pl);
         }
         // ---- (d) value chunks: out tile = Wm . value window (the key window is done with)
         stage_store(VS, 16);
@@ -756,7 +733,7 @@ deform_fused_wmat_kernel(const T *__restrict__ q, const T *__restrict__ key,
                 stage_load(true, (g + 1) * d, d);
                 load_q(g + 1);
             }
-            if (16 * wave < cvalid && !(SAPA_WMAT_SKIP & 2)) {
+            if (16 * wave < cvalid) {
                 // two accumulators: consecutive instructions do not wait for each other
                 f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -800,7 +777,7 @@ deform_fused_wmat_kernel(const T *__restrict__ q, const T *__restrict__ key,
                 __syncthreads();
             }
             // a row of 16 lanes stores its pixel's 64 channels: 256 contiguous bytes
-            if (spx.active && 4 * sq < cvalid && !(SAPA_WMAT_SKIP & 8))
+            if (spx.active && 4 * sq < cvalid)
                 __builtin_nontemporal_store(Q4::narrow(*(const f32x4 *)(Sl + srow * VS + 4 * sq)),
                                             (Raw *)(out + spx.hp * C + cbase + 4 * sq));
             if (vc + 1 < nVc) {
@@ -850,7 +827,10 @@ static hipError_t launch_wmat_t(const void *q, const void *key, const void *valu
 // hipErrorNotSupported otherwise.
 hipError_t deform_fused_nhwc_launch(const void *q, const void *key, const void *value,
                                     const void *offset, void *out, int B, int Cq, int C, int H,
-                                    int W, int P, int s, int G, int dtype, hipStream_t st) {
+                                    int W, int P, int s, int G, int dtype, hipStream_t st,
+                                    const char **kernel) {
+    const char *unused;
+    if (!kernel) kernel = &unused;
     // the query / key channels of a group are one LDS chunk
     if (P > 16 * dnhwc::MAXSETS || (Cq / G) % 4 != 0 || Cq / G > 64 || (C / G) % 4 != 0)
         return hipErrorNotSupported;
@@ -866,6 +846,7 @@ hipError_t deform_fused_nhwc_launch(const void *q, const void *key, const void *
     // B=8, C=256, G=4, d=32, 64x64 -> 128x128: P = 9 259 against 248 us, P = 5 257
     // against 225 us, P = 25 292 against 450 us.
     // (SAPA_DNHWC_GATHER: a tuning build with the gather formulation throughout.)
+    *kernel = "deform_fused_nhwc_kernel";
 #ifndef SAPA_DNHWC_GATHER
     if (P <= 12)
 #endif
@@ -876,6 +857,13 @@ hipError_t deform_fused_nhwc_launch(const void *q, const void *key, const void *
         default: return hipErrorNotSupported;
     }
 #ifndef SAPA_DNHWC_GATHER
+    // 16-bit tensors whose groups are whole 16-byte pieces: the 16-bit matrix instructions
+    if (dtype != 0) {
+        *kernel = "deform_fused_wmat16_kernel";
+        const hipError_t e = deform_fused_wmat16_launch(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, dtype, st);
+        if (e != hipErrorNotSupported) return e;
+    }
+    *kernel = "deform_fused_wmat_kernel";
     switch (dtype) {
         case 0: return dnhwc::launch_wmat_t<float>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);
         case 2: return dnhwc::launch_wmat_t<f16_t>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);

@@ -29,7 +29,12 @@ SHAPES = [(2, 2, 4, 8, 5, 7, 9, 2, 1.0), (1, 4, 32, 64, 8, 8, 25, 2, 0.75), (1, 
           # chunk (72 = 64 + 8) and a short single one (20); s = 4 and s = 1 with part of
           # the samples outside the window; odd extents
           (1, 2, 8, 12, 14, 13, 16, 2, 6.0), (1, 1, 64, 72, 6, 5, 20, 2, 1.5), (1, 2, 48, 20, 7, 9, 13, 4, 2.5),
-          (2, 1, 12, 36, 11, 6, 29, 1, 3.0)]
+          (2, 1, 12, 36, 11, 6, 29, 1, 3.0),
+          # channels per group in whole 16-byte pieces: 16-bit tensors take the 16-bit matrix
+          # instructions -- far offsets with 16 lanes per pixel, 48 channels padded to 64 at
+          # s = 4, s = 1, the full 32 points over three groups, three value chunks (64 + 64 + 8)
+          (1, 2, 8, 16, 14, 13, 16, 2, 6.0), (1, 2, 48, 24, 7, 9, 13, 4, 2.5), (2, 1, 16, 40, 11, 6, 29, 1, 3.0),
+          (2, 3, 24, 8, 9, 11, 32, 2, 1.0), (1, 1, 64, 136, 5, 7, 21, 2, 1.5)]
 IDS = ['-'.join(map(str, s)) for s in SHAPES]
 
 
@@ -95,6 +100,28 @@ def test_guard_failures_and_image_border(P):
     off_far = torch.full_like(off, 100.0)
     got = sapa_amd.deform_sapa_fused(*cl(q, key, v, off_far), P, s, G)
     assert torch.count_nonzero(got) == 0
+
+
+@pytest.mark.parametrize('dtype,rel', [(torch.bfloat16, BF16_REL), (torch.float16, F16_REL)])
+def test_guard_failures_on_the_16bit_matrix_kernel(coracle, dtype, rel):
+    """The same border case where 16-bit tensors take the 16-bit matrix
+    instructions (8 channels per group, 17 points), and the name of the
+    kernel that ran."""
+    from sapa_amd import _lib
+    B, G, d, cg, H, W, P, s = 1, 2, 8, 8, 6, 7, 17, 2
+    g = gen(505)
+    q, key, v, off = inputs(g, B, G, d, cg, H, W, P, s, 1.0, dtype=dtype)
+    off = (off.float() + 5.0 * torch.sign(randn(g, *off.shape))).to(dtype)
+    got = sapa_amd.deform_sapa_fused(*cl(q, key, v, off), P, s, G)
+    assert _lib.last_kernel() == 'deform_fused_wmat16_kernel'
+    want = coracle.deform_sapa_fused(q.float(), key.float(), v.float(), off.float(), P, s, G, 'f32')
+    assert_rel_rms_close(got.float(), want, rel, 'fused')
+    got = sapa_amd.deform_sapa_fused(*cl(q, key, v, torch.full_like(off, 100.0)), P, s, G)
+    assert torch.count_nonzero(got) == 0
+    # groups that are not whole 16-byte pieces stay on the kernel for any channel count
+    q, key, v, off = inputs(g, B, G, 4, 12, H, W, P, s, 1.0, dtype=dtype)
+    sapa_amd.deform_sapa_fused(*cl(q, key, v, off), P, s, G)
+    assert _lib.last_kernel() == 'deform_fused_wmat_kernel'
 
 
 def test_layout_errors_and_backward():
