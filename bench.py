@@ -67,10 +67,10 @@ MEASURED_TRAFFIC = {
                                           'sapa_b_nhwc16_kernel'),
     ('deform_p25', 'fp32', 'nchw'): (829340888, 'profiles/sapa_d_lds_fused_deform_p25_fp32.md', 'deform_lds_kernel'),
     ('deform_p9', 'fp32', 'nchw'): (402514487, 'profiles/sapa_d_lds_fused_deform_p9_fp32.md', 'deform_lds_kernel'),
-    ('deform_p25', 'fp32', 'channels_last'): (356787493, 'profiles/sapa_d_nhwc_fused_deform_p25_fp32.md',
+    ('deform_p25', 'fp32', 'channels_last'): (356742233, 'profiles/sapa_d_nhwc_fused_deform_p25_fp32.md',
                                               'deform_fused_wmat_kernel'),
-    ('deform_p25', 'bf16', 'channels_last'): (178502923, 'profiles/sapa_d_nhwc_fused_deform_p25_bf16.md',
-                                              'deform_fused_wmat_kernel'),
+    ('deform_p25', 'bf16', 'channels_last'): (178450680, 'profiles/sapa_d_wmat16_fused_deform_p25_bf16.md',
+                                              'deform_fused_wmat16_kernel'),
 }
 
 

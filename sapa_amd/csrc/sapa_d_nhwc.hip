@@ -489,6 +489,9 @@ static hipError_t launch_t(const void *q, const void *key, const void *value, co
 // (lane % 16, lane / 16) operand layout; half a wave per pixel, one lane per
 // point, for the per-sample work.
 constexpr int TPW = 4;          // tile edge, hi-res pixels
+#ifndef SAPA_DNHWC_GATHER_MAXP
+#define SAPA_DNHWC_GATHER_MAXP 7
+#endif
 
 template <typename T, int S, int DP>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3)))
@@ -610,11 +613,13 @@ deform_fused_wmat_kernel(const T *__restrict__ q, const T *__restrict__ key,
         }
     };
 
+    __shared__ int fb_flag;         // some point of the tile left the window (this group)
     stage_load(true, 0, d);
     load_q(0);
     for (int g = 0; g < G; ++g) {
         // ---- (a) key window and an empty weight matrix
         stage_store(KS, DP / 4);
+        if (tid == 0) fb_flag = 0;
         for (int i = tid; i < NPX * WS / 4; i += NT) ((f32x4 *)Wl)[i] = f32x4{0.f, 0.f, 0.f, 0.f};
         __syncthreads();
         // the group's first value chunk and the offsets travel during the similarity
@@ -697,7 +702,11 @@ deform_fused_wmat_kernel(const T *__restrict__ q, const T *__restrict__ key,
             // softmax over the pixel's points = the lanes pt < P of its group of NL lanes
             const float mx = reduce_lanes<true, NL>(pt < P ? lg : -__builtin_huge_valf());
             const float e = pt < P ? exp_(lg - mx) : 0.f;
-            const float att = e * (1.f / reduce_lanes<false, NL>(e));
+            // 1 / sum: the hardware reciprocal (1 ulp) and one Newton step
+            const float sum = reduce_lanes<false, NL>(e);
+            float rs = __builtin_amdgcn_rcpf(sum);
+            rs = fma_(fma_(-sum, rs, 1.f), rs, rs);
+            const float att = e * rs;
             fatt[ps] = att;
             if (in) {
                 // Wm holds 2^30-scaled integers: every entry and every row sum is at
@@ -707,10 +716,10 @@ deform_fused_wmat_kernel(const T *__restrict__ q, const T *__restrict__ key,
                 // contribution, 2^-31, is below that of an fp32 weight near 1
                 u32 *wp = (u32 *)Wl + pi * WS + cell;
                 const float sc = att * WSCALE;
-                __hip_atomic_fetch_add(wp, (u32)__float2uint_rn(sc * t.w1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                __hip_atomic_fetch_add(wp + 1, (u32)__float2uint_rn(sc * t.w2), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                __hip_atomic_fetch_add(wp + WW, (u32)__float2uint_rn(sc * t.w3), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                __hip_atomic_fetch_add(wp + WW + 1, (u32)__float2uint_rn(sc * t.w4), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                __hip_atomic_fetch_add(wp, (u32)fma_(sc, t.w1, 0.5f), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                __hip_atomic_fetch_add(wp + 1, (u32)fma_(sc, t.w2, 0.5f), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                __hip_atomic_fetch_add(wp + WW, (u32)fma_(sc, t.w3, 0.5f), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                __hip_atomic_fetch_add(wp + WW + 1, (u32)fma_(sc, t.w4, 0.5f), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             }
         };
         if (narrow) {
@@ -721,7 +730,9 @@ deform_fused_wmat_kernel(const T *__restrict__ q, const T *__restrict__ key,
         }
         // ---- (d) value chunks: out tile = Wm . value window (the key window is done with)
         stage_store(VS, 16);
-        const bool any_fb = __syncthreads_or(fb[0] || fb[1]);
+        if (fb[0] || fb[1]) fb_flag = 1;
+        __syncthreads();
+        const bool any_fb = fb_flag != 0;
         for (int vc = 0; vc < nVc; ++vc) {
             const int cbase = g * cg + vc * CHK;
             const int cvalid = cg - vc * CHK < CHK ? cg - vc * CHK : CHK;
@@ -758,8 +769,12 @@ deform_fused_wmat_kernel(const T *__restrict__ q, const T *__restrict__ key,
                 for (int ps = 0; ps < 2; ++ps) {
                     if (!fb[ps]) continue;
                     const int pi = narrow ? srow : ps * 8 + half;
+                    // (opaque to the compiler, which would otherwise set these taps up
+                    // ahead of the branch, for every tile)
+                    float kh = fkh[ps], kw = fkw[ps];
+                    asm volatile("" : "+v"(kh), "+v"(kw));
                     Tap<float> tp = {};
-                    tap_setup(fkh[ps], fkw[ps], H, W, tp);
+                    tap_setup(kh, kw, H, W, tp);
                     const T *vp = value + (long)n * lpix * C + cbase;
                     for (int c = 0; c < cvalid; ++c) {
                         const float v1 = tp.m1 ? (float)vp[(long)tp.i1 * C + c] : 0.f;
@@ -841,36 +856,36 @@ hipError_t deform_fused_nhwc_launch(const void *q, const void *key, const void *
     for (const void *p : ptrs)
         if ((uintptr_t)p % (4 * esize) != 0) return hipErrorNotSupported;
     if ((uintptr_t)offset % (2 * esize) != 0) return hipErrorNotSupported;
-    // Few points: the matrix formulation's fixed work per tile (two products over the
-    // whole window whatever P is) outweighs the gathers it saves; measured at
-    // B=8, C=256, G=4, d=32, 64x64 -> 128x128: P = 9 259 against 248 us, P = 5 257
-    // against 225 us, P = 25 292 against 450 us.
-    // (SAPA_DNHWC_GATHER: a tuning build with the gather formulation throughout.)
-    *kernel = "deform_fused_nhwc_kernel";
 #ifndef SAPA_DNHWC_GATHER
-    if (P <= 12)
+    // 16-bit tensors whose groups are whole 16-byte pieces: the 16-bit matrix
+    // instructions, for any number of points
+    if (dtype != 0) {
+        *kernel = "deform_fused_wmat16_kernel";
+        const hipError_t e = deform_fused_wmat16_launch(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, dtype, st);
+        if (e != hipErrorNotSupported) return e;
+    }
+    // Few points: the fp32 matrix formulation's fixed work per tile (two products over
+    // the whole window whatever P is) outweighs the gathers it saves; measured at
+    // B=8, C=256, G=4, d=32, 64x64 -> 128x128, fp32: P = 5 236 against 211 us, P = 9
+    // 237 against 249 us, P = 12 238 against 277 us, P = 25 268 against 450 us.
+    // (SAPA_DNHWC_GATHER: a tuning build with the gather formulation throughout.)
+    if (P > SAPA_DNHWC_GATHER_MAXP) {
+        *kernel = "deform_fused_wmat_kernel";
+        switch (dtype) {
+            case 0: return dnhwc::launch_wmat_t<float>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);
+            case 2: return dnhwc::launch_wmat_t<f16_t>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);
+            case 3: return dnhwc::launch_wmat_t<bf16_t>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);
+            default: return hipErrorNotSupported;
+        }
+    }
 #endif
+    *kernel = "deform_fused_nhwc_kernel";
     switch (dtype) {
         case 0: return dnhwc::launch_t<float>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);
         case 2: return dnhwc::launch_t<f16_t>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);
         case 3: return dnhwc::launch_t<bf16_t>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);
         default: return hipErrorNotSupported;
     }
-#ifndef SAPA_DNHWC_GATHER
-    // 16-bit tensors whose groups are whole 16-byte pieces: the 16-bit matrix instructions
-    if (dtype != 0) {
-        *kernel = "deform_fused_wmat16_kernel";
-        const hipError_t e = deform_fused_wmat16_launch(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, dtype, st);
-        if (e != hipErrorNotSupported) return e;
-    }
-    *kernel = "deform_fused_wmat_kernel";
-    switch (dtype) {
-        case 0: return dnhwc::launch_wmat_t<float>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);
-        case 2: return dnhwc::launch_wmat_t<f16_t>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);
-        case 3: return dnhwc::launch_wmat_t<bf16_t>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);
-        default: return hipErrorNotSupported;
-    }
-#endif
 }
 
 }  // namespace sapa

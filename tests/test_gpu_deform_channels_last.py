@@ -23,8 +23,8 @@ SHAPES = [(2, 2, 4, 8, 5, 7, 9, 2, 1.0), (1, 4, 32, 64, 8, 8, 25, 2, 0.75), (1, 
           (1, 2, 8, 132, 4, 6, 16, 1, 1.0), (2, 3, 4, 4, 3, 5, 17, 4, 1.0), (1, 2, 8, 8, 9, 9, 32, 2, 1.0),
           (1, 1, 4, 4, 1, 1, 1, 2, 1.0),
           # offsets far beyond the +-4 cells of the LDS window: the global-memory path
-          (1, 2, 8, 12, 14, 13, 9, 2, 6.0),
-          # more than 12 points take the matrix formulation: the same far offsets; 64 and 48
+          (1, 2, 8, 12, 14, 13, 7, 2, 6.0), (1, 2, 8, 12, 14, 13, 9, 2, 6.0),
+          # more than 7 points take the matrix formulation: the same far offsets; 64 and 48
           # query / key channels per group (the padded instance), a ragged second value
           # chunk (72 = 64 + 8) and a short single one (20); s = 4 and s = 1 with part of
           # the samples outside the window; odd extents
@@ -83,7 +83,7 @@ def test_matches_contiguous_path_at_a_larger_shape():
     torch.testing.assert_close(got.contiguous(), want, rtol=2e-5, atol=2e-5)
 
 
-@pytest.mark.parametrize('P', [9, 17])      # the gather kernel / the matrix formulation
+@pytest.mark.parametrize('P', [5, 9, 17])   # the gather kernel / the matrix formulation (16 and 32 lanes per pixel)
 def test_guard_failures_and_image_border(P):
     """Offsets that push most points out of the image: those points keep logit
     0, take part in the softmax and contribute nothing."""
