@@ -60,7 +60,7 @@ __device__ __forceinline__ void softmax_inplace(A (&v)[N]) {
     for (int i = 0; i < N; ++i) v[i] *= inv;
 }
 
-// max / sum of a value over the aligned group of N = 16 or 32 lanes a lane is in.
+// max / sum of a value over the aligned group of N = 8, 16 or 32 lanes a lane is in.
 // The maximum is written as one DPP instruction per step: from the builtin the
 // compiler makes three (a move and two canonicalising maxima).  The s_nop covers
 // the two wait states a DPP read needs after the VALU write of its source.
@@ -74,7 +74,7 @@ __device__ __forceinline__ float reduce_lanes(float v) {
         SAPA_MAX_DPP(x.f, "quad_perm:[1,0,3,2]");      // lane ^ 1
         SAPA_MAX_DPP(x.f, "quad_perm:[2,3,0,1]");      // lane ^ 2
         SAPA_MAX_DPP(x.f, "row_half_mirror");          // the other quad of 8
-        SAPA_MAX_DPP(x.f, "row_mirror");               // the other 8 of the row
+        if (N >= 16) SAPA_MAX_DPP(x.f, "row_mirror");  // the other 8 of the row
         if (N == 32) {
             y.i = __builtin_amdgcn_ds_swizzle(x.i, 0x401F);    // lane ^ 16
             asm volatile("v_max_f32 %0, %1, %2" : "=v"(x.f) : "v"(x.f), "v"(y.f));
@@ -88,7 +88,7 @@ __device__ __forceinline__ float reduce_lanes(float v) {
     step(__builtin_amdgcn_mov_dpp(x.i, 0xB1, 0xf, 0xf, true));     // lane ^ 1 (quad_perm [1,0,3,2])
     step(__builtin_amdgcn_mov_dpp(x.i, 0x4E, 0xf, 0xf, true));     // lane ^ 2 (quad_perm [2,3,0,1])
     step(__builtin_amdgcn_mov_dpp(x.i, 0x141, 0xf, 0xf, true));    // the other quad of 8 (row_half_mirror)
-    step(__builtin_amdgcn_mov_dpp(x.i, 0x140, 0xf, 0xf, true));    // the other 8 of the row (row_mirror)
+    if (N >= 16) step(__builtin_amdgcn_mov_dpp(x.i, 0x140, 0xf, 0xf, true));   // the other 8 of the row (row_mirror)
     if (N == 32) step(__builtin_amdgcn_ds_swizzle(x.i, 0x401F));   // lane ^ 16
     return x.f;
 }
