@@ -318,8 +318,20 @@ def main():
                               out.data_ptr(), B, G * d, C, H, W, P, s, G, code,
                               stream.cuda_stream), entry)
             return step
-        step = fused_step('sapa_deform_fused_forward_nhwc' if args.layout == 'channels_last'
-                          else 'sapa_deform_fused_forward', q, key, v, out, off)
+        # contiguous tensors through the matrix-form kernels (key and value copied to
+        # channels-last order in a workspace): what sapa_amd.deform_sapa_fused does by
+        # default for 16-bit tensors, on request (matrix_form=True) for fp32
+        ws_bytes = lib.sapa_deform_fused_forward_workspace(B, G * d, C, H, W, P, s, G, code)
+        ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+
+        def ws_step():
+            _lib.check(lib.sapa_deform_fused_forward_ws(
+                q.data_ptr(), key.data_ptr(), v.data_ptr(), off.data_ptr(), out.data_ptr(), ws.data_ptr(),
+                B, G * d, C, H, W, P, s, G, 0, code, stream.cuda_stream), 'sapa_deform_fused_forward_ws')
+        main_is_ws = args.layout == 'nchw' and ws_bytes > 0 and dtype != torch.float32
+        step = ws_step if main_is_ws else fused_step(
+            'sapa_deform_fused_forward_nhwc' if args.layout == 'channels_last' else 'sapa_deform_fused_forward',
+            q, key, v, out, off)
     else:
         def fused_step(entry, q, key, v, out):
             fn = getattr(lib, entry)
@@ -387,6 +399,17 @@ def main():
         cl_kernel = _lib.last_kernel()
         err_cl = (cl[3][:1].float() - out[:1].float()).abs().max().item()
         del cl
+
+    matrix_form = None
+    if deform and args.layout == 'nchw' and ws_bytes > 0 and not main_is_ws and args.direction == 'forward' \
+            and not args.only_main:
+        ref_out = out[:1].clone()
+        ms_m, _ = timed(ws_step)
+        matrix_form = {'ms_per_step': ms_m, 'kernel': _lib.last_kernel(), 'workspace_bytes': ws_bytes,
+                       'max_abs_diff_vs_main_image0': (out[:1].float() - ref_out.float()).abs().max().item(),
+                       'note': 'the same contiguous tensors through sapa_deform_fused_forward_ws '
+                               '(sapa_amd.deform_sapa_fused(..., matrix_form=True))'}
+        step()      # the main line's result back into `out` for the checks below
 
     if args.calibration_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
@@ -467,6 +490,13 @@ def main():
             'max_abs_diff_vs_nchw_image0': err_cl,
             'note': 'same workload and algorithmic bytes, every tensor in torch.channels_last '
                     'order (python bench.py --layout channels_last makes this the main line)'}
+    if matrix_form is not None:
+        matrix_form['value'] = pix / (matrix_form['ms_per_step'] * 1e-3) / 1e9
+        matrix_form['roofline_frac'] = abytes / (matrix_form['ms_per_step'] * 1e-3) / 1e9 / HBM_PEAK_GBS
+        rec['matrix_form'] = matrix_form
+    if deform and not train and main_is_ws:
+        rec['config']['workspace_bytes'] = ws_bytes
+        rec['config']['entry'] = 'sapa_deform_fused_forward_ws (key / value copied to channels-last order inside the timed call)'
     if not args.no_cpu_baseline and not train:
         from oracle import torch_oracle
         if deform:

@@ -289,6 +289,33 @@ int sapa_deform_fused_forward_nhwc(const void *query, const void *key,
                                    int B, int Cq, int C, int H, int W,
                                    int P, int s, int G, int dtype, void *stream);
 
+/* sapa_deform_fused_forward (same contiguous tensors, same result up to the
+ * order of the sums) through the matrix-form kernels that serve the
+ * channels-last entry point: the low-res key and value are first copied into
+ * channels-last order in `workspace`, query / offset / out are used in place.
+ * At B=8, C=256, G=4, d=32, P=25, 64x64 -> 128x128 this is 1.5x (fp32) to 2.5x
+ * (bf16) faster than sapa_deform_fused_forward.  It replaces the same reference
+ * calls (dqk.forward -> softmax -> dav.forward, sapa_deform.py:51-53).
+ * sapa_deform_fused_forward_workspace: bytes of device memory the call needs,
+ * 0 when this path does not serve the case (use sapa_deform_fused_forward).
+ * workspace: at least that many bytes, aligned to 256; contents undefined
+ * before and after.  SAPA_ERR_UNSUPPORTED when the size is 0 or workspace NULL.
+ * offset_layout as in sapa_deform_fused_forward_from below: the offsets are
+ * read from the hi-res tensor or in place from the low-res convolution output.
+ * Served: s in {1, 2, 4}, Cq / G (at most 64) and C / G multiples of 4, and
+ * enough points for it to pay: 6 <= P <= 32 for SAPA_F16 / BF16 with Cq / G and
+ * C / G multiples of 8, 15 <= P <= 32 otherwise (SAPA_F32 included).  The sums
+ * run per window cell instead of per point: fp32 results differ from
+ * sapa_deform_fused_forward at rounding level (no further from the
+ * double-precision result than it). */
+long long sapa_deform_fused_forward_workspace(int B, int Cq, int C, int H, int W,
+                                              int P, int s, int G, int dtype);
+int sapa_deform_fused_forward_ws(const void *query, const void *key,
+                                 const void *value, const void *offset, void *out,
+                                 void *workspace, int B, int Cq, int C, int H, int W,
+                                 int P, int s, int G, int offset_layout, int dtype,
+                                 void *stream);
+
 /* The three sampled forward operators reading the offsets in the layout
  * `offset_layout` (sapa_offset_layout) names; with SAPA_OFFSET_HIRES they are
  * the functions above.  They replace

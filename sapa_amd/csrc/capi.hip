@@ -476,6 +476,31 @@ int sapa_deform_fused_forward_nhwc(const void *query, const void *key, const voi
     return finish(e);
 }
 
+long long sapa_deform_fused_forward_workspace(int B, int Cq, int C, int H, int W, int P, int s,
+                                              int G, int dtype) {
+    if (check_deform_args(B, Cq, C, H, W, P, s, G, dtype) != SAPA_OK) return 0;
+    return deform_fused_nchw_workspace(B, Cq, C, H, W, P, s, G, dtype);
+}
+
+int sapa_deform_fused_forward_ws(const void *query, const void *key, const void *value,
+                                 const void *offset, void *out, void *workspace, int B, int Cq,
+                                 int C, int H, int W, int P, int s, int G, int offset_layout,
+                                 int dtype, void *stream) {
+    const int rc = check_deform_args(B, Cq, C, H, W, P, s, G, dtype);
+    if (rc != SAPA_OK) return rc;
+    if (offset_layout < SAPA_OFFSET_HIRES || offset_layout > SAPA_OFFSET_NEAREST)
+        return SAPA_ERR_INVALID_ARGUMENT;
+    if (B == 0) return SAPA_OK;
+    if (!query || !key || !value || !offset || !out) return SAPA_ERR_INVALID_ARGUMENT;
+    const char *name = "";
+    const hipError_t e0 = deform_fused_nchw_ws_launch(query, key, value, offset, out, workspace, B, Cq, C,
+                                                      H, W, P, s, G, offset_layout, dtype,
+                                                      (hipStream_t)stream, &name);
+    const hipError_t e = took(name, e0);
+    if (e == hipErrorNotSupported) return SAPA_ERR_UNSUPPORTED;
+    return finish(e);
+}
+
 int sapa_deform_qk_backward(const void *grad_out, const void *query, const void *key,
                             const void *offset, void *grad_query, void *grad_key,
                             void *grad_offset, int B, int Cq, int H, int W, int P, int s, int G,

@@ -73,12 +73,30 @@ hipError_t deform_fused_nhwc_launch(const void *q, const void *key, const void *
                                     int W, int P, int s, int G, int dtype, hipStream_t st,
                                     const char **kernel = nullptr);
 
+// sapa_d_nhwc.hip: contiguous (NCHW) tensors through the matrix-form kernels:
+// key and value are copied into channels-last order in `workspace` (256-byte
+// aligned, deform_fused_nchw_workspace() bytes; 0 = this path does not serve the
+// case), q / offset / out are used in place; olayout: where the offsets are read
+// from (deform_tap.hpp: OffsetLayout).  hipErrorNotSupported otherwise.
+long deform_fused_nchw_workspace(int B, int Cq, int C, int H, int W, int P, int s, int G, int dtype);
+hipError_t deform_fused_nchw_ws_launch(const void *q, const void *key, const void *value,
+                                       const void *offset, void *out, void *workspace, int B, int Cq,
+                                       int C, int H, int W, int P, int s, int G, int olayout,
+                                       int dtype, hipStream_t st, const char **kernel = nullptr);
+
+// sapa_layout.hip: contiguous [B, C, HW] -> channels-last [B, HW, C]; esize 2 or 4 bytes
+hipError_t nchw_to_nhwc_launch(const void *src, void *dst, int B, int C, long HW, int esize,
+                               hipStream_t st);
+
 // sapa_d_wmat16.hip: the same operator for f16 / bf16 on the 16-bit matrix
-// instructions; channels per group multiples of 8, tensors aligned to 16 bytes,
-// P <= 32.  hipErrorNotSupported otherwise.
+// instructions; channels per group multiples of 8, key / value channels-last and
+// aligned to 16 bytes, P <= 32.  nchw: query, offset and out are contiguous
+// [B, channels, sH, sW] tensors instead of channels-last ones.
+// hipErrorNotSupported otherwise.
 hipError_t deform_fused_wmat16_launch(const void *q, const void *key, const void *value,
                                       const void *offset, void *out, int B, int Cq, int C, int H,
-                                      int W, int P, int s, int G, int dtype, hipStream_t st);
+                                      int W, int P, int s, int G, int dtype, hipStream_t st,
+                                      bool nchw = false, int olayout = 0);
 
 // sapa_b_dot2.hip: qk, qk+softmax and fused for f16 / bf16 tensors on the
 // two-term dot-product instructions (K = 5, s = 2); hipErrorNotSupported

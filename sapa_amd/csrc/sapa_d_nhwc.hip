@@ -493,12 +493,15 @@ constexpr int TPW = 4;          // tile edge, hi-res pixels
 #define SAPA_DNHWC_GATHER_MAXP 7
 #endif
 
-template <typename T, int S, int DP>
+// NCHW: query, offset and out are contiguous [B, channels, sH, sW] tensors (the
+// reference's layout); key and value are channels-last either way (the launcher
+// hands copies in that order to this kernel).
+template <typename T, int S, int DP, bool NCHW>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3)))
 deform_fused_wmat_kernel(const T *__restrict__ q, const T *__restrict__ key,
                          const T *__restrict__ value, const T *__restrict__ offset,
                          T *__restrict__ out, int Cq, int C, int H, int W, int P, int G,
-                         int tiles_x, int tiles_y, int nblocks, int per_xcd) {
+                         int tiles_x, int tiles_y, int nblocks, int per_xcd, int olayout) {
     constexpr int TPL = (TPW + S - 1) / S;                   // parents of a tile per axis
     constexpr int WW = TPL + 2 * RCH + 1, NPOS = WW * WW;    // window cells
     constexpr int KP = (NPOS + 15) / 16 * 16, NKB = KP / 16; // cells padded to blocks of 16
@@ -534,13 +537,15 @@ deform_fused_wmat_kernel(const T *__restrict__ q, const T *__restrict__ key,
 
     // pixel i of the tile (row-major 4 x 4): inside the image?  its flat hi-res
     // index, clamped for loads, and its parent
-    struct Pix { bool active; long hp; int ph, pw; };
+    struct Pix { bool active; long hp; int pp, ph, pw; };
+    const long hpl = (long)hH * hW;                                  // a hi-res channel plane (NCHW)
     auto pixel = [&](int i) __attribute__((always_inline)) {
         const int qh = y0 + i / TPW, qw = x0 + i % TPW;
         Pix r;
         r.active = qh < hH && qw < hW;
         const int ch = qh < hH ? qh : hH - 1, cw = qw < hW ? qw : hW - 1;
-        r.hp = (long)n * hH * hW + (long)ch * hW + cw;
+        r.pp = ch * hW + cw;
+        r.hp = (long)n * hH * hW + r.pp;
         r.ph = ch / S;
         r.pw = cw / S;
         return r;
@@ -608,8 +613,18 @@ deform_fused_wmat_kernel(const T *__restrict__ q, const T *__restrict__ key,
 #pragma unroll
         for (int s16 = 0; s16 < DP / 16; ++s16) {
             qa[s16] = Raw{};
-            if (mpx.active && 16 * s16 + 4 * mk < d)
-                qa[s16] = *(const Raw *)(q + mpx.hp * Cq + g * d + 16 * s16 + 4 * mk);
+            if (mpx.active && 16 * s16 + 4 * mk < d) {
+                if (NCHW) {
+                    // 4 channel planes, one element each
+                    const T *qp = q + ((long)n * Cq + g * d + 16 * s16 + 4 * mk) * hpl + mpx.pp;
+                    union { T h[4]; Raw r; } x;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) x.h[e] = qp[e * hpl];
+                    qa[s16] = x.r;
+                } else {
+                    qa[s16] = *(const Raw *)(q + mpx.hp * Cq + g * d + 16 * s16 + 4 * mk);
+                }
+            }
         }
     };
 
@@ -628,14 +643,36 @@ deform_fused_wmat_kernel(const T *__restrict__ q, const T *__restrict__ key,
         // the tile; else half a wave per pixel, two passes
         const bool narrow = P <= 16;
         f32x2 off2[2] = {f32x2{0.f, 0.f}, f32x2{0.f, 0.f}};
+        // (dx, dy) of point pt of pixel px
+        auto load_offset = [&](const Pix &px, int pt) __attribute__((always_inline)) {
+            if (NCHW) {
+                // channel cx = dx, cx + 1 = dy of the point, from the hi-res tensor or
+                // from the low-res one it is a pixel shuffle / a nearest interpolation
+                // of (deform_tap.hpp: OffsetLayout)
+                const long cx = (long)n * 2 * G * P + 2L * ((long)g * P + pt);
+                const T *op;
+                long dy;
+                if (olayout == OFFSET_PIXEL_SHUFFLE) {
+                    const int qh = px.pp / hW, qw = px.pp % hW;
+                    op = offset + (cx * (S * S) + (qh % S) * S + qw % S) * lpix + (long)px.ph * W + px.pw;
+                    dy = (long)(S * S) * lpix;
+                } else if (olayout == OFFSET_NEAREST) {
+                    op = offset + cx * lpix + (long)px.ph * W + px.pw;
+                    dy = lpix;
+                } else {
+                    op = offset + cx * hpl + px.pp;
+                    dy = hpl;
+                }
+                return f32x2{(float)op[0], (float)op[dy]};
+            }
+            return Q4::load_pair(offset + px.hp * (2L * G * P) + 2L * ((long)g * P + pt));
+        };
         if (narrow) {
-            if (spx.active && sq < P)
-                off2[0] = Q4::load_pair(offset + spx.hp * (2L * G * P) + 2L * ((long)g * P + sq));
+            if (spx.active && sq < P) off2[0] = load_offset(spx, sq);
         } else {
 #pragma unroll
             for (int ps = 0; ps < 2; ++ps)
-                if (bpx[ps].active && pl < P)
-                    off2[ps] = Q4::load_pair(offset + bpx[ps].hp * (2L * G * P) + 2L * ((long)g * P + pl));
+                if (bpx[ps].active && pl < P) off2[ps] = load_offset(bpx[ps], pl);
         }
 
         // ---- (b) Sim = q . key over the window: this wave's blocks of 16 cells
@@ -686,7 +723,8 @@ deform_fused_wmat_kernel(const T *__restrict__ q, const T *__restrict__ key,
                 Tap<float> tp = {};
                 tap_setup(kh, kw, H, W, tp);
                 const T *kp = key + (long)n * lpix * Cq + g * d;
-                const T *qp = q + px.hp * Cq + g * d;
+                const T *qp = NCHW ? q + ((long)n * Cq + g * d) * hpl + px.pp : q + px.hp * Cq + g * d;
+                const long qcs = NCHW ? hpl : 1;        // from one channel of the pixel to the next
                 for (int c = 0; c < d; ++c) {
                     const float v1 = tp.m1 ? (float)kp[(long)tp.i1 * Cq + c] : 0.f;
                     const float v2 = tp.m2 ? (float)kp[(long)tp.i2 * Cq + c] : 0.f;
@@ -696,7 +734,7 @@ deform_fused_wmat_kernel(const T *__restrict__ q, const T *__restrict__ key,
                     v = fma_(tp.w2, v2, v);
                     v = fma_(tp.w3, v3, v);
                     v = fma_(tp.w4, v4, v);
-                    lg = fma_(v, (float)qp[c], lg);
+                    lg = fma_(v, (float)qp[c * qcs], lg);
                 }
             }
             // softmax over the pixel's points = the lanes pt < P of its group of NL lanes
@@ -791,10 +829,30 @@ deform_fused_wmat_kernel(const T *__restrict__ q, const T *__restrict__ key,
                 }
                 __syncthreads();
             }
-            // a row of 16 lanes stores its pixel's 64 channels: 256 contiguous bytes
-            if (spx.active && 4 * sq < cvalid)
+            if (NCHW) {
+                // a thread stores one row of the tile in one channel plane: 4
+                // contiguous pixels.  Plain stores: the rest of each line comes from
+                // the neighbouring tiles, and the L2 puts the pieces together.
+                const int ch = tid / TPW, row = tid % TPW, qh = y0 + row;
+                if (ch < cvalid && qh < hH) {
+                    const f32x4 v = {Sl[(row * TPW + 0) * VS + ch], Sl[(row * TPW + 1) * VS + ch],
+                                     Sl[(row * TPW + 2) * VS + ch], Sl[(row * TPW + 3) * VS + ch]};
+                    union { T h[4]; Raw r; } x;
+                    x.r = Q4::narrow(v);
+                    T *op = out + ((long)n * C + cbase + ch) * hpl + (long)qh * hW + x0;
+                    if (hW % TPW == 0 && (uintptr_t)out % sizeof(Raw) == 0) {
+                        *(Raw *)op = x.r;
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < TPW; ++e)
+                            if (x0 + e < hW) op[e] = x.h[e];
+                    }
+                }
+            } else if (spx.active && 4 * sq < cvalid) {
+                // a row of 16 lanes stores its pixel's 64 channels: 256 contiguous bytes
                 __builtin_nontemporal_store(Q4::narrow(*(const f32x4 *)(Sl + srow * VS + 4 * sq)),
                                             (Raw *)(out + spx.hp * C + cbase + 4 * sq));
+            }
             if (vc + 1 < nVc) {
                 __syncthreads();        // everyone is done with this chunk's window and tile
                 stage_store(VS, 16);
@@ -804,29 +862,29 @@ deform_fused_wmat_kernel(const T *__restrict__ q, const T *__restrict__ key,
     }
 }
 
-template <typename T, int S, int DP>
+template <typename T, int S, int DP, bool NCHW>
 static hipError_t launch_wmat(const void *q, const void *key, const void *value, const void *offset,
                               void *out, int B, int Cq, int C, int H, int W, int P, int G,
-                              hipStream_t st) {
+                              hipStream_t st, int olayout) {
     const int tiles_x = (W * S + TPW - 1) / TPW, tiles_y = (H * S + TPW - 1) / TPW;
     const long nb = (long)tiles_x * tiles_y * B;
     if (nb > (1L << 30)) return hipErrorNotSupported;
     const int per_xcd = (int)((nb + 7) / 8);
-    hipLaunchKernelGGL((deform_fused_wmat_kernel<T, S, DP>), dim3(per_xcd * 8), dim3(256), 0, st,
+    hipLaunchKernelGGL((deform_fused_wmat_kernel<T, S, DP, NCHW>), dim3(per_xcd * 8), dim3(256), 0, st,
                        (const T *)q, (const T *)key, (const T *)value, (const T *)offset, (T *)out,
-                       Cq, C, H, W, P, G, tiles_x, tiles_y, (int)nb, per_xcd);
+                       Cq, C, H, W, P, G, tiles_x, tiles_y, (int)nb, per_xcd, olayout);
     return hipGetLastError();
 }
 
-template <typename T>
+template <typename T, bool NCHW = false>
 static hipError_t launch_wmat_t(const void *q, const void *key, const void *value, const void *offset,
                                 void *out, int B, int Cq, int C, int H, int W, int P, int s, int G,
-                                hipStream_t st) {
+                                hipStream_t st, int olayout = OFFSET_HIRES) {
     const int d = Cq / G;
 #define SAPA_WMAT(SV)                                                                               \
     case SV:                                                                                        \
-        return d <= 32 ? launch_wmat<T, SV, 32>(q, key, value, offset, out, B, Cq, C, H, W, P, G, st) \
-                       : launch_wmat<T, SV, 64>(q, key, value, offset, out, B, Cq, C, H, W, P, G, st);
+        return d <= 32 ? launch_wmat<T, SV, 32, NCHW>(q, key, value, offset, out, B, Cq, C, H, W, P, G, st, olayout) \
+                       : launch_wmat<T, SV, 64, NCHW>(q, key, value, offset, out, B, Cq, C, H, W, P, G, st, olayout);
     switch (s) {
         SAPA_WMAT(1) SAPA_WMAT(2) SAPA_WMAT(4)
         default: return hipErrorNotSupported;
@@ -884,6 +942,66 @@ hipError_t deform_fused_nhwc_launch(const void *q, const void *key, const void *
         case 0: return dnhwc::launch_t<float>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);
         case 2: return dnhwc::launch_t<f16_t>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);
         case 3: return dnhwc::launch_t<bf16_t>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);
+        default: return hipErrorNotSupported;
+    }
+}
+
+// ---- contiguous (NCHW) callers through the matrix-form kernels -------------
+// The kernels above read q and the offsets and write the output in place in
+// the contiguous layout (NCHW = true); only the low-res key and value are
+// copied into channels-last order first, into a workspace of the caller.
+
+static long align256(long x) { return (x + 255) / 256 * 256; }
+
+// Bytes of workspace, or 0 when the contiguous-layout kernels serve the case
+// (shapes the matrix form does not cover, or too few points for it to pay).
+long deform_fused_nchw_workspace(int B, int Cq, int C, int H, int W, int P, int s, int G, int dtype) {
+    if (dtype != 0 && dtype != 2 && dtype != 3) return 0;
+    if (s != 1 && s != 2 && s != 4) return 0;
+    if (G <= 0 || Cq % G != 0 || C % G != 0) return 0;
+    const int d = Cq / G, cg = C / G;
+    if (P > 32 || d % 4 != 0 || d > 64 || cg % 4 != 0) return 0;
+    const int esize = dtype == 0 ? 4 : 2;
+    const long plane = (long)H * W * esize;
+    if (plane * Cq >= (1L << 31) || plane * C >= (1L << 31)) return 0;
+    if ((long)H * s * W * s >= (1L << 31)) return 0;
+    // Where this path is the faster one (B=8, C=256, G=4, d=32, 64x64 -> 128x128, us,
+    // the two copies included, against the contiguous-layout kernels): fp32 P = 25
+    // 336 / 498, P = 9 296 / 212; bf16 on the 16-bit kernel P = 25 218 / 471, P = 9
+    // 161 / 199, P = 5 156 / 154.
+    const bool wm16 = dtype != 0 && d % 8 == 0 && cg % 8 == 0;
+    if (P < (wm16 ? 6 : 15)) return 0;
+    return align256((long)B * plane * Cq) + align256((long)B * plane * C);
+}
+
+hipError_t deform_fused_nchw_ws_launch(const void *q, const void *key, const void *value,
+                                       const void *offset, void *out, void *workspace, int B, int Cq,
+                                       int C, int H, int W, int P, int s, int G, int olayout,
+                                       int dtype, hipStream_t st, const char **kernel) {
+    const char *unused;
+    if (!kernel) kernel = &unused;
+    if (olayout != OFFSET_HIRES && olayout != OFFSET_PIXEL_SHUFFLE && olayout != OFFSET_NEAREST)
+        return hipErrorNotSupported;
+    if (!workspace || (uintptr_t)workspace % 256 != 0) return hipErrorNotSupported;
+    if (deform_fused_nchw_workspace(B, Cq, C, H, W, P, s, G, dtype) == 0) return hipErrorNotSupported;
+    const int esize = dtype == 0 ? 4 : 2;
+    const long lpix = (long)H * W;
+    char *key_cl = (char *)workspace;
+    char *value_cl = key_cl + align256((long)B * lpix * Cq * esize);
+    hipError_t e = nchw_to_nhwc_launch(key, key_cl, B, Cq, lpix, esize, st);
+    if (e != hipSuccess) return e;
+    e = nchw_to_nhwc_launch(value, value_cl, B, C, lpix, esize, st);
+    if (e != hipSuccess) return e;
+    if (dtype != 0) {
+        *kernel = "deform_fused_wmat16_kernel";
+        e = deform_fused_wmat16_launch(q, key_cl, value_cl, offset, out, B, Cq, C, H, W, P, s, G, dtype, st, true, olayout);
+        if (e != hipErrorNotSupported) return e;
+    }
+    *kernel = "deform_fused_wmat_kernel";
+    switch (dtype) {
+        case 0: return dnhwc::launch_wmat_t<float, true>(q, key_cl, value_cl, offset, out, B, Cq, C, H, W, P, s, G, st, olayout);
+        case 2: return dnhwc::launch_wmat_t<f16_t, true>(q, key_cl, value_cl, offset, out, B, Cq, C, H, W, P, s, G, st, olayout);
+        case 3: return dnhwc::launch_wmat_t<bf16_t, true>(q, key_cl, value_cl, offset, out, B, Cq, C, H, W, P, s, G, st, olayout);
         default: return hipErrorNotSupported;
     }
 }

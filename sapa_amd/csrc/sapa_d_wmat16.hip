@@ -134,12 +134,15 @@ __device__ __forceinline__ u32x4 narrow8(f32x4 a, f32x4 b) {
 #ifndef SAPA_WM16_VPAD
 #define SAPA_WM16_VPAD 8
 #endif
-template <typename T, int S, int TH, int TW, int DP>
+// NCHW: query, offset and out are contiguous [B, channels, sH, sW] tensors (the
+// reference's layout); key and value are channels-last either way (the launcher
+// hands copies in that order to this kernel).
+template <typename T, int S, int TH, int TW, int DP, bool NCHW>
 __global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(SAPA_WM16_WPE, SAPA_WM16_WPE)))
 deform_fused_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key,
                            const T *__restrict__ value, const T *__restrict__ offset,
                            T *__restrict__ out, int Cq, int C, int H, int W, int P, int G,
-                           int tiles_x, int tiles_y, int nblocks, int per_xcd) {
+                           int tiles_x, int tiles_y, int nblocks, int per_xcd, int olayout) {
     constexpr int NPX = TH * TW, NMB = NPX / 16;             // pixels, blocks of 16 matrix rows
     constexpr int WWY = (TH + S - 1) / S + 2 * RCH + 1;      // window cells per axis
     constexpr int WWX = (TW + S - 1) / S + 2 * RCH + 1;
@@ -179,13 +182,15 @@ deform_fused_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key,
 
     // pixel i of the tile (row-major): inside the image?  its flat hi-res index,
     // clamped for loads, and its parent
-    struct Pix { bool active; long hp; int ph, pw; };
+    struct Pix { bool active; long hp; int pp, ph, pw; };
+    const long hpl = (long)hH * hW;                                  // a hi-res channel plane (NCHW)
     auto pixel = [&](int i) __attribute__((always_inline)) {
         const int qh = y0 + i / TW, qw = x0 + i % TW;
         Pix r;
         r.active = qh < hH && qw < hW;
         const int ch = qh < hH ? qh : hH - 1, cw = qw < hW ? qw : hW - 1;
-        r.hp = (long)n * hH * hW + (long)ch * hW + cw;
+        r.pp = ch * hW + cw;
+        r.hp = (long)n * hH * hW + r.pp;
         r.ph = ch / S;
         r.pw = cw / S;
         return r;
@@ -256,8 +261,18 @@ deform_fused_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key,
 #pragma unroll
             for (int ks = 0; ks < DP / 32; ++ks) {
                 qa[mb][ks] = u32x4{0u, 0u, 0u, 0u};
-                if (px.active && 32 * ks + 8 * mk < d)
-                    qa[mb][ks] = *(const u32x4 *)(q + px.hp * Cq + g * d + 32 * ks + 8 * mk);
+                if (px.active && 32 * ks + 8 * mk < d) {
+                    if (NCHW) {
+                        // 8 channel planes, one element each
+                        const T *qp = q + ((long)n * Cq + g * d + 32 * ks + 8 * mk) * hpl + px.pp;
+                        union { T h[8]; u32x4 u; } x;
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) x.h[e] = qp[e * hpl];
+                        qa[mb][ks] = x.u;
+                    } else {
+                        qa[mb][ks] = *(const u32x4 *)(q + px.hp * Cq + g * d + 32 * ks + 8 * mk);
+                    }
+                }
             }
         }
     };
@@ -280,8 +295,33 @@ deform_fused_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key,
             offnext[ps] = 0u;
             if (ps < nsp) {
                 const Pix px = pixel(ps * ppp + prow);
-                if (px.active && pt < P)
-                    offnext[ps] = *(const u32 *)(offset + px.hp * (2L * G * P) + 2L * ((long)g * P + pt));
+                if (px.active && pt < P) {
+                    if (NCHW) {
+                        // channel cx = dx, cx + 1 = dy of the point, from the hi-res tensor
+                        // or from the low-res one it is a pixel shuffle / a nearest
+                        // interpolation of (deform_tap.hpp: OffsetLayout)
+                        const long cx = (long)n * 2 * G * P + 2L * ((long)g * P + pt);
+                        const T *op;
+                        long dy;
+                        if (olayout == OFFSET_PIXEL_SHUFFLE) {
+                            const int qh = px.pp / hW, qw = px.pp % hW;
+                            op = offset + (cx * (S * S) + (qh % S) * S + qw % S) * lpix + (long)px.ph * W + px.pw;
+                            dy = (long)(S * S) * lpix;
+                        } else if (olayout == OFFSET_NEAREST) {
+                            op = offset + cx * lpix + (long)px.ph * W + px.pw;
+                            dy = lpix;
+                        } else {
+                            op = offset + cx * hpl + px.pp;
+                            dy = hpl;
+                        }
+                        union { T h[2]; u32 u; } x;
+                        x.h[0] = op[0];
+                        x.h[1] = op[dy];
+                        offnext[ps] = x.u;
+                    } else {
+                        offnext[ps] = *(const u32 *)(offset + px.hp * (2L * G * P) + 2L * ((long)g * P + pt));
+                    }
+                }
             }
         }
     };
@@ -353,7 +393,8 @@ deform_fused_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key,
                 Tap<float> tp = {};
                 tap_setup(kh, kw, H, W, tp);
                 const T *kp = key + (long)n * lpix * Cq + g * d;
-                const T *qp = q + px.hp * Cq + g * d;
+                const T *qp = NCHW ? q + ((long)n * Cq + g * d) * hpl + px.pp : q + px.hp * Cq + g * d;
+                const long qcs = NCHW ? hpl : 1;        // from one channel of the pixel to the next
                 for (int c = 0; c < d; ++c) {
                     const float v1 = tp.m1 ? (float)kp[(long)tp.i1 * Cq + c] : 0.f;
                     const float v2 = tp.m2 ? (float)kp[(long)tp.i2 * Cq + c] : 0.f;
@@ -363,7 +404,7 @@ deform_fused_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key,
                     v = fma_(tp.w2, v2, v);
                     v = fma_(tp.w3, v3, v);
                     v = fma_(tp.w4, v4, v);
-                    lg = fma_(v, (float)qp[c], lg);
+                    lg = fma_(v, (float)qp[c * qcs], lg);
                 }
             }
             // softmax over the pixel's points = the lanes pt < P of its group of NL lanes
@@ -482,15 +523,44 @@ deform_fused_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key,
                 }
                 __syncthreads();
             }
-            // 8 lanes store a pixel's 64 channels: 128 contiguous bytes
+            if (NCHW) {
+                // a thread stores one row of the tile in one channel plane: TW
+                // contiguous pixels.  Plain stores: the rest of each line comes from
+                // the neighbouring tiles, and the L2 puts the pieces together.
+                static_assert(TW == 4 || TW == 8, "a tile row is one 8- or 16-byte store");
+                typedef u32 RowVec __attribute__((ext_vector_type(TW / 2)));
+                const bool ovec = hW % TW == 0 && (uintptr_t)out % (TW * sizeof(T)) == 0;
 #pragma unroll
-            for (int sp = 0; sp < (NPX + 31) / 32; ++sp) {
-                const int pi = sp * 32 + tid / 8;
-                if (NPX % 32 != 0 && pi >= NPX) break;
-                const Pix px = pixel(pi);
-                if (px.active && 8 * c8 < cvalid) {
-                    const f32x4 *op = (const f32x4 *)(Ol + pi * OS + 8 * c8);
-                    __builtin_nontemporal_store(narrow8<T>(op[0], op[1]), (u32x4 *)(out + px.hp * C + cbase + 8 * c8));
+                for (int it = 0; it < (CHK * TH + NT - 1) / NT; ++it) {
+                    const int item = it * NT + tid;
+                    const int ch = item / TH, row = item % TH;
+                    if ((CHK * TH) % NT != 0 && item >= CHK * TH) break;
+                    const int qh = y0 + row;
+                    if (ch < cvalid && qh < hH) {
+                        union { T h[TW]; RowVec v; } x;
+#pragma unroll
+                        for (int e = 0; e < TW; ++e) x.h[e] = (T)Ol[(row * TW + e) * OS + ch];
+                        T *op = out + ((long)n * C + cbase + ch) * hpl + (long)qh * hW + x0;
+                        if (ovec && x0 + TW <= hW) {
+                            *(RowVec *)op = x.v;
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < TW; ++e)
+                                if (x0 + e < hW) op[e] = x.h[e];
+                        }
+                    }
+                }
+            } else {
+                // 8 lanes store a pixel's 64 channels: 128 contiguous bytes
+#pragma unroll
+                for (int sp = 0; sp < (NPX + 31) / 32; ++sp) {
+                    const int pi = sp * 32 + tid / 8;
+                    if (NPX % 32 != 0 && pi >= NPX) break;
+                    const Pix px = pixel(pi);
+                    if (px.active && 8 * c8 < cvalid) {
+                        const f32x4 *op = (const f32x4 *)(Ol + pi * OS + 8 * c8);
+                        __builtin_nontemporal_store(narrow8<T>(op[0], op[1]), (u32x4 *)(out + px.hp * C + cbase + 8 * c8));
+                    }
                 }
             }
             if (vc + 1 < nVc) {
@@ -502,17 +572,17 @@ deform_fused_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key,
     }
 }
 
-template <typename T, int S, int TH, int TW, int DP>
+template <typename T, int S, int TH, int TW, int DP, bool NCHW>
 static hipError_t launch_tile(const void *q, const void *key, const void *value, const void *offset,
                               void *out, int B, int Cq, int C, int H, int W, int P, int G,
-                              hipStream_t st) {
+                              hipStream_t st, int olayout) {
     const int tiles_x = (W * S + TW - 1) / TW, tiles_y = (H * S + TH - 1) / TH;
     const long nb = (long)tiles_x * tiles_y * B;
     if (nb > (1L << 30)) return hipErrorNotSupported;
     const int per_xcd = (int)((nb + 7) / 8);
-    hipLaunchKernelGGL((deform_fused_wmat16_kernel<T, S, TH, TW, DP>), dim3(per_xcd * 8), dim3(NT), 0, st,
+    hipLaunchKernelGGL((deform_fused_wmat16_kernel<T, S, TH, TW, DP, NCHW>), dim3(per_xcd * 8), dim3(NT), 0, st,
                        (const T *)q, (const T *)key, (const T *)value, (const T *)offset, (T *)out,
-                       Cq, C, H, W, P, G, tiles_x, tiles_y, (int)nb, per_xcd);
+                       Cq, C, H, W, P, G, tiles_x, tiles_y, (int)nb, per_xcd, olayout);
     return hipGetLastError();
 }
 
@@ -520,15 +590,15 @@ static hipError_t launch_tile(const void *q, const void *key, const void *value,
 #define SAPA_WM16_TILE 4, 4
 #endif
 
-template <typename T>
+template <typename T, bool NCHW>
 static hipError_t launch_t(const void *q, const void *key, const void *value, const void *offset,
                            void *out, int B, int Cq, int C, int H, int W, int P, int s, int G,
-                           hipStream_t st) {
+                           hipStream_t st, int olayout) {
     const int d = Cq / G;
 #define SAPA_WM16(SV)                                                                                  \
     case SV:                                                                                           \
-        return d <= 32 ? launch_tile<T, SV, SAPA_WM16_TILE, 32>(q, key, value, offset, out, B, Cq, C, H, W, P, G, st) \
-                       : launch_tile<T, SV, SAPA_WM16_TILE, 64>(q, key, value, offset, out, B, Cq, C, H, W, P, G, st);
+        return d <= 32 ? launch_tile<T, SV, SAPA_WM16_TILE, 32, NCHW>(q, key, value, offset, out, B, Cq, C, H, W, P, G, st, olayout) \
+                       : launch_tile<T, SV, SAPA_WM16_TILE, 64, NCHW>(q, key, value, offset, out, B, Cq, C, H, W, P, G, st, olayout);
     switch (s) {
         SAPA_WM16(1) SAPA_WM16(2) SAPA_WM16(4)
         default: return hipErrorNotSupported;
@@ -538,22 +608,30 @@ static hipError_t launch_t(const void *q, const void *key, const void *value, co
 
 }  // namespace dwm16
 
-// f16 / bf16 channels-last tensors, s in {1, 2, 4}, P <= 32, channels per group
-// (Cq / G and C / G) multiples of 8, Cq / G <= 64, tensors aligned to 16 bytes,
-// one image's key / value tensor below 2^31 bytes.  hipErrorNotSupported otherwise.
+// f16 / bf16 tensors, s in {1, 2, 4}, P <= 32, channels per group (Cq / G and
+// C / G) multiples of 8, Cq / G <= 64, one image's key / value tensor below 2^31
+// bytes.  key and value in channels-last order, aligned to 16 bytes; query, offset
+// and out either channels-last too (query and out aligned to 16 bytes, offset to
+// 4) or, nchw = true, contiguous [B, channels, sH, sW] with one plane below 2^31
+// elements, the offsets in the layout olayout names (deform_tap.hpp).
+// hipErrorNotSupported otherwise.
 hipError_t deform_fused_wmat16_launch(const void *q, const void *key, const void *value,
                                       const void *offset, void *out, int B, int Cq, int C, int H,
-                                      int W, int P, int s, int G, int dtype, hipStream_t st) {
+                                      int W, int P, int s, int G, int dtype, hipStream_t st, bool nchw, int olayout) {
     if (dtype != 2 && dtype != 3) return hipErrorNotSupported;
     if (P > 32 || (Cq / G) % 8 != 0 || Cq / G > 64 || (C / G) % 8 != 0) return hipErrorNotSupported;
     const long plane = (long)H * W * 2;
     if (plane * Cq >= (1L << 31) || plane * C >= (1L << 31)) return hipErrorNotSupported;
-    const void *ptrs[4] = {q, key, value, out};
-    for (const void *p : ptrs)
-        if ((uintptr_t)p % 16 != 0) return hipErrorNotSupported;
-    if ((uintptr_t)offset % 4 != 0) return hipErrorNotSupported;
-    return dtype == 2 ? dwm16::launch_t<f16_t>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st)
-                      : dwm16::launch_t<bf16_t>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st);
+    if ((uintptr_t)key % 16 != 0 || (uintptr_t)value % 16 != 0) return hipErrorNotSupported;
+    if (nchw) {
+        // the pixel index within a plane and the row stores use 32-bit arithmetic
+        if ((long)H * s * W * s >= (1L << 31)) return hipErrorNotSupported;
+        return dtype == 2 ? dwm16::launch_t<f16_t, true>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st, olayout)
+                          : dwm16::launch_t<bf16_t, true>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st, olayout);
+    }
+    if ((uintptr_t)q % 16 != 0 || (uintptr_t)out % 16 != 0 || (uintptr_t)offset % 4 != 0) return hipErrorNotSupported;
+    return dtype == 2 ? dwm16::launch_t<f16_t, false>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st, OFFSET_HIRES)
+                      : dwm16::launch_t<bf16_t, false>(q, key, value, offset, out, B, Cq, C, H, W, P, s, G, st, OFFSET_HIRES);
 }
 
 }  // namespace sapa

@@ -1,0 +1,53 @@
+// Layout helpers: a contiguous [B, C, H*W] tensor copied into channels-last
+// order [B, H*W, C].  The matrix-form SAPA-D kernels read their low-res key and
+// value windows in channels-last order (a window cell's channels are one
+// contiguous piece); for callers with the reference's contiguous tensors
+// (deformsapa/deformsapa/src/cuda/deform_qk_cuda.cpp:37-43: CHECK_CONTIGUOUS)
+// these two small tensors are copied into a caller-provided workspace first,
+// while the large hi-res tensors are read and written in place.
+#include "kernels.hpp"
+
+namespace sapa {
+
+namespace layout {
+
+// 64 pixels x 64 channels per workgroup through LDS: reads run along the
+// pixels of a channel plane, writes along the channels of a pixel.
+template <typename U>
+__global__ void __launch_bounds__(256)
+nchw_to_nhwc_kernel(const U *__restrict__ src, U *__restrict__ dst, int C, long HW) {
+    __shared__ U tile[64][65];
+    const long p0 = (long)blockIdx.x * 64;
+    const int c0 = (int)blockIdx.y * 64;
+    const long n = blockIdx.z;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int c = ty; c < 64; c += 4)
+        tile[c][tx] = (c0 + c < C && p0 + tx < HW) ? src[(n * C + c0 + c) * HW + p0 + tx] : (U)0;
+    __syncthreads();
+    for (int p = ty; p < 64; p += 4)
+        if (c0 + tx < C && p0 + p < HW) dst[(n * HW + p0 + p) * C + c0 + tx] = tile[tx][p];
+}
+
+}  // namespace layout
+
+// esize: bytes per element, 2 or 4.  hipErrorNotSupported otherwise, or for more
+// than 65535 images or 64-channel blocks.
+hipError_t nchw_to_nhwc_launch(const void *src, void *dst, int B, int C, long HW, int esize,
+                               hipStream_t st) {
+    if (B <= 0 || C <= 0 || HW <= 0) return hipSuccess;
+    const long gx = (HW + 63) / 64;
+    const int gy = (C + 63) / 64;
+    if (gx > 0x7fffffffL || gy > 65535 || B > 65535) return hipErrorNotSupported;
+    const dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)B);
+    if (esize == 2)
+        hipLaunchKernelGGL(layout::nchw_to_nhwc_kernel<unsigned short>, grid, dim3(256), 0, st,
+                           (const unsigned short *)src, (unsigned short *)dst, C, HW);
+    else if (esize == 4)
+        hipLaunchKernelGGL(layout::nchw_to_nhwc_kernel<unsigned>, grid, dim3(256), 0, st, (const unsigned *)src,
+                           (unsigned *)dst, C, HW);
+    else
+        return hipErrorNotSupported;
+    return hipGetLastError();
+}
+
+}  // namespace sapa

@@ -208,7 +208,7 @@ class DeformSAPAFusedFunction(Function):
 
     @staticmethod
     def forward(ctx, query, key, value, offset, num_point, scale_factor, groups,
-                offset_layout='hires'):
+                offset_layout='hires', matrix_form=None):
         if offset_layout not in OFFSET_LAYOUTS:
             raise ValueError('offset_layout must be one of %s' % sorted(OFFSET_LAYOUTS))
         assert scale_factor >= 1
@@ -247,10 +247,27 @@ class DeformSAPAFusedFunction(Function):
                            key.size(1), c, h, w, num_point, scale_factor, groups,
                            _lib.dtype_code(value))
         else:
-            _lib.call('sapa_deform_fused_forward_from', value.device, _lib.ptr(query),
-                      _lib.ptr(key), _lib.ptr(value), _lib.ptr(offset), _lib.ptr(output), n,
-                      key.size(1), c, h, w, num_point, scale_factor, groups,
-                      OFFSET_LAYOUTS[offset_layout], _lib.dtype_code(value))
+            # contiguous tensors: through the matrix-form kernels where they serve the
+            # case (key and value go through a workspace in channels-last order),
+            # else the contiguous-layout kernels
+            shape = (n, key.size(1), c, h, w, num_point, scale_factor, groups, _lib.dtype_code(value))
+            nbytes = _lib.lib().sapa_deform_fused_forward_workspace(*shape)
+            if matrix_form is None:
+                # fp32 keeps the reference's order of sums unless asked otherwise
+                matrix_form = value.dtype != torch.float32
+            elif matrix_form and nbytes == 0:
+                raise _lib.SapaUnsupported('deform_sapa_fused(matrix_form=True): this configuration is served '
+                                           'by the contiguous-layout kernels only')
+            if matrix_form and nbytes > 0:
+                ws = torch.empty(nbytes, dtype=torch.uint8, device=value.device)
+                _lib.call('sapa_deform_fused_forward_ws', value.device, _lib.ptr(query),
+                          _lib.ptr(key), _lib.ptr(value), _lib.ptr(offset), _lib.ptr(output),
+                          _lib.ptr(ws), *shape[:-1], OFFSET_LAYOUTS[offset_layout], shape[-1])
+            else:
+                _lib.call('sapa_deform_fused_forward_from', value.device, _lib.ptr(query),
+                          _lib.ptr(key), _lib.ptr(value), _lib.ptr(offset), _lib.ptr(output), n,
+                          key.size(1), c, h, w, num_point, scale_factor, groups,
+                          OFFSET_LAYOUTS[offset_layout], _lib.dtype_code(value))
 
         if any(t.requires_grad for t in (query, key, value, offset)):
             ctx.save_for_backward(query, key, value, offset)
@@ -263,10 +280,16 @@ class DeformSAPAFusedFunction(Function):
         gq, gk, gv, goff = _deform_fused_backward(
             grad_output, query, key, value, offset, ctx.num_point, ctx.scale_factor, ctx.groups,
             ctx.offset_layout)
-        return gq, gk, gv, goff, None, None, None, None
+        return gq, gk, gv, goff, None, None, None, None, None
 
 
 def deform_sapa_fused(query, key, value, offset, num_point, scale_factor, groups,
-                      offset_layout='hires'):
+                      offset_layout='hires', matrix_form=None):
+    """deform_qk -> softmax over the points -> deform_av (sapa_deform.py:51-53) in one
+    launch.  matrix_form (contiguous tensors): True = through the matrix-form kernels
+    (sums per window cell: rounding-level differences from the reference's order in
+    fp32; SapaUnsupported where they do not serve the configuration), False = the
+    reference's order of sums, None = matrix form for 16-bit tensors where it is the
+    faster one, the reference's order for fp32."""
     return DeformSAPAFusedFunction.apply(query, key, value, offset, num_point, scale_factor,
-                                         groups, offset_layout)
+                                         groups, offset_layout, matrix_form)

@@ -272,6 +272,12 @@ def test_c4_deform_against_oracle(coracle, P):
                                         images=(0, 3, B - 1))
     exact = per_image(coracle.deform_sapa_fused, [t.double() for t in sub(q, key, v, off)], P, s, G, 'f64')
     assert_no_worse_than_reference_order(got_cl[list(imgs)], want_f, exact, f'c4 P={P} fused channels_last')
+    if P >= 15:
+        # contiguous tensors through the same matrix-form kernel (key and value via a workspace)
+        fused_m = lambda a, b, c, o: sapa_amd.deform_sapa_fused(a, b, c, o, P, s, G, matrix_form=True)
+        got_m = assert_batch_equals_images(fused_m, (qd, kd, vd, od), f'c4 P={P} fused matrix form', images=(0, 3, B - 1))
+        assert got_m.is_contiguous()
+        assert_no_worse_than_reference_order(got_m[list(imgs)], want_f, exact, f'c4 P={P} fused matrix form')
     # 16-bit tensors, contiguous and channels_last
     hq, hk, hv, ho = (t.to(torch.bfloat16) for t in (qd, kd, vd, od))
     exact16 = per_image(coracle.deform_sapa_fused, [t[list(imgs)].double().cpu() for t in (hq, hk, hv, ho)],

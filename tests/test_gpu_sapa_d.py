@@ -61,6 +61,72 @@ def test_deform_fused_fp32(coracle, shape):
     torch.testing.assert_close(got.double(), want64, rtol=1e-4, atol=1e-5)
 
 
+# Contiguous tensors through the matrix-form kernels (key and value copied to
+# channels-last order in a workspace, q / offset / out used in place).
+# B, G, dq, cg, H, W, P, s, offset scale: far offsets with 16 lanes per pixel and
+# rows that are no multiple of the 4-pixel tile (26 and 6 pixels wide); 48 channels
+# padded to 64 at s = 4; s = 1; three value chunks (64 + 64 + 8); groups that are
+# not whole 16-byte pieces (16-bit tensors then stay on the fp32-in-LDS kernel)
+MATRIX_SHAPES = [(1, 4, 32, 64, 8, 8, 25, 2, 0.75), (2, 2, 8, 16, 14, 13, 16, 2, 6.0),
+                 (1, 2, 48, 24, 7, 9, 15, 4, 2.5), (2, 1, 16, 40, 11, 6, 29, 1, 3.0),
+                 (1, 1, 64, 136, 5, 7, 21, 2, 1.5), (1, 2, 12, 20, 6, 5, 17, 2, 1.0)]
+MATRIX_IDS = ['-'.join(map(str, s)) for s in MATRIX_SHAPES]
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('shape', MATRIX_SHAPES, ids=MATRIX_IDS)
+def test_deform_fused_matrix_form_on_contiguous_tensors(coracle, shape, dtype):
+    from sapa_amd import _lib
+    B, G, dq, cg, H, W, P, s, oscale = shape
+    q, key, v, off, _ = make(gen(230), shape[:8], off_scale=oscale)
+    q, key, v, off = (t.to(dtype) for t in (q, key, v, off))
+    want = coracle.deform_sapa_fused(q.float(), key.float(), v.float(), off.float(), P, s, G, 'f32')
+    got = sapa_amd.deform_sapa_fused(*dev(q, key, v, off), P, s, G, matrix_form=True)
+    kernel = _lib.last_kernel()
+    assert got.is_contiguous() and got.dtype == dtype and got.shape == want.shape
+    if dtype == torch.float32:
+        assert kernel == 'deform_fused_wmat_kernel'
+        if dq <= 8:
+            assert_f32_close(got, want, 'matrix form')
+        else:   # the reference's own check tolerance (deformsapa/deformsapa/forward_check.py)
+            torch.testing.assert_close(got.cpu(), want, rtol=1e-5, atol=1e-5)
+        # the default for fp32 stays the reference's order of sums
+        plain = sapa_amd.deform_sapa_fused(*dev(q, key, v, off), P, s, G)
+        assert _lib.last_kernel() != kernel
+        assert_f32_close(plain, want, 'default path')
+    else:
+        assert kernel == ('deform_fused_wmat16_kernel' if dq % 8 == 0 and cg % 8 == 0 else 'deform_fused_wmat_kernel')
+        assert_rel_rms_close(got.float(), want, BF16_REL if dtype == torch.bfloat16 else F16_REL, 'matrix form')
+        # 16-bit tensors take it by default
+        auto = sapa_amd.deform_sapa_fused(*dev(q, key, v, off), P, s, G)
+        assert _lib.last_kernel() == kernel and torch.equal(auto, got)
+        sapa_amd.deform_sapa_fused(*dev(q, key, v, off), P, s, G, matrix_form=False)
+        assert _lib.last_kernel() != kernel
+    # the offsets read in place from the low-res convolution output (sapa_deform.py:44-47)
+    from sapa_amd.deform_func import expand_offset
+    for layout in ('pixel_shuffle', 'nearest'):
+        lo = _lowres_offsets(gen(233), shape[:8], layout, dtype=dtype).to(DEV)
+        hi = expand_offset(lo, s, layout).contiguous()
+        a = sapa_amd.deform_sapa_fused(*dev(q, key, v), hi, P, s, G, matrix_form=True)
+        b = sapa_amd.deform_sapa_fused(*dev(q, key, v), lo, P, s, G, layout, matrix_form=True)
+        assert _lib.last_kernel() == kernel and torch.equal(a, b), layout
+
+
+def test_deform_fused_matrix_form_limits():
+    """Too few points for the matrix form to pay, fp64, and the low-res offset
+    layouts stay on the contiguous-layout kernels; asking for it explicitly raises."""
+    from sapa_amd import _lib
+    shape = (1, 2, 8, 8, 6, 7, 5, 2)
+    q, key, v, off, _ = make(gen(231), shape)
+    with pytest.raises(_lib.SapaUnsupported):
+        sapa_amd.deform_sapa_fused(*dev(q, key, v, off), 5, 2, 2, matrix_form=True)
+    h = sapa_amd.deform_sapa_fused(*dev(*(t.half() for t in (q, key, v, off))), 5, 2, 2)
+    assert _lib.last_kernel() not in ('deform_fused_wmat_kernel', 'deform_fused_wmat16_kernel') and h.dtype == torch.float16
+    q, key, v, off, _ = make(gen(232), (1, 2, 8, 8, 6, 7, 17, 2), dtype=torch.float64)
+    with pytest.raises(_lib.SapaUnsupported):
+        sapa_amd.deform_sapa_fused(*dev(q, key, v, off), 17, 2, 2, matrix_form=True)
+
+
 def test_golden_vectors():
     G = golden()
     t = lambda a: torch.from_numpy(a)
@@ -283,10 +349,13 @@ def test_offsets_read_in_place_fp64_and_bf16():
         q, key, v, _, _ = make(g, shape, dtype=dtype)
         lo = _lowres_offsets(g, shape, 'pixel_shuffle', dtype=dtype)
         q, key, v, lo = dev(q, key, v, lo)
-        want = sapa_amd.deform_sapa_fused(q, key, v, expand_offset(lo, s, 'pixel_shuffle').contiguous(),
-                                          P, s, G)
-        got = sapa_amd.deform_sapa_fused(q, key, v, lo, P, s, G, 'pixel_shuffle')
-        assert torch.equal(got, want), str(dtype)
+        # on either kernel family (bf16: the matrix form by default) the result is the
+        # same bit for bit as with the hi-res offsets written out first
+        for mf in (None, False):
+            want = sapa_amd.deform_sapa_fused(q, key, v, expand_offset(lo, s, 'pixel_shuffle').contiguous(),
+                                              P, s, G, matrix_form=mf)
+            got = sapa_amd.deform_sapa_fused(q, key, v, lo, P, s, G, 'pixel_shuffle', matrix_form=mf)
+            assert torch.equal(got, want), f'{dtype} matrix_form={mf}'
 
 
 @pytest.mark.parametrize('layout', ['pixel_shuffle', 'nearest'])
