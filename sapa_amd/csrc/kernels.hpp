@@ -84,9 +84,10 @@ hipError_t deform_fused_nchw_ws_launch(const void *q, const void *key, const voi
                                        int C, int H, int W, int P, int s, int G, int olayout,
                                        int dtype, hipStream_t st, const char **kernel = nullptr);
 
-// sapa_layout.hip: contiguous [B, C, HW] -> channels-last [B, HW, C]; esize 2 or 4 bytes
-hipError_t nchw_to_nhwc_launch(const void *src, void *dst, int B, int C, long HW, int esize,
-                               hipStream_t st);
+// sapa_layout.hip: contiguous [B, C, HW] -> channels-last [B, HW, C] for two tensors
+// of the same B and HW in one launch (C1 = 0: one); esize 2 or 4 bytes
+hipError_t nchw_to_nhwc_launch(const void *src0, void *dst0, int C0, const void *src1, void *dst1,
+                               int C1, int B, long HW, int esize, hipStream_t st);
 
 // sapa_d_wmat16.hip: the same operator for f16 / bf16 on the 16-bit matrix
 // instructions; channels per group multiples of 8, key / value channels-last and

@@ -988,9 +988,7 @@ hipError_t deform_fused_nchw_ws_launch(const void *q, const void *key, const voi
     const long lpix = (long)H * W;
     char *key_cl = (char *)workspace;
     char *value_cl = key_cl + align256((long)B * lpix * Cq * esize);
-    hipError_t e = nchw_to_nhwc_launch(key, key_cl, B, Cq, lpix, esize, st);
-    if (e != hipSuccess) return e;
-    e = nchw_to_nhwc_launch(value, value_cl, B, C, lpix, esize, st);
+    hipError_t e = nchw_to_nhwc_launch(key, key_cl, Cq, value, value_cl, C, B, lpix, esize, st);
     if (e != hipSuccess) return e;
     if (dtype != 0) {
         *kernel = "deform_fused_wmat16_kernel";

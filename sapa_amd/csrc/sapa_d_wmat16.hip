@@ -164,6 +164,8 @@ deform_fused_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key,
     __shared__ __attribute__((aligned(16))) T Xl[XSZ];              // key window, then value window
     __shared__ __attribute__((aligned(16))) u32 SWl[NPX * WS];      // Sim (fp32), then Wm, then its 16-bit split
     __shared__ __attribute__((aligned(16))) float Ol[NPX * OS];     // output tile
+    constexpr int QSB = DP + 8;     // elements per pixel of the q tile (contiguous-layout callers)
+    __shared__ __attribute__((aligned(16))) T Ql[NCHW ? NPX * QSB : 8];
     float *const Sl = (float *)SWl;
 
     const int logical = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
@@ -252,28 +254,62 @@ deform_fused_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key,
 #pragma unroll
         for (int p = 0; p < NPV; ++p) *(u32x4 *)(Xl + (p * 32 + tid / 8) * VSB + 8 * c8) = st[p];
     };
-    // q of pixel 16 mb + mi as the A operand: channels 32 ks + 8 mk .. + 7 of the group
-    u32x4 qa[NMB][DP / 32];
+    // q of pixel 16 mb + mi as the A operand: channels 32 ks + 8 mk .. + 7 of the group.
+    // Channels-last: 16 contiguous bytes of global memory per lane.  Contiguous
+    // layout: the tile's q (NPX pixels x d channel planes) comes in once per
+    // workgroup, a thread fetching pairs of x-neighbours of one plane, and goes
+    // through LDS as [pixel][channel], from where every wave reads its operands.
+    u32x4 qa[NCHW ? 1 : NMB][DP / 32];
+    constexpr int QN = NCHW ? NPX * DP / 2 / NT : 1;     // pixel pairs per thread
+    static_assert(!NCHW || (NPX * DP / 2) % NT == 0, "the q tile divides over the threads");
+    u32 qraw[QN];
+    const bool q32 = hW % 2 == 0 && (uintptr_t)q % 4 == 0;           // pairs are aligned dwords
     auto load_q = [&](int g) __attribute__((always_inline)) {
+        if (NCHW) {
 #pragma unroll
-        for (int mb = 0; mb < NMB; ++mb) {
-            const Pix px = pixel(16 * mb + mi);
-#pragma unroll
-            for (int ks = 0; ks < DP / 32; ++ks) {
-                qa[mb][ks] = u32x4{0u, 0u, 0u, 0u};
-                if (px.active && 32 * ks + 8 * mk < d) {
-                    if (NCHW) {
-                        // 8 channel planes, one element each
-                        const T *qp = q + ((long)n * Cq + g * d + 32 * ks + 8 * mk) * hpl + px.pp;
-                        union { T h[8]; u32x4 u; } x;
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) x.h[e] = qp[e * hpl];
-                        qa[mb][ks] = x.u;
+            for (int i = 0; i < QN; ++i) {
+                const int item = i * NT + tid;
+                const int ch = item / (NPX / 2), pr = item % (NPX / 2);
+                const int qh = y0 + pr / (TW / 2), qw = x0 + 2 * (pr % (TW / 2));
+                qraw[i] = 0u;
+                if (ch < d && qh < hH && qw < hW) {
+                    const T *qp = q + ((long)n * Cq + g * d + ch) * hpl + (long)qh * hW + qw;
+                    if (q32) {
+                        qraw[i] = *(const u32 *)qp;
                     } else {
-                        qa[mb][ks] = *(const u32x4 *)(q + px.hp * Cq + g * d + 32 * ks + 8 * mk);
+                        union { T h[2]; u32 u; } x;
+                        x.u = 0u;
+                        x.h[0] = qp[0];
+                        if (qw + 1 < hW) x.h[1] = qp[1];
+                        qraw[i] = x.u;
                     }
                 }
             }
+        } else {
+#pragma unroll
+            for (int mb = 0; mb < NMB; ++mb) {
+                const Pix px = pixel(16 * mb + mi);
+#pragma unroll
+                for (int ks = 0; ks < DP / 32; ++ks) {
+                    qa[mb][ks] = u32x4{0u, 0u, 0u, 0u};
+                    if (px.active && 32 * ks + 8 * mk < d)
+                        qa[mb][ks] = *(const u32x4 *)(q + px.hp * Cq + g * d + 32 * ks + 8 * mk);
+                }
+            }
+        }
+    };
+    // (contiguous layout) the fetched pairs into the q tile; channels d .. DP hold zeros
+    auto stage_store_q = [&]() __attribute__((always_inline)) {
+        if (!NCHW) return;
+#pragma unroll
+        for (int i = 0; i < QN; ++i) {
+            const int item = i * NT + tid;
+            const int ch = item / (NPX / 2), pr = item % (NPX / 2);
+            const int pi = (pr / (TW / 2)) * TW + 2 * (pr % (TW / 2));
+            union { u32 u; T h[2]; } x;
+            x.u = qraw[i];
+            Ql[pi * QSB + ch] = x.h[0];
+            Ql[(pi + 1) * QSB + ch] = x.h[1];
         }
     };
 
@@ -333,6 +369,7 @@ deform_fused_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key,
     for (int g = 0; g < G; ++g) {
         // ---- (a) key window
         stage_store_key();
+        stage_store_q();
         if (tid == 0) fb_flag = 0;
         __syncthreads();
         // the group's first value chunk travels during the similarity and the sampling
@@ -354,7 +391,10 @@ deform_fused_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key,
             for (int mb = 0; mb < NMB; ++mb) {
                 f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int ks = 0; ks < DP / 32; ++ks) acc = Half<T>::mma(qa[mb][ks], b[ks], acc);
+                for (int ks = 0; ks < DP / 32; ++ks) {
+                    const u32x4 a = NCHW ? *(const u32x4 *)(Ql + (16 * mb + mi) * QSB + 32 * ks + 8 * mk) : qa[NCHW ? 0 : mb][ks];
+                    acc = Half<T>::mma(a, b[ks], acc);
+                }
 #pragma unroll
                 for (int r = 0; r < 4; ++r) Sl[(16 * mb + 4 * mk + r) * WS + 16 * nb + mi] = acc[r];
             }

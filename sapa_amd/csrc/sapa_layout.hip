@@ -12,13 +12,20 @@ namespace sapa {
 namespace layout {
 
 // 64 pixels x 64 channels per workgroup through LDS: reads run along the
-// pixels of a channel plane, writes along the channels of a pixel.
+// pixels of a channel plane, writes along the channels of a pixel.  Two tensors
+// of the same extent [B, C*, HW] in one launch: blockIdx.y < yblocks0 works on
+// the first.
 template <typename U>
 __global__ void __launch_bounds__(256)
-nchw_to_nhwc_kernel(const U *__restrict__ src, U *__restrict__ dst, int C, long HW) {
+nchw_to_nhwc_kernel(const U *__restrict__ src0, U *__restrict__ dst0, int C0, int yblocks0,
+                    const U *__restrict__ src1, U *__restrict__ dst1, int C1, long HW) {
     __shared__ U tile[64][65];
+    const bool first = (int)blockIdx.y < yblocks0;
+    const U *src = first ? src0 : src1;
+    U *dst = first ? dst0 : dst1;
+    const int C = first ? C0 : C1;
     const long p0 = (long)blockIdx.x * 64;
-    const int c0 = (int)blockIdx.y * 64;
+    const int c0 = ((int)blockIdx.y - (first ? 0 : yblocks0)) * 64;
     const long n = blockIdx.z;
     const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
     for (int c = ty; c < 64; c += 4)
@@ -30,21 +37,23 @@ nchw_to_nhwc_kernel(const U *__restrict__ src, U *__restrict__ dst, int C, long 
 
 }  // namespace layout
 
-// esize: bytes per element, 2 or 4.  hipErrorNotSupported otherwise, or for more
-// than 65535 images or 64-channel blocks.
-hipError_t nchw_to_nhwc_launch(const void *src, void *dst, int B, int C, long HW, int esize,
-                               hipStream_t st) {
-    if (B <= 0 || C <= 0 || HW <= 0) return hipSuccess;
+// Two tensors [B, C0, HW] and [B, C1, HW] (C1 = 0: one) in one launch.  esize:
+// bytes per element, 2 or 4.  hipErrorNotSupported otherwise, or for more than
+// 65535 images or 64-channel blocks.
+hipError_t nchw_to_nhwc_launch(const void *src0, void *dst0, int C0, const void *src1, void *dst1,
+                               int C1, int B, long HW, int esize, hipStream_t st) {
+    if (B <= 0 || C0 <= 0 || HW <= 0) return hipSuccess;
     const long gx = (HW + 63) / 64;
-    const int gy = (C + 63) / 64;
-    if (gx > 0x7fffffffL || gy > 65535 || B > 65535) return hipErrorNotSupported;
-    const dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)B);
+    const int gy0 = (C0 + 63) / 64, gy1 = (C1 + 63) / 64;
+    if (gx > 0x7fffffffL || gy0 + gy1 > 65535 || B > 65535) return hipErrorNotSupported;
+    const dim3 grid((unsigned)gx, (unsigned)(gy0 + gy1), (unsigned)B);
     if (esize == 2)
         hipLaunchKernelGGL(layout::nchw_to_nhwc_kernel<unsigned short>, grid, dim3(256), 0, st,
-                           (const unsigned short *)src, (unsigned short *)dst, C, HW);
+                           (const unsigned short *)src0, (unsigned short *)dst0, C0, gy0,
+                           (const unsigned short *)src1, (unsigned short *)dst1, C1, HW);
     else if (esize == 4)
-        hipLaunchKernelGGL(layout::nchw_to_nhwc_kernel<unsigned>, grid, dim3(256), 0, st, (const unsigned *)src,
-                           (unsigned *)dst, C, HW);
+        hipLaunchKernelGGL(layout::nchw_to_nhwc_kernel<unsigned>, grid, dim3(256), 0, st, (const unsigned *)src0,
+                           (unsigned *)dst0, C0, gy0, (const unsigned *)src1, (unsigned *)dst1, C1, HW);
     else
         return hipErrorNotSupported;
     return hipGetLastError();
