@@ -316,6 +316,28 @@ int sapa_deform_fused_forward_ws(const void *query, const void *key,
                                  int P, int s, int G, int offset_layout, int dtype,
                                  void *stream);
 
+/* Backward pass of sapa_deform_fused_forward in one call: gradients of
+ *   deform_av(softmax(deform_qk(query, key, offset), dim = points), value, offset)
+ * with respect to query, key, value and offset (hi-res layout).  It replaces the
+ * chain dav.backward (deform_av.cpp:50-70) -> softmax backward (ATen) ->
+ * dqk.backward (deform_qk.cpp:50-70) that autograd runs for
+ * SAPADeform.attention (sapa_deform.py:51-53), with the weights recomputed from
+ * query / key.  The attention weights and the gradient of the logits
+ * [B,G,P,sH,sW] are fp32 in `workspace` whatever `dtype` is; SAPA_F16 / BF16
+ * tensors are read and written as they are; the low-res gradients and the two
+ * contributions to grad_offset are summed in fp32 and rounded once.  All four gradients are overwritten; any may be NULL.
+ * sapa_deform_fused_backward_workspace: bytes needed (256-byte aligned), 0 when
+ * the configuration is not served -- SAPA_F64, s outside {1, 2, 4}, P > 48 --
+ * and the caller chains sapa_deform_av_backward / sapa_deform_qk_backward;
+ * SAPA_ERR_UNSUPPORTED then, before anything is written. */
+long long sapa_deform_fused_backward_workspace(int B, int Cq, int C, int H, int W,
+                                               int P, int s, int G, int dtype);
+int sapa_deform_fused_backward(const void *grad_out, const void *query, const void *key,
+                               const void *value, const void *offset, void *workspace,
+                               void *grad_query, void *grad_key, void *grad_value,
+                               void *grad_offset, int B, int Cq, int C, int H, int W,
+                               int P, int s, int G, int dtype, void *stream);
+
 /* The three sampled forward operators reading the offsets in the layout
  * `offset_layout` (sapa_offset_layout) names; with SAPA_OFFSET_HIRES they are
  * the functions above.  They replace

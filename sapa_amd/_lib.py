@@ -44,6 +44,7 @@ SIGNATURES = {
     'sapa_deform_av_backward': [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_deform_fused_forward': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_deform_fused_forward_nhwc': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
+    'sapa_deform_fused_backward': [_vp] * 10 + [_i] * 9 + [_vp],
     'sapa_deform_fused_forward_ws': [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_deform_qk_forward_from': [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_deform_av_forward_from': [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
@@ -93,6 +94,8 @@ def lib():
         handle.sapa_fused_backward_workspace.argtypes = [_i, _i, _i, _i, _i]
         handle.sapa_deform_fused_forward_workspace.restype = _ll
         handle.sapa_deform_fused_forward_workspace.argtypes = [_i] * 9
+        handle.sapa_deform_fused_backward_workspace.restype = _ll
+        handle.sapa_deform_fused_backward_workspace.argtypes = [_i] * 9
         handle.sapa_channel_moments_static_capacity.restype = _ll
         handle.sapa_channel_moments_static_capacity.argtypes = []
         _lib = handle

@@ -553,6 +553,28 @@ int sapa_deform_av_backward(const void *grad_out, const void *attn, const void *
     return SAPA_OK;
 }
 
+long long sapa_deform_fused_backward_workspace(int B, int Cq, int C, int H, int W, int P, int s,
+                                               int G, int dtype) {
+    if (check_deform_args(B, Cq, C, H, W, P, s, G, dtype) != SAPA_OK) return 0;
+    return deform_fused_backward_workspace(B, Cq, C, H, W, P, s, G, dtype);
+}
+
+int sapa_deform_fused_backward(const void *grad_out, const void *query, const void *key,
+                               const void *value, const void *offset, void *workspace,
+                               void *grad_query, void *grad_key, void *grad_value,
+                               void *grad_offset, int B, int Cq, int C, int H, int W, int P, int s,
+                               int G, int dtype, void *stream) {
+    const int rc = check_deform_args(B, Cq, C, H, W, P, s, G, dtype);
+    if (rc != SAPA_OK) return rc;
+    if (B == 0) return SAPA_OK;
+    if (!grad_out || !query || !key || !value || !offset) return SAPA_ERR_INVALID_ARGUMENT;
+    const hipError_t e = deform_fused_backward_launch(grad_out, query, key, value, offset, workspace,
+                                                      grad_query, grad_key, grad_value, grad_offset, B, Cq,
+                                                      C, H, W, P, s, G, dtype, (hipStream_t)stream);
+    if (e == hipErrorNotSupported) return SAPA_ERR_UNSUPPORTED;
+    return finish(e);
+}
+
 long long sapa_channel_moments_workspace(int B, int C, long long HW, int channels_last) {
     if (B <= 0 || C <= 0 || HW <= 0) return 0;
     return channel_moments_workspace(B, C, (long)HW, channels_last != 0);

@@ -73,6 +73,17 @@ hipError_t deform_fused_nhwc_launch(const void *q, const void *key, const void *
                                     int W, int P, int s, int G, int dtype, hipStream_t st,
                                     const char **kernel = nullptr);
 
+// sapa_d_backward.hip: the backward pass of the fused SAPA-D operator in one call;
+// attention weights and logit gradients as fp32 in `workspace` (256-byte aligned,
+// deform_fused_backward_workspace() bytes; 0 = not served), f16 / bf16 tensors read
+// and written as they are.  Any gradient may be NULL.  hipErrorNotSupported otherwise.
+long deform_fused_backward_workspace(int B, int Cq, int C, int H, int W, int P, int s, int G, int dtype);
+hipError_t deform_fused_backward_launch(const void *grad_out, const void *q, const void *key,
+                                        const void *value, const void *offset, void *workspace,
+                                        void *grad_q, void *grad_key, void *grad_value,
+                                        void *grad_offset, int B, int Cq, int C, int H, int W, int P,
+                                        int s, int G, int dtype, hipStream_t st);
+
 // sapa_d_nhwc.hip: contiguous (NCHW) tensors through the matrix-form kernels:
 // key and value are copied into channels-last order in `workspace` (256-byte
 // aligned, deform_fused_nchw_workspace() bytes; 0 = this path does not serve the
@@ -127,7 +138,8 @@ hipError_t lowres_grad_tiled_launch(const void *hi, const void *w, void *out, in
 hipError_t deform_lds_launch(int mode, const void *q, const void *key, const void *attn_in,
                              const void *value, const void *offset, void *out, int B, int Cq, int C,
                              int H, int W, int P, int s, int G, int olayout, int dtype,
-                             hipStream_t st);
+                             hipStream_t st, bool wide = false, bool accumulate = false,
+                             float *partial = nullptr);
 
 // sapa_d.hip.  olayout (OffsetLayout in deform_tap.hpp) says whether `offset`
 // is the hi-res tensor or the low-res tensor it is produced from.
@@ -148,7 +160,7 @@ hipError_t deform_fused_forward_launch(const void *q, const void *key, const voi
 // otherwise.  Accumulates into grad_low.
 hipError_t deform_lowgrad_lds_launch(const void *hi, const void *sc, const void *offset,
                                      void *grad_low, int B, int Cx, int H, int W, int P, int s,
-                                     int G, int dtype, hipStream_t st);
+                                     int G, int dtype, hipStream_t st, bool wide = false);
 
 // grad_low (atomic accumulate, may be null) and grad_offset (store, may be
 // null) of either sampled op: hi = per-channel high-res tensor [B,Cx,sH,sW],

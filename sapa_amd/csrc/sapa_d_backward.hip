@@ -1,0 +1,157 @@
+// Backward pass of the fused SAPA-D operator
+//   out = deform_av(softmax(deform_qk(q, key, offset), dim = points), value, offset)
+// (SAPADeform.attention, sapa_deform.py:51-53) in one call: the chain of the two
+// reference backward functions (deform_qk.cpp:50-70 -> DeformQKBackward,
+// deform_av.cpp:50-70 -> DeformAVBackward) with the softmax between them.
+//
+// The attention weights and the gradient of the logits, [B, G, P, sH, sW], live
+// in the caller's workspace as fp32 whatever the tensors' type is; f16 / bf16
+// features, offsets and gradients are read and written as they are (no fp32
+// copies of them), and the low-res gradients, which are sums of many terms, are
+// accumulated in fp32 and rounded once.
+//
+//   attn        = softmax(deform_qk(q, key))                    sampled similarity
+//   grad_attn   = deform_qk(grad_out, value)                    (the same kernel)
+//   grad_logits = attn * (grad_attn - sum_p attn * grad_attn)
+//   grad_value  = scatter(grad_out, attn);   grad_offset  = d/d offset of the aggregation
+//   grad_query  = deform_av(grad_logits, key)                   sampled aggregation
+//   grad_key    = scatter(q, grad_logits);   grad_offset += d/d offset of the similarity
+#include "kernels.hpp"
+
+namespace sapa {
+
+namespace dbwd {
+
+// grad_logits = attn * (grad_attn - sum_r attn * grad_attn) over the middle axis
+// of [N, R, M], in place on g; one thread per (n, m)
+__global__ void __launch_bounds__(256)
+softmax_backward_kernel(const float *__restrict__ attn, float *__restrict__ g, long N, int R, long M) {
+    const long total = N * M;
+    for (long idx = blockIdx.x * (long)blockDim.x + threadIdx.x; idx < total;
+         idx += (long)gridDim.x * blockDim.x) {
+        const long n = idx / M, m = idx % M;
+        const float *ap = attn + n * R * M + m;
+        float *gp = g + n * R * M + m;
+        float dot = 0.f;
+        for (int j = 0; j < R; ++j) dot = fma_(ap[j * M], gp[j * M], dot);
+        for (int j = 0; j < R; ++j) gp[j * M] = ap[j * M] * (gp[j * M] - dot);
+    }
+}
+
+__global__ void __launch_bounds__(256) zero_kernel(float *__restrict__ x, long n) {
+    for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
+        x[i] = 0.f;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) narrow_kernel(const float *__restrict__ x, T *__restrict__ y, long n) {
+    for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
+        y[i] = (T)x[i];
+}
+
+static unsigned blocks_for(long n) {
+    const long b = (n + 255) / 256;
+    return (unsigned)(b < 1 ? 1 : (b > 65536 ? 65536 : b));
+}
+
+static long align256(long x) { return (x + 255) / 256 * 256; }
+
+}  // namespace dbwd
+
+// Bytes of workspace, or 0 for configurations this call does not serve (the
+// caller then chains the separate backward entry points): f32 / f16 / bf16,
+// s in {1, 2, 4}, P small enough for the LDS kernels.
+long deform_fused_backward_workspace(int B, int Cq, int C, int H, int W, int P, int s, int G, int dtype) {
+    using dbwd::align256;
+    if (dtype != 0 && dtype != 2 && dtype != 3) return 0;
+    if (s != 1 && s != 2 && s != 4) return 0;
+    if (P > 48) return 0;       // [2P][thread] sums of the offset gradient next to the window in LDS
+    const long per_point = (long)B * G * P * H * s * W * s * (long)sizeof(float);
+    long n = 2 * align256(per_point);
+    // 16-bit tensors: fp32 accumulators of the low-res gradients and of the first
+    // half of grad_offset
+    if (dtype != 0) n += align256((long)B * Cq * H * W * 4) + align256((long)B * C * H * W * 4) + align256(2 * per_point);
+    return n;
+}
+
+// Any of the four gradients may be NULL.  hipErrorNotSupported before anything
+// is written when the configuration is not served.
+hipError_t deform_fused_backward_launch(const void *grad_out, const void *q, const void *key,
+                                        const void *value, const void *offset, void *workspace,
+                                        void *grad_q, void *grad_key, void *grad_value,
+                                        void *grad_offset, int B, int Cq, int C, int H, int W, int P,
+                                        int s, int G, int dtype, hipStream_t st) {
+    using namespace dbwd;
+    if (deform_fused_backward_workspace(B, Cq, C, H, W, P, s, G, dtype) == 0) return hipErrorNotSupported;
+    if (!workspace || (uintptr_t)workspace % 256 != 0) return hipErrorNotSupported;
+    const bool wide = dtype != 0;
+    const long hpix = (long)H * s * W * s, lpix = (long)H * W;
+    const long n_pp = (long)B * G * P * hpix;
+    char *w = (char *)workspace;
+    float *attn = (float *)w;
+    float *gl = (float *)(w + align256(n_pp * 4));
+    float *gk32 = wide ? (float *)(w + 2 * align256(n_pp * 4)) : (float *)grad_key;
+    float *gv32 = wide ? (float *)((char *)gk32 + align256((long)B * Cq * lpix * 4)) : (float *)grad_value;
+    float *goff32 = wide ? (float *)((char *)gv32 + align256((long)B * C * lpix * 4)) : nullptr;
+    const int HIRES = 0;
+    hipError_t e;
+#define SAPA_STEP(call)                  \
+    do {                                 \
+        e = (call);                      \
+        if (e != hipSuccess) return e;   \
+    } while (0)
+
+    // attention weights: sampled similarity (mode 0), softmax over the points
+    SAPA_STEP(deform_lds_launch(0, q, key, nullptr, nullptr, offset, attn, B, Cq, Cq, H, W, P, s, G, HIRES,
+                                dtype, st, wide));
+    SAPA_STEP(softmax_generic_launch(attn, attn, (long)B * G, P, hpix, 0, st));
+    // gradient of the weights: the similarity of grad_out and value
+    SAPA_STEP(deform_lds_launch(0, grad_out, value, nullptr, nullptr, offset, gl, B, C, C, H, W, P, s, G,
+                                HIRES, dtype, st, wide));
+    hipLaunchKernelGGL(softmax_backward_kernel, dim3(blocks_for((long)B * G * hpix)), dim3(256), 0, st, attn,
+                       gl, (long)B * G, P, hpix);
+    SAPA_STEP(hipGetLastError());
+
+    // aggregation: grad_value (scatter) and its share of grad_offset
+    if (grad_offset)
+        SAPA_STEP(deform_lds_launch(3, grad_out, value, attn, nullptr, offset, grad_offset, B, C, C, H, W, P, s,
+                                    G, HIRES, dtype, st, wide, false, goff32));
+    if (grad_value) {
+        hipLaunchKernelGGL(zero_kernel, dim3(blocks_for((long)B * C * lpix)), dim3(256), 0, st, gv32,
+                           (long)B * C * lpix);
+        SAPA_STEP(hipGetLastError());
+        SAPA_STEP(deform_lowgrad_lds_launch(grad_out, attn, offset, gv32, B, C, H, W, P, s, G, dtype, st, wide));
+    }
+    // similarity: grad_query (aggregation of key with grad_logits), grad_key
+    // (scatter) and the other share of grad_offset
+    if (grad_q)
+        SAPA_STEP(deform_lds_launch(1, nullptr, nullptr, gl, key, offset, grad_q, B, Cq, Cq, H, W, P, s, G, HIRES,
+                                    dtype, st, wide));
+    if (grad_offset)
+        SAPA_STEP(deform_lds_launch(3, q, key, gl, nullptr, offset, grad_offset, B, Cq, Cq, H, W, P, s, G, HIRES,
+                                    dtype, st, wide, true, goff32));
+    if (grad_key) {
+        hipLaunchKernelGGL(zero_kernel, dim3(blocks_for((long)B * Cq * lpix)), dim3(256), 0, st, gk32,
+                           (long)B * Cq * lpix);
+        SAPA_STEP(hipGetLastError());
+        SAPA_STEP(deform_lowgrad_lds_launch(q, gl, offset, gk32, B, Cq, H, W, P, s, G, dtype, st, wide));
+    }
+    if (wide) {
+        if (grad_key) {
+            const long n = (long)B * Cq * lpix;
+            if (dtype == 2) hipLaunchKernelGGL(narrow_kernel<f16_t>, dim3(blocks_for(n)), dim3(256), 0, st, gk32, (f16_t *)grad_key, n);
+            else hipLaunchKernelGGL(narrow_kernel<bf16_t>, dim3(blocks_for(n)), dim3(256), 0, st, gk32, (bf16_t *)grad_key, n);
+            SAPA_STEP(hipGetLastError());
+        }
+        if (grad_value) {
+            const long n = (long)B * C * lpix;
+            if (dtype == 2) hipLaunchKernelGGL(narrow_kernel<f16_t>, dim3(blocks_for(n)), dim3(256), 0, st, gv32, (f16_t *)grad_value, n);
+            else hipLaunchKernelGGL(narrow_kernel<bf16_t>, dim3(blocks_for(n)), dim3(256), 0, st, gv32, (bf16_t *)grad_value, n);
+            SAPA_STEP(hipGetLastError());
+        }
+    }
+#undef SAPA_STEP
+    return hipSuccess;
+}
+
+}  // namespace sapa

@@ -26,12 +26,17 @@ namespace sapa {
 
 enum DeformMode { DEFORM_QK = 0, DEFORM_AV = 1, DEFORM_FUSED = 2, DEFORM_OFFGRAD = 3 };
 
-template <typename T, int S, int TPW, int TPH, int CH, int MODE>
+// TS: the type of the per-point scalar tensors [B, G, P, sH, sW] -- the logits
+// (out of DEFORM_QK) and attn_in -- which the backward pass keeps in fp32 next to
+// 16-bit features.  accumulate (DEFORM_OFFGRAD): add to what out -- or partial,
+// if given -- holds.
+template <typename T, typename TS, int S, int TPW, int TPH, int CH, int MODE>
 __global__ void __launch_bounds__(TPW *TPH *S *S)
 deform_lds_kernel(const T *__restrict__ q, const T *__restrict__ key,
-                  const T *__restrict__ attn_in, const T *__restrict__ value,
+                  const TS *__restrict__ attn_in, const T *__restrict__ value,
                   const T *__restrict__ offset, T *__restrict__ out, int Cq, int C, int H, int W,
-                  int P, int G, int olayout, int tiles_x, int tiles_y, int nblocks, int per_xcd) {
+                  int P, int G, int olayout, int tiles_x, int tiles_y, int nblocks, int per_xcd,
+                  int accumulate, float *__restrict__ partial) {
     typedef float A;
     typedef float F4 __attribute__((ext_vector_type(4)));
     constexpr int HR = 4;                           // window reach in low-res cells
@@ -96,7 +101,7 @@ deform_lds_kernel(const T *__restrict__ q, const T *__restrict__ key,
         // attention weights), out = grad_offset [B,2GP,sH,sW].  Per point the
         // two running sums live in LDS next to each other ([2P][thread]).
         const long ch0 = (long)b * Cq + (long)g * d;
-        const T *sp = attn_in + ((long)b * GP + (long)g * P) * hplane + pix;
+        const TS *sp = attn_in + ((long)b * GP + (long)g * P) * hplane + pix;
         for (int c0 = 0; c0 < d; c0 += CH) {
             const int nvalid = d - c0 < CH ? d - c0 : CH;
             A qv[CH];
@@ -159,7 +164,14 @@ deform_lds_kernel(const T *__restrict__ q, const T *__restrict__ key,
         }
         if (active) {
             T *o = out + ((((long)b * GP + (long)g * P)) << 1) * hplane + pix;
-            for (int p = 0; p < 2 * P; ++p) o[(long)p * hplane] = (T)lgt[p * NT];
+            // `partial` (same shape as out, fp32): the first of two contributions is
+            // parked there instead of out, the second adds it and rounds once
+            float *po = partial ? partial + ((((long)b * GP + (long)g * P)) << 1) * hplane + pix : nullptr;
+            for (int p = 0; p < 2 * P; ++p) {
+                const A prev = !accumulate ? (A)0 : po ? (A)po[(long)p * hplane] : (A)o[(long)p * hplane];
+                if (po && !accumulate) po[(long)p * hplane] = lgt[p * NT];
+                else o[(long)p * hplane] = (T)(lgt[p * NT] + prev);
+            }
         }
         return;
     }
@@ -228,11 +240,11 @@ deform_lds_kernel(const T *__restrict__ q, const T *__restrict__ key,
             const A inv = (A)1 / sum;
             for (int p = 0; p < P; ++p) lgt[p * NT] *= inv;
         } else if (active) {
-            T *o = out + ((long)b * GP + (long)g * P) * hplane + pix;
-            for (int p = 0; p < P; ++p) o[(long)p * hplane] = (T)lgt[p * NT];
+            TS *o = (TS *)out + ((long)b * GP + (long)g * P) * hplane + pix;
+            for (int p = 0; p < P; ++p) o[(long)p * hplane] = (TS)lgt[p * NT];
         }
     } else {
-        const T *ap = attn_in + ((long)b * GP + (long)g * P) * hplane + pix;
+        const TS *ap = attn_in + ((long)b * GP + (long)g * P) * hplane + pix;
         for (int p = 0; p < P; ++p) lgt[p * NT] = (A)ap[(long)p * hplane];
     }
 
@@ -297,10 +309,11 @@ deform_lds_kernel(const T *__restrict__ q, const T *__restrict__ key,
 }
 
 // ------------------------------------------------------------------ launcher
-template <typename T, int S, int TPW, int TPH, int CH>
+template <typename T, typename TS, int S, int TPW, int TPH, int CH>
 static hipError_t launch_geom(int mode, const void *q, const void *key, const void *attn_in,
                               const void *value, const void *offset, void *out, int B, int Cq,
-                              int C, int H, int W, int P, int G, int olayout, hipStream_t st) {
+                              int C, int H, int W, int P, int G, int olayout, hipStream_t st,
+                              int accumulate, float *partial) {
     constexpr int HR = 4, NT = TPW * TPH * S * S;
     constexpr int WW = TPW + 2 * HR + 1, WH = TPH + 2 * HR + 1, CST = CH + 4;
     const size_t smem =
@@ -315,15 +328,15 @@ static hipError_t launch_geom(int mode, const void *q, const void *key, const vo
 #define SAPA_DL_CASE(M)                                                                       \
     case M:                                                                                   \
         if (big && hipFuncSetAttribute(                                                       \
-                       reinterpret_cast<const void *>(&deform_lds_kernel<T, S, TPW, TPH, CH, M>), \
+                       reinterpret_cast<const void *>(&deform_lds_kernel<T, TS, S, TPW, TPH, CH, M>), \
                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) { \
             (void)hipGetLastError();                                                          \
             return hipErrorNotSupported;                                                      \
         }                                                                                     \
-        hipLaunchKernelGGL((deform_lds_kernel<T, S, TPW, TPH, CH, M>), grid, block, smem, st, \
-                           (const T *)q, (const T *)key, (const T *)attn_in,                  \
+        hipLaunchKernelGGL((deform_lds_kernel<T, TS, S, TPW, TPH, CH, M>), grid, block, smem, st, \
+                           (const T *)q, (const T *)key, (const TS *)attn_in,                 \
                            (const T *)value, (const T *)offset, (T *)out, Cq, C, H, W, P, G,  \
-                           olayout, tiles_x, tiles_y, (int)nb, per_xcd);                      \
+                           olayout, tiles_x, tiles_y, (int)nb, per_xcd, accumulate, partial); \
         break;
     switch (mode) {
         SAPA_DL_CASE(DEFORM_QK) SAPA_DL_CASE(DEFORM_AV) SAPA_DL_CASE(DEFORM_FUSED)
@@ -334,24 +347,25 @@ static hipError_t launch_geom(int mode, const void *q, const void *key, const vo
     return hipGetLastError();
 }
 
-template <typename T>
+template <typename T, typename TS>
 static hipError_t launch_t(int mode, const void *q, const void *key, const void *attn_in,
                            const void *value, const void *offset, void *out, int B, int Cq, int C,
-                           int H, int W, int P, int s, int G, int olayout, hipStream_t st) {
+                           int H, int W, int P, int s, int G, int olayout, hipStream_t st,
+                           int accumulate, float *partial) {
 #ifdef SAPA_DLDS_TUNE
-    if (s == 2) return launch_geom<T, 2, SAPA_DLDS_TUNE>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, G, olayout, st);
+    if (s == 2) return launch_geom<T, TS, 2, SAPA_DLDS_TUNE>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, G, olayout, st, accumulate, partial);
     return hipErrorNotSupported;
 #else
     switch (s) {
-        case 1: return launch_geom<T, 1, 16, 16, 8>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, G, olayout, st);
+        case 1: return launch_geom<T, TS, 1, 16, 16, 8>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, G, olayout, st, accumulate, partial);
         case 2:
             // few points leave LDS room for a 16 x 8-parent tile (512 threads): a
             // smaller share of halo cells per staged window (measured at P = 9: 12 % faster;
             // at P = 25 the [P][thread] logits of 512 threads cost a workgroup per CU)
             if (P <= 12 && W > 8)
-                return launch_geom<T, 2, 16, 8, 16>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, G, olayout, st);
-            return launch_geom<T, 2, 8, 8, 16>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, G, olayout, st);
-        case 4: return launch_geom<T, 4, 4, 4, 16>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, G, olayout, st);
+                return launch_geom<T, TS, 2, 16, 8, 16>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, G, olayout, st, accumulate, partial);
+            return launch_geom<T, TS, 2, 8, 8, 16>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, G, olayout, st, accumulate, partial);
+        case 4: return launch_geom<T, TS, 4, 4, 4, 16>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, G, olayout, st, accumulate, partial);
         default: return hipErrorNotSupported;
     }
 #endif
@@ -360,16 +374,26 @@ static hipError_t launch_t(int mode, const void *q, const void *key, const void 
 // mode: 0 = deform_qk (out = logits), 1 = deform_av (attn_in given),
 // 2 = fused, 3 = gradient of the offsets (q = per-channel high-res tensor,
 // key = sampled tensor, attn_in = per-point scalar, out = grad_offset).  hipErrorNotSupported: no instance for (s, dtype) or P too large
-// for the LDS budget; the caller then takes the global-memory kernels.
+// for the LDS budget; the caller then takes the global-memory kernels.  wide:
+// the per-point tensors (attn_in, the logits) are fp32 next to 16-bit features;
+// accumulate: mode 3 adds to grad_offset; partial (fp32, grad_offset's shape):
+// the first contribution is kept there unrounded until the second adds it.
 hipError_t deform_lds_launch(int mode, const void *q, const void *key, const void *attn_in,
                              const void *value, const void *offset, void *out, int B, int Cq, int C,
                              int H, int W, int P, int s, int G, int olayout, int dtype,
-                             hipStream_t st) {
+                             hipStream_t st, bool wide, bool accumulate, float *partial) {
+    // the fused mode has no per-point tensor in memory
+    if (wide && mode == DEFORM_FUSED) return hipErrorNotSupported;
+    const int acc = accumulate ? 1 : 0;
     switch (dtype) {
-        case 0: return launch_t<float>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, s, G, olayout, st);
+        case 0: return launch_t<float, float>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, s, G, olayout, st, acc, partial);
 #ifndef SAPA_DLDS_TUNE
-        case 2: return launch_t<f16_t>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, s, G, olayout, st);
-        case 3: return launch_t<bf16_t>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, s, G, olayout, st);
+        case 2:
+            return wide ? launch_t<f16_t, float>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, s, G, olayout, st, acc, partial)
+                        : launch_t<f16_t, f16_t>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, s, G, olayout, st, acc, partial);
+        case 3:
+            return wide ? launch_t<bf16_t, float>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, s, G, olayout, st, acc, partial)
+                        : launch_t<bf16_t, bf16_t>(mode, q, key, attn_in, value, offset, out, B, Cq, C, H, W, P, s, G, olayout, st, acc, partial);
 #endif
         default: return hipErrorNotSupported;
     }

@@ -28,10 +28,12 @@
 
 namespace sapa {
 
-template <int S, int TPW, int TPH, int CH>
+// T: the features' and the offsets' type, TS: the per-point scalars' (fp32 next
+// to 16-bit features in the fused backward pass); grad_low is fp32 either way.
+template <typename T, typename TS, int S, int TPW, int TPH, int CH>
 __global__ void __launch_bounds__(TPW *TPH *S *S)
-deform_lowgrad_lds_kernel(const float *__restrict__ hi, const float *__restrict__ sc,
-                          const float *__restrict__ offset, float *__restrict__ grad_low, int Cx,
+deform_lowgrad_lds_kernel(const T *__restrict__ hi, const TS *__restrict__ sc,
+                          const T *__restrict__ offset, float *__restrict__ grad_low, int Cx,
                           int H, int W, int P, int G, int tiles_x, int tiles_y, int nblocks,
                           int per_xcd) {
     constexpr int HR = 4;                           // window reach in low-res cells
@@ -62,8 +64,8 @@ deform_lowgrad_lds_kernel(const float *__restrict__ hi, const float *__restrict_
     const float ph = (float)(cqh / S), pw = (float)(cqw / S);
     const int wx0 = tx * TPW - HR, wy0 = ty * TPH - HR;
     const long k0 = (long)b * GP + (long)g * P;
-    const float *op = offset + (k0 << 1) * hplane + pix;
-    const float *sp = sc + k0 * hplane + pix;
+    const T *op = offset + (k0 << 1) * hplane + pix;
+    const TS *sp = sc + k0 * hplane + pix;
     const long ch0 = (long)b * Cx + (long)g * cg;
 
     for (int i = tid; i < CH * WIN; i += NT) acc[i] = 0;
@@ -76,7 +78,7 @@ deform_lowgrad_lds_kernel(const float *__restrict__ hi, const float *__restrict_
     bool scbad = false;
     if (active)
         for (int p = 0; p < P; ++p) {
-            const float a = fabsf(sp[(long)p * hplane]);
+            const float a = fabsf((float)sp[(long)p * hplane]);
             scbad |= !(a < __builtin_huge_valf());
             scmax = fmaxf(scmax, a);
         }
@@ -91,7 +93,7 @@ deform_lowgrad_lds_kernel(const float *__restrict__ hi, const float *__restrict_
         bool bad = scbad;
 #pragma unroll
         for (int ch = 0; ch < CH; ++ch) {
-            hv[ch] = (active && ch < nvalid) ? hi[(ch0 + c0 + ch) * hplane + pix] : 0.f;
+            hv[ch] = (active && ch < nvalid) ? (float)hi[(ch0 + c0 + ch) * hplane + pix] : 0.f;
             const float a = fabsf(hv[ch]);
             bad |= !(a < __builtin_huge_valf());
             hmax = fmaxf(hmax, a);
@@ -118,14 +120,14 @@ deform_lowgrad_lds_kernel(const float *__restrict__ hi, const float *__restrict_
 
         if (active) {
             // the next point's offsets and scalar are fetched while this one is scattered
-            float ow = op[0], oh = op[hplane], sn = sp[0];
+            float ow = (float)op[0], oh = (float)op[hplane], sn = (float)sp[0];
             for (int p = 0; p < P; ++p) {
                 const float kw = pw + ow, kh = ph + oh, scv = sn;
                 {
                     const int pn = p + 1 < P ? p + 1 : p;
-                    ow = op[(long)(2 * pn) * hplane];
-                    oh = op[(long)(2 * pn + 1) * hplane];
-                    sn = sp[(long)pn * hplane];
+                    ow = (float)op[(long)(2 * pn) * hplane];
+                    oh = (float)op[(long)(2 * pn + 1) * hplane];
+                    sn = (float)sp[(long)pn * hplane];
                 }
                 Tap<float> tap;
                 if (!tap_setup(kh, kw, H, W, tap)) continue;
@@ -183,7 +185,7 @@ deform_lowgrad_lds_kernel(const float *__restrict__ hi, const float *__restrict_
     }
 }
 
-template <int S, int TPW, int TPH, int CH>
+template <typename T, typename TS, int S, int TPW, int TPH, int CH>
 static hipError_t deform_lowgrad_launch_geom(const void *hi, const void *sc, const void *offset, void *grad_low, int B,
                        int Cx, int H, int W, int P, int G, hipStream_t st) {
     constexpr int NT = TPW * TPH * S * S;
@@ -191,24 +193,33 @@ static hipError_t deform_lowgrad_launch_geom(const void *hi, const void *sc, con
     const long nb = (long)tiles_x * tiles_y * G * B;
     if (nb > (1L << 30)) return hipErrorNotSupported;
     const int per_xcd = (int)((nb + 7) / 8);
-    hipLaunchKernelGGL((deform_lowgrad_lds_kernel<S, TPW, TPH, CH>), dim3(per_xcd * 8), dim3(NT),
-                       0, st, (const float *)hi, (const float *)sc, (const float *)offset,
+    hipLaunchKernelGGL((deform_lowgrad_lds_kernel<T, TS, S, TPW, TPH, CH>), dim3(per_xcd * 8), dim3(NT),
+                       0, st, (const T *)hi, (const TS *)sc, (const T *)offset,
                        (float *)grad_low, Cx, H, W, P, G, tiles_x, tiles_y, (int)nb, per_xcd);
     return hipGetLastError();
 }
 
-// fp32, s in {1, 2, 4}; hipErrorNotSupported otherwise (the caller then takes
-// the per-term atomic kernel).  grad_low is accumulated into.
-hipError_t deform_lowgrad_lds_launch(const void *hi, const void *sc, const void *offset,
-                                     void *grad_low, int B, int Cx, int H, int W, int P, int s,
-                                     int G, int dtype, hipStream_t st) {
-    if (dtype != 0) return hipErrorNotSupported;
+template <typename T, typename TS>
+static hipError_t deform_lowgrad_lds_t(const void *hi, const void *sc, const void *offset, void *grad_low,
+                                       int B, int Cx, int H, int W, int P, int s, int G, hipStream_t st) {
     switch (s) {
-        case 1: return deform_lowgrad_launch_geom<1, 16, 16, 4>(hi, sc, offset, grad_low, B, Cx, H, W, P, G, st);
-        case 2: return deform_lowgrad_launch_geom<2, 8, 8, 8>(hi, sc, offset, grad_low, B, Cx, H, W, P, G, st);
-        case 4: return deform_lowgrad_launch_geom<4, 4, 4, 8>(hi, sc, offset, grad_low, B, Cx, H, W, P, G, st);
+        case 1: return deform_lowgrad_launch_geom<T, TS, 1, 16, 16, 4>(hi, sc, offset, grad_low, B, Cx, H, W, P, G, st);
+        case 2: return deform_lowgrad_launch_geom<T, TS, 2, 8, 8, 8>(hi, sc, offset, grad_low, B, Cx, H, W, P, G, st);
+        case 4: return deform_lowgrad_launch_geom<T, TS, 4, 4, 4, 8>(hi, sc, offset, grad_low, B, Cx, H, W, P, G, st);
         default: return hipErrorNotSupported;
     }
+}
+
+// fp32 tensors, or (wide) f16 / bf16 features and offsets with fp32 per-point
+// scalars; s in {1, 2, 4}; hipErrorNotSupported otherwise (the caller then takes
+// the per-term atomic kernel).  grad_low is fp32 and is accumulated into.
+hipError_t deform_lowgrad_lds_launch(const void *hi, const void *sc, const void *offset,
+                                     void *grad_low, int B, int Cx, int H, int W, int P, int s,
+                                     int G, int dtype, hipStream_t st, bool wide) {
+    if (dtype == 0) return deform_lowgrad_lds_t<float, float>(hi, sc, offset, grad_low, B, Cx, H, W, P, s, G, st);
+    if (wide && dtype == 2) return deform_lowgrad_lds_t<f16_t, float>(hi, sc, offset, grad_low, B, Cx, H, W, P, s, G, st);
+    if (wide && dtype == 3) return deform_lowgrad_lds_t<bf16_t, float>(hi, sc, offset, grad_low, B, Cx, H, W, P, s, G, st);
+    return hipErrorNotSupported;
 }
 
 }  // namespace sapa

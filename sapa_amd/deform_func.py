@@ -173,7 +173,27 @@ def _reduce_offset_grad(grad_hi, scale_factor, layout):
     return grad_hi.view(b, c, hh // s, s, hw // s, s).sum(dim=(3, 5))
 
 
-def _deform_fused_backward(grad_output, query, key, value, offset, P, s, G, offset_layout):
+def _native_fused_backward(grad_output, query, key, value, offset, P, s, G, needs):
+    """sapa_deform_fused_backward on contiguous tensors with hi-res offsets: the whole
+    chain in one call, fp32 [B,G,P,sH,sW] intermediates in a workspace, 16-bit tensors
+    read and written as they are.  None where the entry point does not serve the
+    configuration (fp64, up_factor 3, many points)."""
+    n, c, h, w = value.size()
+    shape = (n, key.size(1), c, h, w, P, s, G, _lib.dtype_code(value))
+    nbytes = _lib.lib().sapa_deform_fused_backward_workspace(*shape)
+    if nbytes == 0 or not all(t.dtype == value.dtype for t in (grad_output, query, key, offset)):
+        return None
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=value.device)
+    grads = [_lib.new_out(t) if need else None
+             for t, need in zip((query, key, value, offset), needs)]
+    _lib.call('sapa_deform_fused_backward', value.device, _lib.ptr(grad_output), _lib.ptr(query),
+              _lib.ptr(key), _lib.ptr(value), _lib.ptr(offset), _lib.ptr(ws),
+              *(_lib.ptr(g) if g is not None else None for g in grads), *shape)
+    return grads
+
+
+def _deform_fused_backward(grad_output, query, key, value, offset, P, s, G, offset_layout,
+                           needs=(True, True, True, True)):
     """Gradients of deform_av(softmax(deform_qk(q, k, off), dim=2), v, off)
     with respect to q, k, v and the offset tensor in its own layout."""
     with torch.no_grad():
@@ -182,6 +202,12 @@ def _deform_fused_backward(grad_output, query, key, value, offset, P, s, G, offs
         query, key, value = query.contiguous(), key.contiguous(), value.contiguous()
         grad_output = grad_output.contiguous()
         offset = expand_offset(offset, s, offset_layout).contiguous()
+        native = _native_fused_backward(grad_output, query, key, value, offset, P, s, G, needs)
+        if native is not None:
+            gq, gk, gv, goff = native
+            if goff is not None:
+                goff = _reduce_offset_grad(goff, s, offset_layout)
+            return gq, gk, gv, goff
         # 16-bit tensors: the logits are recomputed from fp32 copies so that, like
         # the forward kernel's, they are not rounded to 16 bits before the softmax
         wide = _compute_dtype(query)
@@ -279,7 +305,7 @@ class DeformSAPAFusedFunction(Function):
         query, key, value, offset = ctx.saved_tensors
         gq, gk, gv, goff = _deform_fused_backward(
             grad_output, query, key, value, offset, ctx.num_point, ctx.scale_factor, ctx.groups,
-            ctx.offset_layout)
+            ctx.offset_layout, tuple(ctx.needs_input_grad[:4]))
         return gq, gk, gv, goff, None, None, None, None, None
 
 

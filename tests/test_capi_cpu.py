@@ -31,7 +31,8 @@ def test_library_exports_every_declared_symbol():
     # (the workspace query returns a size, not a status: bound separately)
     ops = [n for n in names if not n.startswith('sapa_hip_')
            and n not in ('sapa_channel_moments_workspace', 'sapa_channel_moments_static_capacity',
-                         'sapa_fused_backward_workspace', 'sapa_deform_fused_forward_workspace')]
+                         'sapa_fused_backward_workspace', 'sapa_deform_fused_forward_workspace',
+                         'sapa_deform_fused_backward_workspace')]
     assert sorted(ops) == sorted(_lib.SIGNATURES)
     h = _lib.lib()
     assert h.sapa_channel_moments_workspace(16, 256, 67200, 0) > 0
@@ -42,6 +43,13 @@ def test_library_exports_every_declared_symbol():
     assert h.sapa_deform_fused_forward_workspace(8, 128, 256, 64, 64, 25, 2, 4, _lib.DTYPES[torch.bfloat16]) == 8 * 4096 * (128 + 256) * 2
     assert h.sapa_deform_fused_forward_workspace(8, 128, 256, 64, 64, 5, 2, 4, _lib.DTYPES[torch.float32]) == 0
     assert h.sapa_deform_fused_forward_workspace(8, 128, 256, 64, 64, 25, 2, 4, _lib.DTYPES[torch.float64]) == 0
+    # two fp32 [B,G,P,sH,sW] tensors; 16-bit tensors: plus fp32 accumulators of the low-res gradients
+    # and of half of grad_offset
+    per_point = 8 * 4 * 25 * 128 * 128 * 4
+    assert h.sapa_deform_fused_backward_workspace(8, 128, 256, 64, 64, 25, 2, 4, _lib.DTYPES[torch.float32]) == 2 * per_point
+    assert (h.sapa_deform_fused_backward_workspace(8, 128, 256, 64, 64, 25, 2, 4, _lib.DTYPES[torch.bfloat16])
+            == 4 * per_point + 8 * 4096 * (128 + 256) * 4)
+    assert h.sapa_deform_fused_backward_workspace(8, 128, 256, 64, 64, 25, 3, 4, _lib.DTYPES[torch.float32]) == 0
 
 
 def test_abi_version_and_status_strings():

@@ -238,6 +238,92 @@ def test_backward_vs_oracle(coracle, shape):
         torch.testing.assert_close(od.grad.cpu(), goff, **tol)
 
 
+def _deform_fused_backward_oracle(coracle, go, q, key, v, off, P, s, G):
+    """deform_av_backward -> softmax backward -> deform_qk_backward in float64
+    on the given values (the chain autograd runs for sapa_deform.py:51-53)."""
+    go, q, key, v, off = (t.double() for t in (go, q, key, v, off))
+    attn = torch.softmax(coracle.deform_qk(q, key, off, P, s, G, 'f64'), dim=2)
+    ga, gv, goff_av = coracle.deform_av_backward(go, attn, v, off, P, s, G, 'f64')
+    gl = attn * (ga - (ga * attn).sum(dim=2, keepdim=True))
+    gq, gk, goff_qk = coracle.deform_qk_backward(gl, q, key, off, P, s, G, 'f64')
+    return gq, gk, gv, goff_av + goff_qk
+
+
+# B, G, dq, cg, H, W, P, s, offset scale: partial tiles and chunks; offsets beyond the
+# LDS window; s = 4 and s = 1
+BACKWARD_SHAPES = [(2, 2, 8, 12, 9, 11, 9, 2, 1.0), (1, 4, 5, 3, 7, 6, 17, 2, 6.0),
+                   (1, 1, 4, 6, 5, 4, 5, 4, 2.0), (1, 2, 6, 4, 10, 9, 13, 1, 1.5)]
+
+
+@pytest.mark.parametrize('dtype,tol', [(torch.float32, dict(rtol=1e-4, atol=2e-5)),
+                                        (torch.bfloat16, 1.5e-2), (torch.float16, 2e-3)])
+@pytest.mark.parametrize('shape', BACKWARD_SHAPES, ids=['-'.join(map(str, s)) for s in BACKWARD_SHAPES])
+def test_deform_fused_backward_entry_point(coracle, shape, dtype, tol):
+    """sapa_deform_fused_backward through the C ABI: the four gradients against the
+    float64 oracle chain on the same (rounded) inputs; fp32 intermediates for 16-bit
+    tensors, only the gradients themselves are rounded to 16 bits.  Offsets sit away
+    from integers, where the bilinear sample has a kink."""
+    from sapa_amd import _lib
+    B, G, dq, cg, H, W, P, s, oscale = shape
+    g = gen(240)
+    q, key, v, off, _ = make(g, shape[:8], off_scale=oscale)
+    frac = off - off.floor()
+    off = off.floor() + frac.clamp(0.2, 0.8)        # the 16-bit rounding must not cross an integer
+    go = randn(g, B, G * cg, H * s, W * s)
+    q, key, v, off, go = (t.to(dtype) for t in (q, key, v, off, go))
+    qd, kd, vd, od, god = dev(q, key, v, off, go)
+    h = _lib.lib()
+    args = (B, G * dq, G * cg, H, W, P, s, G, _lib.DTYPES[dtype])
+    nbytes = h.sapa_deform_fused_backward_workspace(*args)
+    assert nbytes > 0
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=DEV)
+    grads = [torch.full_like(t, float('nan')) for t in (qd, kd, vd, od)]
+    assert _lib.call_status('sapa_deform_fused_backward', DEV, _lib.ptr(god), _lib.ptr(qd), _lib.ptr(kd),
+                            _lib.ptr(vd), _lib.ptr(od), _lib.ptr(ws), *(_lib.ptr(t) for t in grads), *args) == 0
+    want = _deform_fused_backward_oracle(coracle, go.float(), q.float(), key.float(), v.float(), off.float(), P, s, G)
+    for got, w, name in zip(grads, want, ('grad_query', 'grad_key', 'grad_value', 'grad_offset')):
+        assert torch.isfinite(got).all(), name
+        if dtype == torch.float32:
+            torch.testing.assert_close(got.cpu().double(), w, msg=lambda m: f'{name}: {m}', **tol)
+        else:
+            assert_rel_rms_close(got.float().cpu(), w, tol, f'{name} {dtype}')
+    # only grad_key and grad_offset wanted: the other buffers stay as they are
+    gq2, gv2 = torch.full_like(qd, 7.0), torch.full_like(vd, 7.0)
+    gk2, go2 = torch.full_like(kd, float('nan')), torch.full_like(od, float('nan'))
+    assert _lib.call_status('sapa_deform_fused_backward', DEV, _lib.ptr(god), _lib.ptr(qd), _lib.ptr(kd),
+                            _lib.ptr(vd), _lib.ptr(od), _lib.ptr(ws), None, _lib.ptr(gk2), None, _lib.ptr(go2),
+                            *args) == 0
+    assert (gq2 == 7).all() and (gv2 == 7).all() and torch.equal(go2, grads[3])
+    torch.testing.assert_close(gk2.float(), grads[1].float(), rtol=1e-5, atol=1e-6)   # float atomics: order varies
+    # the autograd route takes the same entry point, also with the offsets read in
+    # place from a low-res tensor (their gradient is folded back to its layout)
+    leaves = [t.clone().requires_grad_() for t in (qd, kd, vd, od)]
+    sapa_amd.deform_sapa_fused(*leaves, P, s, G).backward(god)
+    for leaf, got, name in zip(leaves, grads, ('grad_query', 'grad_key', 'grad_value', 'grad_offset')):
+        torch.testing.assert_close(leaf.grad.float(), got.float(), rtol=1e-5, atol=1e-6, msg=lambda m: f'{name}: {m}')
+
+
+def test_deform_fused_backward_limits():
+    from sapa_amd import _lib
+    h = _lib.lib()
+    f32, f64 = _lib.DTYPES[torch.float32], _lib.DTYPES[torch.float64]
+    assert h.sapa_deform_fused_backward_workspace(1, 8, 8, 4, 4, 9, 3, 2, f32) == 0     # up_factor 3
+    assert h.sapa_deform_fused_backward_workspace(1, 8, 8, 4, 4, 9, 2, 2, f64) == 0
+    assert h.sapa_deform_fused_backward_workspace(1, 8, 8, 4, 4, 49, 2, 2, f32) == 0    # many points
+    x = torch.zeros(1, 8, 8, 8, device=DEV)
+    lo = torch.zeros(1, 8, 4, 4, device=DEV)
+    off = torch.zeros(1, 2 * 2 * 9, 12, 12, device=DEV)
+    ws = torch.empty(256, dtype=torch.uint8, device=DEV)
+    assert _lib.call_status('sapa_deform_fused_backward', DEV, _lib.ptr(x), _lib.ptr(x), _lib.ptr(lo), _lib.ptr(lo),
+                            _lib.ptr(off), _lib.ptr(ws), _lib.ptr(x), None, None, None,
+                            1, 8, 8, 4, 4, 9, 3, 2, f32) == _lib.UNSUPPORTED
+    # such configurations still train through the separate backward entry points
+    q = torch.randn(1, 8, 12, 12, device=DEV, requires_grad=True)
+    k = torch.randn(1, 8, 4, 4, device=DEV, requires_grad=True)
+    sapa_amd.deform_sapa_fused(q, k, k.detach(), off, 9, 3, 2).sum().backward()
+    assert torch.isfinite(q.grad).all() and torch.isfinite(k.grad).all()
+
+
 def test_gradcheck_reference_shapes():
     """deformsapa/deformsapa/grad_check.py:8-35: float64 gradcheck at its
     shapes, offsets in [0,1) so no sample sits on a bilinear kink.  The
