@@ -66,8 +66,15 @@ hipError_t deform_lowgrad_any(const void *hi, const void *sc, const void *low, c
         else if (e != hipErrorNotSupported) return e;
     }
     if (grad_low) {
-        const hipError_t e =
-            deform_lowgrad_lds_launch(hi, sc, offset, grad_low, B, Cx, H, W, P, s, G, dtype, st);
+        // the matrix-product form first (SAPA_SCATTER_MAT_OFF: a tuning build without it),
+        // then the LDS-window scatter
+#ifdef SAPA_SCATTER_MAT_OFF
+        hipError_t e = hipErrorNotSupported;
+#else
+        hipError_t e = deform_scatter_mat_launch(hi, sc, offset, grad_low, B, Cx, H, W, P, s, G, dtype, st);
+#endif
+        if (e == hipErrorNotSupported)
+            e = deform_lowgrad_lds_launch(hi, sc, offset, grad_low, B, Cx, H, W, P, s, G, dtype, st);
         if (e == hipSuccess) grad_low = nullptr;
         else if (e != hipErrorNotSupported) return e;
     }

@@ -73,6 +73,14 @@ hipError_t deform_fused_nhwc_launch(const void *q, const void *key, const void *
                                     int W, int P, int s, int G, int dtype, hipStream_t st,
                                     const char **kernel = nullptr);
 
+// sapa_d_scatter.hip: the same gradient (grad_key / grad_value of the sampled
+// operators) as a matrix product per region; fp32 tensors, or (wide) f16 / bf16
+// features with fp32 per-point scalars; s in {1, 2, 4}, P <= 32; grad_low fp32,
+// accumulated into.  hipErrorNotSupported otherwise.
+hipError_t deform_scatter_mat_launch(const void *hi, const void *sc, const void *offset, void *grad_low,
+                                     int B, int Cx, int H, int W, int P, int s, int G, int dtype,
+                                     hipStream_t st, bool wide = false);
+
 // sapa_d_backward.hip: the backward pass of the fused SAPA-D operator in one call;
 // attention weights and logit gradients as fp32 in `workspace` (256-byte aligned,
 // deform_fused_backward_workspace() bytes; 0 = not served), f16 / bf16 tensors read

@@ -56,6 +56,21 @@ static unsigned blocks_for(long n) {
 
 static long align256(long x) { return (x + 255) / 256 * 256; }
 
+// grad_low += scatter(hi, sc): the matrix-product form where it applies, else the
+// LDS-window scatter
+static hipError_t scatter_low(const void *hi, const void *sc, const void *offset, void *grad_low, int B,
+                              int Cx, int H, int W, int P, int s, int G, int dtype, hipStream_t st,
+                              bool wide) {
+#ifdef SAPA_SCATTER_MAT_OFF
+    hipError_t e = hipErrorNotSupported;
+#else
+    hipError_t e = deform_scatter_mat_launch(hi, sc, offset, grad_low, B, Cx, H, W, P, s, G, dtype, st, wide);
+#endif
+    if (e == hipErrorNotSupported)
+        e = deform_lowgrad_lds_launch(hi, sc, offset, grad_low, B, Cx, H, W, P, s, G, dtype, st, wide);
+    return e;
+}
+
 }  // namespace dbwd
 
 // Bytes of workspace, or 0 for configurations this call does not serve (the
@@ -120,7 +135,7 @@ hipError_t deform_fused_backward_launch(const void *grad_out, const void *q, con
         hipLaunchKernelGGL(zero_kernel, dim3(blocks_for((long)B * C * lpix)), dim3(256), 0, st, gv32,
                            (long)B * C * lpix);
         SAPA_STEP(hipGetLastError());
-        SAPA_STEP(deform_lowgrad_lds_launch(grad_out, attn, offset, gv32, B, C, H, W, P, s, G, dtype, st, wide));
+        SAPA_STEP(scatter_low(grad_out, attn, offset, gv32, B, C, H, W, P, s, G, dtype, st, wide));
     }
     // similarity: grad_query (aggregation of key with grad_logits), grad_key
     // (scatter) and the other share of grad_offset
@@ -134,7 +149,7 @@ hipError_t deform_fused_backward_launch(const void *grad_out, const void *q, con
         hipLaunchKernelGGL(zero_kernel, dim3(blocks_for((long)B * Cq * lpix)), dim3(256), 0, st, gk32,
                            (long)B * Cq * lpix);
         SAPA_STEP(hipGetLastError());
-        SAPA_STEP(deform_lowgrad_lds_launch(q, gl, offset, gk32, B, Cq, H, W, P, s, G, dtype, st, wide));
+        SAPA_STEP(scatter_low(q, gl, offset, gk32, B, Cq, H, W, P, s, G, dtype, st, wide));
     }
     if (wide) {
         if (grad_key) {
