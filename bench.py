@@ -65,8 +65,13 @@ MEASURED_TRAFFIC = {
     ('stress', 'bf16', 'nchw'): (380752179, 'profiles/sapa_b_mfma_fused_stress_bf16.md', 'sapa_b_mfma_kernel'),
     ('stress', 'bf16', 'channels_last'): (323093471, 'profiles/sapa_b_nhwc16_fused_stress_bf16.md',
                                           'sapa_b_nhwc16_kernel'),
-    ('deform_p25', 'fp32', 'nchw'): (829340888, 'profiles/sapa_d_lds_fused_deform_p25_fp32.md', 'deform_lds_kernel'),
-    ('deform_p9', 'fp32', 'nchw'): (402514487, 'profiles/sapa_d_lds_fused_deform_p9_fp32.md', 'deform_lds_kernel'),
+    ('deform_p25', 'fp32', 'nchw'): (513060882, 'profiles/sapa_d_wmat_fused_deform_p25_fp32_nchw.md',
+                                     'deform_fused_wmat_kernel'),
+    ('deform_p25', 'bf16', 'nchw'): (228826463, 'profiles/sapa_d_wmat16_fused_deform_p25_bf16_nchw.md',
+                                     'deform_fused_wmat16_kernel'),
+    ('deform_p25', 'fp32', 'nchw_reference_order'): (829727510, 'profiles/sapa_d_lds_fused_deform_p25_fp32.md',
+                                                     'deform_lds_kernel'),
+    ('deform_p9', 'fp32', 'nchw'): (401608116, 'profiles/sapa_d_lds_fused_deform_p9_fp32.md', 'deform_lds_kernel'),
     ('deform_p25', 'fp32', 'channels_last'): (356742233, 'profiles/sapa_d_nhwc_fused_deform_p25_fp32.md',
                                               'deform_fused_wmat_kernel'),
     ('deform_p25', 'bf16', 'channels_last'): (178450680, 'profiles/sapa_d_wmat16_fused_deform_p25_bf16.md',
@@ -259,6 +264,10 @@ def main():
     ap.add_argument('--settle-ms', type=float, default=40.0,
                     help='GPU time (ms) of untimed launches of the same step before the warm-up '
                          'steps, to let the power management settle after idle; 0 = none')
+    ap.add_argument('--reference-order', action='store_true',
+                    help='SAPA-D, contiguous tensors: time sapa_deform_fused_forward (sums in the '
+                         "reference's order) as the main line instead of the matrix-form path that "
+                         'sapa_amd.deform_sapa_fused takes by default where it is faster')
     ap.add_argument('--only-main', action='store_true',
                     help='skip the channels_last timing that a default (contiguous) SAPA-B / SAPA-D '
                          'forward line carries along (e.g. under a profiler)')
@@ -320,7 +329,7 @@ def main():
             return step
         # contiguous tensors through the matrix-form kernels (key and value copied to
         # channels-last order in a workspace): what sapa_amd.deform_sapa_fused does by
-        # default for 16-bit tensors, on request (matrix_form=True) for fp32
+        # default where it is the faster path (16-bit tensors from 6 points, fp32 from 15)
         ws_bytes = lib.sapa_deform_fused_forward_workspace(B, G * d, C, H, W, P, s, G, code)
         ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
 
@@ -328,7 +337,7 @@ def main():
             _lib.check(lib.sapa_deform_fused_forward_ws(
                 q.data_ptr(), key.data_ptr(), v.data_ptr(), off.data_ptr(), out.data_ptr(), ws.data_ptr(),
                 B, G * d, C, H, W, P, s, G, 0, code, stream.cuda_stream), 'sapa_deform_fused_forward_ws')
-        main_is_ws = args.layout == 'nchw' and ws_bytes > 0 and dtype != torch.float32
+        main_is_ws = args.layout == 'nchw' and ws_bytes > 0 and not args.reference_order
         step = ws_step if main_is_ws else fused_step(
             'sapa_deform_fused_forward_nhwc' if args.layout == 'channels_last' else 'sapa_deform_fused_forward',
             q, key, v, out, off)
@@ -400,15 +409,15 @@ def main():
         err_cl = (cl[3][:1].float() - out[:1].float()).abs().max().item()
         del cl
 
-    matrix_form = None
-    if deform and args.layout == 'nchw' and ws_bytes > 0 and not main_is_ws and args.direction == 'forward' \
-            and not args.only_main:
-        ref_out = out[:1].clone()
-        ms_m, _ = timed(ws_step)
-        matrix_form = {'ms_per_step': ms_m, 'kernel': _lib.last_kernel(), 'workspace_bytes': ws_bytes,
-                       'max_abs_diff_vs_main_image0': (out[:1].float() - ref_out.float()).abs().max().item(),
-                       'note': 'the same contiguous tensors through sapa_deform_fused_forward_ws '
-                               '(sapa_amd.deform_sapa_fused(..., matrix_form=True))'}
+    reference_order = None
+    if deform and main_is_ws and args.direction == 'forward' and not args.only_main:
+        # the same contiguous tensors through the kernel that keeps the reference's order of sums
+        ws_out = out[:1].clone()
+        ms_r, _ = timed(fused_step('sapa_deform_fused_forward', q, key, v, out, off))
+        reference_order = {'ms_per_step': ms_r, 'kernel': _lib.last_kernel(),
+                           'max_abs_diff_vs_main_image0': (out[:1].float() - ws_out.float()).abs().max().item(),
+                           'note': 'sapa_deform_fused_forward (sapa_amd.deform_sapa_fused(..., matrix_form=False)); '
+                                   'python bench.py --reference-order makes this the main line'}
         step()      # the main line's result back into `out` for the checks below
 
     if args.calibration_copy:
@@ -449,7 +458,8 @@ def main():
         kern = 'several (see profiles/)'
     traffic = traffic_source = None
     if not train:
-        traffic, traffic_source = measured_traffic(args.workload, args.dtype, args.layout, main_kernel)
+        tlayout = 'nchw_reference_order' if deform and args.layout == 'nchw' and args.reference_order else args.layout
+        traffic, traffic_source = measured_traffic(args.workload, args.dtype, tlayout, main_kernel)
     achieved = abytes / (ms * 1e-3) / 1e9
     rec = {
         'metric': f'upsampled Gpix/s, {what}, 1 GPU',
@@ -490,10 +500,10 @@ def main():
             'max_abs_diff_vs_nchw_image0': err_cl,
             'note': 'same workload and algorithmic bytes, every tensor in torch.channels_last '
                     'order (python bench.py --layout channels_last makes this the main line)'}
-    if matrix_form is not None:
-        matrix_form['value'] = pix / (matrix_form['ms_per_step'] * 1e-3) / 1e9
-        matrix_form['roofline_frac'] = abytes / (matrix_form['ms_per_step'] * 1e-3) / 1e9 / HBM_PEAK_GBS
-        rec['matrix_form'] = matrix_form
+    if reference_order is not None:
+        reference_order['value'] = pix / (reference_order['ms_per_step'] * 1e-3) / 1e9
+        reference_order['roofline_frac'] = abytes / (reference_order['ms_per_step'] * 1e-3) / 1e9 / HBM_PEAK_GBS
+        rec['reference_order'] = reference_order
     if deform and not train and main_is_ws:
         rec['config']['workspace_bytes'] = ws_bytes
         rec['config']['entry'] = 'sapa_deform_fused_forward_ws (key / value copied to channels-last order inside the timed call)'

@@ -608,23 +608,56 @@ deform_fused_wmat_kernel(const T *__restrict__ q, const T *__restrict__ key,
         }
     };
     // q of pixel mi as the A operand: channels 16 s + 4 mk .. + 3 of the group, s < DP / 16
+    // Channels-last: 4 contiguous elements of global memory per lane.  Contiguous
+    // layout: the tile's q (16 pixels x d channel planes) comes in once per workgroup,
+    // a thread fetching one tile row (4 x-neighbours) of one plane, and goes through
+    // LDS as [pixel][channel], from where every wave reads its operands.
     Raw qa[DP / 16];
+    constexpr int QS = DP + 4;                                       // floats per pixel of the q tile
+    static_assert(NPX * QS <= NPX * WS, "the q tile fits the weight matrix's buffer");
+    float *const Ql = Wl;           // (contiguous layout) the q tile, until the similarity has its operands
+    constexpr int QN = NCHW ? (TPW * DP + NT - 1) / NT : 1;          // tile rows per thread
+    Raw qrow[QN];
+    const bool qvec = hW % TPW == 0 && (uintptr_t)q % sizeof(Raw) == 0;
     auto load_q = [&](int g) __attribute__((always_inline)) {
+        if (NCHW) {
 #pragma unroll
-        for (int s16 = 0; s16 < DP / 16; ++s16) {
-            qa[s16] = Raw{};
-            if (mpx.active && 16 * s16 + 4 * mk < d) {
-                if (NCHW) {
-                    // 4 channel planes, one element each
-                    const T *qp = q + ((long)n * Cq + g * d + 16 * s16 + 4 * mk) * hpl + mpx.pp;
-                    union { T h[4]; Raw r; } x;
+            for (int i = 0; i < QN; ++i) {
+                const int item = i * NT + tid, ch = item / TPW, qh = y0 + item % TPW;
+                qrow[i] = Raw{};
+                if (ch < d && qh < hH) {        // (ch < d <= DP: also the bound of the items)
+                    const T *qp = q + ((long)n * Cq + g * d + ch) * hpl + (long)qh * hW + x0;
+                    if (qvec) {
+                        qrow[i] = *(const Raw *)qp;
+                    } else {
+                        union { T h[4]; Raw r; } x;
+                        x.r = Raw{};
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) x.h[e] = qp[e * hpl];
-                    qa[s16] = x.r;
-                } else {
-                    qa[s16] = *(const Raw *)(q + mpx.hp * Cq + g * d + 16 * s16 + 4 * mk);
+                        for (int e = 0; e < TPW; ++e)
+                            if (x0 + e < hW) x.h[e] = qp[e];
+                        qrow[i] = x.r;
+                    }
                 }
             }
+        } else {
+#pragma unroll
+            for (int s16 = 0; s16 < DP / 16; ++s16) {
+                qa[s16] = Raw{};
+                if (mpx.active && 16 * s16 + 4 * mk < d)
+                    qa[s16] = *(const Raw *)(q + mpx.hp * Cq + g * d + 16 * s16 + 4 * mk);
+            }
+        }
+    };
+    // (contiguous layout) the fetched rows into the q tile; channels d .. DP hold zeros
+    auto stage_store_q = [&]() __attribute__((always_inline)) {
+        if (!NCHW) return;
+#pragma unroll
+        for (int i = 0; i < QN; ++i) {
+            const int item = i * NT + tid, ch = item / TPW, row = item % TPW;
+            if (TPW * DP % NT != 0 && ch >= DP) break;
+            const f32x4 v = Q4::widen(qrow[i]);
+#pragma unroll
+            for (int e = 0; e < TPW; ++e) Ql[(row * TPW + e) * QS + ch] = v[e];
         }
     };
 
@@ -634,8 +667,10 @@ deform_fused_wmat_kernel(const T *__restrict__ q, const T *__restrict__ key,
     for (int g = 0; g < G; ++g) {
         // ---- (a) key window and an empty weight matrix
         stage_store(KS, DP / 4);
+        stage_store_q();
         if (tid == 0) fb_flag = 0;
-        for (int i = tid; i < NPX * WS / 4; i += NT) ((f32x4 *)Wl)[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (!NCHW)
+            for (int i = tid; i < NPX * WS / 4; i += NT) ((f32x4 *)Wl)[i] = f32x4{0.f, 0.f, 0.f, 0.f};
         __syncthreads();
         // the group's first value chunk and the offsets travel during the similarity
         stage_load(false, g * cg, cg < CHK ? cg : CHK);
@@ -679,7 +714,13 @@ deform_fused_wmat_kernel(const T *__restrict__ q, const T *__restrict__ key,
         {
             f32x4 a4[DP / 16];
 #pragma unroll
-            for (int s16 = 0; s16 < DP / 16; ++s16) a4[s16] = Q4::widen(qa[s16]);
+            for (int s16 = 0; s16 < DP / 16; ++s16)
+                a4[s16] = NCHW ? *(const f32x4 *)(Ql + mi * QS + 16 * s16 + 4 * mk) : Q4::widen(qa[s16]);
+            if (NCHW) {
+                // every wave has its operands: the buffer becomes the empty weight matrix
+                __syncthreads();
+                for (int i = tid; i < NPX * WS / 4; i += NT) ((f32x4 *)Wl)[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
             for (int nb = wave; nb < NKB; nb += 4) {
                 f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll

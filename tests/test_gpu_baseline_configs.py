@@ -265,19 +265,24 @@ def test_c4_deform_against_oracle(coracle, P):
     assert torch.equal(out[list(imgs)].cpu(), want)
     # fused, both memory orders
     fused = lambda a, b, c, o: sapa_amd.deform_sapa_fused(a, b, c, o, P, s, G)
-    got = assert_batch_equals_images(fused, (qd, kd, vd, od), f'c4 P={P} fused', images=(0, 3, B - 1))
+    fused_r = lambda a, b, c, o: sapa_amd.deform_sapa_fused(a, b, c, o, P, s, G, matrix_form=False)
+    got = assert_batch_equals_images(fused_r, (qd, kd, vd, od), f'c4 P={P} fused', images=(0, 3, B - 1))
     want_f = per_image(coracle.deform_sapa_fused, sub(q, key, v, off), P, s, G, 'f32')
-    assert_f32_close(got[list(imgs)].cpu(), want_f, f'c4 P={P} fused')
+    assert_f32_close(got[list(imgs)].cpu(), want_f, f'c4 P={P} fused, reference order')
     got_cl = assert_batch_equals_images(fused, as_cl(qd, kd, vd, od), f'c4 P={P} fused channels_last',
                                         images=(0, 3, B - 1))
     exact = per_image(coracle.deform_sapa_fused, [t.double() for t in sub(q, key, v, off)], P, s, G, 'f64')
     assert_no_worse_than_reference_order(got_cl[list(imgs)], want_f, exact, f'c4 P={P} fused channels_last')
+    # contiguous tensors, the default route: the matrix-form kernel from 15 points on (key and
+    # value via a workspace), the reference's order of sums below
+    got_m = assert_batch_equals_images(fused, (qd, kd, vd, od), f'c4 P={P} fused default', images=(0, 3, B - 1))
+    assert got_m.is_contiguous()
     if P >= 15:
-        # contiguous tensors through the same matrix-form kernel (key and value via a workspace)
-        fused_m = lambda a, b, c, o: sapa_amd.deform_sapa_fused(a, b, c, o, P, s, G, matrix_form=True)
-        got_m = assert_batch_equals_images(fused_m, (qd, kd, vd, od), f'c4 P={P} fused matrix form', images=(0, 3, B - 1))
-        assert got_m.is_contiguous()
+        from sapa_amd import _lib
+        assert _lib.last_kernel() == 'deform_fused_wmat_kernel'
         assert_no_worse_than_reference_order(got_m[list(imgs)], want_f, exact, f'c4 P={P} fused matrix form')
+    else:
+        assert torch.equal(got_m, got)
     # 16-bit tensors, contiguous and channels_last
     hq, hk, hv, ho = (t.to(torch.bfloat16) for t in (qd, kd, vd, od))
     exact16 = per_image(coracle.deform_sapa_fused, [t[list(imgs)].double().cpu() for t in (hq, hk, hv, ho)],
@@ -301,8 +306,11 @@ def test_c4_regular_grid_offsets_reduce_to_sapa_b():
     qd, kd, vd, od = dev(q, key, v, off)
     assert torch.equal(sapa_amd.deform_qk(qd, kd, od, K * K, s, 1).squeeze(1), sapa_amd.qk(qd, kd, K, s))
     want = sapa_amd.sapa_fused(qd, kd, vd, K, s)
-    assert_f32_close(sapa_amd.deform_sapa_fused(qd, kd, vd, od, K * K, s, 1), want, 'regular grid, contiguous')
+    assert_f32_close(sapa_amd.deform_sapa_fused(qd, kd, vd, od, K * K, s, 1, matrix_form=False), want,
+                     'regular grid, contiguous, reference order')
     exact = sapa_amd.sapa_fused(qd.double(), kd.double(), vd.double(), K, s)
+    assert_no_worse_than_reference_order(sapa_amd.deform_sapa_fused(qd, kd, vd, od, K * K, s, 1), want, exact,
+                                         'regular grid, contiguous, matrix form')
     assert_no_worse_than_reference_order(sapa_amd.deform_sapa_fused(*as_cl(qd, kd, vd, od), K * K, s, 1), want,
                                          exact, 'regular grid, channels_last')
 

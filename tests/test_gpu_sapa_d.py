@@ -90,10 +90,12 @@ def test_deform_fused_matrix_form_on_contiguous_tensors(coracle, shape, dtype):
             assert_f32_close(got, want, 'matrix form')
         else:   # the reference's own check tolerance (deformsapa/deformsapa/forward_check.py)
             torch.testing.assert_close(got.cpu(), want, rtol=1e-5, atol=1e-5)
-        # the default for fp32 stays the reference's order of sums
-        plain = sapa_amd.deform_sapa_fused(*dev(q, key, v, off), P, s, G)
+        # the reference's order of sums on request
+        plain = sapa_amd.deform_sapa_fused(*dev(q, key, v, off), P, s, G, matrix_form=False)
         assert _lib.last_kernel() != kernel
-        assert_f32_close(plain, want, 'default path')
+        assert_f32_close(plain, want, 'reference order')
+        auto = sapa_amd.deform_sapa_fused(*dev(q, key, v, off), P, s, G)
+        assert _lib.last_kernel() == kernel and torch.equal(auto, got)
     else:
         assert kernel == ('deform_fused_wmat16_kernel' if dq % 8 == 0 and cg % 8 == 0 else 'deform_fused_wmat_kernel')
         assert_rel_rms_close(got.float(), want, BF16_REL if dtype == torch.bfloat16 else F16_REL, 'matrix form')
