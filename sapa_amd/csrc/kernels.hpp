@@ -81,6 +81,16 @@ hipError_t deform_scatter_mat_launch(const void *hi, const void *sc, const void 
                                      int B, int Cx, int H, int W, int P, int s, int G, int dtype,
                                      hipStream_t st, bool wide = false);
 
+// The per-pixel part of the fused SAPA-D backward in the matrix form of the
+// forward kernel (sapa_d_bwdmat.hip): attention weights and gradient of the
+// logits (fp32 [B, G, P, sH, sW], for the scatter kernels), grad_offset and
+// grad_query (either may be NULL).  key_cl, value_cl: channels-last copies.
+bool deform_bwd_wmat_serves(int B, int Cq, int C, int H, int W, int P, int s, int G, int dtype);
+hipError_t deform_bwd_wmat_launch(const void *grad_out, const void *q, const void *key_cl,
+                                  const void *value_cl, const void *offset, float *attn_ws,
+                                  float *gl_ws, void *grad_q, void *grad_offset, int B, int Cq, int C,
+                                  int H, int W, int P, int s, int G, int dtype, hipStream_t st);
+
 // sapa_d_backward.hip: the backward pass of the fused SAPA-D operator in one call;
 // attention weights and logit gradients as fp32 in `workspace` (256-byte aligned,
 // deform_fused_backward_workspace() bytes; 0 = not served), f16 / bf16 tensors read

@@ -71,6 +71,18 @@ static hipError_t scatter_low(const void *hi, const void *sc, const void *offset
     return e;
 }
 
+// The per-pixel part of the chain (attention weights, gradient of the logits,
+// grad_offset, grad_query) in one matrix-form kernel instead of five launches
+// of per-pixel gathers.  (B=8, C=256, G=4, d=32, 64x64 -> 128x128, fp32: the
+// whole backward call with / without it, us: P = 25 ... ; P = 9 ...; P = 5 ...)
+static bool matrix_stage(int B, int Cq, int C, int H, int W, int P, int s, int G, int dtype) {
+#ifdef SAPA_BWD_MAT_OFF
+    return false;
+#else
+    return deform_bwd_wmat_serves(B, Cq, C, H, W, P, s, G, dtype);
+#endif
+}
+
 }  // namespace dbwd
 
 // Bytes of workspace, or 0 for configurations this call does not serve (the
@@ -83,9 +95,16 @@ long deform_fused_backward_workspace(int B, int Cq, int C, int H, int W, int P, 
     if (P > 48) return 0;       // [2P][thread] sums of the offset gradient next to the window in LDS
     const long per_point = (long)B * G * P * H * s * W * s * (long)sizeof(float);
     long n = 2 * align256(per_point);
-    // 16-bit tensors: fp32 accumulators of the low-res gradients and of the first
-    // half of grad_offset
-    if (dtype != 0) n += align256((long)B * Cq * H * W * 4) + align256((long)B * C * H * W * 4) + align256(2 * per_point);
+    // 16-bit tensors: fp32 accumulators of the low-res gradients
+    if (dtype != 0) n += align256((long)B * Cq * H * W * 4) + align256((long)B * C * H * W * 4);
+    if (dbwd::matrix_stage(B, Cq, C, H, W, P, s, G, dtype)) {
+        // channels-last copies of key and value for the matrix-form kernel
+        const long esize = dtype == 0 ? 4 : 2;
+        n += align256((long)B * Cq * H * W * esize) + align256((long)B * C * H * W * esize);
+    } else if (dtype != 0) {
+        // the first half of grad_offset in fp32
+        n += align256(2 * per_point);
+    }
     return n;
 }
 
@@ -107,7 +126,9 @@ hipError_t deform_fused_backward_launch(const void *grad_out, const void *q, con
     float *gl = (float *)(w + align256(n_pp * 4));
     float *gk32 = wide ? (float *)(w + 2 * align256(n_pp * 4)) : (float *)grad_key;
     float *gv32 = wide ? (float *)((char *)gk32 + align256((long)B * Cq * lpix * 4)) : (float *)grad_value;
-    float *goff32 = wide ? (float *)((char *)gv32 + align256((long)B * C * lpix * 4)) : nullptr;
+    char *rest = wide ? (char *)gv32 + align256((long)B * C * lpix * 4) : w + 2 * align256(n_pp * 4);
+    const bool mat = matrix_stage(B, Cq, C, H, W, P, s, G, dtype);
+    float *goff32 = wide && !mat ? (float *)rest : nullptr;
     const int HIRES = 0;
     hipError_t e;
 #define SAPA_STEP(call)                  \
@@ -116,35 +137,43 @@ hipError_t deform_fused_backward_launch(const void *grad_out, const void *q, con
         if (e != hipSuccess) return e;   \
     } while (0)
 
-    // attention weights: sampled similarity (mode 0), softmax over the points
-    SAPA_STEP(deform_lds_launch(0, q, key, nullptr, nullptr, offset, attn, B, Cq, Cq, H, W, P, s, G, HIRES,
-                                dtype, st, wide));
-    SAPA_STEP(softmax_generic_launch(attn, attn, (long)B * G, P, hpix, 0, st));
-    // gradient of the weights: the similarity of grad_out and value
-    SAPA_STEP(deform_lds_launch(0, grad_out, value, nullptr, nullptr, offset, gl, B, C, C, H, W, P, s, G,
-                                HIRES, dtype, st, wide));
-    hipLaunchKernelGGL(softmax_backward_kernel, dim3(blocks_for((long)B * G * hpix)), dim3(256), 0, st, attn,
-                       gl, (long)B * G, P, hpix);
-    SAPA_STEP(hipGetLastError());
-
-    // aggregation: grad_value (scatter) and its share of grad_offset
-    if (grad_offset)
-        SAPA_STEP(deform_lds_launch(3, grad_out, value, attn, nullptr, offset, grad_offset, B, C, C, H, W, P, s,
-                                    G, HIRES, dtype, st, wide, false, goff32));
+    if (mat) {
+        const long esize = wide ? 2 : 4;
+        char *key_cl = rest, *value_cl = rest + align256((long)B * Cq * lpix * esize);
+        SAPA_STEP(nchw_to_nhwc_launch(key, key_cl, Cq, value, value_cl, C, B, lpix, (int)esize, st));
+        SAPA_STEP(deform_bwd_wmat_launch(grad_out, q, key_cl, value_cl, offset, attn, gl, grad_q, grad_offset, B,
+                                         Cq, C, H, W, P, s, G, dtype, st));
+    } else {
+        // attention weights: sampled similarity (mode 0), softmax over the points
+        SAPA_STEP(deform_lds_launch(0, q, key, nullptr, nullptr, offset, attn, B, Cq, Cq, H, W, P, s, G, HIRES,
+                                    dtype, st, wide));
+        SAPA_STEP(softmax_generic_launch(attn, attn, (long)B * G, P, hpix, 0, st));
+        // gradient of the weights: the similarity of grad_out and value
+        SAPA_STEP(deform_lds_launch(0, grad_out, value, nullptr, nullptr, offset, gl, B, C, C, H, W, P, s, G,
+                                    HIRES, dtype, st, wide));
+        hipLaunchKernelGGL(softmax_backward_kernel, dim3(blocks_for((long)B * G * hpix)), dim3(256), 0, st, attn,
+                           gl, (long)B * G, P, hpix);
+        SAPA_STEP(hipGetLastError());
+        // grad_offset: the aggregation's share, then the similarity's
+        if (grad_offset) {
+            SAPA_STEP(deform_lds_launch(3, grad_out, value, attn, nullptr, offset, grad_offset, B, C, C, H, W, P, s,
+                                        G, HIRES, dtype, st, wide, false, goff32));
+            SAPA_STEP(deform_lds_launch(3, q, key, gl, nullptr, offset, grad_offset, B, Cq, Cq, H, W, P, s, G, HIRES,
+                                        dtype, st, wide, true, goff32));
+        }
+        // grad_query: aggregation of key with the gradient of the logits
+        if (grad_q)
+            SAPA_STEP(deform_lds_launch(1, nullptr, nullptr, gl, key, offset, grad_q, B, Cq, Cq, H, W, P, s, G, HIRES,
+                                        dtype, st, wide));
+    }
+    // the low-res gradients: grad_value (attention weights x grad_out) and
+    // grad_key (gradient of the logits x query), scattered
     if (grad_value) {
         hipLaunchKernelGGL(zero_kernel, dim3(blocks_for((long)B * C * lpix)), dim3(256), 0, st, gv32,
                            (long)B * C * lpix);
         SAPA_STEP(hipGetLastError());
         SAPA_STEP(scatter_low(grad_out, attn, offset, gv32, B, C, H, W, P, s, G, dtype, st, wide));
     }
-    // similarity: grad_query (aggregation of key with grad_logits), grad_key
-    // (scatter) and the other share of grad_offset
-    if (grad_q)
-        SAPA_STEP(deform_lds_launch(1, nullptr, nullptr, gl, key, offset, grad_q, B, Cq, Cq, H, W, P, s, G, HIRES,
-                                    dtype, st, wide));
-    if (grad_offset)
-        SAPA_STEP(deform_lds_launch(3, q, key, gl, nullptr, offset, grad_offset, B, Cq, Cq, H, W, P, s, G, HIRES,
-                                    dtype, st, wide, true, goff32));
     if (grad_key) {
         hipLaunchKernelGGL(zero_kernel, dim3(blocks_for((long)B * Cq * lpix)), dim3(256), 0, st, gk32,
                            (long)B * Cq * lpix);
