@@ -77,9 +77,11 @@ hipError_t deform_fused_nhwc_launch(const void *q, const void *key, const void *
 // operators) as a matrix product per region; fp32 tensors, or (wide) f16 / bf16
 // features with fp32 per-point scalars; s in {1, 2, 4}, P <= 32; grad_low fp32,
 // accumulated into.  hipErrorNotSupported otherwise.
+// channels_last_out: grad_low is a [B, H, W, Cx] fp32 buffer instead of the contiguous tensor.
+bool deform_scatter_mat_serves(int B, int Cx, int H, int W, int P, int s, int G, int dtype);
 hipError_t deform_scatter_mat_launch(const void *hi, const void *sc, const void *offset, void *grad_low,
                                      int B, int Cx, int H, int W, int P, int s, int G, int dtype,
-                                     hipStream_t st, bool wide = false);
+                                     hipStream_t st, bool wide = false, bool channels_last_out = false);
 
 // The per-pixel part of the fused SAPA-D backward in the matrix form of the
 // forward kernel (sapa_d_bwdmat.hip): attention weights and gradient of the
@@ -117,6 +119,8 @@ hipError_t deform_fused_nchw_ws_launch(const void *q, const void *key, const voi
 // of the same B and HW in one launch (C1 = 0: one); esize 2 or 4 bytes
 hipError_t nchw_to_nhwc_launch(const void *src0, void *dst0, int C0, const void *src1, void *dst1,
                                int C1, int B, long HW, int esize, hipStream_t st);
+// channels-last fp32 [B, HW, C] -> contiguous [B, C, HW] of dtype f32 / f16 / bf16 (0 / 2 / 3)
+hipError_t nhwc_f32_to_nchw_launch(const float *src, void *dst, int C, int B, long HW, int dtype, hipStream_t st);
 
 // sapa_d_wmat16.hip: the same operator for f16 / bf16 on the 16-bit matrix
 // instructions; channels per group multiples of 8, key / value channels-last and

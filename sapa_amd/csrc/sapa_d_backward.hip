@@ -56,19 +56,36 @@ static unsigned blocks_for(long n) {
 
 static long align256(long x) { return (x + 255) / 256 * 256; }
 
-// grad_low += scatter(hi, sc): the matrix-product form where it applies, else the
-// LDS-window scatter
-static hipError_t scatter_low(const void *hi, const void *sc, const void *offset, void *grad_low, int B,
-                              int Cx, int H, int W, int P, int s, int G, int dtype, hipStream_t st,
-                              bool wide) {
+// One low-res gradient (grad_key from q and the gradient of the logits, grad_value
+// from grad_out and the attention weights), a sum of many terms: accumulated in
+// fp32 in `acc` and rounded once.  The matrix-product scatter, where it applies,
+// accumulates in channels-last order (a cell's channels in one piece: its final
+// atomics then fall on two cache lines per instruction instead of one per window
+// row and channel) and a transposing pass writes the tensor; else the LDS-window
+// scatter accumulates in the tensor's own order.
+static hipError_t low_gradient(const void *hi, const void *sc, const void *offset, float *acc, void *grad_low,
+                               int B, int Cx, int H, int W, int P, int s, int G, int dtype, hipStream_t st) {
+    const bool wide = dtype != 0;
+    const long n = (long)B * Cx * H * W;
 #ifdef SAPA_SCATTER_MAT_OFF
-    hipError_t e = hipErrorNotSupported;
+    const bool mat = false;
 #else
-    hipError_t e = deform_scatter_mat_launch(hi, sc, offset, grad_low, B, Cx, H, W, P, s, G, dtype, st, wide);
+    const bool mat = deform_scatter_mat_serves(B, Cx, H, W, P, s, G, dtype);
 #endif
-    if (e == hipErrorNotSupported)
-        e = deform_lowgrad_lds_launch(hi, sc, offset, grad_low, B, Cx, H, W, P, s, G, dtype, st, wide);
-    return e;
+    float *const target = (mat || wide) ? acc : (float *)grad_low;
+    hipLaunchKernelGGL(zero_kernel, dim3(blocks_for(n)), dim3(256), 0, st, target, n);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    if (mat) {
+        e = deform_scatter_mat_launch(hi, sc, offset, acc, B, Cx, H, W, P, s, G, dtype, st, wide, true);
+        if (e != hipSuccess) return e;
+        return nhwc_f32_to_nchw_launch(acc, grad_low, Cx, B, (long)H * W, dtype, st);
+    }
+    e = deform_lowgrad_lds_launch(hi, sc, offset, target, B, Cx, H, W, P, s, G, dtype, st, wide);
+    if (e != hipSuccess || !wide) return e;
+    if (dtype == 2) hipLaunchKernelGGL(narrow_kernel<f16_t>, dim3(blocks_for(n)), dim3(256), 0, st, acc, (f16_t *)grad_low, n);
+    else hipLaunchKernelGGL(narrow_kernel<bf16_t>, dim3(blocks_for(n)), dim3(256), 0, st, acc, (bf16_t *)grad_low, n);
+    return hipGetLastError();
 }
 
 // The per-pixel part of the chain (attention weights, gradient of the logits,
@@ -95,8 +112,8 @@ long deform_fused_backward_workspace(int B, int Cq, int C, int H, int W, int P, 
     if (P > 48) return 0;       // [2P][thread] sums of the offset gradient next to the window in LDS
     const long per_point = (long)B * G * P * H * s * W * s * (long)sizeof(float);
     long n = 2 * align256(per_point);
-    // 16-bit tensors: fp32 accumulators of the low-res gradients
-    if (dtype != 0) n += align256((long)B * Cq * H * W * 4) + align256((long)B * C * H * W * 4);
+    // fp32 accumulators of the low-res gradients
+    n += align256((long)B * Cq * H * W * 4) + align256((long)B * C * H * W * 4);
     if (dbwd::matrix_stage(B, Cq, C, H, W, P, s, G, dtype)) {
         // channels-last copies of key and value for the matrix-form kernel
         const long esize = dtype == 0 ? 4 : 2;
@@ -124,9 +141,9 @@ hipError_t deform_fused_backward_launch(const void *grad_out, const void *q, con
     char *w = (char *)workspace;
     float *attn = (float *)w;
     float *gl = (float *)(w + align256(n_pp * 4));
-    float *gk32 = wide ? (float *)(w + 2 * align256(n_pp * 4)) : (float *)grad_key;
-    float *gv32 = wide ? (float *)((char *)gk32 + align256((long)B * Cq * lpix * 4)) : (float *)grad_value;
-    char *rest = wide ? (char *)gv32 + align256((long)B * C * lpix * 4) : w + 2 * align256(n_pp * 4);
+    float *gk32 = (float *)(w + 2 * align256(n_pp * 4));
+    float *gv32 = (float *)((char *)gk32 + align256((long)B * Cq * lpix * 4));
+    char *rest = (char *)gv32 + align256((long)B * C * lpix * 4);
     const bool mat = matrix_stage(B, Cq, C, H, W, P, s, G, dtype);
     float *goff32 = wide && !mat ? (float *)rest : nullptr;
     const int HIRES = 0;
@@ -168,32 +185,8 @@ hipError_t deform_fused_backward_launch(const void *grad_out, const void *q, con
     }
     // the low-res gradients: grad_value (attention weights x grad_out) and
     // grad_key (gradient of the logits x query), scattered
-    if (grad_value) {
-        hipLaunchKernelGGL(zero_kernel, dim3(blocks_for((long)B * C * lpix)), dim3(256), 0, st, gv32,
-                           (long)B * C * lpix);
-        SAPA_STEP(hipGetLastError());
-        SAPA_STEP(scatter_low(grad_out, attn, offset, gv32, B, C, H, W, P, s, G, dtype, st, wide));
-    }
-    if (grad_key) {
-        hipLaunchKernelGGL(zero_kernel, dim3(blocks_for((long)B * Cq * lpix)), dim3(256), 0, st, gk32,
-                           (long)B * Cq * lpix);
-        SAPA_STEP(hipGetLastError());
-        SAPA_STEP(scatter_low(q, gl, offset, gk32, B, Cq, H, W, P, s, G, dtype, st, wide));
-    }
-    if (wide) {
-        if (grad_key) {
-            const long n = (long)B * Cq * lpix;
-            if (dtype == 2) hipLaunchKernelGGL(narrow_kernel<f16_t>, dim3(blocks_for(n)), dim3(256), 0, st, gk32, (f16_t *)grad_key, n);
-            else hipLaunchKernelGGL(narrow_kernel<bf16_t>, dim3(blocks_for(n)), dim3(256), 0, st, gk32, (bf16_t *)grad_key, n);
-            SAPA_STEP(hipGetLastError());
-        }
-        if (grad_value) {
-            const long n = (long)B * C * lpix;
-            if (dtype == 2) hipLaunchKernelGGL(narrow_kernel<f16_t>, dim3(blocks_for(n)), dim3(256), 0, st, gv32, (f16_t *)grad_value, n);
-            else hipLaunchKernelGGL(narrow_kernel<bf16_t>, dim3(blocks_for(n)), dim3(256), 0, st, gv32, (bf16_t *)grad_value, n);
-            SAPA_STEP(hipGetLastError());
-        }
-    }
+    if (grad_value) SAPA_STEP(low_gradient(grad_out, attn, offset, gv32, grad_value, B, C, H, W, P, s, G, dtype, st));
+    if (grad_key) SAPA_STEP(low_gradient(q, gl, offset, gk32, grad_key, B, Cq, H, W, P, s, G, dtype, st));
 #undef SAPA_STEP
     return hipSuccess;
 }

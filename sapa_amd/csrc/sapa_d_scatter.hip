@@ -37,18 +37,59 @@ namespace sapa {
 
 namespace dscat {
 
+#ifndef SAPA_SCAT_PROBE
+#define SAPA_SCAT_PROBE 0
+#endif
+
 typedef unsigned u32;
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int RCH = 4;          // window reach around the region's parents, in low-res cells
-constexpr int NT = 256;
+
+// Tensor elements through a buffer descriptor, widened to float: an offset with
+// bit 31 set lies beyond every descriptor and returns 0 without touching memory,
+// so a load needs no branch around it (and the compiler can count the loads in
+// flight: with loads in branches it waits for all of them at every use).
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+constexpr unsigned OOB = 0x80000000u;
+template <typename T> struct Ld;
+template <> struct Ld<float> {
+    static __device__ __forceinline__ float one(__amdgpu_buffer_rsrc_t r, unsigned off) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, off, 0, 0));
+    }
+    static __device__ __forceinline__ void four(__amdgpu_buffer_rsrc_t r, unsigned off, float (&v)[4]) {
+        union { u32x4 u; float f[4]; } x;
+        x.u = __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = x.f[e];
+    }
+};
+template <typename H> struct Ld16 {
+    static __device__ __forceinline__ float one(__amdgpu_buffer_rsrc_t r, unsigned off) {
+        return (float)__builtin_bit_cast(H, (unsigned short)__builtin_amdgcn_raw_buffer_load_b16(r, off, 0, 0));
+    }
+    static __device__ __forceinline__ void four(__amdgpu_buffer_rsrc_t r, unsigned off, float (&v)[4]) {
+        union { u32x2 u; H h[4]; } x;
+        x.u = __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = (float)x.h[e];
+    }
+};
+template <> struct Ld<f16_t> : Ld16<f16_t> {};
+template <> struct Ld<bf16_t> : Ld16<bf16_t> {};
+constexpr int NT = 512;         // 4 waves that accumulate the products + 4 waves that build their operands
+constexpr int NTP = 256;        // threads of either kind
 constexpr int CHK = 64;         // channels per workgroup
 constexpr int SPX = 16;         // pixels per step
 constexpr int GS = CHK + 16;    // floats per pixel of the staged hi tile: 16 mod 64, so that the
                                 // 4 pixels a matrix operand read touches fall on disjoint banks
 
-template <typename T, typename TS, int S, int RG>
-__global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2)))
+// CLO: grad_low is a channels-last fp32 buffer [B, H, W, Cx] (a cell's channels in
+// one piece: the final atomics of a wave then fall on two cache lines instead of
+// one per window row and channel); else the contiguous [B, Cx, H, W] tensor.
+template <typename T, typename TS, int S, int RG, bool CLO>
+__global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4)))
 deform_scatter_mat_kernel(const T *__restrict__ hi, const TS *__restrict__ sc,
                           const T *__restrict__ offset, float *__restrict__ grad_low, int Cx, int H,
                           int W, int P, int G, int regions_x, int regions_y, int nchunks, int nblocks,
@@ -61,13 +102,15 @@ deform_scatter_mat_kernel(const T *__restrict__ hi, const TS *__restrict__ sc,
     constexpr int NSTEP = RG * RG / SPX;
     static_assert(RG % S == 0 && (RG * RG) % SPX == 0 && SPX % RG == 0 || RG % SPX == 0, "whole steps");
     static_assert(WSR % 64 == 48, "bank layout of the weight rows");
+    static_assert(NSTEP % 2 == 0, "the steps take the two buffers in turn");
 
     constexpr int TS_ = 65;         // floats per channel row of the epilogue's transposition buffer
-    constexpr int WLN = SPX * WSR > CHK * TS_ ? SPX * WSR : CHK * TS_;
-    __shared__ __attribute__((aligned(16))) int Wl[WLN];            // Wm rows of the step, scaled integers
-    __shared__ __attribute__((aligned(16))) float Gl[SPX * GS];     // hi of the step's pixels [pixel][channel]
-    __shared__ float invl[SPX];                                     // 1 / scale of each row
-    __shared__ u32 badmask;                                         // pixels of the step that go the direct way
+    static_assert(2 * SPX * WSR >= CHK * TS_, "the transposition buffer fits the weight rows' buffers");
+    // two sets of buffers: the producer waves fill one for step s while the consumer
+    // waves multiply the other (step s - 1)
+    __shared__ __attribute__((aligned(16))) int Wl2[2 * SPX * WSR];     // Wm rows of a step, scaled integers
+    __shared__ __attribute__((aligned(16))) float Gl2[2 * SPX * GS];    // hi of a step's pixels [pixel][channel]
+    __shared__ float invl2[2 * SPX];                                    // 1 / scale of each row
 
     const int logical = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
     if (logical >= nblocks) return;
@@ -78,7 +121,8 @@ deform_scatter_mat_kernel(const T *__restrict__ hi, const TS *__restrict__ sc,
     rest /= nchunks;
     const int g = rest % G, n = rest / G;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const bool producer = threadIdx.x >= NTP;
+    const int tid = threadIdx.x & (NTP - 1), lane = tid & 63, wave = tid >> 6;   // within the 4 waves of a kind
     const int mi = lane & 15, mk = lane >> 4;
     const int hH = H * S, hW = W * S, cg = Cx / G;
     const long lpix = (long)H * W, hpl = (long)hH * hW;
@@ -95,89 +139,91 @@ deform_scatter_mat_kernel(const T *__restrict__ hi, const TS *__restrict__ sc,
         qh = y0 + lin / RG;
         qw = x0 + lin % RG;
     };
+    // The step's pixels belong to one or two rows of parents, and a sample within
+    // RCH cells of its parent lands on the window rows b0 .. b1 (the band), i.e. on
+    // the cell blocks cb0 .. cb1: only those take part in the step's product.  A
+    // sample that lands elsewhere in the window goes the direct way.
+    auto band = [&](int step, int &b0, int &b1, int &cb0, int &cb1) __attribute__((always_inline)) {
+        b0 = (step * SPX / RG) / S;
+        b1 = ((step * SPX + SPX - 1) / RG) / S + 2 * RCH + 1;
+        cb0 = b0 * WWR / 16;
+        cb1 = ((b1 + 1) * WWR - 1) / 16;
+    };
 
-    // ---- hi tile of a step: thread t brings channel t % 64, pixels 4 (t / 64) .. + 3
-    const int gch = tid & 63, gq = tid >> 6;
+    // ===== producer waves: wave w owns pixels 4 w .. 4 w + 3 of every step -- their hi
+    // values (lane = channel), their rows of Wm (zeroed, then filled by the wave's
+    // own lanes: LDS operations of one wave execute in order, so no barrier sits
+    // between the two) and their scales
     const bool vec4 = hW % 4 == 0 && (uintptr_t)hi % (4 * sizeof(T)) == 0;
-    float greg[4];
-    auto load_hi = [&](int step) __attribute__((always_inline)) {
+    // the chunk's planes of hi, the group's scalars and offsets (byte offsets below 2^31: the launcher checks)
+    const __amdgpu_buffer_rsrc_t hrsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(hi + ch0 * hpl), 0, (int)(cvalid * hpl * (long)sizeof(T)), 0x00020000);
+    const __amdgpu_buffer_rsrc_t srsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(sc + k0 * hpl), 0, (int)(P * hpl * (long)sizeof(TS)), 0x00020000);
+    const __amdgpu_buffer_rsrc_t orsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(offset + (k0 << 1) * hpl), 0, (int)(2 * P * hpl * (long)sizeof(T)), 0x00020000);
+    // what a step needs from global memory, fetched two steps ahead (two sets in turn)
+    struct Pre { float greg[4], scr[2], oxr[2], oyr[2]; };
+    auto load_hi = [&](int step, Pre &pre) __attribute__((always_inline)) {
         int qh, qw;
-        step_pixel(step, 4 * gq, qh, qw);
+        step_pixel(step, 4 * wave, qh, qw);
+        const bool row_ok = lane < cvalid && qh < hH;
+        const unsigned off = (unsigned)(((long)lane * hpl + (long)qh * hW + qw) * (long)sizeof(T));
+        if (vec4) {     // (uniform) whole aligned vectors: inside the image or outside as a whole
+            Ld<T>::four(hrsrc, row_ok && qw < hW ? off : OOB, pre.greg);
+        } else {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) greg[e] = 0.f;
-        if (gch < cvalid && qh < hH) {
-            const T *hp = hi + (ch0 + gch) * hpl + (long)qh * hW + qw;
-            if (vec4 && qw + 3 < hW) {
-                struct alignas(4 * sizeof(T)) V4 { T v[4]; };
-                const V4 x = *(const V4 *)hp;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) greg[e] = (float)x.v[e];
-            } else {
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (qw + e < hW) greg[e] = (float)hp[e];
-            }
+            for (int e = 0; e < 4; ++e)
+                pre.greg[e] = Ld<T>::one(hrsrc, row_ok && qw + e < hW ? off + e * (unsigned)sizeof(T) : OOB);
         }
     };
-    // into LDS; a value that is not finite is replaced by 0 there and its pixel marked
-    auto store_hi = [&]() __attribute__((always_inline)) {
+    // per-sample view: P <= 16 -> 16 lanes per pixel, one pass over the wave's 4
+    // pixels; else 32 lanes per pixel, two passes
+    const bool narrow = P <= 16;
+    const int pt = narrow ? (lane & 15) : (lane & 31);
+    const int npass = narrow ? 1 : 2;
+    // this lane's pixel of the step in pass ps
+    auto sample_pixel = [&](int ps) __attribute__((always_inline)) {
+        return 4 * wave + (narrow ? lane >> 4 : 2 * ps + (lane >> 5));
+    };
+    auto load_samples = [&](int step, Pre &pre) __attribute__((always_inline)) {
+#pragma unroll
+        for (int ps = 0; ps < 2; ++ps) {
+            int qh, qw;
+            step_pixel(step, sample_pixel(ps), qh, qw);
+            const bool ok = ps < npass && pt < P && qh < hH && qw < hW;
+            const long pp = (long)pt * hpl + (long)qh * hW + qw;        // the point's plane of sc
+            const long po = pp + (long)pt * hpl;                        // its dx plane of the offsets
+            pre.scr[ps] = Ld<TS>::one(srsrc, ok ? (unsigned)(pp * (long)sizeof(TS)) : OOB);
+            pre.oxr[ps] = Ld<T>::one(orsrc, ok ? (unsigned)(po * (long)sizeof(T)) : OOB);
+            pre.oyr[ps] = Ld<T>::one(orsrc, ok ? (unsigned)((po + hpl) * (long)sizeof(T)) : OOB);
+        }
+    };
+    auto produce = [&](int step, Pre &pre) __attribute__((always_inline)) {
+        const float (&scr)[2] = pre.scr, (&oxr)[2] = pre.oxr, (&oyr)[2] = pre.oyr;
+        int *const Wl = Wl2 + (step & 1) * SPX * WSR;
+        float *const Gl = Gl2 + (step & 1) * SPX * GS;
+        float *const invl = invl2 + (step & 1) * SPX;
+        int b0, b1, cb0, cb1;
+        band(step, b0, b1, cb0, cb1);
+        // ---- empty weight rows; the hi values, a value that is not finite replaced
+        // by 0 and its pixel marked (bit e of bad: pixel 4 w + e)
+        {
+            int __attribute__((ext_vector_type(4))) *rows = (int __attribute__((ext_vector_type(4))) *)(Wl + 4 * wave * WSR);
+            for (int i = lane; i < 4 * WSR / 4; i += 64) rows[i] = {0, 0, 0, 0};
+        }
         u32 bad = 0;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const bool fin = __builtin_fabsf(greg[e]) < __builtin_huge_valf();
-            bad |= fin ? 0u : 1u << (4 * gq + e);
-            Gl[(4 * gq + e) * GS + gch] = fin ? greg[e] : 0.f;
+            const bool fin = __builtin_fabsf(pre.greg[e]) < __builtin_huge_valf();
+            bad |= __builtin_amdgcn_ballot_w64(!fin) != 0 ? 1u << e : 0u;
+            Gl[(4 * wave + e) * GS + lane] = fin ? pre.greg[e] : 0.f;
         }
-        if (bad) atomicOr(&badmask, bad);
-    };
-
-    // ---- per-sample view: P <= 16 -> 16 lanes per pixel, one pass per step; else 32, two
-    const bool narrow = P <= 16;
-    const int pt = narrow ? (tid & 15) : (tid & 31);
-    const int prow = narrow ? (tid >> 4) : (tid >> 5);
-    const int npass = narrow ? 1 : 2, ppp = narrow ? 16 : 8;
-    // the scalar and the offsets of this lane's point, per pass, fetched a step ahead
-    float scr[2], oxr[2], oyr[2];
-    auto load_samples = [&](int step) __attribute__((always_inline)) {
-#pragma unroll
-        for (int ps = 0; ps < 2; ++ps) {
-            scr[ps] = oxr[ps] = oyr[ps] = 0.f;
-            if (ps < npass && pt < P) {
-                int qh, qw;
-                step_pixel(step, ps * ppp + prow, qh, qw);
-                if (qh < hH && qw < hW) {
-                    const long pp = (long)qh * hW + qw;
-                    scr[ps] = (float)sc[(k0 + pt) * hpl + pp];
-                    const T *op = offset + ((k0 + pt) << 1) * hpl + pp;
-                    oxr[ps] = (float)op[0];
-                    oyr[ps] = (float)op[hpl];
-                }
-            }
-        }
-    };
-
-    f32x4 D[CBI][CHK / 16];
-#pragma unroll
-    for (int cbi = 0; cbi < CBI; ++cbi)
-#pragma unroll
-        for (int nb = 0; nb < CHK / 16; ++nb) D[cbi][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-    if (tid == 0) badmask = 0;
-    load_hi(0);
-    load_samples(0);
-    __syncthreads();
-
-    for (int step = 0; step < NSTEP; ++step) {
-        // ---- (a) empty weight rows, the step's hi tile
-        for (int i = tid; i < SPX * WSR / 4; i += NT) ((int __attribute__((ext_vector_type(4))) *)Wl)[i] = {0, 0, 0, 0};
-        store_hi();
-        __syncthreads();
-
-        // ---- (b) per (pixel, point): the corners' shares of sc into the pixel's row
-        const u32 bad = badmask;
+        // ---- per (pixel, point): the corners' shares of sc into the pixel's row
         auto sample = [&](auto nl, int ps) __attribute__((always_inline)) {
             constexpr int NL = decltype(nl)::value;
-            const int t = ps * (NT / NL) + tid / NL;
+            const int t = sample_pixel(ps);
+            const bool isbad = bad >> (t & 3) & 1;
             int qh, qw;
             step_pixel(step, t, qh, qw);
             const bool live = qh < hH && qw < hW && pt < P;
@@ -189,11 +235,11 @@ deform_scatter_mat_kernel(const T *__restrict__ hi, const TS *__restrict__ sc,
             (void)__builtin_frexpf(l1, &ex);
             const float scale = __builtin_ldexpf(1.f, 30 - ex);
             if (pt == 0) invl[t] = (finite && l1 > 0.f) ? __builtin_ldexpf(1.f, ex - 30) : 0.f;
-            if (!live || (scv == 0.f && !(bad >> t & 1))) return;
+            if (!live || (scv == 0.f && !isbad)) return;
             const float kw = (float)(qw / S) + oxr[ps], kh = (float)(qh / S) + oyr[ps];
             const WinTap<float> wt = win_tap<float>(kh, kw, H, W, wy0, wx0, WWR, WWR);
             if (!wt.guard) return;
-            if (wt.inwin && finite && !(bad >> t & 1)) {
+            if (wt.inwin && wt.hl >= b0 && wt.hl < b1 && finite && !isbad) {
                 int *wp = Wl + t * WSR + wt.hl * WWR + wt.wl;
                 const float sv = scv * scale;
                 __hip_atomic_fetch_add(wp, (int)__builtin_rintf(sv * wt.w1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -201,84 +247,156 @@ deform_scatter_mat_kernel(const T *__restrict__ hi, const TS *__restrict__ sc,
                 __hip_atomic_fetch_add(wp + WWR, (int)__builtin_rintf(sv * wt.w3), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                 __hip_atomic_fetch_add(wp + WWR + 1, (int)__builtin_rintf(sv * wt.w4), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             } else {
-                // the reference's own way: one float atomic per term (rare)
+                // the reference's own way: one float atomic per term (rare).  (The
+                // position is made opaque: its taps are set up in this branch only.)
+                float fkh = kh, fkw = kw;
+                asm volatile("" : "+v"(fkh), "+v"(fkw));
                 Tap<float> tp = {};
-                tap_setup(kh, kw, H, W, tp);
+                tap_setup(fkh, fkw, H, W, tp);
                 const T *hp = hi + ch0 * hpl + (long)qh * hW + qw;
+                // element (cell i, channel c of the chunk) of grad_low
+                const long cstep = CLO ? Cx : 1, chstep = CLO ? 1 : lpix;
+                float *const g0 = grad_low + (CLO ? (long)n * lpix * Cx + (long)g * cg + c0 : ch0 * lpix);
                 for (int c = 0; c < cvalid; ++c) {
-                    float *gp = grad_low + (ch0 + c) * lpix;
+                    float *gp = g0 + c * chstep;
                     const float tv = (float)hp[c * hpl] * scv;
-                    if (tp.m1) unsafeAtomicAdd(gp + tp.i1, tp.w1 * tv);
-                    if (tp.m2) unsafeAtomicAdd(gp + tp.i2, tp.w2 * tv);
-                    if (tp.m3) unsafeAtomicAdd(gp + tp.i3, tp.w3 * tv);
-                    if (tp.m4) unsafeAtomicAdd(gp + tp.i4, tp.w4 * tv);
+                    if (tp.m1) unsafeAtomicAdd(gp + tp.i1 * cstep, tp.w1 * tv);
+                    if (tp.m2) unsafeAtomicAdd(gp + tp.i2 * cstep, tp.w2 * tv);
+                    if (tp.m3) unsafeAtomicAdd(gp + tp.i3 * cstep, tp.w3 * tv);
+                    if (tp.m4) unsafeAtomicAdd(gp + tp.i4 * cstep, tp.w4 * tv);
                 }
             }
         };
-        if (narrow) {
+        if (SAPA_SCAT_PROBE & 2) {
+        } else if (narrow) {
             sample(std::integral_constant<int, 16>{}, 0);
         } else {
             sample(std::integral_constant<int, 32>{}, 0);
             sample(std::integral_constant<int, 32>{}, 1);
         }
-        __syncthreads();
-
-        // ---- (c) D[cell][channel] += Wm^T . hi over the step's 16 pixels; the next
-        // step's loads travel meanwhile
-        if (tid == 0) badmask = 0;
-        if (step + 1 < NSTEP) {
-            load_hi(step + 1);
-            load_samples(step + 1);
+        // the loads of the step after the next go out (into the set this step has used up)
+        if (step + 2 < NSTEP && !(SAPA_SCAT_PROBE & 8)) {
+            load_hi(step + 2, pre);
+            load_samples(step + 2, pre);
         }
-#pragma unroll
-        for (int ks = 0; ks < SPX / 4; ++ks) {
-            const float inv = invl[4 * ks + mk];
-            float b[CHK / 16];
-#pragma unroll
-            for (int nb = 0; nb < CHK / 16; ++nb) b[nb] = Gl[(4 * ks + mk) * GS + 16 * nb + mi];
-#pragma unroll
-            for (int cbi = 0; cbi < CBI; ++cbi) {
-                const int cb = wave + 4 * cbi;
-                if (cb < NCB) {
-                    const float a = (float)Wl[(4 * ks + mk) * WSR + 16 * cb + mi] * inv;
-#pragma unroll
-                    for (int nb = 0; nb < CHK / 16; ++nb)
-                        if (16 * nb < cvalid)       // (uniform) a short chunk skips its empty channel blocks
-                            D[cbi][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b[nb], D[cbi][nb], 0, 0, 0);
-                }
-            }
-        }
-        __syncthreads();
-    }
+    };
 
     // ---- the region's sums into grad_low.  D[cbi][nb][r] = cell 16 cb + 4 mk + r,
     // channel 16 nb + mi: as it stands a wave's 64 lanes would hit 64 channel planes,
-    // one atomic per cache line.  Through LDS ([channel][64 cells], the 4 waves'
-    // blocks of a round side by side) the lanes of an instruction run along the
-    // cells of one channel instead -- runs of up to WWR consecutive floats.
-    float *const Tl = (float *)Wl;
-#pragma unroll
-    for (int cbi = 0; cbi < CBI; ++cbi) {
+    // one atomic per cache line.  The 64 cells x 64 channels of a round (the 4
+    // consumer waves' blocks side by side) go through LDS, after which all 8 waves
+    // issue the atomics with their lanes along what is contiguous in grad_low:
+    // the cells of one channel (contiguous layout: runs of up to WWR floats), or the
+    // channels of one cell (channels-last buffer: 256 bytes).
+    float *const Tl = (float *)Wl2;
+    constexpr int TSC = 68;         // floats per cell row of the channels-last form: 4 x 68 = 16 mod 64
+    static_assert(2 * SPX * WSR >= 64 * TSC, "the transposition buffer fits the weight rows' buffers");
+    auto stash = [&](int cbi, const f32x4 (&Dc)[CHK / 16]) __attribute__((always_inline)) {
 #pragma unroll
         for (int nb = 0; nb < CHK / 16; ++nb)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) Tl[(16 * nb + mi) * TS_ + 16 * wave + 4 * mk + r] = D[cbi][nb][r];
-        __syncthreads();
-        // lane <-> cell 64 cbi + lane; this wave: channels 16 wave .. + 15
-        const int cell = 64 * cbi + lane;
-        const int gy = wy0 + cell / WWR, gx = wx0 + cell % WWR;
-        const bool ok = cell < NPOS && gy >= 0 && gy < H && gx >= 0 && gx < W;
-        float *gp = grad_low + (ch0 + 16 * wave) * lpix + (long)gy * W + gx;
+            for (int r = 0; r < 4; ++r) {
+                if (CLO) Tl[(16 * wave + 4 * mk + r) * TSC + 16 * nb + mi] = Dc[nb][r];
+                else Tl[(16 * nb + mi) * TS_ + 16 * wave + 4 * mk + r] = Dc[nb][r];
+            }
+    };
+    auto flush = [&](int cbi) __attribute__((always_inline)) {
+        const int w8 = (int)(threadIdx.x >> 6);
+        if (CLO) {
+            // this wave: cells 8 w8 .. + 7 of the round; lane <-> channel
+            float *const g0 = grad_low + (long)n * lpix * Cx + (long)g * cg + c0 + lane;
 #pragma unroll 4
-        for (int c = 0; c < 16; ++c) {
-            const float v = Tl[(16 * wave + c) * TS_ + lane];
-            if (ok && 16 * wave + c < cvalid && v != 0.f) unsafeAtomicAdd(gp + c * lpix, v);
+            for (int c = 0; c < 8; ++c) {
+                const int cell = 64 * cbi + 8 * w8 + c;
+                const int gy = wy0 + cell / WWR, gx = wx0 + cell % WWR;
+                const bool ok = cell < NPOS && gy >= 0 && gy < H && gx >= 0 && gx < W;
+                const float v = Tl[(8 * w8 + c) * TSC + lane];
+                if (ok && lane < cvalid && v != 0.f) unsafeAtomicAdd(g0 + ((long)gy * W + gx) * Cx, v);
+            }
+        } else {
+            // lane <-> cell 64 cbi + lane; this wave: channels 8 w8 .. + 7
+            const int cell = 64 * cbi + lane;
+            const int gy = wy0 + cell / WWR, gx = wx0 + cell % WWR;
+            const bool ok = cell < NPOS && gy >= 0 && gy < H && gx >= 0 && gx < W;
+            float *gp = grad_low + (ch0 + 8 * w8) * lpix + (long)gy * W + gx;
+#pragma unroll 4
+            for (int c = 0; c < 8; ++c) {
+                const float v = Tl[(8 * w8 + c) * TS_ + lane];
+                if (ok && 8 * w8 + c < cvalid && v != 0.f && !(SAPA_SCAT_PROBE & 4)) unsafeAtomicAdd(gp + c * lpix, v);
+            }
         }
-        __syncthreads();
+    };
+
+    // The two kinds of waves run their own code from here on and meet at the
+    // barriers (the same number on both paths): in iteration i step i is produced
+    // while step i - 1 is consumed.  (One loop with both roles in it would keep the
+    // consumers' accumulators alive in the producers' registers.)
+    if (producer) {
+        Pre pre0, pre1;
+        load_hi(0, pre0);
+        load_samples(0, pre0);
+        load_hi(1, pre1);
+        load_samples(1, pre1);
+        for (int i = 0; i <= NSTEP; i += 2) {
+            if (i < NSTEP) produce(i, pre0);
+            __syncthreads();
+            if (i + 1 < NSTEP) produce(i + 1, pre1);
+            __syncthreads();
+        }
+        for (int cbi = 0; cbi < CBI; ++cbi) {
+            __syncthreads();
+            flush(cbi);
+            __syncthreads();
+        }
+    } else {
+        // ===== consumer waves: D[cell][channel] += Wm^T . hi over a step's 16 pixels
+        f32x4 D[CBI][CHK / 16];
+#pragma unroll
+        for (int cbi = 0; cbi < CBI; ++cbi)
+#pragma unroll
+            for (int nb = 0; nb < CHK / 16; ++nb) D[cbi][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+        auto consume = [&](int step) __attribute__((always_inline)) {
+            const int *const Wl = Wl2 + (step & 1) * SPX * WSR;
+            const float *const Gl = Gl2 + (step & 1) * SPX * GS;
+            const float *const invl = invl2 + (step & 1) * SPX;
+            int b0, b1, cb0, cb1;
+            band(step, b0, b1, cb0, cb1);
+#pragma unroll
+            for (int ks = 0; ks < ((SAPA_SCAT_PROBE & 1) ? 0 : SPX / 4); ++ks) {
+                const float inv = invl[4 * ks + mk];
+                float b[CHK / 16];
+#pragma unroll
+                for (int nb = 0; nb < CHK / 16; ++nb) b[nb] = Gl[(4 * ks + mk) * GS + 16 * nb + mi];
+#pragma unroll
+                for (int cbi = 0; cbi < CBI; ++cbi) {
+                    const int cb = wave + 4 * cbi;
+                    if (cb >= cb0 && cb <= cb1) {
+                        const float a = (float)Wl[(4 * ks + mk) * WSR + 16 * cb + mi] * inv;
+#pragma unroll
+                        for (int nb = 0; nb < CHK / 16; ++nb)
+                            if (16 * nb < cvalid)       // (uniform) a short chunk skips its empty channel blocks
+                                D[cbi][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b[nb], D[cbi][nb], 0, 0, 0);
+                    }
+                }
+            }
+        };
+        for (int i = 0; i <= NSTEP; i += 2) {
+            if (i > 0) consume(i - 1);
+            __syncthreads();
+            if (i < NSTEP) consume(i);
+            __syncthreads();
+        }
+#pragma unroll
+        for (int cbi = 0; cbi < CBI; ++cbi) {
+            stash(cbi, D[cbi]);
+            __syncthreads();
+            flush(cbi);
+            __syncthreads();
+        }
     }
 }
 
-template <typename T, typename TS, int S, int RG>
+template <typename T, typename TS, int S, int RG, bool CLO>
 static hipError_t launch_geom(const void *hi, const void *sc, const void *offset, void *grad_low, int B,
                               int Cx, int H, int W, int P, int G, hipStream_t st) {
     const int regions_x = (W * S + RG - 1) / RG, regions_y = (H * S + RG - 1) / RG;
@@ -286,7 +404,7 @@ static hipError_t launch_geom(const void *hi, const void *sc, const void *offset
     const long nb = (long)regions_x * regions_y * nchunks * G * B;
     if (nb > (1L << 30)) return hipErrorNotSupported;
     const int per_xcd = (int)((nb + 7) / 8);
-    hipLaunchKernelGGL((deform_scatter_mat_kernel<T, TS, S, RG>), dim3(per_xcd * 8), dim3(NT), 0, st,
+    hipLaunchKernelGGL((deform_scatter_mat_kernel<T, TS, S, RG, CLO>), dim3(per_xcd * 8), dim3(NT), 0, st,
                        (const T *)hi, (const TS *)sc, (const T *)offset, (float *)grad_low, Cx, H, W, P, G,
                        regions_x, regions_y, nchunks, (int)nb, per_xcd);
     return hipGetLastError();
@@ -294,33 +412,50 @@ static hipError_t launch_geom(const void *hi, const void *sc, const void *offset
 
 template <typename T, typename TS>
 static hipError_t launch_t(const void *hi, const void *sc, const void *offset, void *grad_low, int B, int Cx,
-                           int H, int W, int P, int s, int G, hipStream_t st) {
+                           int H, int W, int P, int s, int G, hipStream_t st, bool clo) {
+#define SAPA_SCAT(SV, RGV)                                                                                     \
+    case SV:                                                                                                   \
+        return clo ? launch_geom<T, TS, SV, RGV, true>(hi, sc, offset, grad_low, B, Cx, H, W, P, G, st)        \
+                   : launch_geom<T, TS, SV, RGV, false>(hi, sc, offset, grad_low, B, Cx, H, W, P, G, st);
     switch (s) {
-        case 1: return launch_geom<T, TS, 1, 8>(hi, sc, offset, grad_low, B, Cx, H, W, P, G, st);
-        case 2: return launch_geom<T, TS, 2, 16>(hi, sc, offset, grad_low, B, Cx, H, W, P, G, st);
-        case 4: return launch_geom<T, TS, 4, 16>(hi, sc, offset, grad_low, B, Cx, H, W, P, G, st);
+        SAPA_SCAT(1, 8)
+        SAPA_SCAT(2, 16)
+        SAPA_SCAT(4, 16)
         default: return hipErrorNotSupported;
     }
+#undef SAPA_SCAT
 }
 
 }  // namespace dscat
 
-// fp32 tensors, or (wide) f16 / bf16 features and offsets with fp32 per-point
-// scalars; s in {1, 2, 4}, P <= 32; grad_low is fp32 and is accumulated into.
-// hipErrorNotSupported otherwise.
-hipError_t deform_scatter_mat_launch(const void *hi, const void *sc, const void *offset, void *grad_low,
-                                     int B, int Cx, int H, int W, int P, int s, int G, int dtype,
-                                     hipStream_t st, bool wide) {
-    if (P > 32 || (long)H * s * W * s >= (1L << 31)) return hipErrorNotSupported;
+// Whether deform_scatter_mat_launch serves the configuration (dtype as the C ABI
+// numbers them; 16-bit features go with fp32 scalars).
+bool deform_scatter_mat_serves(int B, int Cx, int H, int W, int P, int s, int G, int dtype) {
+    if (dtype != 0 && dtype != 2 && dtype != 3) return false;
+    if (s != 1 && s != 2 && s != 4) return false;
+    if (P < 1 || P > 32 || G <= 0 || Cx % G != 0 || (long)H * s * W * s >= (1L << 31)) return false;
+    // byte offsets within a group's planes of the scalars, the offsets and a chunk of hi stay below 2^31
+    if (2L * P * H * s * W * s * 4 >= (1L << 31) || 64L * H * s * W * s * 4 >= (1L << 31)) return false;
     // The two products over the region's whole window are a fixed cost; the LDS-window
     // scatter's cost grows with points x channels.  Measured at B=8, G=4, 64 channels per
     // group, 64x64 -> 128x128 (us, this kernel / that one): P = 2 342 / 227, P = 5 349 / 452,
     // P = 9 352 / 770, P = 25 400 / 2052.
     const int cg = Cx / G;
-    if ((long)P * (cg < 64 ? cg : 64) < 256) return hipErrorNotSupported;
-    if (dtype == 0) return dscat::launch_t<float, float>(hi, sc, offset, grad_low, B, Cx, H, W, P, s, G, st);
-    if (wide && dtype == 2) return dscat::launch_t<f16_t, float>(hi, sc, offset, grad_low, B, Cx, H, W, P, s, G, st);
-    if (wide && dtype == 3) return dscat::launch_t<bf16_t, float>(hi, sc, offset, grad_low, B, Cx, H, W, P, s, G, st);
+    return (long)P * (cg < 64 ? cg : 64) >= 256;
+}
+
+// fp32 tensors, or (wide) f16 / bf16 features and offsets with fp32 per-point
+// scalars; s in {1, 2, 4}, P <= 32; grad_low is fp32 and is accumulated into: the
+// contiguous [B, Cx, H, W] tensor, or (channels_last_out) a [B, H, W, Cx] buffer.
+// hipErrorNotSupported otherwise.
+hipError_t deform_scatter_mat_launch(const void *hi, const void *sc, const void *offset, void *grad_low,
+                                     int B, int Cx, int H, int W, int P, int s, int G, int dtype,
+                                     hipStream_t st, bool wide, bool channels_last_out) {
+    if (!deform_scatter_mat_serves(B, Cx, H, W, P, s, G, dtype)) return hipErrorNotSupported;
+    const bool clo = channels_last_out;
+    if (dtype == 0) return dscat::launch_t<float, float>(hi, sc, offset, grad_low, B, Cx, H, W, P, s, G, st, clo);
+    if (wide && dtype == 2) return dscat::launch_t<f16_t, float>(hi, sc, offset, grad_low, B, Cx, H, W, P, s, G, st, clo);
+    if (wide && dtype == 3) return dscat::launch_t<bf16_t, float>(hi, sc, offset, grad_low, B, Cx, H, W, P, s, G, st, clo);
     return hipErrorNotSupported;
 }
 

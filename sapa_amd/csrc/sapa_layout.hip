@@ -35,6 +35,23 @@ nchw_to_nhwc_kernel(const U *__restrict__ src0, U *__restrict__ dst0, int C0, in
         if (c0 + tx < C && p0 + p < HW) dst[(n * HW + p0 + p) * C + c0 + tx] = tile[tx][p];
 }
 
+// The way back for an fp32 accumulation buffer: channels-last [B, HW, C] floats
+// into a contiguous [B, C, HW] tensor of type T (rounded once).
+template <typename T>
+__global__ void __launch_bounds__(256)
+nhwc_f32_to_nchw_kernel(const float *__restrict__ src, T *__restrict__ dst, int C, long HW) {
+    __shared__ float tile[64][65];
+    const long p0 = (long)blockIdx.x * 64;
+    const int c0 = (int)blockIdx.y * 64;
+    const long n = blockIdx.z;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int p = ty; p < 64; p += 4)
+        tile[p][tx] = (c0 + tx < C && p0 + p < HW) ? src[(n * HW + p0 + p) * C + c0 + tx] : 0.f;
+    __syncthreads();
+    for (int c = ty; c < 64; c += 4)
+        if (c0 + c < C && p0 + tx < HW) dst[(n * C + c0 + c) * HW + p0 + tx] = (T)tile[tx][c];
+}
+
 }  // namespace layout
 
 // Two tensors [B, C0, HW] and [B, C1, HW] (C1 = 0: one) in one launch.  esize:
@@ -56,6 +73,19 @@ hipError_t nchw_to_nhwc_launch(const void *src0, void *dst0, int C0, const void 
                            (unsigned *)dst0, C0, gy0, (const unsigned *)src1, (unsigned *)dst1, C1, HW);
     else
         return hipErrorNotSupported;
+    return hipGetLastError();
+}
+
+hipError_t nhwc_f32_to_nchw_launch(const float *src, void *dst, int C, int B, long HW, int dtype, hipStream_t st) {
+    if (B <= 0 || C <= 0 || HW <= 0) return hipSuccess;
+    const long gx = (HW + 63) / 64;
+    const int gy = (C + 63) / 64;
+    if (gx > 0x7fffffffL || gy > 65535 || B > 65535) return hipErrorNotSupported;
+    const dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)B);
+    if (dtype == 0) hipLaunchKernelGGL(layout::nhwc_f32_to_nchw_kernel<float>, grid, dim3(256), 0, st, src, (float *)dst, C, HW);
+    else if (dtype == 2) hipLaunchKernelGGL(layout::nhwc_f32_to_nchw_kernel<f16_t>, grid, dim3(256), 0, st, src, (f16_t *)dst, C, HW);
+    else if (dtype == 3) hipLaunchKernelGGL(layout::nhwc_f32_to_nchw_kernel<bf16_t>, grid, dim3(256), 0, st, src, (bf16_t *)dst, C, HW);
+    else return hipErrorNotSupported;
     return hipGetLastError();
 }
 

@@ -43,17 +43,18 @@ def test_library_exports_every_declared_symbol():
     assert h.sapa_deform_fused_forward_workspace(8, 128, 256, 64, 64, 25, 2, 4, _lib.DTYPES[torch.bfloat16]) == 8 * 4096 * (128 + 256) * 2
     assert h.sapa_deform_fused_forward_workspace(8, 128, 256, 64, 64, 5, 2, 4, _lib.DTYPES[torch.float32]) == 0
     assert h.sapa_deform_fused_forward_workspace(8, 128, 256, 64, 64, 25, 2, 4, _lib.DTYPES[torch.float64]) == 0
-    # two fp32 [B,G,P,sH,sW] tensors and channels-last copies of key and value for the matrix-form
-    # stage; 16-bit tensors: plus fp32 accumulators of the low-res gradients.  Groups the matrix-form
-    # stage does not serve (5 channels): no copies, but half of grad_offset in fp32 for 16-bit tensors
+    # two fp32 [B,G,P,sH,sW] tensors, fp32 accumulators of the two low-res gradients and
+    # channels-last copies of key and value for the matrix-form stage.  Groups that stage does not
+    # serve (5 channels): no copies, but half of grad_offset in fp32 for 16-bit tensors
     per_point = 8 * 4 * 25 * 128 * 128 * 4
     low = 8 * 4096 * (128 + 256)
-    assert h.sapa_deform_fused_backward_workspace(8, 128, 256, 64, 64, 25, 2, 4, _lib.DTYPES[torch.float32]) == 2 * per_point + low * 4
+    assert h.sapa_deform_fused_backward_workspace(8, 128, 256, 64, 64, 25, 2, 4, _lib.DTYPES[torch.float32]) == 2 * per_point + low * 4 + low * 4
     assert (h.sapa_deform_fused_backward_workspace(8, 128, 256, 64, 64, 25, 2, 4, _lib.DTYPES[torch.bfloat16])
             == 2 * per_point + low * 4 + low * 2)
-    assert h.sapa_deform_fused_backward_workspace(8, 20, 256, 64, 64, 25, 2, 4, _lib.DTYPES[torch.float32]) == 2 * per_point
+    low5 = 8 * 4096 * (20 + 256)
+    assert h.sapa_deform_fused_backward_workspace(8, 20, 256, 64, 64, 25, 2, 4, _lib.DTYPES[torch.float32]) == 2 * per_point + low5 * 4
     assert (h.sapa_deform_fused_backward_workspace(8, 20, 256, 64, 64, 25, 2, 4, _lib.DTYPES[torch.bfloat16])
-            == 4 * per_point + 8 * 4096 * (20 + 256) * 4)
+            == 4 * per_point + low5 * 4)
     assert h.sapa_deform_fused_backward_workspace(8, 128, 256, 64, 64, 25, 3, 4, _lib.DTYPES[torch.float32]) == 0
 
 
