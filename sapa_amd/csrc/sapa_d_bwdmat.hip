@@ -315,9 +315,12 @@ deform_bwd_wmat_kernel(const T *__restrict__ grad_out, const T *__restrict__ q,
                 v1 = gp[0], v2 = gp[1], v3 = gp[WW], v4 = gp[WW + 1];
             }
             if (m.fb) {
-                // the same eight products straight from global memory (rare)
+                // the same eight products straight from global memory (rare; the
+                // position is made opaque, so that its taps are set up in this branch only)
+                float fkh = kh, fkw = kw;
+                asm volatile("" : "+v"(fkh), "+v"(fkw));
                 Tap<float> tp = {};
-                tap_setup(kh, kw, H, W, tp);
+                tap_setup(fkh, fkw, H, W, tp);
                 const T *kp = key + (long)n * lpix * Cq + g * d;
                 const T *qp = q_n + (long)(g * d) * hpl + px.pp;
                 for (int c = 0; c < d; ++c) {
@@ -379,6 +382,28 @@ deform_bwd_wmat_kernel(const T *__restrict__ grad_out, const T *__restrict__ q,
                     op[hpl] = (T)gh;
                 }
             }
+            if (grad_q) {
+                // ---- (d) Wg[pixel][cell] += gl * corner weight, as integers scaled by
+                // 2^30 / sum_p |gl| of the pixel: every partial sum stays within 2^30, the
+                // adds are exact in any order and run at the rate of plain LDS writes.
+                // Wg takes the place of G': the rows of this pass's pixels (NPP of them,
+                // read and written by this wave only, whose LDS operations execute in
+                // order) are emptied here, after the reads above.
+                constexpr int NPP = 64 / NL;
+                f32x4 *rows = (f32x4 *)(Gl + (pi - (lane / NL)) * WS);
+                for (int i = lane; i < NPP * WS / 4; i += 64) rows[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+                const float sc = l1[ps] > 0.f ? WSCALE / l1[ps] : 0.f;
+                // (a sum that is not finite reaches the result through this factor)
+                if (pt == 0) invl[pi] = l1[ps] * (1.f / WSCALE);
+                if (m.in) {
+                    u32 *wp = (u32 *)Gl + pi * WS + m.cell;
+                    const float x = gl * sc;
+                    __hip_atomic_fetch_add(wp, (u32)(int)__builtin_rintf(x * m.w1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    __hip_atomic_fetch_add(wp + 1, (u32)(int)__builtin_rintf(x * m.w2), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    __hip_atomic_fetch_add(wp + WW, (u32)(int)__builtin_rintf(x * m.w3), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    __hip_atomic_fetch_add(wp + WW + 1, (u32)(int)__builtin_rintf(x * m.w4), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                }
+            }
         };
         if (narrow) {
             sample(std::integral_constant<int, 16>{}, 0, srow, spx, sq);
@@ -393,33 +418,7 @@ deform_bwd_wmat_kernel(const T *__restrict__ grad_out, const T *__restrict__ q,
             gorow = load_tile_row(go_n + (long)((g + 1) * cg) * hpl, cv0);
         }
         if (grad_q) {
-            // ---- (d) Wg[pixel][cell] += gl * corner weight, as integers scaled by
-            // 2^30 / sum_p |gl| of the pixel: every partial sum stays within 2^30, the
-            // adds are exact in any order and run at the rate of plain LDS writes
-            __syncthreads();        // Sim and G' are done with
-            for (int i = tid; i < NPX * WS / 4; i += NT) ((f32x4 *)Gl)[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-            __syncthreads();
-            auto scatter = [&](int ps, int pi, int pt) __attribute__((always_inline)) {
-                const Smp &m = sm[ps];
-                const float sc = l1[ps] > 0.f ? WSCALE / l1[ps] : 0.f;
-                // (a sum that is not finite reaches the result through this factor)
-                if (pt == 0) invl[pi] = l1[ps] * (1.f / WSCALE);
-                if (m.in) {
-                    u32 *wp = (u32 *)Gl + pi * WS + m.cell;
-                    const float x = m.gl * sc;
-                    __hip_atomic_fetch_add(wp, (u32)(int)__builtin_rintf(x * m.w1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                    __hip_atomic_fetch_add(wp + 1, (u32)(int)__builtin_rintf(x * m.w2), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                    __hip_atomic_fetch_add(wp + WW, (u32)(int)__builtin_rintf(x * m.w3), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                    __hip_atomic_fetch_add(wp + WW + 1, (u32)(int)__builtin_rintf(x * m.w4), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                }
-            };
-            if (narrow) {
-                scatter(0, srow, sq);
-            } else {
-                scatter(0, half, pl);
-                scatter(1, 8 + half, pl);
-            }
-            __syncthreads();
+            __syncthreads();        // the rows of Wg are complete; Sim is done with
             // ---- (e) grad_query tile = Wg . key window: wave = (channel block, share of the cells)
             {
                 const int cb = wave % NCB, ks = wave / NCB;
