@@ -14,15 +14,18 @@
 //   grad_low[cell][c] += sum_pixels Wm[pixel][cell] * hi[pixel][c]        (Wm^T . hi)
 //
 // A workgroup owns a region of RG x RG hi-res pixels of one (image, group,
-// 64-channel chunk) and walks over it 16 pixels at a time: the rows of Wm for
-// those pixels are built in LDS (integer adds of per-row-scaled values: exact in
-// any order, and several times the rate of LDS float atomics), their hi values
-// are staged next to them, and v_mfma_f32_16x16x4f32 accumulates
+// 64-channel chunk) and walks over it 16 pixels (a step) at a time: the rows of
+// Wm for those pixels are built in LDS (integer adds of per-row-scaled values:
+// exact in any order, and several times the rate of LDS float atomics), their hi
+// values are staged next to them, and v_mfma_f32_16x16x4f32 accumulates
 // [cells of the region's window] x [64 channels] in registers over all 256
-// pixels.  One global float atomic per window cell and channel at the end adds
-// the region's sums to grad_low (the caller zero-fills it), as the LDS-window
-// kernel of sapa_d_lowgrad.hip does -- which needs four 64-bit LDS atomics per
-// sample AND channel where this kernel needs four 32-bit ones per sample.
+// pixels.  Half of the workgroup's 8 waves build the operands of step s while the
+// other half multiplies those of step s - 1 (two sets of LDS buffers, one barrier
+// per step), so that the vector and the matrix pipe work at the same time.  One
+// global float atomic per window cell and channel at the end adds the region's
+// sums to grad_low (the caller zero-fills it), as the LDS-window kernel of
+// sapa_d_lowgrad.hip does -- which needs four 64-bit LDS atomics per sample AND
+// channel where this kernel needs four 32-bit ones per sample.
 //
 // Samples that leave the region's window (offsets beyond +-4 cells), and all
 // samples of a pixel whose scalars or hi values are not finite (an inf / NaN
@@ -37,6 +40,8 @@ namespace sapa {
 
 namespace dscat {
 
+// Timing builds (wrong results): 1 = no matrix products, 2 = no per-sample phase,
+// 4 = no final atomics, 8 = no loads after the first two steps
 #ifndef SAPA_SCAT_PROBE
 #define SAPA_SCAT_PROBE 0
 #endif
@@ -311,7 +316,7 @@ deform_scatter_mat_kernel(const T *__restrict__ hi, const TS *__restrict__ sc,
                 const int gy = wy0 + cell / WWR, gx = wx0 + cell % WWR;
                 const bool ok = cell < NPOS && gy >= 0 && gy < H && gx >= 0 && gx < W;
                 const float v = Tl[(8 * w8 + c) * TSC + lane];
-                if (ok && lane < cvalid && v != 0.f) unsafeAtomicAdd(g0 + ((long)gy * W + gx) * Cx, v);
+                if (ok && lane < cvalid && v != 0.f && !(SAPA_SCAT_PROBE & 4)) unsafeAtomicAdd(g0 + ((long)gy * W + gx) * Cx, v);
             }
         } else {
             // lane <-> cell 64 cbi + lane; this wave: channels 8 w8 .. + 7
