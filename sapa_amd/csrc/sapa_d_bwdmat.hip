@@ -165,11 +165,16 @@ deform_bwd_wmat_kernel(const T *__restrict__ grad_out, const T *__restrict__ q,
     // ---- hi-res tiles: 16 pixels x up to 64 channel planes of q or grad_out, a
     // thread fetching one tile row (4 x-neighbours) of one plane; zeros for
     // channels past nch and rows / columns past the image
+    // (addresses are worked out at each use from opaque copies of the thread's
+    // indices: hoisted out of the loops as 64-bit pointers they are spilled, and
+    // the spill stores of every workgroup are memory traffic)
     auto load_tile_row = [&](const T *base, int nch) __attribute__((always_inline)) {
         Raw r = Raw{};
-        const int qh = y0 + trow;
-        if (tch < nch && qh < hH) {
-            const T *p = base + (long)tch * hpl + (long)qh * hW + x0;
+        int tch_o = tch, trow_o = trow;
+        asm volatile("" : "+v"(tch_o), "+v"(trow_o));
+        const int qh = y0 + trow_o;
+        if (tch_o < nch && qh < hH) {
+            const T *p = base + (long)tch_o * hpl + (long)qh * hW + x0;
             if (hvec) {
                 r = *(const Raw *)p;
             } else {
@@ -246,7 +251,9 @@ deform_bwd_wmat_kernel(const T *__restrict__ grad_out, const T *__restrict__ q,
         const bool narrow = P <= 16;
         f32x2 off2[2] = {f32x2{0.f, 0.f}, f32x2{0.f, 0.f}};
         auto load_offset = [&](const Pix &px, int pt) __attribute__((always_inline)) {
-            const T *op = off_n + 2L * ((long)g * P + pt) * hpl + px.pp;
+            int pp = px.pp;
+            asm volatile("" : "+v"(pp));
+            const T *op = off_n + 2L * ((long)g * P + pt) * hpl + pp;
             return f32x2{(float)op[0], (float)op[hpl]};
         };
         if (narrow) {
@@ -289,6 +296,7 @@ deform_bwd_wmat_kernel(const T *__restrict__ grad_out, const T *__restrict__ q,
         float l1[2] = {0.f, 0.f};
         auto sample = [&](auto nl, int ps, int pi, const Pix &px, int pt) __attribute__((always_inline)) {
             constexpr int NL = decltype(nl)::value;
+            asm volatile("" : "+v"(pi));        // (its LDS rows' addresses: not kept across the groups)
             const bool live = px.active && pt < P;
             const float kw = (float)px.pw + off2[ps][0], kh = (float)px.ph + off2[ps][1];
             const bool guard = kh > -1.f && kh < (float)H && kw > -1.f && kw < (float)W;
@@ -361,7 +369,9 @@ deform_bwd_wmat_kernel(const T *__restrict__ grad_out, const T *__restrict__ q,
             m.gl = pt < P ? gl : 0.f;
             l1[ps] = reduce_lanes<false, NL>(m.in ? __builtin_fabsf(gl) : 0.f);
             if (live) {
-                const long pidx = (((long)n * G + g) * P + pt) * hpl + px.pp;
+                int pp = px.pp;
+                asm volatile("" : "+v"(pp));
+                const long pidx = (((long)n * G + g) * P + pt) * hpl + pp;
                 attn_ws[pidx] = att;
                 gl_ws[pidx] = gl;
                 if (grad_offset) {
@@ -377,7 +387,7 @@ deform_bwd_wmat_kernel(const T *__restrict__ grad_out, const T *__restrict__ q,
                         gw = fma_(gl, dsw, att * dvw);
                         gh = fma_(gl, dsh, att * dvh);
                     }
-                    T *op = grad_offset + ((long)n * 2 * G * P + 2L * ((long)g * P + pt)) * hpl + px.pp;
+                    T *op = grad_offset + ((long)n * 2 * G * P + 2L * ((long)g * P + pt)) * hpl + pp;
                     op[0] = (T)gw;
                     op[hpl] = (T)gh;
                 }

@@ -325,12 +325,44 @@ deform_fused_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key,
     // group before it is aggregated, and stay as loaded until their use: nothing
     // waits for them where they are issued
     u32 offraw[NSP], offnext[NSP];
+    // Contiguous hi-res offsets whose tile rows are whole aligned vectors come in as
+    // such: thread t fetches the 4 x-neighbours of tile row (t / 2) % 4 in the dx
+    // (t even) or dy plane of point t / 8 -- one 8-byte load per thread instead of
+    // four 2-byte ones, and a quarter of the memory requests -- through a buffer
+    // descriptor (out-of-range offset = no access), and they reach the lanes that
+    // use them through LDS, as the (dx, dy) pairs the other paths load directly.
+    __shared__ __attribute__((aligned(16))) T Ost[NCHW ? 32 * NPX * 2 : 8];
+    const bool ovec = NCHW && olayout == OFFSET_HIRES && hW % TW == 0 && TW == 4 && TH == 4 &&
+                      (uintptr_t)offset % 8 == 0 && 2L * G * P * hpl * (long)sizeof(T) < (1L << 31);
+    const __amdgpu_buffer_rsrc_t orsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(offset + (long)n * 2 * G * P * hpl), 0, ovec ? (int)(2L * G * P * hpl * (long)sizeof(T)) : 0, 0x00020000);
+    static_assert(NSP >= 2 || !NCHW, "the vector form keeps its 8 bytes in the two offnext registers");
     auto load_offsets = [&](int g) __attribute__((always_inline)) {
+        if (ovec) {
+            // this thread's piece within a group's planes (worked out here each time,
+            // from an opaque copy of the thread index: kept across the kernel it would
+            // cost a register the kernel does not have); the group's first plane
+            // travels as the load's scalar offset
+            int t = tid;
+            asm volatile("" : "+v"(t));
+            const int xy = t & 1, row = (t >> 1) & 3, opt = t >> 3;
+            const u32 ovoff = (opt < P && y0 + row < hH)
+                                  ? (u32)(((2L * opt + xy) * hpl + (long)(y0 + row) * hW + x0) * (long)sizeof(T))
+                                  : 0x80000000u;
+            const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(orsrc, ovoff, (u32)(2L * g * P * hpl * (long)sizeof(T)), 0);
+            offnext[0] = v[0];
+            offnext[NSP > 1 ? 1 : 0] = v[1];
+            return;
+        }
+        // (the addresses are worked out from an opaque copy of the lane's pixel row:
+        // hoisted out of the loop over the groups they would be spilled)
+        int prow_o = prow;
+        asm volatile("" : "+v"(prow_o));
 #pragma unroll
         for (int ps = 0; ps < NSP; ++ps) {
             offnext[ps] = 0u;
             if (ps < nsp) {
-                const Pix px = pixel(ps * ppp + prow);
+                const Pix px = pixel(ps * ppp + prow_o);
                 if (px.active && pt < P) {
                     if (NCHW) {
                         // channel cx = dx, cx + 1 = dy of the point, from the hi-res tensor
@@ -370,6 +402,14 @@ deform_fused_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key,
         // ---- (a) key window
         stage_store_key();
         stage_store_q();
+        if (ovec) {
+            // Ost[point][pixel][dx, dy]
+            const int xy = tid & 1, row = (tid >> 1) & 3, opt = tid >> 3;
+            union { u32x2 u; T h[4]; } x;
+            x.u = u32x2{offnext[0], offnext[NSP > 1 ? 1 : 0]};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) Ost[((opt * NPX) + row * 4 + e) * 2 + xy] = x.h[e];
+        }
         if (tid == 0) fb_flag = 0;
         __syncthreads();
         // the group's first value chunk travels during the similarity and the sampling
@@ -378,6 +418,7 @@ deform_fused_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key,
 #pragma unroll
         for (int ps = 0; ps < NSP; ++ps) {
             offraw[ps] = offnext[ps];
+            if (ovec) offraw[ps] = ps < nsp ? ((const u32 *)Ost)[pt * NPX + ps * ppp + prow] : 0u;
             off2[ps] = widen_pair<T>(offraw[ps]);
         }
 
