@@ -632,8 +632,13 @@ deform_fused_wmat_kernel(const T *__restrict__ q, const T *__restrict__ key,
         const bool narrow = P <= 16;
         f32x2 off2[2] = {f32x2{0.f, 0.f}, f32x2{0.f, 0.f}};
         // (dx, dy) of point pt of pixel px
-        auto load_offset = [&](const Pix &px, int pt) __attribute__((always_inline)) {
+        auto load_offset = [&](const Pix &pxc, int pt) __attribute__((always_inline)) {
             if (NCHW) {
+                // (opaque copies: the addresses below, hoisted out of the loop over the
+                // groups as 64-bit pointers, would be spilled -- and the spill stores of
+                // every workgroup are memory traffic)
+                Pix px = pxc;
+                asm volatile("" : "+v"(px.pp), "+v"(px.ph), "+v"(px.pw));
                 // channel cx = dx, cx + 1 = dy of the point, from the hi-res tensor or
                 // from the low-res one it is a pixel shuffle / a nearest interpolation
                 // of (deform_tap.hpp: OffsetLayout)
@@ -653,7 +658,7 @@ deform_fused_wmat_kernel(const T *__restrict__ q, const T *__restrict__ key,
                 }
                 return f32x2{(float)op[0], (float)op[dy]};
             }
-            return Q4::load_pair(offset + px.hp * (2L * G * P) + 2L * ((long)g * P + pt));
+            return Q4::load_pair(offset + pxc.hp * (2L * G * P) + 2L * ((long)g * P + pt));
         };
         if (narrow) {
             if (spx.active && sq < P) off2[0] = load_offset(spx, sq);
