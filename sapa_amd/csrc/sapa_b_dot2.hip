@@ -316,11 +316,15 @@ sapa_b_dot2_kernel(const T *__restrict__ q, const T *__restrict__ key,
                     for (int cx = 0; cx < S; ++cx)
                         dot[cy * S + cx] = fma_(a[cy * S + cx][k], v[cx], dot[cy * S + cx]);
                 }
+            // (through an opaque copy of the pointer: the compiler would otherwise keep
+            // the first pass's K*K loads for this one and spill them)
+            const float *ap2 = ap;
+            asm volatile("" : "+v"(ap2));
 #pragma unroll
             for (int k = 0; k < KK; ++k)
 #pragma unroll
                 for (int cy = 0; cy < S; ++cy) {
-                    const f32x2 v = *(const f32x2 *)(ap + (long)k * hplane + (long)cy * hW);
+                    const f32x2 v = *(const f32x2 *)(ap2 + (long)k * hplane + (long)cy * hW);
 #pragma unroll
                     for (int cx = 0; cx < S; ++cx)
                         a[cy * S + cx][k] = v[cx] * (a[cy * S + cx][k] - dot[cy * S + cx]);

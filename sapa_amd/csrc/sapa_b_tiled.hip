@@ -351,11 +351,15 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
                     for (int cx = 0; cx < S; ++cx)
                         dot[cy * S + cx] = fma_(a[cy * S + cx][k], (A)v.v[cx], dot[cy * S + cx]);
                 }
+            // (through an opaque copy of the pointer: the compiler would otherwise keep
+            // the first pass's K*K loads for this one and spill them)
+            const TA *ap2 = ap;
+            asm volatile("" : "+v"(ap2));
 #pragma unroll
             for (int k = 0; k < KK; ++k)
 #pragma unroll
                 for (int cy = 0; cy < CY; ++cy) {
-                    const VecA v = *(const VecA *)(ap + (long)k * hplane + (long)cy * hW);
+                    const VecA v = *(const VecA *)(ap2 + (long)k * hplane + (long)cy * hW);
 #pragma unroll
                     for (int cx = 0; cx < S; ++cx)
                         a[cy * S + cx][k] = (A)v.v[cx] * (a[cy * S + cx][k] - dot[cy * S + cx]);
