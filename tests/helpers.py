@@ -52,3 +52,14 @@ def ulp_report(got, want):
     got, want = got.detach().cpu().float(), want.detach().cpu().float()
     sp = torch.abs(torch.nextafter(want, torch.full_like(want, float('inf'))) - want)
     return ((got - want).abs() / sp).max().item()
+
+
+def deform_fused_backward_oracle(coracle, go, q, key, v, off, P, s, G):
+    """deform_av_backward -> softmax backward -> deform_qk_backward in float64
+    on the given values (the chain autograd runs for sapa_deform.py:51-53)."""
+    go, q, key, v, off = (t.double() for t in (go, q, key, v, off))
+    attn = torch.softmax(coracle.deform_qk(q, key, off, P, s, G, 'f64'), dim=2)
+    ga, gv, goff_av = coracle.deform_av_backward(go, attn, v, off, P, s, G, 'f64')
+    gl = attn * (ga - (ga * attn).sum(dim=2, keepdim=True))
+    gq, gk, goff_qk = coracle.deform_qk_backward(gl, q, key, off, P, s, G, 'f64')
+    return gq, gk, gv, goff_av + goff_qk

@@ -32,7 +32,8 @@ import torch
 import torch.nn.functional as F
 
 import sapa_amd
-from helpers import BF16_REL, F32_ATOL, F32_RTOL, assert_f32_close, assert_rel_rms_close, gen, randn
+from helpers import (BF16_REL, F32_ATOL, F32_RTOL, assert_f32_close, assert_rel_rms_close,
+                     deform_fused_backward_oracle, gen, randn)
 
 pytestmark = pytest.mark.gpu
 DEV = 'cuda:0'
@@ -290,6 +291,58 @@ def test_c4_deform_against_oracle(coracle, P):
     assert_rel_rms_close(fused(hq, hk, hv, ho)[list(imgs)].float(), exact16, BF16_REL, f'c4 P={P} bf16')
     assert_rel_rms_close(fused(*as_cl(hq, hk, hv, ho))[list(imgs)].float(), exact16, BF16_REL,
                          f'c4 P={P} bf16 channels_last')
+
+
+@pytest.mark.parametrize('dtype,P', [(torch.float32, 25), (torch.float32, 9), (torch.bfloat16, 25)])
+def test_c4_deform_backward_against_oracle(coracle, dtype, P):
+    """The training step of config 4 at its own sizes: the gradients of
+    sum(out * grad_out) through deform_sapa_fused (one sapa_deform_fused_backward call:
+    the matrix-form kernel for the per-pixel part, the matrix-product scatter for the
+    low-res gradients) against the float64 oracle chain on two images, and the whole
+    batch against the same call image by image -- bit for bit where no atomics are
+    involved (grad_query, grad_offset), to fp32 rounding where the order of the sums
+    varies (grad_key, grad_value)."""
+    B, s, G = 8, 2, 4
+    q, key, v, off, _ = c4_inputs(B, P, 450 + P)
+    frac = off - off.floor()
+    off = off.floor() + frac.clamp(0.2, 0.8)        # 16-bit rounding must not cross a bilinear kink
+    go = randn(gen(460 + P), B, 256, 128, 128)
+    q, key, v, off, go = (t.to(dtype) for t in (q, key, v, off, go))
+
+    def grads(*ts):
+        leaves = [t.clone().requires_grad_() for t in ts[:4]]
+        sapa_amd.deform_sapa_fused(*leaves, P, s, G).backward(ts[4])
+        return [t.grad for t in leaves]
+
+    def grads_separate(*ts):
+        leaves = [t.clone().requires_grad_() for t in ts[:4]]
+        a, b, c, o = leaves
+        attn = torch.softmax(sapa_amd.deform_qk(a, b, o, P, s, G), dim=2)
+        sapa_amd.deform_av(attn, c, o, P, s, G).backward(ts[4])
+        return [t.grad for t in leaves]
+
+    full = grads(*dev(q, key, v, off, go))
+    names = ('grad_query', 'grad_key', 'grad_value', 'grad_offset')
+    for n in (0, B - 1):
+        one = grads(*dev(*(t[n:n + 1] for t in (q, key, v, off, go))))
+        for name, a, b in zip(names, full, one):
+            if name in ('grad_query', 'grad_offset'):
+                assert torch.equal(a[n:n + 1], b), f'{name}: image {n} of the batch differs from the image alone'
+            else:
+                torch.testing.assert_close(a[n:n + 1].float(), b.float(), msg=lambda m: f'{name} image {n}: {m}',
+                                           rtol=1e-5 if dtype == torch.float32 else 2.0 ** -7, atol=1e-5)
+        want = deform_fused_backward_oracle(coracle, *(t[n:n + 1].float() for t in (go, q, key, v, off)), P, s, G)
+        if dtype == torch.float32:
+            # fp32: sums per window cell instead of per point and channel -- no further
+            # from the double-precision result than the chain of the separate operators,
+            # whose kernels keep the reference's order
+            ref = grads_separate(*dev(*(t[n:n + 1] for t in (q, key, v, off, go))))
+            for name, got, r, w in zip(names, full, ref, want):
+                assert_no_worse_than_reference_order(got[n:n + 1], r, w, f'c4 backward P={P} {name} image {n}')
+        else:
+            for name, got, w in zip(names, full, want):
+                assert_rel_rms_close(got[n:n + 1].float().cpu().double(), w, 1.5e-2,
+                                     f'c4 backward P={P} bf16 {name} image {n}')
 
 
 def test_c4_regular_grid_offsets_reduce_to_sapa_b():

@@ -9,8 +9,8 @@ import torch
 import torch.nn.functional as F
 
 import sapa_amd
-from helpers import (BF16_REL, F16_REL, assert_f32_close, assert_rel_rms_close, gen, golden,
-                     randn, ulp_report)
+from helpers import (BF16_REL, F16_REL, assert_f32_close, assert_rel_rms_close, deform_fused_backward_oracle,
+                     gen, golden, randn, ulp_report)
 
 pytestmark = pytest.mark.gpu
 DEV = 'cuda:0'
@@ -240,17 +240,6 @@ def test_backward_vs_oracle(coracle, shape):
         torch.testing.assert_close(od.grad.cpu(), goff, **tol)
 
 
-def _deform_fused_backward_oracle(coracle, go, q, key, v, off, P, s, G):
-    """deform_av_backward -> softmax backward -> deform_qk_backward in float64
-    on the given values (the chain autograd runs for sapa_deform.py:51-53)."""
-    go, q, key, v, off = (t.double() for t in (go, q, key, v, off))
-    attn = torch.softmax(coracle.deform_qk(q, key, off, P, s, G, 'f64'), dim=2)
-    ga, gv, goff_av = coracle.deform_av_backward(go, attn, v, off, P, s, G, 'f64')
-    gl = attn * (ga - (ga * attn).sum(dim=2, keepdim=True))
-    gq, gk, goff_qk = coracle.deform_qk_backward(gl, q, key, off, P, s, G, 'f64')
-    return gq, gk, gv, goff_av + goff_qk
-
-
 # B, G, dq, cg, H, W, P, s, offset scale: partial tiles and chunks; offsets beyond the
 # LDS window; s = 4 and s = 1
 # (B, G, d, cg, H, W, P, s, offset scale).  The first four: one shape the matrix-form
@@ -292,7 +281,7 @@ def test_deform_fused_backward_entry_point(coracle, shape, dtype, tol):
     grads = [torch.full_like(t, float('nan')) for t in (qd, kd, vd, od)]
     assert _lib.call_status('sapa_deform_fused_backward', DEV, _lib.ptr(god), _lib.ptr(qd), _lib.ptr(kd),
                             _lib.ptr(vd), _lib.ptr(od), _lib.ptr(ws), *(_lib.ptr(t) for t in grads), *args) == 0
-    want = _deform_fused_backward_oracle(coracle, go.float(), q.float(), key.float(), v.float(), off.float(), P, s, G)
+    want = deform_fused_backward_oracle(coracle, go.float(), q.float(), key.float(), v.float(), off.float(), P, s, G)
     for got, w, name in zip(grads, want, ('grad_query', 'grad_key', 'grad_value', 'grad_offset')):
         assert torch.isfinite(got).all(), name
         if dtype == torch.float32:
