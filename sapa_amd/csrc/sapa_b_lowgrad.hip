@@ -26,6 +26,8 @@
 // S children of a parent row with one S-wide LDS access.  Each child row has
 // its own running sum over k in ascending order, one FMA per term; the row
 // sums are added at the end.
+#include <type_traits>
+
 #include "kernels.hpp"
 
 namespace sapa {
@@ -66,8 +68,16 @@ lowgrad_gather_kernel(const T *__restrict__ hi, const WT *__restrict__ w,
     static_assert(NLD <= 32, "validity mask is 32 bits");
     typedef typename FVec<VEC>::type V;
     typedef typename FVec<S>::type V2;
+    // 16-bit tensors stay 16-bit in LDS (a dword = the two children of a parent in a
+    // row): the kernel is bound by the bytes it reads from LDS, and widening at the
+    // use -- a shift and a mask for bf16, two conversions for f16 -- costs less than
+    // those bytes
+    constexpr bool PACK = sizeof(T) == 2;
+    constexpr int LW = PACK ? 2 : 1;                     // pixels per LDS dword
+    static_assert(!PACK || (S == 2 && VEC % 2 == 0), "a dword holds the two children of a parent row");
+    typedef unsigned RawV __attribute__((ext_vector_type(VEC / 2 > 0 ? VEC / 2 : 1)));   // VEC 16-bit elements
 
-    __shared__ __attribute__((aligned(16))) float win[2 * CH * PS];
+    __shared__ __attribute__((aligned(16))) float win[2 * CH * PS / LW];
 
     const int logical = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
     if (logical >= nblocks) return;
@@ -105,7 +115,8 @@ lowgrad_gather_kernel(const T *__restrict__ hi, const WT *__restrict__ w,
     // staging: element e of a chunk = (channel, window row, vector in the row)
     const int wy0 = (ty * TH - R) * S, wx0 = (tx * TW - R) * S;   // window origin, high-res
     const T *hp = hi + (long)n * C * hplane;
-    V stage[NLD];
+    typedef typename std::conditional<PACK, RawV, V>::type StageV;
+    StageV stage[NLD];
     unsigned okmask = 0;
     auto issue = [&](int c0) {
         okmask = 0;
@@ -120,7 +131,8 @@ lowgrad_gather_kernel(const T *__restrict__ hi, const WT *__restrict__ w,
             const bool ok =
                 e < CH * NV && c0 + ch < cend && gy >= 0 && gy < hH && gx >= 0 && gx < hW;
             const long off = ok ? (long)(c0 + ch) * hplane + (long)gy * hW + gx : 0;
-            stage[i] = load_wide<T, VEC>(hp + off);
+            if constexpr (PACK) stage[i] = *(const RawV *)(hp + off);
+            else stage[i] = load_wide<T, VEC>(hp + off);
             okmask |= (unsigned)ok << i;
         }
     };
@@ -131,9 +143,9 @@ lowgrad_gather_kernel(const T *__restrict__ hi, const WT *__restrict__ w,
             if (e < CH * NV) {
                 const int ch = e / NV, rem = e % NV;
                 const int row = rem / (WW / VEC), col = rem % (WW / VEC) * VEC;
-                V v = stage[i];
-                if (!((okmask >> i) & 1)) v = (V)(0.f);
-                *(V *)(buf + ch * PS + row * RS + col) = v;
+                StageV v = stage[i];
+                if (!((okmask >> i) & 1)) v = StageV{};
+                *(StageV *)(buf + (ch * PS + row * RS + col) / LW) = v;
             }
         }
     };
@@ -143,7 +155,7 @@ lowgrad_gather_kernel(const T *__restrict__ hi, const WT *__restrict__ w,
     __syncthreads();
 
     // the children of window parent (ly + 2r - ky, lx + 2r - kx) feed entry k
-    const float *base = win + (ly + 2 * R) * S * RS + (lx + 2 * R) * S;
+    const float *base = win + ((ly + 2 * R) * S * RS + (lx + 2 * R) * S) / LW;
     const bool live = x < W && y < H;
     const long lplane = (long)H * W;
     T *op = out + (long)n * C * lplane + (long)(y < H ? y : 0) * W + (x < W ? x : 0);
@@ -151,7 +163,7 @@ lowgrad_gather_kernel(const T *__restrict__ hi, const WT *__restrict__ w,
     for (int c0 = cbeg; c0 < cend; c0 += CH, parity ^= 1) {
         const bool more = c0 + CH < cend;
         if (more) issue(c0 + CH);
-        const float *buf = base + parity * CH * PS;
+        const float *buf = base + parity * (CH * PS / LW);
 #pragma unroll 1
         for (int ch = 0; ch < CH; ++ch) {
             float acc[S];   // one running sum per child row: two shorter FMA chains
@@ -161,14 +173,27 @@ lowgrad_gather_kernel(const T *__restrict__ hi, const WT *__restrict__ w,
             for (int k = 0; k < KK; ++k)
 #pragma unroll
                 for (int cy = 0; cy < S; ++cy) {
-                    const V2 h =
-                        *(const V2 *)(buf + ch * PS + (cy - (k / K) * S) * RS - (k % K) * S);
+                    V2 h;
+                    if constexpr (PACK) {
+                        const unsigned u = *(const unsigned *)(buf + (ch * PS + (cy - (k / K) * S) * RS - (k % K) * S) / LW);
+                        if constexpr (std::is_same<T, bf16_t>::value) {
+                            h[0] = __builtin_bit_cast(float, u << 16);
+                            h[1] = __builtin_bit_cast(float, u & 0xffff0000u);
+                        } else {
+                            union { unsigned u; T t[2]; } x;
+                            x.u = u;
+                            h[0] = (float)x.t[0];
+                            h[1] = (float)x.t[1];
+                        }
+                    } else {
+                        h = *(const V2 *)(buf + ch * PS + (cy - (k / K) * S) * RS - (k % K) * S);
+                    }
                     acc[cy] = __builtin_fmaf(wr[k][cy * S], h[0], acc[cy]);
                     acc[cy] = __builtin_fmaf(wr[k][cy * S + 1], h[1], acc[cy]);
                 }
             if (live && c0 + ch < cend) op[(long)(c0 + ch) * lplane] = (T)(acc[0] + acc[1]);
         }
-        if (more) commit(win + (parity ^ 1) * CH * PS);
+        if (more) commit(win + (parity ^ 1) * (CH * PS / LW));
         __syncthreads();
     }
 }
@@ -198,8 +223,16 @@ template <typename T, typename WT, int K, int VEC>
 static hipError_t lowgrad_launch_k(const void *hi, const void *w, void *out, int B, int C, int H, int W,
                     hipStream_t st) {
     const bool wide = (W + 31) / 32 * 32 * 0.9 <= (W + 15) / 16 * 16;
-    return wide ? lowgrad_launch_geom<T, WT, K, 2, 2, 2, 2, VEC>(hi, w, out, B, C, H, W, st)
-                : lowgrad_launch_geom<T, WT, K, 2, 1, 2, 2, VEC>(hi, w, out, B, C, H, W, st);
+    // channels per chunk (a barrier per chunk): 16-bit tensors take half the LDS per channel
+#ifndef SAPA_LOWGRAD_CH16
+#define SAPA_LOWGRAD_CH16 4
+#endif
+#ifndef SAPA_LOWGRAD_CH32
+#define SAPA_LOWGRAD_CH32 2
+#endif
+    constexpr int CHN = sizeof(T) == 2 ? SAPA_LOWGRAD_CH16 : SAPA_LOWGRAD_CH32;
+    return wide ? lowgrad_launch_geom<T, WT, K, 2, 2, 2, CHN, VEC>(hi, w, out, B, C, H, W, st)
+                : lowgrad_launch_geom<T, WT, K, 2, 1, 2, CHN, VEC>(hi, w, out, B, C, H, W, st);
 }
 
 template <typename T, typename WT>
