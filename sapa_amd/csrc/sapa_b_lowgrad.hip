@@ -230,9 +230,10 @@ static hipError_t lowgrad_launch_k(const void *hi, const void *w, void *out, int
 #ifndef SAPA_LOWGRAD_CH32
 #define SAPA_LOWGRAD_CH32 2
 #endif
-    constexpr int CHN = sizeof(T) == 2 ? SAPA_LOWGRAD_CH16 : SAPA_LOWGRAD_CH32;
+    // (with 2-element staging loads 4 channels per chunk do not fit the registers)
+    constexpr int CHN = sizeof(T) == 2 ? (VEC == 4 ? SAPA_LOWGRAD_CH16 : 2) : SAPA_LOWGRAD_CH32;
     return wide ? lowgrad_launch_geom<T, WT, K, 2, 2, 2, CHN, VEC>(hi, w, out, B, C, H, W, st)
-                : lowgrad_launch_geom<T, WT, K, 2, 1, 2, CHN, VEC>(hi, w, out, B, C, H, W, st);
+                : lowgrad_launch_geom<T, WT, K, 2, 1, 2, sizeof(T) == 2 ? 2 : CHN, VEC>(hi, w, out, B, C, H, W, st);
 }
 
 template <typename T, typename WT>
