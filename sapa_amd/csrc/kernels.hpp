@@ -117,8 +117,11 @@ hipError_t deform_fused_nchw_ws_launch(const void *q, const void *key, const voi
 
 // sapa_layout.hip: contiguous [B, C, HW] -> channels-last [B, HW, C] for two tensors
 // of the same B and HW in one launch (C1 = 0: one); esize 2 or 4 bytes
+// zero0 / zero1: optional fp32 buffers of the same extents, cleared by the same launch when the
+// vector form of the kernel applies (*zeroed tells)
 hipError_t nchw_to_nhwc_launch(const void *src0, void *dst0, int C0, const void *src1, void *dst1,
-                               int C1, int B, long HW, int esize, hipStream_t st);
+                               int C1, int B, long HW, int esize, hipStream_t st, float *zero0 = nullptr,
+                               float *zero1 = nullptr, bool *zeroed = nullptr);
 // channels-last fp32 [B, HW, C] -> contiguous [B, C, HW] of dtype f32 / f16 / bf16 (0 / 2 / 3)
 hipError_t nhwc_f32_to_nchw_launch(const float *src, void *dst, int C, int B, long HW, int dtype, hipStream_t st);
 

@@ -63,19 +63,28 @@ static long align256(long x) { return (x + 255) / 256 * 256; }
 // atomics then fall on two cache lines per instruction instead of one per window
 // row and channel) and a transposing pass writes the tensor; else the LDS-window
 // scatter accumulates in the tensor's own order.
+static bool low_gradient_channels_last(int B, int Cx, int H, int W, int P, int s, int G, int dtype) {
+#ifdef SAPA_SCATTER_MAT_OFF
+    return false;
+#else
+    return deform_scatter_mat_serves(B, Cx, H, W, P, s, G, dtype);
+#endif
+}
+
+// (cleared: `acc` was cleared by an earlier launch already -- channels-last accumulation only)
 static hipError_t low_gradient(const void *hi, const void *sc, const void *offset, float *acc, void *grad_low,
-                               int B, int Cx, int H, int W, int P, int s, int G, int dtype, hipStream_t st) {
+                               int B, int Cx, int H, int W, int P, int s, int G, int dtype, hipStream_t st,
+                               bool cleared) {
     const bool wide = dtype != 0;
     const long n = (long)B * Cx * H * W;
-#ifdef SAPA_SCATTER_MAT_OFF
-    const bool mat = false;
-#else
-    const bool mat = deform_scatter_mat_serves(B, Cx, H, W, P, s, G, dtype);
-#endif
+    const bool mat = low_gradient_channels_last(B, Cx, H, W, P, s, G, dtype);
     float *const target = (mat || wide) ? acc : (float *)grad_low;
-    hipLaunchKernelGGL(zero_kernel, dim3(blocks_for(n)), dim3(256), 0, st, target, n);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
+    hipError_t e = hipSuccess;
+    if (!(mat && cleared)) {
+        hipLaunchKernelGGL(zero_kernel, dim3(blocks_for(n)), dim3(256), 0, st, target, n);
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
     if (mat) {
         e = deform_scatter_mat_launch(hi, sc, offset, acc, B, Cx, H, W, P, s, G, dtype, st, wide, true);
         if (e != hipSuccess) return e;
@@ -147,6 +156,7 @@ hipError_t deform_fused_backward_launch(const void *grad_out, const void *q, con
     const bool mat = matrix_stage(B, Cq, C, H, W, P, s, G, dtype);
     float *goff32 = wide && !mat ? (float *)rest : nullptr;
     const int HIRES = 0;
+    bool cleared = false;
     hipError_t e;
 #define SAPA_STEP(call)                  \
     do {                                 \
@@ -157,7 +167,12 @@ hipError_t deform_fused_backward_launch(const void *grad_out, const void *q, con
     if (mat) {
         const long esize = wide ? 2 : 4;
         char *key_cl = rest, *value_cl = rest + align256((long)B * Cq * lpix * esize);
-        SAPA_STEP(nchw_to_nhwc_launch(key, key_cl, Cq, value, value_cl, C, B, lpix, (int)esize, st));
+        // (the accumulators of grad_key / grad_value have the copies' extents and, where
+        // they are channels-last, their order: cleared by the same launch)
+        SAPA_STEP(nchw_to_nhwc_launch(key, key_cl, Cq, value, value_cl, C, B, lpix, (int)esize, st,
+                                      grad_key && low_gradient_channels_last(B, Cq, H, W, P, s, G, dtype) ? gk32 : nullptr,
+                                      grad_value && low_gradient_channels_last(B, C, H, W, P, s, G, dtype) ? gv32 : nullptr,
+                                      &cleared));
         SAPA_STEP(deform_bwd_wmat_launch(grad_out, q, key_cl, value_cl, offset, attn, gl, grad_q, grad_offset, B,
                                          Cq, C, H, W, P, s, G, dtype, st));
     } else {
@@ -185,8 +200,8 @@ hipError_t deform_fused_backward_launch(const void *grad_out, const void *q, con
     }
     // the low-res gradients: grad_value (attention weights x grad_out) and
     // grad_key (gradient of the logits x query), scattered
-    if (grad_value) SAPA_STEP(low_gradient(grad_out, attn, offset, gv32, grad_value, B, C, H, W, P, s, G, dtype, st));
-    if (grad_key) SAPA_STEP(low_gradient(q, gl, offset, gk32, grad_key, B, Cq, H, W, P, s, G, dtype, st));
+    if (grad_value) SAPA_STEP(low_gradient(grad_out, attn, offset, gv32, grad_value, B, C, H, W, P, s, G, dtype, st, cleared));
+    if (grad_key) SAPA_STEP(low_gradient(q, gl, offset, gk32, grad_key, B, Cq, H, W, P, s, G, dtype, st, cleared));
 #undef SAPA_STEP
     return hipSuccess;
 }

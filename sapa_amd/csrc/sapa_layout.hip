@@ -42,12 +42,14 @@ nchw_to_nhwc_kernel(const U *__restrict__ src0, U *__restrict__ dst0, int C0, in
 template <typename U>
 __global__ void __launch_bounds__(256)
 nchw_to_nhwc_vec_kernel(const U *__restrict__ src0, U *__restrict__ dst0, int C0, int yblocks0,
-                        const U *__restrict__ src1, U *__restrict__ dst1, int C1, long HW) {
+                        const U *__restrict__ src1, U *__restrict__ dst1, int C1, long HW,
+                        float *__restrict__ zero0, float *__restrict__ zero1) {
     struct alignas(4 * sizeof(U)) V4 { U v[4]; };
     __shared__ U tile[64][65];
     const bool first = (int)blockIdx.y < yblocks0;
     const U *src = first ? src0 : src1;
     U *dst = first ? dst0 : dst1;
+    float *zero = first ? zero0 : zero1;
     const int C = first ? C0 : C1;
     const long p0 = (long)blockIdx.x * 64;
     const int c0 = ((int)blockIdx.y - (first ? 0 : yblocks0)) * 64;
@@ -69,6 +71,12 @@ nchw_to_nhwc_vec_kernel(const U *__restrict__ src0, U *__restrict__ dst0, int C0
 #pragma unroll
             for (int e = 0; e < 4; ++e) x.v[e] = tile[4 * cq + e][p];
             *(V4 *)(dst + (n * HW + p0 + p) * C + c0 + 4 * cq) = x;
+            // an fp32 buffer of the same extent cleared on the way (the accumulator of
+            // the tensor's gradient: one launch less)
+            if (zero) {
+                struct alignas(16) F4 { float v[4]; };
+                *(F4 *)(zero + (n * HW + p0 + p) * C + c0 + 4 * cq) = F4{};
+            }
         }
     }
 }
@@ -124,24 +132,30 @@ nhwc_f32_to_nchw_vec_kernel(const float *__restrict__ src, T *__restrict__ dst, 
 }  // namespace layout
 
 // Two tensors [B, C0, HW] and [B, C1, HW] (C1 = 0: one) in one launch.  esize:
-// bytes per element, 2 or 4.  hipErrorNotSupported otherwise, or for more than
+// bytes per element, 2 or 4.  zero0 / zero1 (may be NULL): fp32 buffers of the two
+// tensors' extents that the vector form of the kernel clears on the way; *zeroed
+// says whether it did.  hipErrorNotSupported otherwise, or for more than
 // 65535 images or 64-channel blocks.
 hipError_t nchw_to_nhwc_launch(const void *src0, void *dst0, int C0, const void *src1, void *dst1,
-                               int C1, int B, long HW, int esize, hipStream_t st) {
+                               int C1, int B, long HW, int esize, hipStream_t st, float *zero0, float *zero1,
+                               bool *zeroed) {
+    if (zeroed) *zeroed = false;
     if (B <= 0 || C0 <= 0 || HW <= 0) return hipSuccess;
     const long gx = (HW + 63) / 64;
     const int gy0 = (C0 + 63) / 64, gy1 = (C1 + 63) / 64;
     if (gx > 0x7fffffffL || gy0 + gy1 > 65535 || B > 65535) return hipErrorNotSupported;
     const dim3 grid((unsigned)gx, (unsigned)(gy0 + gy1), (unsigned)B);
     const uintptr_t ptrs = (uintptr_t)src0 | (uintptr_t)dst0 | (uintptr_t)src1 | (uintptr_t)dst1;
-    if (HW % 4 == 0 && C0 % 4 == 0 && C1 % 4 == 0 && ptrs % (4 * (uintptr_t)esize) == 0 && (esize == 2 || esize == 4)) {
+    if (HW % 4 == 0 && C0 % 4 == 0 && C1 % 4 == 0 && ptrs % (4 * (uintptr_t)esize) == 0 && (esize == 2 || esize == 4) &&
+        ((uintptr_t)zero0 | (uintptr_t)zero1) % 16 == 0) {
         if (esize == 2)
             hipLaunchKernelGGL(layout::nchw_to_nhwc_vec_kernel<unsigned short>, grid, dim3(256), 0, st,
                                (const unsigned short *)src0, (unsigned short *)dst0, C0, gy0,
-                               (const unsigned short *)src1, (unsigned short *)dst1, C1, HW);
+                               (const unsigned short *)src1, (unsigned short *)dst1, C1, HW, zero0, zero1);
         else
             hipLaunchKernelGGL(layout::nchw_to_nhwc_vec_kernel<unsigned>, grid, dim3(256), 0, st, (const unsigned *)src0,
-                               (unsigned *)dst0, C0, gy0, (const unsigned *)src1, (unsigned *)dst1, C1, HW);
+                               (unsigned *)dst0, C0, gy0, (const unsigned *)src1, (unsigned *)dst1, C1, HW, zero0, zero1);
+        if (zeroed) *zeroed = true;
         return hipGetLastError();
     }
     if (esize == 2)
