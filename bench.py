@@ -65,9 +65,9 @@ MEASURED_TRAFFIC = {
     ('stress', 'bf16', 'nchw'): (380752179, 'profiles/sapa_b_mfma_fused_stress_bf16.md', 'sapa_b_mfma_kernel'),
     ('stress', 'bf16', 'channels_last'): (323093471, 'profiles/sapa_b_nhwc16_fused_stress_bf16.md',
                                           'sapa_b_nhwc16_kernel'),
-    ('deform_p25', 'fp32', 'nchw'): (459465979, 'profiles/sapa_d_wmat_fused_deform_p25_fp32_nchw.md',
+    ('deform_p25', 'fp32', 'nchw'): (459885490, 'profiles/sapa_d_wmat_fused_deform_p25_fp32_nchw.md',
                                      'deform_fused_wmat_kernel'),
-    ('deform_p25', 'bf16', 'nchw'): (228860561, 'profiles/sapa_d_wmat16_fused_deform_p25_bf16_nchw.md',
+    ('deform_p25', 'bf16', 'nchw'): (228880702, 'profiles/sapa_d_wmat16_fused_deform_p25_bf16_nchw.md',
                                      'deform_fused_wmat16_kernel'),
     ('deform_p25', 'fp32', 'nchw_reference_order'): (829727510, 'profiles/sapa_d_lds_fused_deform_p25_fp32.md',
                                                      'deform_lds_kernel'),
