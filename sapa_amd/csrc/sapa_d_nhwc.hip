@@ -965,11 +965,18 @@ long deform_fused_nchw_workspace(int B, int Cq, int C, int H, int W, int P, int 
     if (plane * Cq >= (1L << 31) || plane * C >= (1L << 31)) return 0;
     if ((long)H * s * W * s >= (1L << 31)) return 0;
     // Where this path is the faster one (B=8, C=256, G=4, d=32, 64x64 -> 128x128, us,
-    // the two copies included, against the contiguous-layout kernels): fp32 P = 25
-    // 336 / 498, P = 9 296 / 212; bf16 on the 16-bit kernel P = 25 218 / 471, P = 9
-    // 161 / 199, P = 5 156 / 154.
+    // the copy included, against the contiguous-layout kernels): fp32 P = 25 317 / 491,
+    // P = 14 289 / 304, P = 12 282 / 247 (that kernel's wider tile up to 12 points), P = 8
+    // 278 / 197; bf16 on the 16-bit kernel P = 25 194 / 470, P = 9 141 / 199, P = 5 145 / 159,
+    // P = 4 138 / 142, P = 3 137 / 130.
     const bool wm16 = dtype != 0 && d % 8 == 0 && cg % 8 == 0;
-    if (P < (wm16 ? 6 : 15)) return 0;
+#ifndef SAPA_DNCHW_MINP16
+#define SAPA_DNCHW_MINP16 4
+#endif
+#ifndef SAPA_DNCHW_MINP32
+#define SAPA_DNCHW_MINP32 13
+#endif
+    if (P < (wm16 ? SAPA_DNCHW_MINP16 : SAPA_DNCHW_MINP32)) return 0;
     return align256((long)B * plane * Cq) + align256((long)B * plane * C);
 }
 

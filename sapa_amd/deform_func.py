@@ -315,6 +315,6 @@ def deform_sapa_fused(query, key, value, offset, num_point, scale_factor, groups
     (sums per window cell: rounding-level differences from the reference's order in
     fp32, no further from the exact result; SapaUnsupported where they do not serve the
     configuration), False = the reference's order of sums, None = the matrix form
-    where it is the faster path (16-bit tensors from 6 points, fp32 from 15)."""
+    where it is the faster path (16-bit tensors from 4 points, fp32 from 13)."""
     return DeformSAPAFusedFunction.apply(query, key, value, offset, num_point, scale_factor,
                                          groups, offset_layout, matrix_form)

@@ -118,11 +118,11 @@ def test_deform_fused_matrix_form_limits():
     """Too few points for the matrix form to pay, fp64, and the low-res offset
     layouts stay on the contiguous-layout kernels; asking for it explicitly raises."""
     from sapa_amd import _lib
-    shape = (1, 2, 8, 8, 6, 7, 5, 2)
+    shape = (1, 2, 8, 8, 6, 7, 3, 2)
     q, key, v, off, _ = make(gen(231), shape)
     with pytest.raises(_lib.SapaUnsupported):
-        sapa_amd.deform_sapa_fused(*dev(q, key, v, off), 5, 2, 2, matrix_form=True)
-    h = sapa_amd.deform_sapa_fused(*dev(*(t.half() for t in (q, key, v, off))), 5, 2, 2)
+        sapa_amd.deform_sapa_fused(*dev(q, key, v, off), 3, 2, 2, matrix_form=True)
+    h = sapa_amd.deform_sapa_fused(*dev(*(t.half() for t in (q, key, v, off))), 3, 2, 2)
     assert _lib.last_kernel() not in ('deform_fused_wmat_kernel', 'deform_fused_wmat16_kernel') and h.dtype == torch.float16
     q, key, v, off, _ = make(gen(232), (1, 2, 8, 8, 6, 7, 17, 2), dtype=torch.float64)
     with pytest.raises(_lib.SapaUnsupported):
