@@ -27,6 +27,7 @@
 // its own running sum over k in ascending order, one FMA per term; the row
 // sums are added at the end.
 #include <type_traits>
+#include <utility>
 
 #include "kernels.hpp"
 
@@ -198,6 +199,217 @@ lowgrad_gather_kernel(const T *__restrict__ hi, const WT *__restrict__ w,
     }
 }
 
+// ---------------------------------------------------------------------------
+// The same sums with the products owned by the PARENTS.  A lane is one parent
+// (py, px) and keeps its own K*K x S*S weights; per channel it reads its four
+// children of `hi` straight from global memory (every element of `hi` belongs to
+// exactly one parent: no staging, no reuse to organise) and forms
+//
+//   t[ky][kx] = sum over children j of w[(ky,kx)][j] * hi[j]      (K*K*S*S FMAs)
+//
+// which is what this parent adds to cell (py - r + ky, px - r + kx).  The sum over
+// kx is an exchange between x-neighbours: a row of 16 lanes holds 16 consecutive
+// parents, and a DPP row shift hands t[ky][kx] of lane L + r - kx to lane L (K - 1
+// shifted adds per ky).  The sum over ky crosses lane rows and waves and goes through
+// LDS: K floats written and K read per lane and channel, against the K*K*S*S floats
+// the gather above reads per output element -- the gather is bound by exactly those
+// LDS bytes, this form by its vector instructions.  The price is a halo: the r
+// outermost parents on every side of a tile of 16 x TH lanes do not complete their
+// cells (they lack neighbours), so a tile delivers (16 - 2r) x (TH - 2r) cells and
+// neighbouring tiles overlap.  Deterministic: fixed order, no atomics.
+template <typename F, int... I>
+__device__ __forceinline__ void lg_static_for_impl(F &&f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+    lg_static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+template <int SH>   // lane L receives v of lane L + SH of its row of 16 lanes (0 where there is none)
+__device__ __forceinline__ float row_shift(float v) {
+    union { float f; int i; } x, y;
+    x.f = v;
+    y.i = __builtin_amdgcn_mov_dpp(x.i, SH > 0 ? 0x100 + SH : 0x110 - SH, 0xf, 0xf, true);   // row_shl / row_shr
+    return y.f;
+}
+
+template <typename T, typename WT, int K, int NW, int CH>
+__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(3, 3)))
+lowgrad_shift_kernel(const T *__restrict__ hi, const WT *__restrict__ w, T *__restrict__ out, int C,
+                     int H, int W, int tiles_x, int tiles_y, int nblocks, int per_xcd, int cgroups,
+                     int cper) {
+    constexpr int S = 2, KK = K * K, R = (K - 1) / 2, NJ = S * S;
+    constexpr int TH = 4 * NW;                       // lane rows of a tile
+    constexpr int VX = 16 - 2 * R, VY = TH - 2 * R;  // cells a tile completes
+    constexpr int ROWS = TH + 2 * R;                 // exchange rows incl. an unwritten halo, so that
+    constexpr int PL = ROWS * 16;                    // every lane reads at constant distances
+    constexpr bool PACK = sizeof(T) == 2;
+    typedef typename std::conditional<PACK, unsigned, typename FVec<2>::type>::type Raw;   // one child row
+    typedef typename FVec<2>::type V2;
+
+    __shared__ float xbuf[2 * CH * K * PL];
+
+    const int logical = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
+    if (logical >= nblocks) return;
+    const int tx = logical % tiles_x;
+    const int ty = (logical / tiles_x) % tiles_y;
+    const int cg = (logical / (tiles_x * tiles_y)) % cgroups;
+    const int n = logical / (tiles_x * tiles_y * cgroups);
+    const int cbeg = cg * cper, cend = cbeg + cper < C ? cbeg + cper : C;
+
+    const int tid = threadIdx.x, lx = tid % 16, ly = tid / 16;
+    const int x = tx * VX - R + lx, y = ty * VY - R + ly;    // this lane's parent, and its cell
+    const bool inside = x >= 0 && x < W && y >= 0 && y < H;
+    const int hW = W * S;
+    const long hplane = (long)H * S * hW;
+
+    // the parent's weights; a parent outside the image has none
+    float wr[KK][NJ];
+    {
+        const WT *wp = w + (long)n * KK * hplane + (inside ? (long)(y * S) * hW + x * S : 0);
+#pragma unroll
+        for (int k = 0; k < KK; ++k)
+#pragma unroll
+            for (int cy = 0; cy < S; ++cy) {
+                const V2 v = load_wide<WT, S>(wp + (long)k * hplane + (long)cy * hW);
+#pragma unroll
+                for (int cx = 0; cx < S; ++cx) wr[k][cy * S + cx] = inside ? v[cx] : 0.f;
+            }
+    }
+
+    // the children: two rows of S elements per channel, through a descriptor over the
+    // image (offset 2^31 = outside: the hardware returns zeros); the channel travels as
+    // the scalar offset
+    const __amdgpu_buffer_rsrc_t hrsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(hi + (long)n * C * hplane), 0, (int)((long)C * hplane * (long)sizeof(T)), 0x00020000);
+    const unsigned off0 = inside ? (unsigned)((y * S) * hW + x * S) * (unsigned)sizeof(T) : 0x80000000u;
+    const unsigned off1 = inside ? off0 + (unsigned)hW * (unsigned)sizeof(T) : 0x80000000u;
+    const unsigned planeb = (unsigned)hplane * (unsigned)sizeof(T);
+#ifndef SAPA_LOWGRAD_SHIFT_PF
+#define SAPA_LOWGRAD_SHIFT_PF 1
+#endif
+    constexpr int PF = SAPA_LOWGRAD_SHIFT_PF;     // chunks in flight ahead of the one in work
+    auto issue = [&](Raw (&nxt)[CH][S], int c0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int ch = 0; ch < CH; ++ch) {
+            const bool ok = c0 + ch < cend;
+            const unsigned soff = (unsigned)(ok ? c0 + ch : 0) * planeb;
+            const unsigned o0 = ok ? off0 : 0x80000000u, o1 = ok ? off1 : 0x80000000u;
+            if constexpr (PACK) {
+                nxt[ch][0] = __builtin_amdgcn_raw_buffer_load_b32(hrsrc, o0, soff, 0);
+                nxt[ch][1] = __builtin_amdgcn_raw_buffer_load_b32(hrsrc, o1, soff, 0);
+            } else {
+                union { unsigned u __attribute__((ext_vector_type(2))); V2 f; } a, b;
+                a.u = __builtin_amdgcn_raw_buffer_load_b64(hrsrc, o0, soff, 0);
+                b.u = __builtin_amdgcn_raw_buffer_load_b64(hrsrc, o1, soff, 0);
+                nxt[ch][0] = a.f;
+                nxt[ch][1] = b.f;
+            }
+        }
+    };
+    auto widen = [&](Raw r) __attribute__((always_inline)) {
+        if constexpr (PACK) {
+            V2 h;
+            if constexpr (std::is_same<T, bf16_t>::value) {
+                h[0] = __builtin_bit_cast(float, r << 16);
+                h[1] = __builtin_bit_cast(float, r & 0xffff0000u);
+            } else {
+                union { unsigned u; T t[2]; } v;
+                v.u = r;
+                h[0] = (float)v.t[0];
+                h[1] = (float)v.t[1];
+            }
+            return h;
+        } else {
+            return r;
+        }
+    };
+
+    const bool live = lx >= R && lx < 16 - R && ly >= R && ly < TH - R && x < W && y < H;
+    const long lplane = (long)H * W;
+    T *op = out + (long)n * C * lplane + (live ? (long)y * W + x : 0);
+    float *const wrow = xbuf + (ly + R) * 16 + lx;          // where this lane writes
+    const float *const rrow = xbuf + (ly + 2 * R) * 16 + lx;   // row ly + 2r - ky holds what cell row ly gets for ky
+
+    // PF + 1 register sets take turns (the loop is unrolled by as many chunks, so that no
+    // load result is ever copied: a copy would wait for its load)
+    auto work = [&](const Raw (&cur)[CH][S], int c0, int parity) __attribute__((always_inline)) {
+        float *const wb = wrow + parity * (CH * K * PL);
+#pragma unroll
+        for (int ch = 0; ch < CH; ++ch) {
+            const V2 ha = widen(cur[ch][0]), hb = widen(cur[ch][1]);
+#pragma unroll
+            for (int ky = 0; ky < K; ++ky) {
+                float t[K];
+#pragma unroll
+                for (int kx = 0; kx < K; ++kx) {
+                    const int k = ky * K + kx;
+                    float v = wr[k][0] * ha[0];
+                    v = __builtin_fmaf(wr[k][1], ha[1], v);
+                    v = __builtin_fmaf(wr[k][2], hb[0], v);
+                    t[kx] = __builtin_fmaf(wr[k][3], hb[1], v);
+                }
+                // cell column L collects t[kx] of the parent R - kx lanes to its right
+                float sum = t[R];
+                static_for<R>([&](auto i) {
+                    constexpr int D = decltype(i)::value + 1;
+                    sum += row_shift<D>(t[R - D]);
+                    sum += row_shift<-D>(t[R + D]);
+                });
+                wb[(ch * K + ky) * PL] = sum;
+            }
+        }
+        __syncthreads();
+        const float *const rb = rrow + parity * (CH * K * PL);
+#pragma unroll
+        for (int ch = 0; ch < CH; ++ch) {
+            float acc = rb[(ch * K) * PL];
+#pragma unroll
+            for (int ky = 1; ky < K; ++ky) acc += rb[(ch * K + ky) * PL - ky * 16];
+            if (live && c0 + ch < cend) op[(long)(c0 + ch) * lplane] = (T)acc;
+        }
+    };
+    Raw sets[PF + 1][CH][S];
+    static_for<PF>([&](auto p) { issue(sets[decltype(p)::value], cbeg + decltype(p)::value * CH); });
+    int parity = 0;
+    for (int c0 = cbeg; c0 < cend; c0 += (PF + 1) * CH) {
+        static_for<PF + 1>([&](auto ui) {
+            constexpr int u = decltype(ui)::value;
+            // (past the last channel: offsets outside the descriptor, no branch around the loads)
+            issue(sets[(u + PF) % (PF + 1)], c0 + (u + PF) * CH);
+            if (c0 + u * CH < cend) {
+                work(sets[u], c0 + u * CH, parity);
+                parity ^= 1;
+            }
+        });
+    }
+}
+
+template <typename T, typename WT, int K, int NW, int CH>
+static hipError_t lowgrad_shift_launch(const void *hi, const void *w, void *out, int B, int C, int H, int W,
+                                       hipStream_t st) {
+    constexpr int R = (K - 1) / 2, VX = 16 - 2 * R, VY = 4 * NW - 2 * R;
+    const int tiles_x = (W + VX - 1) / VX, tiles_y = (H + VY - 1) / VY;
+    const long tiles = (long)tiles_x * tiles_y * B;
+    // the channels of a tile over several workgroups until the grid fills the chip a
+    // few times over (each re-reads the tile's weights)
+#ifndef SAPA_LOWGRAD_SHIFT_MINWG
+#define SAPA_LOWGRAD_SHIFT_MINWG 2048
+#endif
+    int cgroups = 1;
+    const int max_groups = C / (4 * CH) > 0 ? C / (4 * CH) : 1;
+    while (cgroups * 2 <= max_groups && tiles * cgroups < SAPA_LOWGRAD_SHIFT_MINWG) cgroups *= 2;
+    const int cper = ((C + cgroups - 1) / cgroups + CH - 1) / CH * CH;
+    const long nb = tiles * cgroups;
+    if (nb > (1L << 30)) return hipErrorNotSupported;
+    const int per_xcd = (int)((nb + 7) / 8);
+    hipLaunchKernelGGL((lowgrad_shift_kernel<T, WT, K, NW, CH>), dim3(per_xcd * 8), dim3(64 * NW), 0, st,
+                       (const T *)hi, (const WT *)w, (T *)out, C, H, W, tiles_x, tiles_y, (int)nb,
+                       per_xcd, cgroups, cper);
+    return hipGetLastError();
+}
+
 template <typename T, typename WT, int K, int S, int NWX, int NWY, int CH, int VEC>
 static hipError_t lowgrad_launch_geom(const void *hi, const void *w, void *out, int B, int C, int H, int W,
                        hipStream_t st) {
@@ -241,6 +453,31 @@ static hipError_t lowgrad_launch_t(const void *hi, const void *w, void *out, int
                                    int K, hipStream_t st) {
     // vector loads of s = 2 elements
     if ((uintptr_t)hi % (2 * sizeof(T)) || (uintptr_t)w % (2 * sizeof(WT))) return hipErrorNotSupported;
+#ifndef SAPA_LOWGRAD_SHIFT_OFF
+#ifndef SAPA_LOWGRAD_SHIFT_NW
+#define SAPA_LOWGRAD_SHIFT_NW 4
+#endif
+#ifndef SAPA_LOWGRAD_SHIFT_GAIN
+#define SAPA_LOWGRAD_SHIFT_GAIN 0.47
+#endif
+    {
+        // The lane-exchange form costs about half of the gather per lane and channel
+        // (measured), but its tiles deliver (16 - 2r) x (4 NW - 2r) cells for 64 NW
+        // lanes: it is taken where that still leaves it ahead.  It reads `hi` through
+        // a 32-bit buffer descriptor per image.
+        constexpr int NW = SAPA_LOWGRAD_SHIFT_NW;
+        const int R = (K - 1) / 2, vx = 16 - 2 * R, vy = 4 * NW - 2 * R;
+        const double lanes_shift = (double)((W + vx - 1) / vx) * ((H + vy - 1) / vy) * (64 * NW);
+        const bool wide = (W + 31) / 32 * 32 * 0.9 <= (W + 15) / 16 * 16;    // (the gather's choice of tile)
+        const int tw = wide ? 32 : 16;
+        const double lanes_gather = (double)((W + tw - 1) / tw) * ((H + 7) / 8) * (tw * 8);
+        if ((long)C * H * 2 * W * 2 * (long)sizeof(T) < (1L << 31) &&
+            lanes_gather >= SAPA_LOWGRAD_SHIFT_GAIN * lanes_shift) {
+            if (K == 3) return lowgrad_shift_launch<T, WT, 3, NW, 4>(hi, w, out, B, C, H, W, st);
+            return lowgrad_shift_launch<T, WT, 5, NW, 4>(hi, w, out, B, C, H, W, st);
+        }
+    }
+#endif
     if (K == 3) return lowgrad_launch_k<T, WT, 3, 2>(hi, w, out, B, C, H, W, st);
     // 4-element staging loads when the rows of hi allow it (the window starts
     // r * s = 4 pixels left of a tile, which keeps them aligned)
