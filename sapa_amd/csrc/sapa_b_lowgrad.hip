@@ -1,5 +1,6 @@
 // Gradient of the SAPA-B operators with respect to their low-res operand
-// (grad_key of qk, grad_value of av) as an LDS-tiled gather:
+// (grad_key of qk, grad_value of av): an LDS-tiled gather, and further down the
+// same sums with the products owned by the parents (lanes exchange partial sums):
 //
 //   out[n,c,y,x] = sum over window entries k = (ky,kx), i.e. over the parents
 //                  (py,px) = (y + r - ky, x + r - kx) that see cell (y,x) as
