@@ -267,11 +267,16 @@ def test_tiled_lowres_gradients_vs_oracle(coracle, shape):
         torch.testing.assert_close(out_v.cpu().double(), gv, rtol=1e-4, atol=2e-5)
 
 
-def test_tiled_lowres_gradient_integer_inputs_exact():
+# the first shape takes the gather, the others the lane-exchange form (several
+# tiles in x and y, ragged edges, channels not a multiple of the chunk)
+@pytest.mark.parametrize('shape', [(2, 10, 13, 37, 5), (2, 10, 24, 50, 5), (1, 7, 21, 70, 3), (1, 3, 12, 12, 5)],
+                         ids=['gather-13x37', 'shift-24x50', 'shift-21x70-k3', 'shift-12x12'])
+def test_tiled_lowres_gradient_integer_inputs_exact(shape):
     """Integer-valued inputs make every product and sum exact in fp32, so any
-    order of the atomic adds gives the same bits: an index error cannot hide."""
+    order of the sums gives the same bits: an index error cannot hide."""
     g = gen(151)
-    B, C, H, W, K, s = 2, 10, 13, 37, 5, 2
+    B, C, H, W, K = shape
+    s = 2
     attn = torch.randint(-3, 4, (B, K * K, H * s, W * s), generator=g).float()
     go = torch.randint(-3, 4, (B, C, H * s, W * s), generator=g).float()
     v = torch.zeros(B, C, H, W)
