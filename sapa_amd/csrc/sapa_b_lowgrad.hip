@@ -235,8 +235,10 @@ __device__ __forceinline__ float row_shift(float v) {
     return y.f;
 }
 
-template <typename T, typename WT, int K, int NW, int CH>
-__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(3, 3)))
+// NW waves of 16 x 4 lanes stacked in y, CH channels per chunk (one barrier per chunk),
+// register budget for WPE waves per SIMD
+template <typename T, typename WT, int K, int NW, int CH, int WPE>
+__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
 lowgrad_shift_kernel(const T *__restrict__ hi, const WT *__restrict__ w, T *__restrict__ out, int C,
                      int H, int W, int tiles_x, int tiles_y, int nblocks, int per_xcd, int cgroups,
                      int cper) {
@@ -387,7 +389,7 @@ lowgrad_shift_kernel(const T *__restrict__ hi, const WT *__restrict__ w, T *__re
     }
 }
 
-template <typename T, typename WT, int K, int NW, int CH>
+template <typename T, typename WT, int K, int NW, int CH, int WPE>
 static hipError_t lowgrad_shift_launch(const void *hi, const void *w, void *out, int B, int C, int H, int W,
                                        hipStream_t st) {
     constexpr int R = (K - 1) / 2, VX = 16 - 2 * R, VY = 4 * NW - 2 * R;
@@ -405,7 +407,7 @@ static hipError_t lowgrad_shift_launch(const void *hi, const void *w, void *out,
     const long nb = tiles * cgroups;
     if (nb > (1L << 30)) return hipErrorNotSupported;
     const int per_xcd = (int)((nb + 7) / 8);
-    hipLaunchKernelGGL((lowgrad_shift_kernel<T, WT, K, NW, CH>), dim3(per_xcd * 8), dim3(64 * NW), 0, st,
+    hipLaunchKernelGGL((lowgrad_shift_kernel<T, WT, K, NW, CH, WPE>), dim3(per_xcd * 8), dim3(64 * NW), 0, st,
                        (const T *)hi, (const WT *)w, (T *)out, C, H, W, tiles_x, tiles_y, (int)nb,
                        per_xcd, cgroups, cper);
     return hipGetLastError();
@@ -455,9 +457,6 @@ static hipError_t lowgrad_launch_t(const void *hi, const void *w, void *out, int
     // vector loads of s = 2 elements
     if ((uintptr_t)hi % (2 * sizeof(T)) || (uintptr_t)w % (2 * sizeof(WT))) return hipErrorNotSupported;
 #ifndef SAPA_LOWGRAD_SHIFT_OFF
-#ifndef SAPA_LOWGRAD_SHIFT_NW
-#define SAPA_LOWGRAD_SHIFT_NW 4
-#endif
 #ifndef SAPA_LOWGRAD_SHIFT_GAIN
 #define SAPA_LOWGRAD_SHIFT_GAIN 0.47
 #endif
@@ -465,8 +464,11 @@ static hipError_t lowgrad_launch_t(const void *hi, const void *w, void *out, int
         // The lane-exchange form costs about half of the gather per lane and channel
         // (measured), but its tiles deliver (16 - 2r) x (4 NW - 2r) cells for 64 NW
         // lanes: it is taken where that still leaves it ahead.  It reads `hi` through
-        // a 32-bit buffer descriptor per image.
-        constexpr int NW = SAPA_LOWGRAD_SHIFT_NW;
+        // a 32-bit buffer descriptor per image.  16-bit tensors need fewer registers
+        // for their children: four waves per SIMD, hence taller tiles (8 waves, two
+        // workgroups per CU) with chunks of 2 channels; fp32: 4 waves, 4 channels, three
+        // waves per SIMD (at four it spills).
+        constexpr int NW = sizeof(T) == 2 ? 8 : 4, CH = sizeof(T) == 2 ? 2 : 4, WPE = sizeof(T) == 2 ? 4 : 3;
         const int R = (K - 1) / 2, vx = 16 - 2 * R, vy = 4 * NW - 2 * R;
         const double lanes_shift = (double)((W + vx - 1) / vx) * ((H + vy - 1) / vy) * (64 * NW);
         const bool wide = (W + 31) / 32 * 32 * 0.9 <= (W + 15) / 16 * 16;    // (the gather's choice of tile)
@@ -474,8 +476,8 @@ static hipError_t lowgrad_launch_t(const void *hi, const void *w, void *out, int
         const double lanes_gather = (double)((W + tw - 1) / tw) * ((H + 7) / 8) * (tw * 8);
         if ((long)C * H * 2 * W * 2 * (long)sizeof(T) < (1L << 31) &&
             lanes_gather >= SAPA_LOWGRAD_SHIFT_GAIN * lanes_shift) {
-            if (K == 3) return lowgrad_shift_launch<T, WT, 3, NW, 4>(hi, w, out, B, C, H, W, st);
-            return lowgrad_shift_launch<T, WT, 5, NW, 4>(hi, w, out, B, C, H, W, st);
+            if (K == 3) return lowgrad_shift_launch<T, WT, 3, NW, CH, WPE>(hi, w, out, B, C, H, W, st);
+            return lowgrad_shift_launch<T, WT, 5, NW, CH, WPE>(hi, w, out, B, C, H, W, st);
         }
     }
 #endif
