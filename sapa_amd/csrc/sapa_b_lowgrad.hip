@@ -227,6 +227,14 @@ __device__ __forceinline__ void static_for(F &&f) {
     lg_static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
+// lane L receives v of lane L + 1 of the wave (0 for the last lane)
+__device__ __forceinline__ float wave_shift_left(float v) {
+    union { float f; int i; } x, y;
+    x.f = v;
+    y.i = __builtin_amdgcn_mov_dpp(x.i, 0x130, 0xf, 0xf, true);   // wave_shl:1
+    return y.f;
+}
+
 template <int SH>   // lane L receives v of lane L + SH of its row of 16 lanes (0 where there is none)
 __device__ __forceinline__ float row_shift(float v) {
     union { float f; int i; } x, y;
@@ -235,18 +243,20 @@ __device__ __forceinline__ float row_shift(float v) {
     return y.f;
 }
 
-// NW waves of 16 x 4 lanes stacked in y, CH channels per chunk (one barrier per chunk),
+// NW waves of RW x (64 / RW) lanes stacked in y (RW = 16: sums over kx by row shifts;
+// RW = 32: by wave shifts, see below), CH channels per chunk (one barrier per chunk),
 // register budget for WPE waves per SIMD
-template <typename T, typename WT, int K, int NW, int CH, int WPE>
+template <typename T, typename WT, int K, int NW, int CH, int WPE, int RW>
 __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
 lowgrad_shift_kernel(const T *__restrict__ hi, const WT *__restrict__ w, T *__restrict__ out, int C,
                      int H, int W, int tiles_x, int tiles_y, int nblocks, int per_xcd, int cgroups,
                      int cper) {
     constexpr int S = 2, KK = K * K, R = (K - 1) / 2, NJ = S * S;
-    constexpr int TH = 4 * NW;                       // lane rows of a tile
-    constexpr int VX = 16 - 2 * R, VY = TH - 2 * R;  // cells a tile completes
+    constexpr int TH = 64 / RW * NW;                 // lane rows of a tile
+    constexpr int VX = RW - 2 * R, VY = TH - 2 * R;  // cells a tile completes
     constexpr int ROWS = TH + 2 * R;                 // exchange rows incl. an unwritten halo, so that
-    constexpr int PL = ROWS * 16;                    // every lane reads at constant distances
+    constexpr int PL = ROWS * RW + 2 * R;            // every lane reads at constant distances
+    static_assert(RW == 16 || RW == 32 || RW == 64, "a wave is whole rows of lanes");
     constexpr bool PACK = sizeof(T) == 2;
     typedef typename std::conditional<PACK, unsigned, typename FVec<2>::type>::type Raw;   // one child row
     typedef typename FVec<2>::type V2;
@@ -261,7 +271,7 @@ lowgrad_shift_kernel(const T *__restrict__ hi, const WT *__restrict__ w, T *__re
     const int n = logical / (tiles_x * tiles_y * cgroups);
     const int cbeg = cg * cper, cend = cbeg + cper < C ? cbeg + cper : C;
 
-    const int tid = threadIdx.x, lx = tid % 16, ly = tid / 16;
+    const int tid = threadIdx.x, lx = tid % RW, ly = tid / RW;
     const int x = tx * VX - R + lx, y = ty * VY - R + ly;    // this lane's parent, and its cell
     const bool inside = x >= 0 && x < W && y >= 0 && y < H;
     const int hW = W * S;
@@ -329,11 +339,12 @@ lowgrad_shift_kernel(const T *__restrict__ hi, const WT *__restrict__ w, T *__re
         }
     };
 
-    const bool live = lx >= R && lx < 16 - R && ly >= R && ly < TH - R && x < W && y < H;
+    const bool live = lx >= R && lx < RW - R && ly >= R && ly < TH - R && x < W && y < H;
     const long lplane = (long)H * W;
     T *op = out + (long)n * C * lplane + (live ? (long)y * W + x : 0);
-    float *const wrow = xbuf + (ly + R) * 16 + lx;          // where this lane writes
-    const float *const rrow = xbuf + (ly + 2 * R) * 16 + lx;   // row ly + 2r - ky holds what cell row ly gets for ky
+    // where this lane writes (with wave shifts its sum belongs to the cell r lanes to its right)
+    float *const wrow = xbuf + (ly + R) * RW + lx + (RW == 16 ? 0 : R);
+    const float *const rrow = xbuf + (ly + 2 * R) * RW + lx;   // row ly + 2r - ky holds what cell row ly gets for ky
 
     // PF + 1 register sets take turns (the loop is unrolled by as many chunks, so that no
     // load result is ever copied: a copy would wait for its load)
@@ -354,12 +365,23 @@ lowgrad_shift_kernel(const T *__restrict__ hi, const WT *__restrict__ w, T *__re
                     t[kx] = __builtin_fmaf(wr[k][3], hb[1], v);
                 }
                 // cell column L collects t[kx] of the parent R - kx lanes to its right
-                float sum = t[R];
-                static_for<R>([&](auto i) {
-                    constexpr int D = decltype(i)::value + 1;
-                    sum += row_shift<D>(t[R - D]);
-                    sum += row_shift<-D>(t[R + D]);
-                });
+                float sum;
+                if constexpr (RW == 16) {
+                    sum = t[R];
+                    static_for<R>([&](auto i) {
+                        constexpr int D = decltype(i)::value + 1;
+                        sum += row_shift<D>(t[R - D]);
+                        sum += row_shift<-D>(t[R + D]);
+                    });
+                } else {
+                    // rows wider than a DPP row: the running sum moves one lane to the left
+                    // through the whole wave per step, sum[L] = t[0][L + K - 1] + ... +
+                    // t[K - 1][L], which is what cell L + r gets; the last 2r lanes of a row
+                    // pick up the next row's first ones and belong to the halo anyway
+                    sum = t[0];
+#pragma unroll
+                    for (int kx = 1; kx < K; ++kx) sum = wave_shift_left(sum) + t[kx];
+                }
                 wb[(ch * K + ky) * PL] = sum;
             }
         }
@@ -369,7 +391,7 @@ lowgrad_shift_kernel(const T *__restrict__ hi, const WT *__restrict__ w, T *__re
         for (int ch = 0; ch < CH; ++ch) {
             float acc = rb[(ch * K) * PL];
 #pragma unroll
-            for (int ky = 1; ky < K; ++ky) acc += rb[(ch * K + ky) * PL - ky * 16];
+            for (int ky = 1; ky < K; ++ky) acc += rb[(ch * K + ky) * PL - ky * RW];
             if (live && c0 + ch < cend) op[(long)(c0 + ch) * lplane] = (T)acc;
         }
     };
@@ -389,10 +411,10 @@ lowgrad_shift_kernel(const T *__restrict__ hi, const WT *__restrict__ w, T *__re
     }
 }
 
-template <typename T, typename WT, int K, int NW, int CH, int WPE>
+template <typename T, typename WT, int K, int NW, int CH, int WPE, int RW>
 static hipError_t lowgrad_shift_launch(const void *hi, const void *w, void *out, int B, int C, int H, int W,
                                        hipStream_t st) {
-    constexpr int R = (K - 1) / 2, VX = 16 - 2 * R, VY = 4 * NW - 2 * R;
+    constexpr int R = (K - 1) / 2, VX = RW - 2 * R, VY = 64 / RW * NW - 2 * R;
     const int tiles_x = (W + VX - 1) / VX, tiles_y = (H + VY - 1) / VY;
     const long tiles = (long)tiles_x * tiles_y * B;
     // the channels of a tile over several workgroups until the grid fills the chip a
@@ -407,7 +429,7 @@ static hipError_t lowgrad_shift_launch(const void *hi, const void *w, void *out,
     const long nb = tiles * cgroups;
     if (nb > (1L << 30)) return hipErrorNotSupported;
     const int per_xcd = (int)((nb + 7) / 8);
-    hipLaunchKernelGGL((lowgrad_shift_kernel<T, WT, K, NW, CH, WPE>), dim3(per_xcd * 8), dim3(64 * NW), 0, st,
+    hipLaunchKernelGGL((lowgrad_shift_kernel<T, WT, K, NW, CH, WPE, RW>), dim3(per_xcd * 8), dim3(64 * NW), 0, st,
                        (const T *)hi, (const WT *)w, (T *)out, C, H, W, tiles_x, tiles_y, (int)nb,
                        per_xcd, cgroups, cper);
     return hipGetLastError();
@@ -462,22 +484,34 @@ static hipError_t lowgrad_launch_t(const void *hi, const void *w, void *out, int
 #endif
     {
         // The lane-exchange form costs about half of the gather per lane and channel
-        // (measured), but its tiles deliver (16 - 2r) x (4 NW - 2r) cells for 64 NW
+        // (measured), but its tiles deliver (RW - 2r) x (TH - 2r) cells for RW x TH
         // lanes: it is taken where that still leaves it ahead.  It reads `hi` through
         // a 32-bit buffer descriptor per image.  16-bit tensors need fewer registers
-        // for their children: four waves per SIMD, hence taller tiles (8 waves, two
-        // workgroups per CU) with chunks of 2 channels; fp32: 4 waves, 4 channels, three
-        // waves per SIMD (at four it spills).
-        constexpr int NW = sizeof(T) == 2 ? 8 : 4, CH = sizeof(T) == 2 ? 2 : 4, WPE = sizeof(T) == 2 ? 4 : 3;
-        const int R = (K - 1) / 2, vx = 16 - 2 * R, vy = 4 * NW - 2 * R;
-        const double lanes_shift = (double)((W + vx - 1) / vx) * ((H + vy - 1) / vy) * (64 * NW);
+        // for their children: four waves per SIMD, hence tiles of 8 waves (two
+        // workgroups per CU) with chunks of 2 channels, as 32 x 16 lanes (rows of whole
+        // cache lines) unless 16 x 32 wastes clearly fewer lanes on the shape; fp32:
+        // 4 waves of 16 x 4 lanes, 4 channels, three waves per SIMD (at four it spills).
+        constexpr bool H16 = sizeof(T) == 2;
+        constexpr int NW = H16 ? 8 : 4, CH = H16 ? 2 : 4, WPE = H16 ? 4 : 3;
+        const int R = (K - 1) / 2;
+        auto lanes = [&](int rw) {
+            const int vx = rw - 2 * R, vy = 64 / rw * NW - 2 * R;
+            return (double)((W + vx - 1) / vx) * ((H + vy - 1) / vy) * (64 * NW);
+        };
+        const bool rows32 = H16 && lanes(32) <= 1.1 * lanes(16);
+        const double lanes_shift = rows32 ? lanes(32) : lanes(16);
         const bool wide = (W + 31) / 32 * 32 * 0.9 <= (W + 15) / 16 * 16;    // (the gather's choice of tile)
         const int tw = wide ? 32 : 16;
         const double lanes_gather = (double)((W + tw - 1) / tw) * ((H + 7) / 8) * (tw * 8);
         if ((long)C * H * 2 * W * 2 * (long)sizeof(T) < (1L << 31) &&
             lanes_gather >= SAPA_LOWGRAD_SHIFT_GAIN * lanes_shift) {
-            if (K == 3) return lowgrad_shift_launch<T, WT, 3, NW, CH, WPE>(hi, w, out, B, C, H, W, st);
-            return lowgrad_shift_launch<T, WT, 5, NW, CH, WPE>(hi, w, out, B, C, H, W, st);
+            if constexpr (H16) {
+                if (rows32)
+                    return K == 3 ? lowgrad_shift_launch<T, WT, 3, NW, CH, WPE, 32>(hi, w, out, B, C, H, W, st)
+                                  : lowgrad_shift_launch<T, WT, 5, NW, CH, WPE, 32>(hi, w, out, B, C, H, W, st);
+            }
+            return K == 3 ? lowgrad_shift_launch<T, WT, 3, NW, CH, WPE, 16>(hi, w, out, B, C, H, W, st)
+                          : lowgrad_shift_launch<T, WT, 5, NW, CH, WPE, 16>(hi, w, out, B, C, H, W, st);
         }
     }
 #endif

@@ -315,6 +315,41 @@ def test_backward_16bit_tensors():
             assert_rel_rms_close(a.grad.float().cpu(), b.grad.cpu(), rel, str(dt))
 
 
+# 16-bit tensors take the lane-exchange form in rows of 32 lanes (30x70, 33x47 with
+# K = 3) or of 16 (25x42); each shape spans several tiles with ragged edges
+@pytest.mark.parametrize('shape', [(1, 6, 30, 70, 5), (2, 5, 25, 42, 5), (1, 5, 33, 47, 3)],
+                         ids=['rows32-30x70', 'rows16-25x42', 'rows32-33x47-k3'])
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+def test_lowres_gradients_16bit_integer_inputs_exact(shape, dtype):
+    """Small integers are exact in 16 bits, and so is every product and sum in the
+    kernels' fp32: grad_value of 16-bit tensors must equal the integer result bit for
+    bit whichever form and tile geometry serves the shape."""
+    g = gen(153)
+    B, C, H, W, K = shape
+    s = 2
+    attn = torch.randint(-2, 3, (B, K * K, H * s, W * s), generator=g).float()
+    go = torch.randint(-2, 3, (B, C, H * s, W * s), generator=g).float()
+    from sapa_amd import _lib
+    ad, god = attn.to(DEV).to(dtype), go.to(DEV).to(dtype)
+    vd = torch.zeros(B, C, H, W, device=DEV, dtype=dtype)
+    out = torch.full_like(vd, 9.0)
+    _lib.call('sapa_av_backward', vd.device, _lib.ptr(god), _lib.ptr(ad), _lib.ptr(vd), None, _lib.ptr(out),
+              B, C, H, W, K, s, _lib.DTYPES[dtype])
+    want = torch.zeros(B, C, H, W, dtype=torch.float64)
+    r = K // 2
+    a6 = attn.double().view(B, K, K, H, s, W, s)
+    g6 = go.double().view(B, C, H, s, W, s)
+    for ky in range(K):
+        for kx in range(K):
+            contrib = torch.einsum('bhiwj,bchiwj->bchw', a6[:, ky, kx], g6)   # per parent
+            dy, dx = ky - r, kx - r                                          # cell = parent + (dy, dx)
+            ys, xs = slice(max(0, -dy), H - max(0, dy)), slice(max(0, -dx), W - max(0, dx))
+            yd, xd = slice(max(0, dy), H + min(0, dy)), slice(max(0, dx), W + min(0, dx))
+            want[:, :, yd, xd] += contrib[:, :, ys, xs]
+    assert want.abs().max() < 256          # exactly representable in bf16 as well
+    assert torch.equal(out.double().cpu(), want)
+
+
 def _fused_backward_oracle(coracle, go, q, key, v, K, s):
     """float64 chain of the reference's backward (sapa/sapa/sapa_func.py:34-48,79-93
     under sapa_base.py:38-40): av backward, softmax backward, qk backward."""
