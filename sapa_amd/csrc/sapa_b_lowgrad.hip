@@ -297,7 +297,7 @@ lowgrad_shift_kernel(const T *__restrict__ hi, const WT *__restrict__ w, T *__re
     const __amdgpu_buffer_rsrc_t hrsrc = __builtin_amdgcn_make_buffer_rsrc(
         (void *)(hi + (long)n * C * hplane), 0, (int)((long)C * hplane * (long)sizeof(T)), 0x00020000);
     const unsigned off0 = inside ? (unsigned)((y * S) * hW + x * S) * (unsigned)sizeof(T) : 0x80000000u;
-    const unsigned off1 = inside ? off0 + (unsigned)hW * (unsigned)sizeof(T) : 0x80000000u;
+    const unsigned rowb = (unsigned)hW * (unsigned)sizeof(T);    // (outside + a row is still outside)
     const unsigned planeb = (unsigned)hplane * (unsigned)sizeof(T);
 #ifndef SAPA_LOWGRAD_SHIFT_PF
 #define SAPA_LOWGRAD_SHIFT_PF 1
@@ -308,7 +308,7 @@ lowgrad_shift_kernel(const T *__restrict__ hi, const WT *__restrict__ w, T *__re
         for (int ch = 0; ch < CH; ++ch) {
             const bool ok = c0 + ch < cend;
             const unsigned soff = (unsigned)(ok ? c0 + ch : 0) * planeb;
-            const unsigned o0 = ok ? off0 : 0x80000000u, o1 = ok ? off1 : 0x80000000u;
+            const unsigned o0 = ok ? off0 : 0x80000000u, o1 = o0 + rowb;
             if constexpr (PACK) {
                 nxt[ch][0] = __builtin_amdgcn_raw_buffer_load_b32(hrsrc, o0, soff, 0);
                 nxt[ch][1] = __builtin_amdgcn_raw_buffer_load_b32(hrsrc, o1, soff, 0);
@@ -341,7 +341,12 @@ lowgrad_shift_kernel(const T *__restrict__ hi, const WT *__restrict__ w, T *__re
 
     const bool live = lx >= R && lx < RW - R && ly >= R && ly < TH - R && x < W && y < H;
     const long lplane = (long)H * W;
-    T *op = out + (long)n * C * lplane + (live ? (long)y * W + x : 0);
+    // results leave through a descriptor over the image's output planes: a lane without a
+    // cell of its own carries an offset outside it and the hardware drops its store
+    const __amdgpu_buffer_rsrc_t orsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(out + (long)n * C * lplane), 0, (int)((long)C * lplane * (long)sizeof(T)), 0x00020000);
+    const unsigned ooff = live ? (unsigned)(y * W + x) * (unsigned)sizeof(T) : 0x80000000u;
+    const unsigned lplaneb = (unsigned)lplane * (unsigned)sizeof(T);
     // where this lane writes (with wave shifts its sum belongs to the cell r lanes to its right)
     float *const wrow = xbuf + (ly + R) * RW + lx + (RW == 16 ? 0 : R);
     const float *const rrow = xbuf + (ly + 2 * R) * RW + lx;   // row ly + 2r - ky holds what cell row ly gets for ky
@@ -392,7 +397,15 @@ lowgrad_shift_kernel(const T *__restrict__ hi, const WT *__restrict__ w, T *__re
             float acc = rb[(ch * K) * PL];
 #pragma unroll
             for (int ky = 1; ky < K; ++ky) acc += rb[(ch * K + ky) * PL - ky * RW];
-            if (live && c0 + ch < cend) op[(long)(c0 + ch) * lplane] = (T)acc;
+            if (c0 + ch < cend) {
+                const unsigned soff = (unsigned)(c0 + ch) * lplaneb;
+                if constexpr (PACK) {
+                    const T r = (T)acc;
+                    __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, r), orsrc, ooff, soff, 0);
+                } else {
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, acc), orsrc, ooff, soff, 0);
+                }
+            }
         }
     };
     Raw sets[PF + 1][CH][S];
@@ -486,30 +499,26 @@ static hipError_t lowgrad_launch_t(const void *hi, const void *w, void *out, int
         // The lane-exchange form costs about half of the gather per lane and channel
         // (measured), but its tiles deliver (RW - 2r) x (TH - 2r) cells for RW x TH
         // lanes: it is taken where that still leaves it ahead.  It reads `hi` through
-        // a 32-bit buffer descriptor per image.  16-bit tensors need fewer registers
-        // for their children: four waves per SIMD, hence tiles of 8 waves (two
-        // workgroups per CU) with chunks of 2 channels, as 32 x 16 lanes (rows of whole
-        // cache lines) unless 16 x 32 wastes clearly fewer lanes on the shape; fp32:
-        // 4 waves of 16 x 4 lanes, 4 channels, three waves per SIMD (at four it spills).
-        constexpr bool H16 = sizeof(T) == 2;
-        constexpr int NW = H16 ? 8 : 4, CH = H16 ? 2 : 4, WPE = H16 ? 4 : 3;
+        // a 32-bit buffer descriptor per image.  Tiles of 8 waves with chunks of 2
+        // channels keep it within 128 registers (four waves per SIMD, two workgroups per
+        // CU), as 32 x 16 lanes (rows of whole cache lines) unless 16 x 32 wastes
+        // clearly fewer lanes on the shape.
+        constexpr int NW = 8, CH = 2, WPE = 4;
         const int R = (K - 1) / 2;
         auto lanes = [&](int rw) {
             const int vx = rw - 2 * R, vy = 64 / rw * NW - 2 * R;
             return (double)((W + vx - 1) / vx) * ((H + vy - 1) / vy) * (64 * NW);
         };
-        const bool rows32 = H16 && lanes(32) <= 1.1 * lanes(16);
+        const bool rows32 = lanes(32) <= 1.1 * lanes(16);
         const double lanes_shift = rows32 ? lanes(32) : lanes(16);
         const bool wide = (W + 31) / 32 * 32 * 0.9 <= (W + 15) / 16 * 16;    // (the gather's choice of tile)
         const int tw = wide ? 32 : 16;
         const double lanes_gather = (double)((W + tw - 1) / tw) * ((H + 7) / 8) * (tw * 8);
         if ((long)C * H * 2 * W * 2 * (long)sizeof(T) < (1L << 31) &&
             lanes_gather >= SAPA_LOWGRAD_SHIFT_GAIN * lanes_shift) {
-            if constexpr (H16) {
-                if (rows32)
-                    return K == 3 ? lowgrad_shift_launch<T, WT, 3, NW, CH, WPE, 32>(hi, w, out, B, C, H, W, st)
-                                  : lowgrad_shift_launch<T, WT, 5, NW, CH, WPE, 32>(hi, w, out, B, C, H, W, st);
-            }
+            if (rows32)
+                return K == 3 ? lowgrad_shift_launch<T, WT, 3, NW, CH, WPE, 32>(hi, w, out, B, C, H, W, st)
+                              : lowgrad_shift_launch<T, WT, 5, NW, CH, WPE, 32>(hi, w, out, B, C, H, W, st);
             return K == 3 ? lowgrad_shift_launch<T, WT, 3, NW, CH, WPE, 16>(hi, w, out, B, C, H, W, st)
                           : lowgrad_shift_launch<T, WT, 5, NW, CH, WPE, 16>(hi, w, out, B, C, H, W, st);
         }
