@@ -54,6 +54,17 @@ def ulp_report(got, want):
     return ((got - want).abs() / sp).max().item()
 
 
+def fused_backward_oracle(coracle, go, q, key, v, K, s):
+    """float64 chain of the reference's backward (sapa/sapa/sapa_func.py:34-48,79-93
+    under sapa_base.py:38-40): av backward, softmax backward, qk backward."""
+    q, key, v, go = (t.double() for t in (q, key, v, go))
+    attn = torch.softmax(coracle.qk(q, key, K, s, 'f64'), dim=1)
+    ga, gv = coracle.av_backward(go, attn, v, K, s, 'f64')
+    gl = attn * (ga - (ga * attn).sum(dim=1, keepdim=True))
+    gq, gk = coracle.qk_backward(gl, q, key, K, s, 'f64')
+    return gq, gk, gv
+
+
 def deform_fused_backward_oracle(coracle, go, q, key, v, off, P, s, G):
     """deform_av_backward -> softmax backward -> deform_qk_backward in float64
     on the given values (the chain autograd runs for sapa_deform.py:51-53)."""

@@ -16,6 +16,9 @@ sapa_deform.py:51-53); the full batch goes through properties a wrong tile,
 channel slice or batch stride breaks: the batch result equals the per-image
 results bit for bit, a zero query gives the box filter, integer-valued inputs
 give exact logits and sums.  Contiguous and channels_last tensors both.
+The backward passes likewise: c3's low-res gradients on integer-valued tensors
+at the levels' own sizes, bit for bit; the fused backward of one image per
+level against the float64 chain, the batch against its images.
 
 Bars: fp32 |a-b| <= 1e-6 + 1e-5 |b| against the reference-order ('f32')
 oracle; bf16 |a-b| <= 1e-2 max(|b|, rms(b)) against the oracle with double
@@ -33,7 +36,7 @@ import torch.nn.functional as F
 
 import sapa_amd
 from helpers import (BF16_REL, F32_ATOL, F32_RTOL, assert_f32_close, assert_rel_rms_close,
-                     deform_fused_backward_oracle, gen, randn)
+                     deform_fused_backward_oracle, fused_backward_oracle, gen, randn)
 
 pytestmark = pytest.mark.gpu
 DEV = 'cuda:0'
@@ -190,6 +193,77 @@ def test_c3_full_batch_integer_inputs_exact(layout):
         vu = F.unfold(vd[sl].contiguous(), K, padding=K // 2).view(4, 256, K * K, H, W)
         want = torch.einsum('bckhw,bkhiwj->bchiwj', vu, ad[sl].contiguous().view(4, K * K, H, s, W, s))
         assert torch.equal(out[sl].contiguous(), want.reshape(4, 256, s * H, s * W))
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('H,W', C3_LEVELS)
+def test_c3_lowres_gradients_integer_inputs_exact(H, W, dtype):
+    """grad_value and grad_key at the FPN levels' own sizes (C = 256 / d = 64, four
+    images) with small integers in every tensor: products and sums are exact in the
+    kernels' fp32 and in the 16-bit result, whatever form, tile geometry and order
+    serve the shape, so they must equal the shifted sums of the per-parent products
+    (av_cuda_kernel.cu:128-145, qk_cuda_kernel.cu:120-135 written as 25 shifts) bit
+    for bit."""
+    B, K, s = 4, 5, 2
+    g = gen(335)
+    r = K // 2
+    from sapa_amd import _lib
+
+    def shifted_sums(w, hi):
+        C = hi.shape[1]
+        w6 = w.double().view(B, K, K, H, s, W, s)
+        h6 = hi.double().view(B, C, H, s, W, s)
+        want = torch.zeros(B, C, H, W, dtype=torch.float64, device=hi.device)
+        for ky in range(K):
+            for kx in range(K):
+                contrib = torch.einsum('bhiwj,bchiwj->bchw', w6[:, ky, kx], h6)   # per parent
+                dy, dx = ky - r, kx - r                                          # cell = parent + (dy, dx)
+                ys, xs = slice(max(0, -dy), H - max(0, dy)), slice(max(0, -dx), W - max(0, dx))
+                yd, xd = slice(max(0, dy), H + min(0, dy)), slice(max(0, dx), W + min(0, dx))
+                want[:, :, yd, xd] += contrib[:, :, ys, xs]
+        return want
+
+    for C, entry in ((256, 'sapa_av_backward'), (64, 'sapa_qk_backward')):
+        w = torch.randint(-2, 3, (B, K * K, s * H, s * W), generator=g).float().to(DEV)
+        hi = torch.randint(-2, 3, (B, C, s * H, s * W), generator=g).float().to(DEV)
+        want = shifted_sums(w, hi)
+        assert want.abs().max() < 256          # exact in bf16 as well
+        wd, hid = w.to(dtype), hi.to(dtype)
+        low = torch.zeros(B, C, H, W, device=DEV, dtype=dtype)
+        out = torch.full_like(low, 9.0)
+        if entry == 'sapa_av_backward':     # (grad_out, attn, value, grad_attn, grad_value)
+            _lib.call(entry, low.device, _lib.ptr(hid), _lib.ptr(wd), _lib.ptr(low), None, _lib.ptr(out),
+                      B, C, H, W, K, s, _lib.DTYPES[dtype])
+        else:                               # (grad_logits, query, key, grad_query, grad_key)
+            _lib.call(entry, low.device, _lib.ptr(wd), _lib.ptr(hid), _lib.ptr(low), None, _lib.ptr(out),
+                      B, C, H, W, K, s, _lib.DTYPES[dtype])
+        assert torch.equal(out.double(), want), f'{entry} {H}x{W} {dtype}'
+
+
+@pytest.mark.parametrize('H,W', C3_LEVELS)
+def test_c3_fused_backward_against_oracle(coracle, H, W):
+    """One image of each FPN level through sapa_fused(...).backward(): all
+    three gradients against the float64 chain of the reference's backward functions on
+    the same values; the full batch of the level equals its images bit for bit (the
+    kernels have no atomics).  Bar: |a - b| <= 1e-4 max(|b|, rms(b)) -- fp32 sums of up
+    to 6400 products against double sums."""
+    q, key, v = c3_inputs(4, H, W, 336)
+    go = randn(gen(337), 4, 256, 2 * H, 2 * W)
+
+    def grads(qi, ki, vi, gi):
+        ts = [t.clone().requires_grad_() for t in (qi, ki, vi)]
+        sapa_amd.sapa_fused(*ts, 5, 2).backward(gi)
+        return [t.grad for t in ts]
+
+    qd, kd, vd, god = dev(q, key, v, go)
+    full = grads(qd, kd, vd, god)
+    for i in (0, 3):
+        one = grads(qd[i:i + 1], kd[i:i + 1], vd[i:i + 1], god[i:i + 1])
+        for name, a, b in zip(('grad_query', 'grad_key', 'grad_value'), full, one):
+            assert torch.equal(a[i:i + 1], b), f'{name}: image {i} differs between batch and single call'
+    want = fused_backward_oracle(coracle, go[:1], q[:1], key[:1], v[:1], 5, 2)
+    for name, a, b in zip(('grad_query', 'grad_key', 'grad_value'), full, want):
+        assert_rel_rms_close(a[:1].cpu().double(), b, 1e-4, f'c3 {H}x{W} {name}')
 
 
 # ---------------------------------------------------------------- c2: SegFormer-style chain

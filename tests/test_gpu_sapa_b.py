@@ -10,7 +10,7 @@ import torch
 import torch.nn.functional as F
 
 import sapa_amd
-from helpers import (BF16_REL, F16_REL, assert_f32_close, assert_rel_rms_close, gen, golden,
+from helpers import (BF16_REL, F16_REL, assert_f32_close, assert_rel_rms_close, fused_backward_oracle, gen, golden,
                      randn, ulp_report)
 
 pytestmark = pytest.mark.gpu
@@ -350,17 +350,6 @@ def test_lowres_gradients_16bit_integer_inputs_exact(shape, dtype):
     assert torch.equal(out.double().cpu(), want)
 
 
-def _fused_backward_oracle(coracle, go, q, key, v, K, s):
-    """float64 chain of the reference's backward (sapa/sapa/sapa_func.py:34-48,79-93
-    under sapa_base.py:38-40): av backward, softmax backward, qk backward."""
-    q, key, v, go = (t.double() for t in (q, key, v, go))
-    attn = torch.softmax(coracle.qk(q, key, K, s, 'f64'), dim=1)
-    ga, gv = coracle.av_backward(go, attn, v, K, s, 'f64')
-    gl = attn * (ga - (ga * attn).sum(dim=1, keepdim=True))
-    gq, gk = coracle.qk_backward(gl, q, key, K, s, 'f64')
-    return gq, gk, gv
-
-
 @pytest.mark.parametrize('dtype,tol', [(torch.float32, dict(rtol=1e-4, atol=1e-5)),
                                         (torch.bfloat16, 1.5e-2), (torch.float16, 2e-3)])
 def test_fused_backward_entry_point(coracle, dtype, tol):
@@ -380,7 +369,7 @@ def test_fused_backward_entry_point(coracle, dtype, tol):
     args = (B, d, C, H, W, K, s, _lib.DTYPES[dtype])
     assert _lib.call_status('sapa_fused_backward', DEV, _lib.ptr(god), _lib.ptr(qd), _lib.ptr(kd), _lib.ptr(vd),
                             _lib.ptr(ws), _lib.ptr(gq), _lib.ptr(gk), _lib.ptr(gv), *args) == 0
-    want = _fused_backward_oracle(coracle, go.float(), q.float(), key.float(), v.float(), K, s)
+    want = fused_backward_oracle(coracle, go.float(), q.float(), key.float(), v.float(), K, s)
     for got, w, name in zip((gq, gk, gv), want, ('grad_query', 'grad_key', 'grad_value')):
         assert torch.isfinite(got).all(), name
         if dtype == torch.float32:
