@@ -243,6 +243,9 @@ def main():
     ap.add_argument('--steps', type=int, default=200)
     # the GPU's clocks take ~50 ms of work to settle: warm up for about that long
     ap.add_argument('--warmup', type=int, default=200)
+    ap.add_argument('--recompute-attention', action='store_true',
+                    help="--pass train, SAPA-B: the backward pass recomputes the attention weights "
+                         'instead of taking the fp32 ones the forward pass keeps by default')
     ap.add_argument('--dtype', default='fp32', choices=['fp32', 'bf16'])
     ap.add_argument('--workload', default='fpn_large',
                     choices=sorted(WORKLOADS) + sorted(DEFORM_WORKLOADS))
@@ -363,7 +366,7 @@ def main():
                 torch.autograd.grad(y, leaves, go)
         else:
             def step():
-                y = sapa_amd.sapa_fused(q, key, v, K, s)
+                y = sapa_amd.sapa_fused(q, key, v, K, s, save_attention=not args.recompute_attention)
                 torch.autograd.grad(y, leaves, go)
 
     settle = {'ms': args.settle_ms, 'launches': 0}

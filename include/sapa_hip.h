@@ -149,6 +149,27 @@ int sapa_fused_backward(const void *grad_out, const void *query, const void *key
                         void *grad_key, void *grad_value, int B, int d, int C,
                         int H, int W, int K, int s, int dtype, void *stream);
 
+/* The same pair for a training step that keeps the attention weights between its
+ * two passes, as the reference does (QKFunction / AVFunction save their operands,
+ * sapa/sapa/sapa_func.py:28,73, and autograd keeps the softmax output):
+ * sapa_fused_forward_attn writes attn [B,K*K,sH,sW] -- fp32 whatever `dtype` is --
+ * next to out (two launches: the weights, then the aggregation with them; nothing
+ * between them is rounded to 16 bits), and sapa_fused_backward_attn takes that
+ * tensor instead of recomputing it; its workspace holds grad_logits only
+ * (sapa_fused_backward_attn_workspace bytes, half of the other's).  Same results
+ * as sapa_fused_backward on the same operands, one launch less per step and a
+ * faster one in the forward pass of 16-bit tensors; the price is the attn tensor
+ * kept alive.  Same SAPA_ERR_UNSUPPORTED cases. */
+int sapa_fused_forward_attn(const void *query, const void *key, const void *value,
+                            void *attn, void *out, int B, int d, int C, int H, int W,
+                            int K, int s, int dtype, void *stream);
+long long sapa_fused_backward_attn_workspace(int B, int H, int W, int K, int s);
+int sapa_fused_backward_attn(const void *grad_out, const void *query, const void *key,
+                             const void *value, const void *attn, void *workspace,
+                             void *grad_query, void *grad_key, void *grad_value, int B,
+                             int d, int C, int H, int W, int K, int s, int dtype,
+                             void *stream);
+
 /* Softmax over the middle axis of x [N,R,M] -> y [N,R,M] (max-subtracted,
  * fp32 arithmetic for 16-bit types).  Covers the reference's
  * F.softmax(logits, dim=1) on [B,K*K,sH,sW] (sapa_base.py:39: N=B, R=K*K,

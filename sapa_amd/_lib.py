@@ -34,6 +34,8 @@ SIGNATURES = {
     'sapa_qk_softmax_forward': [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_av_backward_logits': [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_fused_backward': [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
+    'sapa_fused_forward_attn': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
+    'sapa_fused_backward_attn': [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_qk_forward_nhwc': [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_qk_softmax_forward_nhwc': [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_av_forward_nhwc': [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
@@ -92,6 +94,8 @@ def lib():
         handle.sapa_channel_moments_workspace.argtypes = [_i, _i, _ll, _i]
         handle.sapa_fused_backward_workspace.restype = _ll
         handle.sapa_fused_backward_workspace.argtypes = [_i, _i, _i, _i, _i]
+        handle.sapa_fused_backward_attn_workspace.restype = _ll
+        handle.sapa_fused_backward_attn_workspace.argtypes = [_i, _i, _i, _i, _i]
         handle.sapa_deform_fused_forward_workspace.restype = _ll
         handle.sapa_deform_fused_forward_workspace.argtypes = [_i] * 9
         handle.sapa_deform_fused_backward_workspace.restype = _ll

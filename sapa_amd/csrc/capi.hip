@@ -271,17 +271,21 @@ long long sapa_fused_backward_workspace(int B, int H, int W, int K, int s) {
     return 2LL * B * K * K * H * s * W * s * (long long)sizeof(float);
 }
 
-int sapa_fused_backward(const void *grad_out, const void *query, const void *key, const void *value,
-                        void *workspace, void *grad_query, void *grad_key, void *grad_value, int B,
-                        int d, int C, int H, int W, int K, int s, int dtype, void *stream) {
+// The chain behind sapa_fused_backward / sapa_fused_backward_attn: `attn_given` = the
+// fp32 weights kept by sapa_fused_forward_attn, or NULL to recompute them into the
+// first half of the workspace.
+static int fused_backward_impl(const void *grad_out, const void *query, const void *key, const void *value,
+                               const float *attn_given, void *workspace, void *grad_query, void *grad_key,
+                               void *grad_value, int B, int d, int C, int H, int W, int K, int s, int dtype,
+                               void *stream) {
     const int rc = check_window_args(B, d, C, H, W, K, s, dtype);
     if (rc != SAPA_OK) return rc;
     if (dtype == SAPA_F64 || K != 5 || s != 2) return SAPA_ERR_UNSUPPORTED;
     if (B == 0) return SAPA_OK;
     if (!grad_out || !query || !key || !value || !workspace) return SAPA_ERR_INVALID_ARGUMENT;
     hipStream_t st = (hipStream_t)stream;
-    float *attn = (float *)workspace;
-    float *grad_logits = attn + (long long)B * K * K * H * s * W * s;
+    float *grad_logits = (float *)workspace + (attn_given ? 0LL : (long long)B * K * K * H * s * W * s);
+    const float *attn = attn_given ? attn_given : (const float *)workspace;
     // every stage on the LDS-tiled kernels with fp32 K*K tensors; a stage they do
     // not cover ends the call before anything the caller keeps has been written
     // by a later stage (the caller recomputes everything on its own path)
@@ -300,7 +304,7 @@ int sapa_fused_backward(const void *grad_out, const void *query, const void *key
             e = sapa_b_tiled_launch(mode, qq, kk, attn_in, nullptr, res, B, ch, 0, H, W, K, s, dtype, st, true);
         return e;
     };
-    SAPA_STAGE(similarity(TILED_QK_SOFTMAX, query, key, nullptr, attn, d));
+    if (!attn_given) SAPA_STAGE(similarity(TILED_QK_SOFTMAX, query, key, nullptr, workspace, d));
     if (grad_value)
         SAPA_STAGE(lowres_grad_tiled_launch(grad_out, attn, grad_value, B, C, H, W, K, s, dtype, st, true));
     if (grad_query || grad_key) {
@@ -312,9 +316,51 @@ int sapa_fused_backward(const void *grad_out, const void *query, const void *key
             SAPA_STAGE(lowres_grad_tiled_launch(query, grad_logits, grad_key, B, d, H, W, K, s, dtype, st,
                                                 true));
     }
-#undef SAPA_STAGE
     return SAPA_OK;
 }
+
+int sapa_fused_backward(const void *grad_out, const void *query, const void *key, const void *value,
+                        void *workspace, void *grad_query, void *grad_key, void *grad_value, int B,
+                        int d, int C, int H, int W, int K, int s, int dtype, void *stream) {
+    return fused_backward_impl(grad_out, query, key, value, nullptr, workspace, grad_query, grad_key,
+                               grad_value, B, d, C, H, W, K, s, dtype, stream);
+}
+
+int sapa_fused_forward_attn(const void *query, const void *key, const void *value, void *attn,
+                            void *out, int B, int d, int C, int H, int W, int K, int s, int dtype,
+                            void *stream) {
+    const int rc = check_window_args(B, d, C, H, W, K, s, dtype);
+    if (rc != SAPA_OK) return rc;
+    if (dtype == SAPA_F64 || K != 5 || s != 2) return SAPA_ERR_UNSUPPORTED;
+    if (B == 0) return SAPA_OK;
+    if (!query || !key || !value || !attn || !out) return SAPA_ERR_INVALID_ARGUMENT;
+    hipStream_t st = (hipStream_t)stream;
+    // the weights once, in fp32, then the aggregation with them: the two launches of
+    // the separate operators, without a 16-bit rounding between them
+    hipError_t e = sapa_b_dot2_launch(TILED_QK_SOFTMAX, query, key, nullptr, nullptr, attn, B, d, 0, H, W, K, s,
+                                      dtype, st, true);
+    if (e == hipErrorNotSupported)
+        e = sapa_b_tiled_launch(TILED_QK_SOFTMAX, query, key, nullptr, nullptr, attn, B, d, 0, H, W, K, s, dtype,
+                                st, true);
+    SAPA_STAGE(e);
+    SAPA_STAGE(sapa_b_tiled_launch(TILED_AV, nullptr, nullptr, attn, value, out, B, 0, C, H, W, K, s, dtype, st,
+                                   true));
+    return SAPA_OK;
+}
+
+long long sapa_fused_backward_attn_workspace(int B, int H, int W, int K, int s) {
+    return sapa_fused_backward_workspace(B, H, W, K, s) / 2;
+}
+
+int sapa_fused_backward_attn(const void *grad_out, const void *query, const void *key, const void *value,
+                             const void *attn, void *workspace, void *grad_query, void *grad_key,
+                             void *grad_value, int B, int d, int C, int H, int W, int K, int s, int dtype,
+                             void *stream) {
+    if (!attn) return SAPA_ERR_INVALID_ARGUMENT;
+    return fused_backward_impl(grad_out, query, key, value, (const float *)attn, workspace, grad_query,
+                               grad_key, grad_value, B, d, C, H, W, K, s, dtype, stream);
+}
+#undef SAPA_STAGE
 
 int sapa_softmax_forward(const void *x, void *y, long long N, int R, long long M, int dtype,
                          void *stream) {

@@ -170,13 +170,27 @@ def qk_softmax(query, key, kernel_size, scale_factor):
     return _qk_softmax_forward(query, key, kernel_size, scale_factor, nhwc)
 
 
-def _fused_backward(grad_output, query, key, value, K, s, needs=(True, True, True)):
+def _fused_backward(grad_output, query, key, value, K, s, needs=(True, True, True), attn=None):
     """Gradients of av(softmax(qk(query, key)), value): the attention weights
-    are recomputed (one launch), then the three operators' gradients chain."""
+    are recomputed (one launch) unless the forward pass kept them (`attn`, fp32),
+    then the three operators' gradients chain."""
     need_q, need_k, need_v = needs
     query, key, value = query.contiguous(), key.contiguous(), value.contiguous()
     grad_output = grad_output.contiguous()
     _lib.require_cuda_contiguous(grad_output=grad_output, query=query, key=key, value=value)
+    if attn is not None:
+        n, c, h, w = value.size()
+        nbytes = _lib.lib().sapa_fused_backward_attn_workspace(n, h, w, K, s)
+        ws = torch.empty(max(nbytes // 4, 1), dtype=torch.float32, device=value.device)
+        grads = [_lib.new_out(t) if need else None
+                 for t, need in ((query, need_q), (key, need_k), (value, need_v))]
+        status = _lib.call_status('sapa_fused_backward_attn', value.device, _lib.ptr(grad_output),
+                                  _lib.ptr(query), _lib.ptr(key), _lib.ptr(value), _lib.ptr(attn), _lib.ptr(ws),
+                                  _lib.ptr(grads[0]), _lib.ptr(grads[1]), _lib.ptr(grads[2]), n, key.size(1),
+                                  c, h, w, K, s, _lib.dtype_code(value))
+        if status != _lib.UNSUPPORTED:
+            return tuple(grads)
+        del ws, grads
     # the whole chain in one library call where the tiled kernels cover it: 16-bit
     # tensors go in and out as they are, the [B,K*K,sH,sW] intermediates stay fp32
     n, c, h, w = value.size()
@@ -218,11 +232,20 @@ def _fused_backward(grad_output, query, key, value, K, s, needs=(True, True, Tru
     return grad_query, grad_key, grad_value
 
 
+# Training steps of sapa_fused keep the fp32 attention weights between the forward and
+# the backward pass (faster: one launch less per step) unless this is False or the call
+# says save_attention=False (less memory: the weights are recomputed).
+SAVE_ATTENTION = True
+
+
 class SAPAFusedFunction(Function):
     """av(softmax(qk(query, key), dim=1), value) -- SAPA.attention
-    (sapa_base.py:38-40) -- as one launch in the forward pass.  The backward
-    pass recomputes the attention weights (one launch) instead of keeping the
-    [B,K*K,sH,sW] tensor alive, then chains the three operators' gradients.
+    (sapa_base.py:38-40) -- as one launch in the forward pass.  When a gradient
+    is wanted and `save_attention` is set (the default, SAVE_ATTENTION), the
+    forward pass runs as two launches that leave the fp32 attention weights
+    [B,K*K,sH,sW] behind for the backward pass, as the reference's autograd graph
+    does; otherwise the backward pass recomputes them (one launch more, nothing
+    kept alive but the operands).  Then the three operators' gradients chain.
 
     query_bias [B, d] (optional): a per-image bias added to every query vector,
     i.e. the result for query + query_bias[:, :, None, None] -- what a 1x1
@@ -231,7 +254,7 @@ class SAPAFusedFunction(Function):
     form the sum."""
 
     @staticmethod
-    def forward(ctx, query, key, value, kernel_size, scale_factor, query_bias=None):
+    def forward(ctx, query, key, value, kernel_size, scale_factor, query_bias=None, save_attention=None):
         assert scale_factor >= 1
         assert query.size(0) == key.size(0) == value.size(0)
         assert query.size(1) == key.size(1)
@@ -250,13 +273,27 @@ class SAPAFusedFunction(Function):
         if query_bias is not None:
             assert query_bias.shape == (n, d) and query_bias.dtype == query.dtype
         ctx.has_bias = query_bias is not None
-        if query.requires_grad or key.requires_grad or value.requires_grad or \
-                (query_bias is not None and query_bias.requires_grad):
-            ctx.save_for_backward(*((query, key, value) + ((query_bias,) if ctx.has_bias else ())))
+        wants_grad = query.requires_grad or key.requires_grad or value.requires_grad or \
+            (query_bias is not None and query_bias.requires_grad)
+        saved = (query, key, value) + ((query_bias,) if ctx.has_bias else ())
+        ctx.has_attn = False
         if query_bias is not None and not nhwc:
             query = query + query_bias[:, :, None, None]
             query_bias = None
         output = _lib.new_out(value, (n, c, h * scale_factor, w * scale_factor), nhwc)
+        if wants_grad and not nhwc and (SAVE_ATTENTION if save_attention is None else save_attention):
+            attn = torch.empty((n, kernel_size * kernel_size, h * scale_factor, w * scale_factor),
+                               dtype=torch.float32, device=value.device)
+            status = _lib.call_status('sapa_fused_forward_attn', value.device, _lib.ptr(query), _lib.ptr(key),
+                                      _lib.ptr(value), _lib.ptr(attn), _lib.ptr(output), n, d, c, h, w,
+                                      kernel_size, scale_factor, _lib.dtype_code(value))
+            if status != _lib.UNSUPPORTED:
+                ctx.has_attn = True
+                ctx.save_for_backward(*(saved + (attn,)))
+                return output
+            del attn
+        if wants_grad:
+            ctx.save_for_backward(*saved)
         if query_bias is not None:
             query_bias = query_bias.contiguous()
             _lib.call_nhwc('sapa_fused_forward_nhwc_qbias', value.device, _lib.ptr(query), _lib.ptr(key),
@@ -279,12 +316,13 @@ class SAPAFusedFunction(Function):
             query = query + ctx.saved_tensors[3][:, :, None, None]
         grad_query, grad_key, grad_value = _fused_backward(
             grad_output, query, key, value, ctx.kernel_size, ctx.scale_factor,
-            (needs[0] or (ctx.has_bias and needs[5]), needs[1], needs[2]))
+            (needs[0] or (ctx.has_bias and needs[5]), needs[1], needs[2]),
+            attn=ctx.saved_tensors[-1] if ctx.has_attn else None)
         if ctx.has_bias and needs[5]:
             wide = torch.float32 if grad_query.dtype in (torch.float16, torch.bfloat16) else None
             grad_bias = grad_query.sum(dim=(2, 3), dtype=wide).to(grad_query.dtype)
-        return (grad_query if needs[0] else None), grad_key, grad_value, None, None, grad_bias
+        return (grad_query if needs[0] else None), grad_key, grad_value, None, None, grad_bias, None
 
 
-def sapa_fused(query, key, value, kernel_size, scale_factor, query_bias=None):
-    return SAPAFusedFunction.apply(query, key, value, kernel_size, scale_factor, query_bias)
+def sapa_fused(query, key, value, kernel_size, scale_factor, query_bias=None, save_attention=None):
+    return SAPAFusedFunction.apply(query, key, value, kernel_size, scale_factor, query_bias, save_attention)

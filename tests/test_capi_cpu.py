@@ -31,7 +31,8 @@ def test_library_exports_every_declared_symbol():
     # (the workspace query returns a size, not a status: bound separately)
     ops = [n for n in names if not n.startswith('sapa_hip_')
            and n not in ('sapa_channel_moments_workspace', 'sapa_channel_moments_static_capacity',
-                         'sapa_fused_backward_workspace', 'sapa_deform_fused_forward_workspace',
+                         'sapa_fused_backward_workspace', 'sapa_fused_backward_attn_workspace',
+                         'sapa_deform_fused_forward_workspace',
                          'sapa_deform_fused_backward_workspace')]
     assert sorted(ops) == sorted(_lib.SIGNATURES)
     h = _lib.lib()
@@ -39,6 +40,7 @@ def test_library_exports_every_declared_symbol():
     assert h.sapa_channel_moments_workspace(0, 256, 67200, 1) == 0
     assert h.sapa_channel_moments_static_capacity() == 8 << 20
     assert h.sapa_fused_backward_workspace(2, 10, 12, 5, 2) == 2 * 2 * 25 * 20 * 24 * 4
+    assert h.sapa_fused_backward_attn_workspace(2, 10, 12, 5, 2) == 2 * 25 * 20 * 24 * 4
     # key [8,128,64,64] + value [8,256,64,64] in bf16; fp32 with few points and fp64: not served
     assert h.sapa_deform_fused_forward_workspace(8, 128, 256, 64, 64, 25, 2, 4, _lib.DTYPES[torch.bfloat16]) == 8 * 4096 * (128 + 256) * 2
     assert h.sapa_deform_fused_forward_workspace(8, 128, 256, 64, 64, 5, 2, 4, _lib.DTYPES[torch.float32]) == 0

@@ -350,6 +350,37 @@ def test_lowres_gradients_16bit_integer_inputs_exact(shape, dtype):
     assert torch.equal(out.double().cpu(), want)
 
 
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16, torch.float16])
+def test_fused_training_step_keeps_attention(dtype):
+    """sapa_fused with gradients wanted: the forward pass that keeps the fp32 attention
+    weights (two launches) against the one-launch forward whose backward recomputes them:
+    the same gradients bit for bit (the kept weights are the recomputed ones), the same
+    output to the type's rounding; one more saved tensor, [B,K*K,sH,sW] fp32.  K = 3 is
+    not covered by the pair of entry points and silently takes the other path."""
+    g = gen(154)
+    for (B, d, C, H, W, K) in ((2, 16, 24, 13, 22, 5), (1, 8, 12, 9, 14, 3)):
+        s = 2
+        q, key, v = randn(g, B, d, H * s, W * s), randn(g, B, d, H, W), randn(g, B, C, H, W)
+        go = randn(g, B, C, H * s, W * s).to(DEV).to(dtype)
+        res = {}
+        for keep in (True, False):
+            saved = []
+            ts = [t.to(DEV).to(dtype).requires_grad_() for t in (q, key, v)]
+            with torch.autograd.graph.saved_tensors_hooks(lambda t: saved.append(tuple(t.shape)) or t, lambda t: t):
+                out = sapa_amd.sapa_fused(*ts, K, s, save_attention=keep)
+            out.backward(go)
+            res[keep] = (out.detach(), [t.grad for t in ts], saved)
+        kept = (B, K * K, H * s, W * s) in res[True][2]
+        assert kept == (K == 5) and (B, K * K, H * s, W * s) not in res[False][2]
+        for a, b in zip(res[True][1], res[False][1]):
+            assert torch.equal(a, b)
+        if dtype == torch.float32:
+            assert_f32_close(res[True][0], res[False][0], 'output with kept weights')
+        else:
+            assert_rel_rms_close(res[True][0].float(), res[False][0].float(), 2 ** -7 if dtype == torch.bfloat16 else 2 ** -10,
+                                 f'output with kept weights {dtype}')
+
+
 @pytest.mark.parametrize('dtype,tol', [(torch.float32, dict(rtol=1e-4, atol=1e-5)),
                                         (torch.bfloat16, 1.5e-2), (torch.float16, 2e-3)])
 def test_fused_backward_entry_point(coracle, dtype, tol):
