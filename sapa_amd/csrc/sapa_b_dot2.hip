@@ -371,14 +371,22 @@ sapa_b_dot2_kernel(const T *__restrict__ q, const T *__restrict__ key,
             return (float)__builtin_bit_cast(_Float16, (unsigned short)r);
         };
         const u32 *vbase = lds + ly * RSV + wcol / 2;
-        T *op = out + (long)n * C * hplane + hpix;
+        // The results leave through buffer stores whose descriptor covers exactly the
+        // channels of the chunk that exist: idle lanes (offset 2^31) and channels past
+        // the slice fall outside it and the hardware drops them.  No branch around a
+        // store, so the channel loop unrolls with a known number of stores behind the
+        // next chunk's staging loads, and the wait for those loads leaves this chunk's
+        // stores in flight.
+        const u32 ooff = active ? (u32)(hpix * 2) : 0x80000000u;
+        const u32 plane_bytes = (u32)(hplane * 2);
+        __amdgpu_buffer_rsrc_t orsrc;
         auto load_v = [&](const u32 *wc, u32 (&dst)[NPK]) {
 #pragma unroll
             for (int ky = 0; ky < K; ++ky)
 #pragma unroll
                 for (int p = 0; p < KP; ++p) dst[ky * KP + p] = wc[ky * RSV + p];
         };
-        auto channel = [&](int c, const u32 (&vv)[NPK]) {
+        auto channel = [&](int ch, const u32 (&vv)[NPK]) {
             float o[NJ];
 #pragma unroll
             for (int jj = 0; jj < NJ; ++jj) o[jj] = 0;
@@ -391,17 +399,19 @@ sapa_b_dot2_kernel(const T *__restrict__ q, const T *__restrict__ key,
 #pragma unroll
                     for (int jj = 0; jj < NJ; ++jj) o[jj] = fma_(v, a[jj][ky * K + kx], o[jj]);
                 }
-            if (active && c < cend) {
 #pragma unroll
-                for (int cy = 0; cy < S; ++cy)
-                    __builtin_nontemporal_store(pack2<T>(o[cy * S], o[cy * S + 1]),
-                                                (u32 *)(op + (long)c * hplane + (long)cy * hW));
-            }
+            for (int cy = 0; cy < S; ++cy)
+                __builtin_amdgcn_raw_buffer_store_b32(pack2<T>(o[cy * S], o[cy * S + 1]), orsrc,
+                                                      ooff + (u32)ch * plane_bytes + (u32)(cy * hW) * 2u, 0,
+                                                      2 /* non-temporal */);
         };
         for (int j = nKc; j < ntot; ++j) {
             if (j + 1 < ntot) stage_load(j + 1);
             const int c0 = cbeg + (j - nKc) * CHV;
             const u32 *wb = vbase + (j & 1) * BUF;
+            const int nleft = cend - c0 < CHV ? cend - c0 : CHV;
+            orsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(out + ((long)n * C + c0) * hplane), 0,
+                                                      (int)((u32)nleft * plane_bytes), 0x00020000);
             // two channels per trip: the next channel's words are read from
             // LDS while the current one is multiplied
             u32 va[NPK], vb[NPK];
@@ -409,10 +419,10 @@ sapa_b_dot2_kernel(const T *__restrict__ q, const T *__restrict__ key,
 #pragma unroll 1
             for (int ch = 0; ch < CHV; ch += 2) {
                 load_v(wb + (ch + 1) * PLV, vb);
-                channel(c0 + ch, va);
+                channel(ch, va);
                 __builtin_amdgcn_sched_barrier(0);
                 load_v(wb + (ch + 2 < CHV ? ch + 2 : ch) * PLV, va);
-                channel(c0 + ch + 1, vb);
+                channel(ch + 1, vb);
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (j + 1 < ntot) stage_store(j + 1);
