@@ -305,6 +305,39 @@ def test_c2_segformer_chain_module_and_operators(coracle):
             x = out
 
 
+@pytest.mark.parametrize('h', [16, 32, 64])
+def test_c2_segformer_stage_backward(coracle, h):
+    """One stage of the chain at its own size (B = 8, C = 256, d = 32, projections
+    ~N(0, .02) of GroupNorm-ed features): the gradients of the fused operator for query,
+    key and value -- batch equal to its images bit for bit, image 0 against the float64
+    chain of the reference's backward functions, |a - b| <= 1e-4 max(|b|, rms(b)) --
+    with the attention weights kept by the forward pass and recomputed (same bits)."""
+    B = 8
+    torch.manual_seed(3)
+    g = gen(201)
+    m = sapa_amd.SAPA(256, embedding_dim=32).to(DEV)
+    x, y = randn(g, B, 256, h, h).to(DEV), randn(g, B, 256, 2 * h, 2 * h).to(DEV)
+    go = randn(g, B, 256, 2 * h, 2 * h).to(DEV)
+    with torch.no_grad():
+        q, k = m.q(m.norm_y(y)).contiguous(), m.k(m.norm_x(x)).contiguous()
+
+    def grads(qi, ki, vi, gi, keep=True):
+        ts = [t.clone().requires_grad_() for t in (qi, ki, vi)]
+        sapa_amd.sapa_fused(*ts, 5, 2, save_attention=keep).backward(gi)
+        return [t.grad for t in ts]
+
+    full = grads(q, k, x, go)
+    for a, b in zip(full, grads(q, k, x, go, keep=False)):
+        assert torch.equal(a, b)
+    for i in (0, B - 1):
+        one = grads(q[i:i + 1], k[i:i + 1], x[i:i + 1], go[i:i + 1])
+        for name, a, b in zip(('grad_query', 'grad_key', 'grad_value'), full, one):
+            assert torch.equal(a[i:i + 1], b), f'c2 {h}: {name} of image {i} differs between batch and single call'
+    want = fused_backward_oracle(coracle, go[:1].cpu(), q[:1].cpu(), k[:1].cpu(), x[:1].cpu(), 5, 2)
+    for name, a, b in zip(('grad_query', 'grad_key', 'grad_value'), full, want):
+        assert_rel_rms_close(a[:1].cpu().double(), b, 1e-4, f'c2 {h}->{2 * h} {name}')
+
+
 # ---------------------------------------------------------------- c4: SAPA-D
 
 def c4_inputs(B, P, seed, G=4):
