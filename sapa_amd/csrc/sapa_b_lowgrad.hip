@@ -209,15 +209,16 @@ lowgrad_gather_kernel(const T *__restrict__ hi, const WT *__restrict__ w,
 //   t[ky][kx] = sum over children j of w[(ky,kx)][j] * hi[j]      (K*K*S*S FMAs)
 //
 // which is what this parent adds to cell (py - r + ky, px - r + kx).  The sum over
-// kx is an exchange between x-neighbours: a row of 16 lanes holds 16 consecutive
-// parents, and a DPP row shift hands t[ky][kx] of lane L + r - kx to lane L (K - 1
-// shifted adds per ky).  The sum over ky crosses lane rows and waves and goes through
-// LDS: K floats written and K read per lane and channel, against the K*K*S*S floats
-// the gather above reads per output element -- the gather is bound by exactly those
-// LDS bytes, this form by its vector instructions.  The price is a halo: the r
-// outermost parents on every side of a tile of 16 x TH lanes do not complete their
-// cells (they lack neighbours), so a tile delivers (16 - 2r) x (TH - 2r) cells and
-// neighbouring tiles overlap.  Deterministic: fixed order, no atomics.
+// kx is an exchange between x-neighbours: a row of RW lanes holds RW consecutive
+// parents, and DPP shifts hand t[ky][kx] of lane L + r - kx to lane L (K - 1 shifted
+// adds per ky: row shifts inside rows of 16 lanes, a running sum on wave shifts in
+// wider rows).  The sum over ky crosses lane rows and waves and goes through LDS:
+// K floats written and K read per lane and channel, against the K*K*S*S floats the
+// gather above reads per output element, which are what bounds the gather.  The
+// price is a halo: the r outermost parents on every side of a tile of RW x TH lanes
+// do not complete their cells (they lack neighbours), so a tile delivers
+// (RW - 2r) x (TH - 2r) cells and neighbouring tiles overlap.  Deterministic: fixed
+// order, no atomics.
 template <typename F, int... I>
 __device__ __forceinline__ void lg_static_for_impl(F &&f, std::integer_sequence<int, I...>) {
     (f(std::integral_constant<int, I>{}), ...);
