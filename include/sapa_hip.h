@@ -324,8 +324,8 @@ int sapa_deform_fused_forward_nhwc(const void *query, const void *key,
  * offset_layout as in sapa_deform_fused_forward_from below: the offsets are
  * read from the hi-res tensor or in place from the low-res convolution output.
  * Served: s in {1, 2, 4}, Cq / G (at most 64) and C / G multiples of 4, and
- * enough points for it to pay: 6 <= P <= 32 for SAPA_F16 / BF16 with Cq / G and
- * C / G multiples of 8, 15 <= P <= 32 otherwise (SAPA_F32 included).  The sums
+ * enough points for it to pay: 4 <= P <= 32 for SAPA_F16 / BF16 with Cq / G and
+ * C / G multiples of 8, 13 <= P <= 32 otherwise (SAPA_F32 included).  The sums
  * run per window cell instead of per point: fp32 results differ from
  * sapa_deform_fused_forward at rounding level (no further from the
  * double-precision result than it). */
@@ -405,7 +405,9 @@ int sapa_channel_moments(const void *x, void *workspace, float *mean_var,
  * sapa_channel_moments_workspace(B, C, HW, channels_last) exceeds the capacity.
  * All calls on one device share that array: calls that overlap in time on the
  * same device (different streams or host threads) race and must be serialised
- * by the caller. */
+ * by the caller.  The first call on each device looks the array's address up
+ * (hipGetSymbolAddress): make that call outside a stream capture; later calls
+ * only launch kernels and may be captured. */
 long long sapa_channel_moments_static_capacity(void);
 int sapa_channel_moments_static(const void *x, float *mean_var,
                                 int B, int C, long long HW, int channels_last,
@@ -434,6 +436,23 @@ int sapa_groupnorm_fold(const float *mean_var, const void *gamma, const void *be
  * SAPA_ERR_UNSUPPORTED otherwise. */
 int sapa_project_nhwc(const void *x, const void *weight, const void *bias, void *out,
                       int B, int C, int O, long long HW, int dtype, void *stream);
+
+/* ------------------------------------------------------------ calibration */
+
+/* A kernel that only moves bytes, for putting the operators' measured rates
+ * beside what the memory system gives a plain stream of the same read : write
+ * mix.  No counterpart in the reference (which has no measurement code).
+ * `units` workgroups; unit u reads the contiguous run
+ * src[u * reads * 4096 ... + reads * 4096) and writes the contiguous run
+ * dst[u * writes * 4096 ... + writes * 4096) (bytes), the written words being a
+ * function of the words read; writes = 0: src is only read (dst needs 4096
+ * bytes per unit and is left untouched unless a 16-byte group of src is
+ * ff..fe in every word).  nontemporal != 0: streaming loads and stores.
+ * (reads, writes) in {(9,16): a fused SAPA-B forward at up_factor 2 with
+ * C = 4 d, (18,32), (8,8), (0,16), (16,0)}; SAPA_ERR_UNSUPPORTED otherwise.
+ * Pointers aligned to 16 bytes. */
+int sapa_stream_mix(const void *src, void *dst, long long units, int reads, int writes,
+                    int nontemporal, void *stream);
 
 #ifdef __cplusplus
 }

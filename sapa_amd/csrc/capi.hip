@@ -690,4 +690,17 @@ int sapa_project_nhwc(const void *x, const void *weight, const void *bias, void 
     return finish(e);
 }
 
+int sapa_stream_mix(const void *src, void *dst, long long units, int reads, int writes,
+                    int nontemporal, void *stream) {
+    if (units < 0 || reads < 0 || writes < 0 || (reads == 0 && writes == 0)) return SAPA_ERR_INVALID_ARGUMENT;
+    if (units > (1LL << 30)) return SAPA_ERR_TOO_LARGE;
+    if (units == 0) return SAPA_OK;
+    if ((reads > 0 && !src) || !dst) return SAPA_ERR_INVALID_ARGUMENT;
+    if (((uintptr_t)src | (uintptr_t)dst) % 16 != 0) return SAPA_ERR_INVALID_ARGUMENT;
+    const hipError_t e = stream_mix_launch(src, dst, (long)units, reads, writes, nontemporal != 0,
+                                           (hipStream_t)stream);
+    if (e == hipErrorNotSupported) return SAPA_ERR_UNSUPPORTED;
+    return finish(e);
+}
+
 }  // extern "C"

@@ -123,12 +123,6 @@ __device__ __forceinline__ void halve(const float (&in)[N], float (&out)[(N + 1)
     }
 }
 
-// SAPA_NHWC_PROBE: timing builds that take the kernel apart (results are wrong):
-// bit 1 = no output stores, bit 2 = one tap instead of K*K in the aggregation
-// (the memory side alone: every load, staging pass, barrier and store stays)
-#ifndef SAPA_NHWC_PROBE
-#define SAPA_NHWC_PROBE 0
-#endif
 #ifdef SAPA_NHWC_WPE
 #define SAPA_NHWC_OCC __attribute__((amdgpu_waves_per_eu(SAPA_NHWC_WPE, SAPA_NHWC_WPE)))
 #else
@@ -377,7 +371,7 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
                 constexpr int t = decltype(it)::value;
                 ring[t] = *(const f32x4 *)(wb + ((t / K) * WW + t % K) * CHK);
             });
-            static_for<SAPA_NHWC_PROBE & 2 ? 1 : KK>([&](auto it) {
+            static_for<KK>([&](auto it) {
                 constexpr int t = decltype(it)::value, ky = t / K, kx = t % K, tn = t + AHEAD;
                 if (tn < KK)
                     ring[tn % (AHEAD + 1)] = *(const f32x4 *)(wb + ((tn / K) * WW + tn % K) * CHK);
@@ -397,9 +391,7 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
             // (one counter, no order between the two kinds), so the stores are
             // issued right after the wait and have a whole chunk to complete.
             if (j + 1 < ntot) stage_store(j + 1);
-            // (probe build, bit 1: the stores depend on a condition on the sums that
-            // never holds, so everything but the store stream stays)
-            if (active && c0 + 4 * li < C && (!(SAPA_NHWC_PROBE & 1) || acc[0][0][0] == 1.2345e30f)) {
+            if (active && c0 + 4 * li < C) {
 #pragma unroll
                 for (int jj = 0; jj < NJ; ++jj)
                     __builtin_nontemporal_store(

@@ -745,7 +745,14 @@ deform_fused_wmat_kernel(const T *__restrict__ q, const T *__restrict__ key,
             rs = fma_(fma_(-sum, rs, 1.f), rs, rs);
             const float att = e * rs;
             fatt[ps] = att;
-            if (in) {
+            // A non-finite logit anywhere in the pixel makes every weight of the pixel NaN
+            // (exp(inf - inf), NaN sums), which the integer entries of Wm cannot carry: such
+            // a point takes the per-sample path below, where its weight multiplies the sample
+            // in floating point, as the reference's attn * val does
+            // (deform_av_cuda_kernel.cu:185-190)
+            const bool nonfinite = live && t.guard && att != att;
+            if (nonfinite) fb[ps] = true;
+            if (in && !nonfinite) {
                 // Wm holds 2^30-scaled integers: every entry and every row sum is at
                 // most 1, integer adds are exact in any order (the result does not
                 // depend on which lane the LDS serves first) and run at the rate of

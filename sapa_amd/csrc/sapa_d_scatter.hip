@@ -40,12 +40,6 @@ namespace sapa {
 
 namespace dscat {
 
-// Timing builds (wrong results): 1 = no matrix products, 2 = no per-sample phase,
-// 4 = no final atomics, 8 = no loads after the first two steps
-#ifndef SAPA_SCAT_PROBE
-#define SAPA_SCAT_PROBE 0
-#endif
-
 typedef unsigned u32;
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
@@ -272,15 +266,14 @@ deform_scatter_mat_kernel(const T *__restrict__ hi, const TS *__restrict__ sc,
                 }
             }
         };
-        if (SAPA_SCAT_PROBE & 2) {
-        } else if (narrow) {
+        if (narrow) {
             sample(std::integral_constant<int, 16>{}, 0);
         } else {
             sample(std::integral_constant<int, 32>{}, 0);
             sample(std::integral_constant<int, 32>{}, 1);
         }
         // the loads of the step after the next go out (into the set this step has used up)
-        if (step + 2 < NSTEP && !(SAPA_SCAT_PROBE & 8)) {
+        if (step + 2 < NSTEP) {
             load_hi(step + 2, pre);
             load_samples(step + 2, pre);
         }
@@ -316,7 +309,7 @@ deform_scatter_mat_kernel(const T *__restrict__ hi, const TS *__restrict__ sc,
                 const int gy = wy0 + cell / WWR, gx = wx0 + cell % WWR;
                 const bool ok = cell < NPOS && gy >= 0 && gy < H && gx >= 0 && gx < W;
                 const float v = Tl[(8 * w8 + c) * TSC + lane];
-                if (ok && lane < cvalid && v != 0.f && !(SAPA_SCAT_PROBE & 4)) unsafeAtomicAdd(g0 + ((long)gy * W + gx) * Cx, v);
+                if (ok && lane < cvalid && v != 0.f) unsafeAtomicAdd(g0 + ((long)gy * W + gx) * Cx, v);
             }
         } else {
             // lane <-> cell 64 cbi + lane; this wave: channels 8 w8 .. + 7
@@ -327,7 +320,7 @@ deform_scatter_mat_kernel(const T *__restrict__ hi, const TS *__restrict__ sc,
 #pragma unroll 4
             for (int c = 0; c < 8; ++c) {
                 const float v = Tl[(8 * w8 + c) * TS_ + lane];
-                if (ok && 8 * w8 + c < cvalid && v != 0.f && !(SAPA_SCAT_PROBE & 4)) unsafeAtomicAdd(gp + c * lpix, v);
+                if (ok && 8 * w8 + c < cvalid && v != 0.f) unsafeAtomicAdd(gp + c * lpix, v);
             }
         }
     };
@@ -367,7 +360,7 @@ deform_scatter_mat_kernel(const T *__restrict__ hi, const TS *__restrict__ sc,
             int b0, b1, cb0, cb1;
             band(step, b0, b1, cb0, cb1);
 #pragma unroll
-            for (int ks = 0; ks < ((SAPA_SCAT_PROBE & 1) ? 0 : SPX / 4); ++ks) {
+            for (int ks = 0; ks < SPX / 4; ++ks) {
                 const float inv = invl[4 * ks + mk];
                 float b[CHK / 16];
 #pragma unroll

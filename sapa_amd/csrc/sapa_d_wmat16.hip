@@ -493,6 +493,11 @@ deform_fused_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key,
             const float e = pt < P ? exp_(lg - mx) : 0.f;
             const float att = e * __builtin_amdgcn_rcpf(reduce_lanes<false, NL>(e));
             fatt[ps] = att;
+            // a non-finite logit makes every weight of the pixel NaN, which the integer
+            // entries of Wm cannot carry: such a point takes the per-sample path, where its
+            // weight multiplies the sample in floating point like the reference's attn * val
+            const bool nonfinite = live && t.guard && att != att;
+            fbmask |= nonfinite ? 1u << ps : 0u;
             // the row becomes Wm: cleared, then the corners' shares as 2^30-scaled
             // integers (every entry and every row sum is at most 1; the rounding of
             // a contribution, 2^-31, is below that of an fp32 weight near 1)
@@ -500,7 +505,7 @@ deform_fused_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key,
 #pragma unroll
             for (int i4 = 0; i4 < (KP / 4 + NL - 1) / NL; ++i4)
                 if (i4 * NL + pt < KP / 4) *(u32x4 *)(wrow + 4 * (i4 * NL + pt)) = u32x4{0u, 0u, 0u, 0u};
-            if (in) {
+            if (in && !nonfinite) {
                 u32 *wp = wrow + cell;
                 const float sc = att * WSCALE;
                 __hip_atomic_fetch_add(wp, (u32)fma_(sc, t.w1, 0.5f), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);

@@ -206,6 +206,12 @@ def _fused_backward(grad_output, query, key, value, K, s, needs=(True, True, Tru
     if status != _lib.UNSUPPORTED:
         return tuple(grads)
     del ws, grads
+    if value.dtype in (torch.float16, torch.bfloat16):
+        # no one-call kernel for this (kernel_size, scale_factor): the chain below in fp32 on
+        # widened copies, so that the weights and the gradient of the logits are rounded to
+        # 16 bits nowhere -- each gradient is rounded once, at the end
+        wide = _fused_backward(grad_output.float(), query.float(), key.float(), value.float(), K, s, needs)
+        return tuple(None if t is None else t.to(value.dtype) for t in wide)
     attn = _qk_softmax_forward(query, key, K, s)
     grad_query = grad_key = grad_logits = None
     if need_q or need_k:

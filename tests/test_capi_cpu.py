@@ -45,6 +45,13 @@ def test_library_exports_every_declared_symbol():
     assert h.sapa_deform_fused_forward_workspace(8, 128, 256, 64, 64, 25, 2, 4, _lib.DTYPES[torch.bfloat16]) == 8 * 4096 * (128 + 256) * 2
     assert h.sapa_deform_fused_forward_workspace(8, 128, 256, 64, 64, 5, 2, 4, _lib.DTYPES[torch.float32]) == 0
     assert h.sapa_deform_fused_forward_workspace(8, 128, 256, 64, 64, 25, 2, 4, _lib.DTYPES[torch.float64]) == 0
+    # the point counts from which the path serves, as include/sapa_hip.h states them:
+    # 16-bit tensors from 4 points, fp32 from 13
+    bf, f32 = _lib.DTYPES[torch.bfloat16], _lib.DTYPES[torch.float32]
+    assert h.sapa_deform_fused_forward_workspace(8, 128, 256, 64, 64, 3, 2, 4, bf) == 0
+    assert h.sapa_deform_fused_forward_workspace(8, 128, 256, 64, 64, 4, 2, 4, bf) == 8 * 4096 * (128 + 256) * 2
+    assert h.sapa_deform_fused_forward_workspace(8, 128, 256, 64, 64, 12, 2, 4, f32) == 0
+    assert h.sapa_deform_fused_forward_workspace(8, 128, 256, 64, 64, 13, 2, 4, f32) == 8 * 4096 * (128 + 256) * 4
     # two fp32 [B,G,P,sH,sW] tensors, fp32 accumulators of the two low-res gradients and
     # channels-last copies of key and value for the matrix-form stage.  Groups that stage does not
     # serve (5 channels): no copies, but half of grad_offset in fp32 for 16-bit tensors

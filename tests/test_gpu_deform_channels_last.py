@@ -74,6 +74,32 @@ def test_16bit_vs_oracle(coracle, shape, dtype, rel):
     assert_rel_rms_close(got.float(), want, rel, 'fused')
 
 
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('layout', ['contiguous', 'channels_last'])
+def test_matrix_form_carries_non_finite_logits(coracle, layout, dtype):
+    """A NaN or +inf in the query makes the logits of that pixel and group
+    non-finite; softmax then gives NaN for every point and the reference's
+    attn * val (deform_av_cuda_kernel.cu:185-190) puts NaN into every channel
+    of the group at that pixel.  The matrix form builds its weight matrix from
+    integers, which cannot carry a NaN: such pixels take the per-sample path."""
+    B, G, d, cg, H, W, P, s = 2, 2, 8, 16, 9, 11, 16, 2
+    q, key, v, off = inputs(gen(503), B, G, d, cg, H, W, P, s, 1.0, dtype=dtype)
+    q[0, 3, 5, 7] = float('nan')            # group 0
+    q[1, d + 2, 10, 3] = float('inf')       # group 1
+    q[1, 1, 0, 0] = float('inf')            # a corner pixel: part of its samples fail the guard
+    want = coracle.deform_sapa_fused(q.float(), key.float(), v.float(), off.float(), P, s, G, 'f32')
+    bad = ~torch.isfinite(want)
+    assert bad.any() and bad.sum() <= 3 * cg, 'whole groups of three pixels at most'
+    args = cl(q, key, v, off) if layout == 'channels_last' else [t.to(DEV) for t in (q, key, v, off)]
+    got = sapa_amd.deform_sapa_fused(*args, P, s, G, matrix_form=True).float().cpu()
+    assert torch.equal(torch.isnan(got), torch.isnan(want))
+    fin = ~bad
+    if dtype == torch.float32:
+        torch.testing.assert_close(got[fin], want[fin], rtol=1e-5, atol=1e-5)
+    else:
+        assert_rel_rms_close(torch.where(fin, got, 0), torch.where(fin, want, 0), BF16_REL, 'finite part')
+
+
 def test_matches_contiguous_path_at_a_larger_shape():
     B, G, d, cg, H, W, P, s = 2, 4, 32, 64, 19, 22, 25, 2
     q, key, v, off = inputs(gen(502), B, G, d, cg, H, W, P, s, 0.75)

@@ -153,20 +153,25 @@ def test_softmax_of_minus_infinity_is_zero():
     torch.testing.assert_close(got5, torch.softmax(x5, 2), rtol=1e-5, atol=1e-7)
 
 
+@pytest.mark.parametrize('C', [16, 128])
 @pytest.mark.parametrize('bad', [float('inf'), float('nan')])
-def test_sampled_gradients_carry_non_finite_values(coracle, bad):
+def test_sampled_gradients_carry_non_finite_values(coracle, bad, C):
     """An inf / NaN in grad_output reaches grad_value through the sampled
     aggregation's gradient, as it does through the reference's atomicAdd
     (deform_av_cuda_kernel.cu:230-292): overflow detection of a loss scaler
-    relies on it.  Finite entries stay within the usual bar."""
+    relies on it.  Finite entries stay within the usual bar.  C = 16 is served
+    by the LDS-window scatter, C = 128 (9 points x 64 channels per group) by
+    the matrix-product scatter; one of the bad pixels has an attention weight
+    of exactly 0, where the reference's 0 * inf gives NaN."""
     g = gen(15)
-    B, C, H, W, P, s, G = 1, 16, 12, 12, 9, 2, 2
+    B, H, W, P, s, G = 1, 12, 12, 9, 2, 2
     attn = torch.softmax(randn(g, B, G, P, H * s, W * s), dim=2)
     v = randn(g, B, C, H, W)
     off = (0.75 * randn(g, B, 2 * G * P, H * s, W * s)).clamp(-4, 4)
     go = randn(g, B, C, H * s, W * s)
     go[0, 3, 10, 9] = bad
-    go[0, 12, 2, 20] = bad
+    go[0, C - 4, 2, 20] = bad
+    attn[0, 0, 4, 10, 9] = 0.0          # group of channel 3
     attn_d, v_d, off_d = (t.to(DEV) for t in (attn, v, off))
     v_d.requires_grad_(True)
     out = sapa_amd.deform_av(attn_d, v_d, off_d, P, s, G)
@@ -180,5 +185,31 @@ def test_sampled_gradients_carry_non_finite_values(coracle, bad):
     if bad == float('inf'):
         assert torch.equal(torch.isnan(got), torch.isnan(want))
         assert torch.equal(got[~fin & ~torch.isnan(want)], want[~fin & ~torch.isnan(want)].float())
-    # channels 3 and 12 only: every other channel is untouched by the bad values
+    # channels 3 and C - 4 only: every other channel is untouched by the bad values
+    torch.testing.assert_close(got[fin], want[fin].float(), rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize('bad', [float('inf'), float('nan')])
+def test_fused_sampled_backward_carries_non_finite_values(coracle, bad):
+    """The same through the one-call backward of the fused operator
+    (sapa_deform_fused_backward: matrix-product scatter, channels-last
+    accumulation): grad_value against the float64 chain."""
+    g = gen(16)
+    B, C, d, H, W, P, s, G = 1, 128, 8, 12, 12, 9, 2, 2
+    q, key = randn(g, B, G * d, H * s, W * s), randn(g, B, G * d, H, W)
+    v = randn(g, B, C, H, W)
+    off = (0.75 * randn(g, B, 2 * G * P, H * s, W * s)).clamp(-4, 4)
+    go = randn(g, B, C, H * s, W * s)
+    go[0, 3, 10, 9] = bad
+    go[0, C - 4, 2, 20] = bad
+    leaves = [t.to(DEV).requires_grad_(True) for t in (q, key, v, off)]
+    sapa_amd.deform_sapa_fused(*leaves, P, s, G).backward(go.to(DEV))
+    got = leaves[2].grad.cpu()
+    attn = coracle.softmax(coracle.deform_qk(q.double(), key.double(), off.double(), P, s, G, 'f64'), 2, 'f64')
+    _, want, _ = coracle.deform_av_backward(go.double(), attn, v.double(), off.double(), P, s, G, 'f64')
+    fin = torch.isfinite(want)
+    assert not fin.all()
+    assert torch.equal(torch.isfinite(got), fin)
+    if bad == float('inf'):
+        assert torch.equal(torch.isnan(got), torch.isnan(want))
     torch.testing.assert_close(got[fin], want[fin].float(), rtol=1e-4, atol=1e-5)

@@ -315,6 +315,28 @@ def test_backward_16bit_tensors():
             assert_rel_rms_close(a.grad.float().cpu(), b.grad.cpu(), rel, str(dt))
 
 
+@pytest.mark.parametrize('K,s', [(7, 4), (3, 2), (5, 4)])
+@pytest.mark.parametrize('dt,rel', [(torch.bfloat16, 1e-2), (torch.float16, 2e-3)])
+def test_backward_16bit_tensors_other_windows(coracle, K, s, dt, rel):
+    """(kernel_size, scale_factor) pairs that the one-call backward does not cover:
+    the chain runs in fp32 on widened copies, so the 16-bit gradients are the
+    rounded float64 chain on the rounded inputs (one rounding, at the end)."""
+    g = gen(154)
+    B, d, C, H, W = 1, 8, 12, 6, 9
+    q, key, v = (randn(g, B, d, H * s, W * s).to(dt), randn(g, B, d, H, W).to(dt), randn(g, B, C, H, W).to(dt))
+    go = randn(g, B, C, H * s, W * s).to(dt)
+    ts = [t.to(DEV).requires_grad_() for t in (q, key, v)]
+    sapa_amd.sapa_fused(*ts, K, s).backward(go.to(DEV))
+    q64, k64, v64, go64 = (t.double() for t in (q, key, v, go))
+    attn = coracle.softmax(coracle.qk(q64, k64, K, s, 'f64'), 1, 'f64')
+    ga, gv = coracle.av_backward(go64, attn, v64, K, s, 'f64')
+    gl = attn * (ga - (ga * attn).sum(1, keepdim=True))
+    gq, gk = coracle.qk_backward(gl, q64, k64, K, s, 'f64')
+    for a, want, name in zip(ts, (gq, gk, gv), ('grad_query', 'grad_key', 'grad_value')):
+        assert a.grad.dtype == dt
+        assert_rel_rms_close(a.grad.float().cpu(), want.float(), rel, f'{name} {dt} K={K} s={s}')
+
+
 # 16-bit tensors take the lane-exchange form in rows of 32 lanes (30x70, 33x47 with
 # K = 3) or of 16 (25x42); each shape spans several tiles with ragged edges
 @pytest.mark.parametrize('shape', [(1, 6, 30, 70, 5), (2, 5, 25, 42, 5), (1, 5, 33, 47, 3)],

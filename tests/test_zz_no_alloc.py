@@ -56,3 +56,40 @@ def test_static_scratch_refuses_what_does_not_fit():
     assert h.sapa_channel_moments_workspace(B, C, HW, 1) > h.sapa_channel_moments_static_capacity()
     # refused on the extents alone: the pointers are never dereferenced
     assert h.sapa_channel_moments_static(x.data_ptr(), mv.data_ptr(), B, C, HW, 1, 0, None) == -3
+
+
+def test_static_scratch_under_graph_capture():
+    """The call allocates nothing and can be recorded into a HIP graph: after one
+    eager call (the library looks its array's address up on the first call on a
+    device, which must therefore happen outside a capture), the call is captured,
+    the allocator's byte count is unchanged, and every replay -- on fresh input,
+    with eager work and synchronisations in between -- equals the workspace form
+    bit for bit."""
+    h = _lib.lib()
+    dev = torch.device('cuda:0')
+    g = torch.Generator(device=dev).manual_seed(6)
+    B, C, H, W = 2, 48, 60, 84
+    x = torch.randn(B, C, H, W, generator=g, device=dev)
+    got = torch.full((B, C, 2), float('nan'), device=dev)
+    need = h.sapa_channel_moments_workspace(B, C, H * W, 0)
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    want = torch.empty_like(got)
+    st = torch.cuda.current_stream(dev).cuda_stream
+    assert h.sapa_channel_moments_static(x.data_ptr(), got.data_ptr(), B, C, H * W, 0, 0, st) == 0
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated(dev)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        cst = torch.cuda.current_stream(dev).cuda_stream
+        assert h.sapa_channel_moments_static(x.data_ptr(), got.data_ptr(), B, C, H * W, 0, 0, cst) == 0
+    assert torch.cuda.memory_allocated(dev) == before
+    for rep in range(3):
+        x.copy_(torch.randn(B, C, H, W, generator=g, device=dev) * (rep + 1) - rep)
+        got.fill_(float('nan'))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert h.sapa_channel_moments(x.data_ptr(), ws.data_ptr(), want.data_ptr(), B, C, H * W, 0, 0, st) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f'replay {rep}: max diff {(got - want).abs().max().item()}'
+    assert torch.cuda.memory_allocated(dev) == before
