@@ -172,22 +172,37 @@ def measured_ceiling(lib, dev, stream, args, timed, write_bytes):
     from sapa_amd import _lib
     unit_w = 16 * 4096
     units = max(write_bytes // unit_w, 1)
-    src = torch.empty(units * 32 * 4096 // 4, dtype=torch.int32, device=dev).fill_(12345)
-    dst = torch.empty(units * 32 * 4096 // 4, dtype=torch.int32, device=dev)
+    src = torch.empty(units * 16 * 4096 // 4, dtype=torch.int32, device=dev).fill_(12345)
+    dst = torch.empty(units * 16 * 4096 // 4, dtype=torch.int32, device=dev)
     res = {}
-    for name, r, w, n, nt in (('mix_9_16_runs_36K_64K_nt', 9, 16, units, 1), ('mix_9_16_runs_36K_64K', 9, 16, units, 0),
-                              ('mix_9_16_runs_72K_128K_nt', 18, 32, units // 2, 1),
-                              ('copy_runs_32K_nt', 8, 8, units * 2, 1), ('fill_runs_64K_nt', 0, 16, units, 1),
-                              ('read_runs_64K_nt', 16, 0, units, 1)):
+    # name: reads, writes (x 4 KiB per unit), units, units per workgroup, streaming loads | 2 * streaming stores
+    for name, r, w, n, reps, nt in (('mix_9_16_runs_36K_64K_streaming', 9, 16, units, 1, 3),
+                                    ('mix_9_16_runs_36K_64K_streaming_loads', 9, 16, units, 1, 1),
+                                    ('mix_9_16_runs_36K_64K_plain', 9, 16, units, 1, 0),
+                                    ('mix_9_16_runs_72K_128K_streaming', 9, 16, units, 2, 3),
+                                    # readers and writers in different workgroups (runs of 128K): units // 32 groups
+                                    ('mix_9_16_readers_and_writers_apart', 9, 16, max(units // 32, 1), 2, 4 | 3),
+                                    ('copy_runs_32K_streaming', 8, 8, units, 1, 3),
+                                    ('fill_runs_256K_plain', 0, 16, units, 4, 0),
+                                    ('read_runs_256K_streaming', 16, 0, units, 4, 1)):
         def step():
-            _lib.check(lib.sapa_stream_mix(src.data_ptr(), dst.data_ptr(), n, r, w, nt, stream.cuda_stream),
+            _lib.check(lib.sapa_stream_mix(src.data_ptr(), dst.data_ptr(), n, r, w, reps, nt, stream.cuda_stream),
                        'sapa_stream_mix')
         ms, _ = timed(step)
-        res[name] = {'ms': ms, 'GB/s': n * (r + w) * 4096 / (ms * 1e-3) / 1e9}
+        moved = n * reps * 25 * 65536 if nt & 4 else n * (r + w) * 4096
+        res[name] = {'ms': ms, 'GB/s': moved / (ms * 1e-3) / 1e9}
     del src, dst
     best = max((k for k in res if k.startswith('mix')), key=lambda k: res[k]['GB/s'])
+    # reads and writes share the memory bus: a stream of both takes about as long as its read
+    # part at the read-only rate plus its write part at the write-only rate
+    rd, wr = res['read_runs_256K_streaming']['GB/s'], res['fill_runs_256K_plain']['GB/s']
+    additive_ms = (units * 9 * 4096 / rd + units * 16 * 4096 / wr) / 1e6
     return {'GB/s': res[best]['GB/s'], 'variant': best, 'kernel': 'stream_mix_kernel (sapa_stream_mix)',
-            'bytes_moved': units * 25 * 4096, 'variants': res}
+            'bytes_moved': units * 25 * 4096,
+            'read_plus_write_floor': {'ms': additive_ms, 'GB/s': units * 25 * 4096 / additive_ms / 1e6,
+                                      'note': 'the mix\'s read bytes at the measured read-only rate plus its '
+                                              'write bytes at the measured fill rate'},
+            'variants': res}
 
 
 def timed_median(fn, budget_s):

@@ -442,16 +442,21 @@ int sapa_project_nhwc(const void *x, const void *weight, const void *bias, void 
 /* A kernel that only moves bytes, for putting the operators' measured rates
  * beside what the memory system gives a plain stream of the same read : write
  * mix.  No counterpart in the reference (which has no measurement code).
- * `units` workgroups; unit u reads the contiguous run
- * src[u * reads * 4096 ... + reads * 4096) and writes the contiguous run
- * dst[u * writes * 4096 ... + writes * 4096) (bytes), the written words being a
- * function of the words read; writes = 0: src is only read (dst needs 4096
- * bytes per unit and is left untouched unless a 16-byte group of src is
- * ff..fe in every word).  nontemporal != 0: streaming loads and stores.
- * (reads, writes) in {(9,16): a fused SAPA-B forward at up_factor 2 with
- * C = 4 d, (18,32), (8,8), (0,16), (16,0)}; SAPA_ERR_UNSUPPORTED otherwise.
+ * Unit u reads the contiguous run src[u * reads * 4096 ... + reads * 4096) and
+ * writes the contiguous run dst[u * writes * 4096 ... + writes * 4096) (bytes),
+ * the written words being a function of the words read; a workgroup takes
+ * `reps` consecutive units (runs `reps` times as long), the next unit's loads
+ * issued before the current unit's stores.  writes = 0: src is only read (dst
+ * needs 4096 bytes per workgroup and is left untouched unless a 16-byte group
+ * of src is ff..fe in every word).  nontemporal: bit 0 = streaming
+ * (non-temporal) loads, bit 1 = streaming stores; bit 2 ((9,16) only): readers
+ * and writers are different workgroups -- `units` groups of 9 workgroups that
+ * each read one run of reps * 65536 bytes of src and 16 that each write one of
+ * dst, nothing written depending on anything read (src needs units * 9 * reps
+ * * 65536 bytes, dst units * 16 * reps * 65536).  (reads, writes) in {(9,16): a fused SAPA-B forward at up_factor 2
+ * with C = 4 d, (8,8), (0,16), (16,0)}; SAPA_ERR_UNSUPPORTED otherwise.
  * Pointers aligned to 16 bytes. */
-int sapa_stream_mix(const void *src, void *dst, long long units, int reads, int writes,
+int sapa_stream_mix(const void *src, void *dst, long long units, int reads, int writes, int reps,
                     int nontemporal, void *stream);
 
 #ifdef __cplusplus

@@ -50,7 +50,7 @@ SIGNATURES = {
     'sapa_deform_fused_forward_ws': [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_deform_qk_forward_from': [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_deform_av_forward_from': [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
-    'sapa_stream_mix': [_vp, _vp, _ll, _i, _i, _i, _vp],
+    'sapa_stream_mix': [_vp, _vp, _ll, _i, _i, _i, _i, _vp],
     'sapa_deform_fused_forward_from': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
 }
 

@@ -36,6 +36,9 @@ bool dtype_ok(int dt) { return dt >= SAPA_F32 && dt <= SAPA_BF16; }
 // 64-bit flat indices and 32-bit in-plane indices cannot overflow
 const long long kMaxElems = 1LL << 40;
 
+// fused fp32 K = 5, s = 2 problems of at most this many low-res cells go to the matrix-pipe kernel
+const long kSmallFusedCells = 12288;
+
 // LDS-tiled SAPA-B kernel for `mode`: the VALU kernel where it has an
 // instance (K = 5, s = 2, where it is the faster one), else the matrix-pipe
 // kernel; hipErrorNotSupported when neither covers the request.
@@ -44,6 +47,13 @@ hipError_t tiled_launch(int mode, const void *q, const void *key, const void *at
                         int s, int dtype, hipStream_t st) {
     hipError_t e = took("sapa_b_dot2_kernel", sapa_b_dot2_launch(mode, q, key, attn_in, value, out, B,
                                                                   d, C, H, W, K, s, dtype, st));
+    // small fp32 problems of the common window: the matrix-pipe kernel's lane-per-child
+    // decomposition fills the chip where the VALU kernel's thread-per-parent one leaves it
+    // latency-bound (B=8, d=32, C=256, fused: 16x16 32 -> 13 us, 32x32 32 -> 23 us)
+    if (e == hipErrorNotSupported && K == 5 && s == 2 && dtype == SAPA_F32 && mode == TILED_FUSED &&
+        (long)B * H * W <= kSmallFusedCells)
+        e = took("sapa_b_mfma_kernel",
+                 sapa_b_mfma_launch(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, dtype, st));
     if (e == hipErrorNotSupported)
         e = took("sapa_b_tiled_kernel",
                  sapa_b_tiled_launch(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, dtype, st));
@@ -690,15 +700,19 @@ int sapa_project_nhwc(const void *x, const void *weight, const void *bias, void 
     return finish(e);
 }
 
-int sapa_stream_mix(const void *src, void *dst, long long units, int reads, int writes,
+int sapa_stream_mix(const void *src, void *dst, long long units, int reads, int writes, int reps,
                     int nontemporal, void *stream) {
-    if (units < 0 || reads < 0 || writes < 0 || (reads == 0 && writes == 0)) return SAPA_ERR_INVALID_ARGUMENT;
+    if (units < 0 || reads < 0 || writes < 0 || reps < 1 || (reads == 0 && writes == 0) || nontemporal < 0 || nontemporal > 7)
+        return SAPA_ERR_INVALID_ARGUMENT;
     if (units > (1LL << 30)) return SAPA_ERR_TOO_LARGE;
     if (units == 0) return SAPA_OK;
     if ((reads > 0 && !src) || !dst) return SAPA_ERR_INVALID_ARGUMENT;
     if (((uintptr_t)src | (uintptr_t)dst) % 16 != 0) return SAPA_ERR_INVALID_ARGUMENT;
-    const hipError_t e = stream_mix_launch(src, dst, (long)units, reads, writes, nontemporal != 0,
-                                           (hipStream_t)stream);
+    // bit 2: readers and writers in different workgroups (`units` = groups of 9 + 16)
+    const hipError_t e = (nontemporal & 4)
+        ? (reads == 9 && writes == 16 ? stream_split_launch(src, dst, (long)units, reps, nontemporal & 3, (hipStream_t)stream)
+                                      : hipErrorNotSupported)
+        : stream_mix_launch(src, dst, (long)units, reads, writes, reps, nontemporal, (hipStream_t)stream);
     if (e == hipErrorNotSupported) return SAPA_ERR_UNSUPPORTED;
     return finish(e);
 }

@@ -59,11 +59,15 @@ hipError_t groupnorm_fold_launch(const float *mean_var, const void *gamma, const
                                  const void *w, const void *bias, void *w_out, void *b_out, int B,
                                  int C, int O, int G, float eps, int dtype, hipStream_t st);
 
-// sapa_stream.hip: a kernel that only moves bytes, `units` workgroups that each read one
-// contiguous run of reads * 4 KiB and write one of writes * 4 KiB (calibration of measured
-// rates); (reads, writes) in {(9,16), (18,32), (8,8), (0,16), (16,0)}, hipErrorNotSupported otherwise
-hipError_t stream_mix_launch(const void *src, void *dst, long units, int reads, int writes, bool nt,
-                             hipStream_t st);
+// sapa_stream.hip: a kernel that only moves bytes, `units` units that each read one
+// contiguous run of reads * 4 KiB and write one of writes * 4 KiB, `reps` consecutive units per
+// workgroup (calibration of measured rates); (reads, writes) in {(9,16), (8,8), (0,16), (16,0)},
+// hipErrorNotSupported otherwise; nt: bit 0 = streaming loads, bit 1 = streaming stores
+hipError_t stream_mix_launch(const void *src, void *dst, long units, int reads, int writes, int reps,
+                             int nt, hipStream_t st);
+// the 9 : 16 mix with readers and writers in different workgroups: `groups` groups of 9 reading
+// and 16 writing workgroups, each with one contiguous run of reps * 64 KiB
+hipError_t stream_split_launch(const void *src, void *dst, long groups, int reps, int nt, hipStream_t st);
 
 // sapa_project.hip: 1x1 projection of a channels-last 16-bit feature with per-image weights
 hipError_t project_nhwc_launch(const void *x, const void *w, const void *bias, void *out, int B,

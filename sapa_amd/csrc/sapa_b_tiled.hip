@@ -94,11 +94,17 @@ __device__ __forceinline__ void store_buffer(__amdgpu_buffer_rsrc_t r, unsigned 
 #ifndef SAPA_TILED_WPE
 #define SAPA_TILED_WPE 3
 #endif
+// fused fp32 problems of at most this many low-res cells take the two-waves-per-band geometry
+#ifndef SAPA_TILED_SMALL_PARENTS
+#define SAPA_TILED_SMALL_PARENTS 24576
+#endif
 // WIDE: the K*K-channel tensors of the call (attn_in; the result of the modes
 // without aggregation) are fp32 while the feature tensors are T -- the form the
 // backward pass of 16-bit tensors keeps its intermediates in
+// (a thread with fewer than S x S children needs fewer registers: four waves per SIMD)
 template <typename T, int K, int S, int CY, int NWX, int NWY, int CH, int VEC, int WLX, int MODE, bool WIDE = false>
-__global__ void __launch_bounds__(64 * NWX * NWY * (S / CY)) __attribute__((amdgpu_waves_per_eu(SAPA_TILED_WPE, SAPA_TILED_WPE)))
+__global__ void __launch_bounds__(64 * NWX * NWY * (S / CY))
+    __attribute__((amdgpu_waves_per_eu(CY < S ? SAPA_TILED_WPE + 1 : SAPA_TILED_WPE, CY < S ? SAPA_TILED_WPE + 1 : SAPA_TILED_WPE)))
 sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
                     const T *__restrict__ attn_in, const T *__restrict__ value,
                     T *__restrict__ out, int d, int C, int H, int W, int tiles_x, int tiles_y,
@@ -281,7 +287,10 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
 #ifndef SAPA_TILED_PF
 #define SAPA_TILED_PF 4
 #endif
-        constexpr int PF = CH < SAPA_TILED_PF ? CH : SAPA_TILED_PF;
+        // (twice as far ahead when a thread has half the children: a channel is then over
+        // in half the time)
+        constexpr int PFW = CY < S ? 2 * SAPA_TILED_PF : SAPA_TILED_PF;
+        constexpr int PF = CH < PFW ? CH : PFW;
         static_assert(CH % PF == 0, "prefetch ring must divide the chunk");
         A qr[PF][NJ];
         auto load_q = [&](int c, A (&dst)[NJ]) {
@@ -521,6 +530,16 @@ static hipError_t launch_t(int mode, bool wide, const void *q, const void *key, 
             return W % vec == 0 && (!key || (uintptr_t)key % a == 0) &&
                    (!value || (uintptr_t)value % a == 0);
         };
+        // Small problems (a few waves per SIMD at most, so a wave's own instruction latencies
+        // show): two waves per band of parent rows, each thread with the two children of one
+        // hi-res row (half the accumulators, twice the waves), 16-channel chunks (half the
+        // barriers).  Measured at B=16, 25x42, d=64, C=256: 80 -> 59 us.
+        if constexpr (sizeof(T) == 4) {
+            if (mode == TILED_FUSED && !wide && (long)B * H * W <= SAPA_TILED_SMALL_PARENTS)
+                return aligned(2)
+                           ? launch_mode<T, 5, 2, 1, 1, 2, 16, 2, 16>(mode, wide, q, key, attn_in, value, out, B, d, C, H, W, st)
+                           : launch_mode<T, 5, 2, 1, 1, 2, 16, 1, 16>(mode, wide, q, key, attn_in, value, out, B, d, C, H, W, st);
+        }
 #define SAPA_GEOM(NWX, NWY, VEC, WLX)                                                            \
     launch_mode<T, 5, 2, 2, NWX, NWY, 8, VEC, WLX>(mode, wide, q, key, attn_in, value, out, B, d, C, H, \
                                                    W, st)

@@ -72,7 +72,6 @@ def assert_batch_equals_images(fn, tensors, what, images=None):
 
 # bounds on the literal comparison of a re-ordered fp32 sum with the reference-order result
 LITERAL_BAR_MAX_FRACTION = 0.02
-LITERAL_MAX_ABS = 1e-4
 
 
 def assert_no_worse_than_reference_order(got, ref32, exact, what):
@@ -88,8 +87,9 @@ def assert_no_worse_than_reference_order(got, ref32, exact, what):
     fp32 orders of one sum differ by their rounding errors, which that bar
     (one fp32 spacing near 0.1) does not absorb where terms cancel, so the
     count is not zero for either order against the other; it is printed and
-    held below LITERAL_BAR_MAX_FRACTION of the elements, and the largest
-    difference below LITERAL_MAX_ABS."""
+    held below LITERAL_BAR_MAX_FRACTION of the elements (the largest
+    difference is printed too; it is bounded by the two errors against the
+    exact result, which are held above)."""
     got, ref32, exact = got.double().cpu(), ref32.double().cpu(), exact.double().cpu()
     e_got, e_ref = (got - exact).abs(), (ref32 - exact).abs()
     bar = F32_ATOL + F32_RTOL * exact.abs()
@@ -110,7 +110,6 @@ def assert_no_worse_than_reference_order(got, ref32, exact, what):
         f"{what}: max error {st['max']:.3e} > 1.25 x reference order {st['max_ref']:.3e}"
     assert st['literal_outside'] <= LITERAL_BAR_MAX_FRACTION * st['n'], \
         f"{what}: {st['literal_outside']} of {st['n']} elements outside 1e-6 + 1e-5 |b| of the reference-order result"
-    assert st['literal_max'] <= LITERAL_MAX_ABS, f"{what}: largest difference to the reference-order result {st['literal_max']:.3e}"
     return st
 
 
