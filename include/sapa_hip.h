@@ -284,6 +284,35 @@ int sapa_deform_av_backward(const void *grad_out, const void *attn,
                             int B, int C, int H, int W, int P, int s, int G,
                             int dtype, void *stream);
 
+/* sapa_deform_qk_backward / sapa_deform_av_backward for SAPA_F16 / SAPA_BF16
+ * tensors, read and written as they are: the half dispatch of the reference's
+ * backward kernels (DeformQKBackwardLauncher, deform_qk_cuda_kernel.cu:298-337;
+ * DeformAVBackwardLauncher, deform_av_cuda_kernel.cu:294-333).  The per-pixel
+ * gradients are computed in fp32 from the 16-bit operands and rounded once; the
+ * low-res gradient (grad_key / grad_value), a sum of many terms, is accumulated
+ * in fp32 in `workspace` and rounded once -- so, unlike the fp32 entry points,
+ * grad_key / grad_value are OVERWRITTEN here and need no zero fill.
+ * sapa_deform_backward_workspace: bytes of device memory either call needs for
+ * Cx = Cq (deform_qk) or C (deform_av) channels; 0 when this path does not serve
+ * the case (s not in {1, 2, 4}, P > 48, other dtypes).  workspace: at least that
+ * many bytes, aligned to 256, contents undefined before and after.
+ * SAPA_ERR_UNSUPPORTED when the size is 0, workspace is NULL, or a kernel's window
+ * does not fit the configuration (nothing the caller relies on is then written:
+ * run the fp32 entry points on widened copies instead).  Any gradient may be NULL. */
+long long sapa_deform_backward_workspace(int B, int Cx, int H, int W,
+                                         int P, int s, int G, int dtype);
+int sapa_deform_qk_backward_ws(const void *grad_out, const void *query,
+                               const void *key, const void *offset, void *workspace,
+                               void *grad_query, void *grad_key, void *grad_offset,
+                               int B, int Cq, int H, int W, int P, int s, int G,
+                               int dtype, void *stream);
+int sapa_deform_av_backward_ws(const void *grad_out, const void *attn,
+                               const void *value, const void *offset, void *workspace,
+                               void *grad_attn, void *grad_value, void *grad_offset,
+                               int B, int C, int H, int W, int P, int s, int G,
+                               int dtype, void *stream);
+
+
 /* Fused sapa_deform_qk_forward -> softmax over P -> sapa_deform_av_forward in
  * one launch (SAPADeform.attention, sapa_deform.py:51-53).  Sample positions
  * and bilinear weights are computed once per (pixel, group, point) and shared

@@ -44,6 +44,8 @@ SIGNATURES = {
     'sapa_deform_qk_backward': [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_deform_av_forward': [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_deform_av_backward': [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
+    'sapa_deform_qk_backward_ws': [_vp] * 8 + [_i] * 8 + [_vp],
+    'sapa_deform_av_backward_ws': [_vp] * 8 + [_i] * 8 + [_vp],
     'sapa_deform_fused_forward': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_deform_fused_forward_nhwc': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_deform_fused_backward': [_vp] * 10 + [_i] * 9 + [_vp],
@@ -101,6 +103,8 @@ def lib():
         handle.sapa_deform_fused_forward_workspace.argtypes = [_i] * 9
         handle.sapa_deform_fused_backward_workspace.restype = _ll
         handle.sapa_deform_fused_backward_workspace.argtypes = [_i] * 9
+        handle.sapa_deform_backward_workspace.restype = _ll
+        handle.sapa_deform_backward_workspace.argtypes = [_i] * 8
         handle.sapa_channel_moments_static_capacity.restype = _ll
         handle.sapa_channel_moments_static_capacity.argtypes = []
         _lib = handle

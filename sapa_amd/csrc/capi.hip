@@ -616,6 +616,41 @@ int sapa_deform_av_backward(const void *grad_out, const void *attn, const void *
     return SAPA_OK;
 }
 
+long long sapa_deform_backward_workspace(int B, int Cx, int H, int W, int P, int s, int G, int dtype) {
+    if (check_deform_args(B, Cx, Cx, H, W, P, s, G, dtype) != SAPA_OK) return 0;
+    return deform_separate_backward_workspace(B, Cx, H, W, P, s, G, dtype);
+}
+
+int sapa_deform_qk_backward_ws(const void *grad_out, const void *query, const void *key,
+                               const void *offset, void *workspace, void *grad_query, void *grad_key,
+                               void *grad_offset, int B, int Cq, int H, int W, int P, int s, int G,
+                               int dtype, void *stream) {
+    const int rc = check_deform_args(B, Cq, Cq, H, W, P, s, G, dtype);
+    if (rc != SAPA_OK) return rc;
+    if (B == 0) return SAPA_OK;
+    if (!grad_out || !query || !key || !offset) return SAPA_ERR_INVALID_ARGUMENT;
+    const hipError_t e = deform_separate_backward_launch(0, query, key, grad_out, offset, workspace, grad_query,
+                                                         grad_key, grad_offset, B, Cq, H, W, P, s, G, dtype,
+                                                         (hipStream_t)stream);
+    if (e == hipErrorNotSupported) return SAPA_ERR_UNSUPPORTED;
+    return finish(e);
+}
+
+int sapa_deform_av_backward_ws(const void *grad_out, const void *attn, const void *value,
+                               const void *offset, void *workspace, void *grad_attn, void *grad_value,
+                               void *grad_offset, int B, int C, int H, int W, int P, int s, int G,
+                               int dtype, void *stream) {
+    const int rc = check_deform_args(B, C, C, H, W, P, s, G, dtype);
+    if (rc != SAPA_OK) return rc;
+    if (B == 0) return SAPA_OK;
+    if (!grad_out || !attn || !value || !offset) return SAPA_ERR_INVALID_ARGUMENT;
+    const hipError_t e = deform_separate_backward_launch(1, grad_out, value, attn, offset, workspace, grad_attn,
+                                                         grad_value, grad_offset, B, C, H, W, P, s, G, dtype,
+                                                         (hipStream_t)stream);
+    if (e == hipErrorNotSupported) return SAPA_ERR_UNSUPPORTED;
+    return finish(e);
+}
+
 long long sapa_deform_fused_backward_workspace(int B, int Cq, int C, int H, int W, int P, int s,
                                                int G, int dtype) {
     if (check_deform_args(B, Cq, C, H, W, P, s, G, dtype) != SAPA_OK) return 0;

@@ -114,6 +114,16 @@ hipError_t deform_fused_backward_launch(const void *grad_out, const void *q, con
                                         void *grad_offset, int B, int Cq, int C, int H, int W, int P,
                                         int s, int G, int dtype, hipStream_t st);
 
+// sapa_d_backward.hip: backward of deform_qk (which = 0: a = query, low = key, pp = grad_out,
+// grad_a_or_pp = grad_query) or deform_av (which = 1: a = grad_out, low = value, pp = attn,
+// grad_a_or_pp = grad_attn) on f16 / bf16 tensors as they are; `workspace` (256-byte aligned,
+// deform_separate_backward_workspace() bytes; 0 = not served) holds fp32 intermediates.
+long deform_separate_backward_workspace(int B, int Cx, int H, int W, int P, int s, int G, int dtype);
+hipError_t deform_separate_backward_launch(int which, const void *a, const void *low, const void *pp,
+                                           const void *offset, void *workspace, void *grad_a_or_pp,
+                                           void *grad_low, void *grad_offset, int B, int Cx, int H, int W,
+                                           int P, int s, int G, int dtype, hipStream_t st);
+
 // sapa_d_nhwc.hip: contiguous (NCHW) tensors through the matrix-form kernels:
 // key and value are copied into channels-last order in `workspace` (256-byte
 // aligned, deform_fused_nchw_workspace() bytes; 0 = this path does not serve the

@@ -558,7 +558,7 @@ hipError_t sapa_b_tiled_launch(int mode, const void *q, const void *key, const v
                                int K, int s, int dtype, hipStream_t st, bool wide) {
     switch (dtype) {
         case 0: return launch_t<float>(mode, wide, q, key, attn_in, value, out, B, d, C, H, W, K, s, st);
-#if !defined(SAPA_TUNE_GEOM) || defined(SAPA_TUNE_ALLTYPES)
+#if (!defined(SAPA_TUNE_GEOM) || defined(SAPA_TUNE_ALLTYPES)) && !defined(SAPA_TUNE_ONLY_F32)
         case 2: return launch_t<f16_t>(mode, wide, q, key, attn_in, value, out, B, d, C, H, W, K, s, st);
         case 3: return launch_t<bf16_t>(mode, wide, q, key, attn_in, value, out, B, d, C, H, W, K, s, st);
 #endif

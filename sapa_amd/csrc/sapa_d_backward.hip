@@ -109,7 +109,77 @@ static bool matrix_stage(int B, int Cq, int C, int H, int W, int P, int s, int G
 #endif
 }
 
+
+
+template <typename T>
+__global__ void __launch_bounds__(256) widen_kernel(const T *__restrict__ x, float *__restrict__ y, long n) {
+    for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
+        y[i] = (float)x[i];
+}
+
+static hipError_t widen(const void *x, float *y, long n, int dtype, hipStream_t st) {
+    if (dtype == 2) hipLaunchKernelGGL(widen_kernel<f16_t>, dim3(blocks_for(n)), dim3(256), 0, st, (const f16_t *)x, y, n);
+    else hipLaunchKernelGGL(widen_kernel<bf16_t>, dim3(blocks_for(n)), dim3(256), 0, st, (const bf16_t *)x, y, n);
+    return hipGetLastError();
+}
+
 }  // namespace dbwd
+
+// ---- the separate sampled operators' backward passes on f16 / bf16 tensors, read and
+// written as they are (the reference dispatches DeformQKBackward / DeformAVBackward on
+// half directly, deform_qk_cuda_kernel.cu:298-337, deform_av_cuda_kernel.cu:294-333).
+// The per-pixel gradients come from the forward kernels with swapped roles on the 16-bit
+// tensors; the low-res gradient, a sum of many terms, is accumulated in fp32 in the
+// workspace (next to an fp32 copy of the per-point tensor, which the scatter kernels
+// take) and rounded once.
+long deform_separate_backward_workspace(int B, int Cx, int H, int W, int P, int s, int G, int dtype) {
+    using dbwd::align256;
+    if (dtype != 2 && dtype != 3) return 0;
+    if (s != 1 && s != 2 && s != 4) return 0;
+    if (P > 48) return 0;
+    return align256((long)B * G * P * H * s * W * s * 4) + align256((long)B * Cx * H * W * 4);
+}
+
+// which = 0: gradients of deform_qk -- a = query, low = key, pp = grad_out [B,G,P,sH,sW];
+//            grad_a = grad_query, grad_low = grad_key;
+// which = 1: gradients of deform_av -- a = grad_out [B,C,sH,sW], low = value, pp = attn;
+//            grad_pp = grad_attn, grad_low = grad_value.
+// Any gradient may be NULL.
+hipError_t deform_separate_backward_launch(int which, const void *a, const void *low, const void *pp,
+                                           const void *offset, void *workspace, void *grad_a_or_pp,
+                                           void *grad_low, void *grad_offset, int B, int Cx, int H, int W,
+                                           int P, int s, int G, int dtype, hipStream_t st) {
+    using namespace dbwd;
+    if (deform_separate_backward_workspace(B, Cx, H, W, P, s, G, dtype) == 0) return hipErrorNotSupported;
+    if (!workspace || (uintptr_t)workspace % 256 != 0) return hipErrorNotSupported;
+    const long n_pp = (long)B * G * P * H * s * W * s;
+    float *pp32 = (float *)workspace;
+    float *acc = (float *)((char *)workspace + align256(n_pp * 4));
+    const int HIRES = 0;
+    hipError_t e;
+#define SAPA_STEP(call)                  \
+    do {                                 \
+        e = (call);                      \
+        if (e != hipSuccess) return e;   \
+    } while (0)
+    if (grad_a_or_pp) {
+        if (which == 0)   // grad_query: the sampled aggregation of key with grad_out as the weights
+            SAPA_STEP(deform_lds_launch(1, nullptr, nullptr, pp, low, offset, grad_a_or_pp, B, Cx, Cx, H, W, P, s, G,
+                                        HIRES, dtype, st));
+        else              // grad_attn: the sampled similarity of grad_out and value
+            SAPA_STEP(deform_lds_launch(0, a, low, nullptr, nullptr, offset, grad_a_or_pp, B, Cx, Cx, H, W, P, s, G,
+                                        HIRES, dtype, st));
+    }
+    if (grad_offset)
+        SAPA_STEP(deform_lds_launch(3, a, low, pp, nullptr, offset, grad_offset, B, Cx, Cx, H, W, P, s, G, HIRES,
+                                    dtype, st));
+    if (grad_low) {
+        SAPA_STEP(widen(pp, pp32, n_pp, dtype, st));
+        SAPA_STEP(low_gradient(a, pp32, offset, acc, grad_low, B, Cx, H, W, P, s, G, dtype, st, false));
+    }
+#undef SAPA_STEP
+    return hipSuccess;
+}
 
 // Bytes of workspace, or 0 for configurations this call does not serve (the
 // caller then chains the separate backward entry points): f32 / f16 / bf16,

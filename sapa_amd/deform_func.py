@@ -15,12 +15,35 @@ from . import _lib
 
 
 def _compute_dtype(t):
-    # the backward kernels exist for fp32 / fp64; 16-bit tensors take the
-    # fp32 kernels and the gradients are rounded back
+    # 16-bit tensors that the native 16-bit backward entry points do not serve
+    # (_backward_16bit) take the fp32 kernels and the gradients are rounded back
     return t.dtype if t.dtype in (torch.float32, torch.float64) else torch.float32
 
 
+def _backward_16bit(entry, grad_output, a, low, offset, P, s, G, needs):
+    """The gradients of one sampled operator on f16 / bf16 tensors as they are
+    (sapa_deform_{qk,av}_backward_ws); None where that path does not serve the
+    configuration.  a: query (deform_qk) or attn (deform_av); low: key or value."""
+    if low.dtype not in (torch.float16, torch.bfloat16):
+        return None
+    go, a, low, off = (t.contiguous() for t in (grad_output, a, low, offset))
+    _lib.require_cuda_contiguous(grad_output=go, a=a, low=low, offset=off)
+    n, c, h, w = low.size()
+    nbytes = _lib.lib().sapa_deform_backward_workspace(n, c, h, w, P, s, G, _lib.dtype_code(low))
+    if nbytes <= 0:
+        return None
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=low.device)
+    grads = [_lib.new_out(t) if need else None for t, need in ((a, needs[0]), (low, needs[1]), (off, needs[2]))]
+    status = _lib.call_status(entry, low.device, _lib.ptr(go), _lib.ptr(a), _lib.ptr(low), _lib.ptr(off),
+                              _lib.ptr(ws), _lib.ptr(grads[0]), _lib.ptr(grads[1]), _lib.ptr(grads[2]),
+                              n, c, h, w, P, s, G, _lib.dtype_code(low))
+    return None if status == _lib.UNSUPPORTED else tuple(grads)
+
+
 def _deform_qk_backward(grad_output, query, key, offset, P, s, G, needs=(True, True, True)):
+    native = _backward_16bit('sapa_deform_qk_backward_ws', grad_output, query, key, offset, P, s, G, needs)
+    if native is not None:
+        return native
     cdt = _compute_dtype(query)
     go, q, k, off = (t.contiguous().to(cdt) for t in (grad_output, query, key, offset))
     gq = _lib.new_out(q) if needs[0] else None
@@ -36,6 +59,9 @@ def _deform_qk_backward(grad_output, query, key, offset, P, s, G, needs=(True, T
 
 
 def _deform_av_backward(grad_output, attn, value, offset, P, s, G, needs=(True, True, True)):
+    native = _backward_16bit('sapa_deform_av_backward_ws', grad_output, attn, value, offset, P, s, G, needs)
+    if native is not None:
+        return native
     cdt = _compute_dtype(value)
     go, a, v, off = (t.contiguous().to(cdt) for t in (grad_output, attn, value, offset))
     ga = _lib.new_out(a) if needs[0] else None

@@ -33,7 +33,7 @@ def test_library_exports_every_declared_symbol():
            and n not in ('sapa_channel_moments_workspace', 'sapa_channel_moments_static_capacity',
                          'sapa_fused_backward_workspace', 'sapa_fused_backward_attn_workspace',
                          'sapa_deform_fused_forward_workspace',
-                         'sapa_deform_fused_backward_workspace')]
+                         'sapa_deform_fused_backward_workspace', 'sapa_deform_backward_workspace')]
     assert sorted(ops) == sorted(_lib.SIGNATURES)
     h = _lib.lib()
     assert h.sapa_channel_moments_workspace(16, 256, 67200, 0) > 0
@@ -45,6 +45,11 @@ def test_library_exports_every_declared_symbol():
     assert h.sapa_deform_fused_forward_workspace(8, 128, 256, 64, 64, 25, 2, 4, _lib.DTYPES[torch.bfloat16]) == 8 * 4096 * (128 + 256) * 2
     assert h.sapa_deform_fused_forward_workspace(8, 128, 256, 64, 64, 5, 2, 4, _lib.DTYPES[torch.float32]) == 0
     assert h.sapa_deform_fused_forward_workspace(8, 128, 256, 64, 64, 25, 2, 4, _lib.DTYPES[torch.float64]) == 0
+    # fp32 copy of the per-point tensor + fp32 accumulator of the low-res gradient; 16-bit tensors only
+    assert (h.sapa_deform_backward_workspace(8, 128, 64, 64, 25, 2, 4, _lib.DTYPES[torch.bfloat16])
+            == 8 * 4 * 25 * 128 * 128 * 4 + 8 * 128 * 4096 * 4)
+    assert h.sapa_deform_backward_workspace(8, 128, 64, 64, 25, 2, 4, _lib.DTYPES[torch.float32]) == 0
+    assert h.sapa_deform_backward_workspace(8, 128, 64, 64, 25, 3, 4, _lib.DTYPES[torch.float16]) == 0
     # the point counts from which the path serves, as include/sapa_hip.h states them:
     # 16-bit tensors from 4 points, fp32 from 13
     bf, f32 = _lib.DTYPES[torch.bfloat16], _lib.DTYPES[torch.float32]

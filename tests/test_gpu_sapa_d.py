@@ -240,6 +240,43 @@ def test_backward_vs_oracle(coracle, shape):
         torch.testing.assert_close(od.grad.cpu(), goff, **tol)
 
 
+SEPARATE_16BIT = [(2, 2, 8, 12, 9, 11, 9, 2, 1.0), (1, 4, 5, 3, 7, 6, 17, 2, 6.0), (1, 1, 4, 6, 5, 4, 5, 4, 2.0),
+                  (1, 2, 6, 4, 10, 9, 13, 1, 1.5), (1, 2, 16, 64, 8, 10, 25, 2, 1.0)]
+
+
+@pytest.mark.parametrize('dtype,rel', [(torch.bfloat16, 1.5e-2), (torch.float16, 2e-3)])
+@pytest.mark.parametrize('shape', SEPARATE_16BIT, ids=['-'.join(map(str, s)) for s in SEPARATE_16BIT])
+def test_separate_backward_16bit_native(coracle, shape, dtype, rel):
+    """deform_qk / deform_av backward on f16 / bf16 tensors through the entry points
+    that read and write them as they are (no fp32 copies of the features): every
+    gradient against the float64 oracle on the rounded inputs, one rounding of the
+    result; and the native path, not the widened fallback, served the call."""
+    from sapa_amd import deform_func
+    B, G, dq, cg, H, W, P, s, oscale = shape
+    g = gen(208)
+    q, key, v, off, attn = make(g, shape[:8], dtype=dtype, off_scale=oscale)
+    go_qk = randn(g, B, G, P, H * s, W * s).to(dtype)
+    go_av = randn(g, B, G * cg, H * s, W * s).to(dtype)
+    d64 = lambda *ts: [t.double() for t in ts]
+
+    # the native entry points take these configurations
+    assert deform_func._backward_16bit('sapa_deform_qk_backward_ws', go_qk.to(DEV), q.to(DEV), key.to(DEV),
+                                       off.to(DEV), P, s, G, (True, True, True)) is not None
+    qd, kd, od = (x.to(DEV).requires_grad_() for x in (q, key, off))
+    sapa_amd.deform_qk(qd, kd, od, P, s, G).backward(go_qk.to(DEV))
+    want = coracle.deform_qk_backward(*d64(go_qk, q, key, off), P, s, G, 'f64')
+    for got, w, name in zip((qd.grad, kd.grad, od.grad), want, ('grad_query', 'grad_key', 'grad_offset')):
+        assert got.dtype == dtype
+        assert_rel_rms_close(got.float().cpu(), w.float(), rel, f'deform_qk {name}')
+
+    ad, vd, od = (x.to(DEV).requires_grad_() for x in (attn, v, off))
+    sapa_amd.deform_av(ad, vd, od, P, s, G).backward(go_av.to(DEV))
+    want = coracle.deform_av_backward(*d64(go_av, attn, v, off), P, s, G, 'f64')
+    for got, w, name in zip((ad.grad, vd.grad, od.grad), want, ('grad_attn', 'grad_value', 'grad_offset')):
+        assert got.dtype == dtype
+        assert_rel_rms_close(got.float().cpu(), w.float(), rel, f'deform_av {name}')
+
+
 # B, G, dq, cg, H, W, P, s, offset scale: partial tiles and chunks; offsets beyond the
 # LDS window; s = 4 and s = 1
 # (B, G, d, cg, H, W, P, s, offset scale).  The first four: one shape the matrix-form
