@@ -93,4 +93,58 @@ __device__ __forceinline__ float reduce_lanes(float v) {
     return x.f;
 }
 
+// ---- vector accesses to the high-res tensors (read or written exactly once: streaming)
+template <typename T, int N>
+struct alignas(sizeof(T) * N) Vec {
+    T v[N];
+};
+
+// Unsigned integer of NB bytes, as the carrier of a streaming access.
+template <int NB> struct Bits;
+template <> struct Bits<2> { typedef unsigned short type; };
+template <> struct Bits<4> { typedef unsigned type; };
+template <> struct Bits<8> { typedef unsigned type __attribute__((ext_vector_type(2))); };
+template <> struct Bits<16> { typedef unsigned type __attribute__((ext_vector_type(4))); };
+
+// The high-res tensors are touched exactly once (q read, output written), so
+// both go around the caches as non-temporal accesses: that leaves L2 to the
+// low-res windows, which neighbouring tiles re-read, and lets partial-line
+// output writes drain without allocating.
+#ifndef SAPA_STREAM_LOADS
+#define SAPA_STREAM_LOADS 1
+#endif
+template <typename T, int N>
+__device__ __forceinline__ Vec<T, N> load_stream(const T *p) {
+    typedef typename Bits<sizeof(T) * N>::type B;
+    union { B b; Vec<T, N> v; } u;
+#if SAPA_STREAM_LOADS
+    u.b = __builtin_nontemporal_load((const B *)p);
+#else
+    u.b = *(const B *)p;
+#endif
+    return u.v;
+}
+template <typename T, int N>
+__device__ __forceinline__ void store_stream(T *p, const Vec<T, N> &v) {
+    typedef typename Bits<sizeof(T) * N>::type B;
+    union { B b; Vec<T, N> v; } u;
+    u.v = v;
+    __builtin_nontemporal_store(u.b, (B *)p);
+}
+
+// The same streaming store through a buffer descriptor: byte offset `off`
+// from the descriptor's base, dropped by the hardware when off + size exceeds
+// the descriptor's extent.
+template <typename T, int N>
+__device__ __forceinline__ void store_buffer(__amdgpu_buffer_rsrc_t r, unsigned off, const Vec<T, N> &v) {
+    typedef typename Bits<sizeof(T) * N>::type B;
+    union { B b; Vec<T, N> v; } u;
+    u.v = v;
+    constexpr int NT_HINT = 2;      // non-temporal
+    if constexpr (sizeof(B) == 2) __builtin_amdgcn_raw_buffer_store_b16(u.b, r, off, 0, NT_HINT);
+    else if constexpr (sizeof(B) == 4) __builtin_amdgcn_raw_buffer_store_b32(u.b, r, off, 0, NT_HINT);
+    else if constexpr (sizeof(B) == 8) __builtin_amdgcn_raw_buffer_store_b64(u.b, r, off, 0, NT_HINT);
+    else __builtin_amdgcn_raw_buffer_store_b128(u.b, r, off, 0, NT_HINT);
+}
+
 }  // namespace sapa

@@ -236,13 +236,25 @@ sapa_b_mfma_kernel(const T *__restrict__ q, const T *__restrict__ key,
     }
 
     if (DO_AV) {
-        T *op = out + (long)n * C * hplane + hpix;
-        const int vbase = lbase + r4 * CS;   // lane with r4 = i fetches channel c0+i
+        // A = the weights (lane 4b+i: child i of parent b, tap k), B = the window values (lane
+        // 4b+j: channel c0+j at tap k of parent b), so lane 4b+j ends up with the 4 children's
+        // results for ITS channel: PXR x-neighbours of 4 / PXR rows, stored as whole vectors.
+        // The stores are buffer stores without a branch: the descriptor covers the channels of
+        // the chunk that exist, idle lanes carry an offset beyond it and the hardware drops them.
+        const int vbase = lbase + r4 * CS;   // lane with r4 = j fetches channel c0+j
+        constexpr int PXR = S >= 4 ? 4 : 2, NROW = 4 / PXR;
+        const int cy0 = (gi * 4) / S, cx0 = (gi * 4) % S;     // first child of the lane's group
+        const long hpg = (long)(py * S + cy0) * hW + (long)px * S + cx0;
+        const unsigned ooff = active ? (unsigned)(hpg * (long)sizeof(T)) : 0x80000000u;
+        const unsigned plane_bytes = (unsigned)(hplane * (long)sizeof(T));
         for (int j = nKc; j < ntot; ++j) {
             if (j + 1 < ntot) stage_load(j + 1);
             const int c0 = cbeg + (j - nKc) * CH;
             const A *wb = lds + (j & 1) * BUF + vbase;
-#pragma unroll 1
+            const int nleft = cend - c0 < CH ? cend - c0 : CH;
+            const __amdgpu_buffer_rsrc_t orsrc = __builtin_amdgcn_make_buffer_rsrc(
+                (void *)(out + ((long)n * C + c0) * hplane), 0, (int)((unsigned)nleft * plane_bytes), 0x00020000);
+#pragma unroll
             for (int cq = 0; cq < CH / 4; ++cq) {
                 const A *wc = wb + cq * 4 * CS;
                 f32x4 o = (f32x4){0.f, 0.f, 0.f, 0.f};
@@ -251,13 +263,16 @@ sapa_b_mfma_kernel(const T *__restrict__ q, const T *__restrict__ key,
 #pragma unroll
                     for (int kx = 0; kx < K; ++kx) {
                         const int k = ky * K + kx;
-                        o = __builtin_amdgcn_mfma_f32_4x4x1f32(wc[ky * RS + kx], w[k / 4][k % 4], o,
+                        o = __builtin_amdgcn_mfma_f32_4x4x1f32(w[k / 4][k % 4], wc[ky * RS + kx], o,
                                                               0, 0, 0);
                     }
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int c = c0 + cq * 4 + i;
-                    if (active && c < cend) store_stream1(op + (long)c * hplane, o[i]);
+                for (int r = 0; r < NROW; ++r) {
+                    Vec<T, PXR> v;
+#pragma unroll
+                    for (int e = 0; e < PXR; ++e) v.v[e] = (T)o[r * PXR + e];
+                    store_buffer<T, PXR>(orsrc, ooff + (unsigned)(cq * 4 + r4) * plane_bytes +
+                                                    (unsigned)(r * hW) * (unsigned)sizeof(T), v);
                 }
             }
             if (j + 1 < ntot) stage_store(j + 1);
@@ -282,6 +297,13 @@ static hipError_t launch_mode(int mode, const void *q, const void *key, const vo
     const int cper = ((C + cgroups - 1) / cgroups + CH - 1) / CH * CH;
     const long nb = (long)tiles_x * tiles_y * B * cgroups;
     if (nb > (1L << 30)) return hipErrorNotSupported;
+    if (mode == TILED_FUSED || mode == TILED_AV) {
+        // the results leave as vectors of 2 (s = 2) or 4 x-neighbours through 32-bit byte
+        // offsets inside one chunk of CH planes
+        const uintptr_t va = (uintptr_t)(sizeof(T) * (S >= 4 ? 4 : 2));
+        if ((uintptr_t)out % va != 0) return hipErrorNotSupported;
+        if ((long)CH * H * S * W * S * (long)sizeof(T) > (1L << 31)) return hipErrorNotSupported;
+    }
     const int per_xcd = (int)((nb + 7) / 8);
     const dim3 grid(per_xcd * 8), block(NT);
 #define SAPA_MM_CASE(M)                                                                        \
