@@ -60,25 +60,28 @@ DEFORM_WORKLOADS = {
 # and the kernel they were measured on.  A run whose dispatched kernel is not
 # that kernel stops with an error instead of printing a stale figure.
 MEASURED_TRAFFIC = {
-    ('fpn_large', 'fp32', 'nchw'): (1819215255, 'profiles/sapa_b_fused_fpn_large_fp32.md', 'sapa_b_tiled_kernel'),
-    ('fpn_large', 'bf16', 'nchw'): (1001271685, 'profiles/sapa_b_fused_fpn_large_bf16.md', 'sapa_b_dot2_kernel'),
-    ('fpn_large', 'fp32', 'channels_last'): (1720501728, 'profiles/sapa_b_nhwc_fused_fpn_large_fp32.md',
+    ('fpn_large', 'fp32', 'nchw'): (1819449685, 'profiles/sapa_b_fused_fpn_large_fp32.md', 'sapa_b_tiled_kernel'),
+    ('fpn_large', 'bf16', 'nchw'): (999139434, 'profiles/sapa_b_fused_fpn_large_bf16.md', 'sapa_b_dot2_kernel'),
+    ('fpn_large', 'fp32', 'channels_last'): (1720502255, 'profiles/sapa_b_nhwc_fused_fpn_large_fp32.md',
                                              'sapa_b_nhwc_kernel'),
-    ('fpn_large', 'bf16', 'channels_last'): (864661437, 'profiles/sapa_b_nhwc_fused_fpn_large_bf16.md',
+    ('fpn_large', 'bf16', 'channels_last'): (864607226, 'profiles/sapa_b_nhwc_fused_fpn_large_bf16.md',
                                              'sapa_b_nhwc16_kernel'),
-    ('stress', 'bf16', 'nchw'): (380752179, 'profiles/sapa_b_mfma_fused_stress_bf16.md', 'sapa_b_mfma_kernel'),
-    ('stress', 'bf16', 'channels_last'): (323093471, 'profiles/sapa_b_nhwc16_fused_stress_bf16.md',
+    ('fpn_small', 'fp32', 'nchw'): (136463102, 'profiles/sapa_b_fused_fpn_small_fp32.md', 'sapa_b_tiled_kernel'),
+    ('segformer_16', 'fp32', 'nchw'): (11933607, 'profiles/sapa_b_mfma_fused_segformer_16_fp32.md',
+                                       'sapa_b_mfma_kernel'),
+    ('stress', 'bf16', 'nchw'): (381156823, 'profiles/sapa_b_mfma_fused_stress_bf16.md', 'sapa_b_mfma_kernel'),
+    ('stress', 'bf16', 'channels_last'): (323149105, 'profiles/sapa_b_nhwc16_fused_stress_bf16.md',
                                           'sapa_b_nhwc16_kernel'),
-    ('deform_p25', 'fp32', 'nchw'): (459885490, 'profiles/sapa_d_wmat_fused_deform_p25_fp32_nchw.md',
+    ('deform_p25', 'fp32', 'nchw'): (459730983, 'profiles/sapa_d_wmat_fused_deform_p25_fp32_nchw.md',
                                      'deform_fused_wmat_kernel'),
-    ('deform_p25', 'bf16', 'nchw'): (228880702, 'profiles/sapa_d_wmat16_fused_deform_p25_bf16_nchw.md',
+    ('deform_p25', 'bf16', 'nchw'): (228881067, 'profiles/sapa_d_wmat16_fused_deform_p25_bf16_nchw.md',
                                      'deform_fused_wmat16_kernel'),
-    ('deform_p25', 'fp32', 'nchw_reference_order'): (829727510, 'profiles/sapa_d_lds_fused_deform_p25_fp32.md',
+    ('deform_p25', 'fp32', 'nchw_reference_order'): (828689742, 'profiles/sapa_d_lds_fused_deform_p25_fp32.md',
                                                      'deform_lds_kernel'),
-    ('deform_p9', 'fp32', 'nchw'): (401608116, 'profiles/sapa_d_lds_fused_deform_p9_fp32.md', 'deform_lds_kernel'),
-    ('deform_p25', 'fp32', 'channels_last'): (356742233, 'profiles/sapa_d_nhwc_fused_deform_p25_fp32.md',
+    ('deform_p9', 'fp32', 'nchw'): (399849952, 'profiles/sapa_d_lds_fused_deform_p9_fp32.md', 'deform_lds_kernel'),
+    ('deform_p25', 'fp32', 'channels_last'): (356737114, 'profiles/sapa_d_nhwc_fused_deform_p25_fp32.md',
                                               'deform_fused_wmat_kernel'),
-    ('deform_p25', 'bf16', 'channels_last'): (178450680, 'profiles/sapa_d_wmat16_fused_deform_p25_bf16.md',
+    ('deform_p25', 'bf16', 'channels_last'): (178447650, 'profiles/sapa_d_wmat16_fused_deform_p25_bf16.md',
                                               'deform_fused_wmat16_kernel'),
 }
 

@@ -36,7 +36,7 @@ bool dtype_ok(int dt) { return dt >= SAPA_F32 && dt <= SAPA_BF16; }
 // 64-bit flat indices and 32-bit in-plane indices cannot overflow
 const long long kMaxElems = 1LL << 40;
 
-// fused fp32 K = 5, s = 2 problems of at most this many low-res cells go to the matrix-pipe kernel
+// fused K = 5, s = 2 problems of at most this many low-res cells go to the matrix-pipe kernel
 const long kSmallFusedCells = 12288;
 
 // LDS-tiled SAPA-B kernel for `mode`: the VALU kernel where it has an
@@ -45,15 +45,16 @@ const long kSmallFusedCells = 12288;
 hipError_t tiled_launch(int mode, const void *q, const void *key, const void *attn_in,
                         const void *value, void *out, int B, int d, int C, int H, int W, int K,
                         int s, int dtype, hipStream_t st) {
-    hipError_t e = took("sapa_b_dot2_kernel", sapa_b_dot2_launch(mode, q, key, attn_in, value, out, B,
-                                                                  d, C, H, W, K, s, dtype, st));
-    // small fp32 problems of the common window: the matrix-pipe kernel's lane-per-child
-    // decomposition fills the chip where the VALU kernel's thread-per-parent one leaves it
-    // latency-bound (B=8, d=32, C=256, fused: 16x16 32 -> 13 us, 32x32 32 -> 23 us)
-    if (e == hipErrorNotSupported && K == 5 && s == 2 && dtype == SAPA_F32 && mode == TILED_FUSED &&
-        (long)B * H * W <= kSmallFusedCells)
+    // small fused problems of the common window first: the matrix-pipe kernel's lane-per-child
+    // decomposition fills the chip where the thread-per-parent kernels leave it latency-bound
+    // (B=8, d=32, C=256, fp32: 16x16 32 -> 12 us, 32x32 32 -> 23 us)
+    hipError_t e = hipErrorNotSupported;
+    if (K == 5 && s == 2 && dtype != SAPA_F64 && mode == TILED_FUSED && (long)B * H * W <= kSmallFusedCells)
         e = took("sapa_b_mfma_kernel",
                  sapa_b_mfma_launch(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, dtype, st));
+    if (e == hipErrorNotSupported)
+        e = took("sapa_b_dot2_kernel", sapa_b_dot2_launch(mode, q, key, attn_in, value, out, B,
+                                                          d, C, H, W, K, s, dtype, st));
     if (e == hipErrorNotSupported)
         e = took("sapa_b_tiled_kernel",
                  sapa_b_tiled_launch(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, dtype, st));

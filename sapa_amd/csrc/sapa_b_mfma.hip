@@ -339,14 +339,12 @@ static hipError_t launch_t(int mode, const void *q, const void *key, const void 
     if (K == KV && s == SV)                                                                    \
         return launch_mode<T, KV, SV, __VA_ARGS__>(mode, q, key, attn_in, value, out, B, d, C, \
                                                    H, W, st);
-    // K = 5, s = 2 in fp32 (the callers send only small problems here: with a lane per child
+    // K = 5, s = 2 (the callers send only small problems here: with a lane per child
     // a launch has four times the waves of the VALU kernel, and a wave alone issues these
     // instructions back to back): 16x4-parent tiles, 16-channel chunks from 4096 cells up
-    if constexpr (sizeof(T) == 4) {
-        if (K == 5 && s == 2 && (long)B * H * W <= 4096)
-            return launch_mode<T, 5, 2, 1, 4, 8, 4>(mode, q, key, attn_in, value, out, B, d, C, H, W, st);
-        SAPA_MM_INST(5, 2, 1, 4, 16, 4)
-    }
+    if (K == 5 && s == 2 && (long)B * H * W <= 4096)
+        return launch_mode<T, 5, 2, 1, 4, 8, 4>(mode, q, key, attn_in, value, out, B, d, C, H, W, st);
+    SAPA_MM_INST(5, 2, 1, 4, 16, 4)
     SAPA_MM_INST(3, 2, 2, 4, 8, 5)
     SAPA_MM_INST(7, 2, 2, 4, 8, 4)
     SAPA_MM_INST(3, 4, 1, 2, 16, 5)

@@ -480,13 +480,11 @@ static hipError_t launch_t(int mode, bool wide, const void *q, const void *key, 
         // Small problems (a few waves per SIMD at most, so a wave's own instruction latencies
         // show): two waves per band of parent rows, each thread with the two children of one
         // hi-res row (half the accumulators, twice the waves), 16-channel chunks (half the
-        // barriers).  Measured at B=16, 25x42, d=64, C=256: 80 -> 59 us.
-        if constexpr (sizeof(T) == 4) {
-            if (mode == TILED_FUSED && !wide && (long)B * H * W <= SAPA_TILED_SMALL_PARENTS)
-                return aligned(2)
-                           ? launch_mode<T, 5, 2, 1, 1, 2, 16, 2, 16>(mode, wide, q, key, attn_in, value, out, B, d, C, H, W, st)
-                           : launch_mode<T, 5, 2, 1, 1, 2, 16, 1, 16>(mode, wide, q, key, attn_in, value, out, B, d, C, H, W, st);
-        }
+        // barriers).  Measured at B=16, 25x42, d=64, C=256, fp32: 80 -> 59 us.
+        if (mode == TILED_FUSED && !wide && (long)B * H * W <= SAPA_TILED_SMALL_PARENTS)
+            return aligned(2)
+                       ? launch_mode<T, 5, 2, 1, 1, 2, 16, 2, 16>(mode, wide, q, key, attn_in, value, out, B, d, C, H, W, st)
+                       : launch_mode<T, 5, 2, 1, 1, 2, 16, 1, 16>(mode, wide, q, key, attn_in, value, out, B, d, C, H, W, st);
 #define SAPA_GEOM(NWX, NWY, VEC, WLX)                                                            \
     launch_mode<T, 5, 2, 2, NWX, NWY, 8, VEC, WLX>(mode, wide, q, key, attn_in, value, out, B, d, C, H, \
                                                    W, st)
