@@ -67,9 +67,9 @@ MEASURED_TRAFFIC = {
     ('fpn_large', 'bf16', 'channels_last'): (864607226, 'profiles/sapa_b_nhwc_fused_fpn_large_bf16.md',
                                              'sapa_b_nhwc16_kernel'),
     ('fpn_small', 'fp32', 'nchw'): (136463102, 'profiles/sapa_b_fused_fpn_small_fp32.md', 'sapa_b_tiled_kernel'),
-    ('segformer_16', 'fp32', 'nchw'): (11933607, 'profiles/sapa_b_mfma_fused_segformer_16_fp32.md',
+    ('segformer_16', 'fp32', 'nchw'): (11936679, 'profiles/sapa_b_mfma_fused_segformer_16_fp32.md',
                                        'sapa_b_mfma_kernel'),
-    ('stress', 'bf16', 'nchw'): (381156823, 'profiles/sapa_b_mfma_fused_stress_bf16.md', 'sapa_b_mfma_kernel'),
+    ('stress', 'bf16', 'nchw'): (371333608, 'profiles/sapa_b_mfma_fused_stress_bf16.md', 'sapa_b_mfma_kernel'),
     ('stress', 'bf16', 'channels_last'): (323149105, 'profiles/sapa_b_nhwc16_fused_stress_bf16.md',
                                           'sapa_b_nhwc16_kernel'),
     ('deform_p25', 'fp32', 'nchw'): (459730983, 'profiles/sapa_d_wmat_fused_deform_p25_fp32_nchw.md',
