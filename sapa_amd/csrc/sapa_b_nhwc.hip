@@ -40,6 +40,7 @@
 // order: results agree with them to rounding (1e-5 relative in fp32), not bit
 // for bit.  Out-of-range window positions are zeros in LDS: logit exactly 0
 // (and part of the softmax), contribution exactly 0.
+#include <type_traits>
 #include <utility>
 
 #include "kernels.hpp"
@@ -152,7 +153,16 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
     typedef Quad<T> Q4;
     typedef typename Q4::raw Raw;
 
-    __shared__ __attribute__((aligned(16))) float lds[2 * BUF];
+    // fp32 windows go from global memory straight into LDS (buffer loads with the LDS
+    // modifier; thread t of pass p fills the 16-byte slot p * NT + t, which is the layout
+    // below): no staging registers and no LDS write instructions.  A wave's load fills 64
+    // consecutive slots, so a buffer is a whole number of those.
+#ifndef SAPA_NHWC_DMA
+#define SAPA_NHWC_DMA 1
+#endif
+    constexpr bool DMA = SAPA_NHWC_DMA && std::is_same<T, float>::value;
+    constexpr int BUFA = DMA ? (BUF + 255) / 256 * 256 : BUF;
+    __shared__ __attribute__((aligned(16))) float lds[2 * BUFA];
 
     const int logical = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
     if (logical >= nblocks) return;
@@ -184,6 +194,8 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
         spix[p] = (pos < NPOS && gy >= 0 && gy < H && gx >= 0 && gx < W) ? gy * W + gx : -1;
     }
     const int sq = tid & 15;                      // channel quad staged by this thread
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    (void)wave_u;
     Raw st[NPASS];
     auto stage_load = [&](int j) {
         const bool is_key = j < nKc;
@@ -198,11 +210,31 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
             const u32 off = (c_ok && spix[p] >= 0)
                                 ? (u32)(spix[p] * nch + c0 + 4 * sq) * (u32)sizeof(T)
                                 : 0x80000000u;
-            st[p] = Q4::buffer_load(r, off);
+            if constexpr (DMA) {
+                // (device pass only: the host pass, which sees this body for the launch
+                // stub, does not know the builtin)
+#if defined(__HIP_DEVICE_COMPILE__)
+                const int slot0 = p * NT + wave_u * 64;      // first slot of this wave's load
+                if ((p + 1) * NT <= NPOS * 16 || slot0 < NPOS * 16)
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                        r, (__attribute__((address_space(3))) void *)(lds + (j & 1) * BUFA + slot0 * 4), 16,
+                        off, 0, 0, 0);
+#endif
+            } else {
+                st[p] = Q4::buffer_load(r, off);
+            }
         }
     };
+    // registers -> LDS; direct-to-LDS: wait for the loads (the counter retires in issue
+    // order, so that is a wait for everything issued before them as well)
     auto stage_store = [&](int j) {
-        float *dst = lds + (j & 1) * BUF;
+        if constexpr (DMA) {
+#if defined(__HIP_DEVICE_COMPILE__)
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#endif
+            return;
+        }
+        float *dst = lds + (j & 1) * BUFA;
 #pragma unroll
         for (int p = 0; p < NPASS; ++p) {
             const int pos = p * (NT / 16) + tid / 16;
@@ -210,6 +242,18 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
         }
     };
 
+    // every wave is done with the current window and the next one is in LDS (direct-to-LDS:
+    // the bare barrier instruction -- the loads were waited for above, and a fence here
+    // would drain the output stores issued since)
+    auto chunk_barrier = [&]() {
+        if constexpr (DMA) {
+#if defined(__HIP_DEVICE_COMPILE__)
+            asm volatile("s_barrier" ::: "memory");
+#endif
+        } else {
+            __syncthreads();
+        }
+    };
     // this row's window origin: tap (ky, kx) of its parent sits at position
     // (wy + ky) * WW + 4 wx + row + kx
     const float *win = lds + ((wy * WW + 4 * wx + row) * CHK + 4 * li);
@@ -245,14 +289,14 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
     if (DO_QK) load_q(0, 0);
     stage_load(0);
     stage_store(0);
-    __syncthreads();
+    chunk_barrier();
 
     if (DO_QK) {
 #pragma unroll
         for (int i = 0; i < NR; ++i) w[i] = 0.f;
         for (int j = 0; j < nKc; ++j) {
             if (j + 1 < ntot) stage_load(j + 1);
-            const float *wb = win + (j & 1) * BUF;
+            const float *wb = win + (j & 1) * BUFA;
 #pragma unroll
             for (int g = 0; g < NG; ++g) {
                 f32x4 qv[4];
@@ -293,7 +337,7 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
                 }
             }
             if (j + 1 < ntot) stage_store(j + 1);
-            __syncthreads();
+            chunk_barrier();
         }
         if (DO_SOFTMAX) {
             // a child's taps lie in this lane's registers of its group and in the
@@ -356,7 +400,7 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
         for (int j = nKc; j < ntot; ++j) {
             if (j + 1 < ntot) stage_load(j + 1);
             const int c0 = (j - nKc) * CHK;
-            const float *wb = win + (j & 1) * BUF;
+            const float *wb = win + (j & 1) * BUFA;
             // acc[g][u][i]: child 4g + i, channel c0 + 4 li + u
             f32x4 acc[NG][4];
 #pragma unroll
@@ -399,7 +443,7 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
                                          acc[jj / 4][2][jj % 4], acc[jj / 4][3][jj % 4]}),
                         (Raw *)(out + child_pixel(jj) * C + c0 + 4 * li));
             }
-            __syncthreads();
+            chunk_barrier();
         }
     }
 }

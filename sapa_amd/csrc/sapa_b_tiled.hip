@@ -71,7 +71,17 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
     // LDS row: two channels side by side, each HALF > WW floats wide (spare
     // columns absorb surplus staging lanes) with HALF = 8 mod 16, so the row
     // stride is 16 mod 32
-    constexpr int HALF = ((WW + VEC - 8 + 15) / 16) * 16 + 8, STRIDE = 2 * HALF;
+#ifndef SAPA_TILED_OPAQUE_BASE
+#define SAPA_TILED_OPAQUE_BASE 1
+#endif
+#ifndef SAPA_TILED_PLAIN_ROWS
+#define SAPA_TILED_PLAIN_ROWS 1
+#endif
+    constexpr bool PAIRED = WLX == 16 || !SAPA_TILED_PLAIN_ROWS;
+    constexpr int HALF = PAIRED ? ((WW + VEC - 8 + 15) / 16) * 16 + 8 : (WW + VEC + 3) / 4 * 4;
+    constexpr int STRIDE = PAIRED ? 2 * HALF : HALF;
+    // float offset of channel ch of a chunk inside a buffer
+    auto ch_off = [](int ch) { return PAIRED ? (ch >> 1) * WH * STRIDE + (ch & 1) * HALF : ch * WH * STRIDE; };
     constexpr int NVR = WW / VEC, NVP = WH * NVR;   // vectors per row / per channel
     // staging threads are split into NSL slices that take every NSL-th channel
     constexpr int NSL = (CH % 4 == 0 && NT >= 4 * NVP && NT % 256 == 0) ? 4
@@ -80,12 +90,12 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
     constexpr int NPOS = (NVP + TPC - 1) / TPC;     // vectors per thread and channel
     constexpr int CPT = CH / NSL;                   // channels per thread
     constexpr int NSTAGE = CPT * NPOS * VEC;
-    constexpr int BUF = (CH / 2) * WH * STRIDE;
+    constexpr int BUF = (PAIRED ? CH / 2 : CH) * WH * STRIDE;
     constexpr int NJ = CY * S;             // children per thread
     constexpr bool DO_QK = MODE != TILED_AV;
     constexpr bool DO_SOFTMAX = MODE == TILED_QK_SOFTMAX || MODE == TILED_FUSED;
     constexpr bool DO_AV = MODE == TILED_AV || MODE == TILED_FUSED;
-    static_assert(WW + VEC <= HALF && STRIDE % 32 == 16, "LDS row layout");
+    static_assert(WW + VEC <= HALF && (!PAIRED || STRIDE % 32 == 16), "LDS row layout");
     static_assert(TPC % 64 == 0 && CH % NSL == 0, "staging slices are whole waves");
     typedef Vec<T, VEC> VecV;
     static_assert(CH % 2 == 0, "channels are staged in pairs");
@@ -97,7 +107,23 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
     typedef Vec<TA, S> VecA;
     const TA *attn_w = reinterpret_cast<const TA *>(attn_in);
 
-    __shared__ __attribute__((aligned(16))) A lds[2 * BUF];
+    // fp32 windows staged as 16-byte vectors go from global memory straight into LDS
+    // (buffer loads with the LDS modifier): no staging registers, no LDS write instructions,
+    // and the hardware's zero for an out-of-range offset is the window's zero padding.
+#ifndef SAPA_TILED_DMA
+#define SAPA_TILED_DMA 1
+#endif
+    constexpr bool DMA = SAPA_TILED_DMA && std::is_same<T, float>::value && VEC == 4;
+    // a wave's load fills 64 consecutive 16-byte slots: buffers are whole numbers of those
+    constexpr int BUFA = DMA ? (BUF + 255) / 256 * 256 : BUF;
+    constexpr int NW = NT / 64, NBLK = BUFA / 256;   // waves; 64-slot blocks per buffer
+    constexpr int NLD = DMA ? (NBLK + NW - 1) / NW : 1;       // loads per wave and chunk
+    // vector memory operations a wave issues per chunk after its staging loads (q loads in
+    // the logits phase, output stores in the aggregation): the staging loads have landed
+    // when no more than these are outstanding
+    constexpr int NAFTER = CH * CY;
+    static_assert(STRIDE % 4 == 0 && HALF % 4 == 0 && NAFTER < 64, "direct-to-LDS staging");
+    __shared__ __attribute__((aligned(16))) A lds[2 * BUFA];
 
     // Workgroups are handed to the 8 XCDs round-robin; give each XCD a
     // contiguous run of tiles so that neighbouring tiles (which share halo
@@ -138,8 +164,10 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
     // window of channels sl, sl+NSL, ... of a chunk, so the per-thread part
     // of each address (in-plane offset, LDS offset, inside-the-image mask) is
     // fixed for the whole kernel and the channel part is wave-uniform.
-    const int sl = tid / TPC, vt = tid % TPC;
-    int g_off[NPOS], l_off[NPOS];
+    // (a slice is whole waves: its number is wave-uniform, and so is every channel address)
+    const int sl = __builtin_amdgcn_readfirstlane(tid / TPC), vt = tid % TPC;
+    unsigned g_off[NPOS];   // byte offset inside a channel plane
+    int l_off[NPOS];
     unsigned g_mask[NPOS];
 #pragma unroll
     for (int i = 0; i < NPOS; ++i) {
@@ -151,29 +179,78 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
         const bool g_ok = l_ok && gy >= 0 && gy < H && gx >= 0 && gx + VEC <= W;
         const int yy = gy < 0 ? 0 : (gy < H ? gy : H - 1);
         const int xx = gx < 0 ? 0 : (gx + VEC <= W ? gx : W - VEC);
-        g_off[i] = yy * W + xx;             // clamped: always a legal address
+        g_off[i] = (unsigned)(yy * W + xx) * (unsigned)sizeof(T);   // clamped: always a legal address
         g_mask[i] = g_ok ? 0xffffffffu : 0u;
         // surplus vectors land in the unread spare columns of row 0
         l_off[i] = l_ok ? row * STRIDE + col : WW;
     }
+    // Direct-to-LDS map: load i of wave w fills slots ((i * NW + w) * 64 + lane) of a buffer;
+    // the slot's place in the LDS layout gives the channel of the chunk and the window
+    // position it holds, i.e. a byte offset from the chunk's first plane -- or 2^31 (out of
+    // any range: the hardware writes zeros) for padding columns, positions outside the
+    // image and the tail of the last block.  Channels past the last one fall outside the
+    // descriptor the same way.
+    const int wave_u = __builtin_amdgcn_readfirstlane(tid >> 6);
+    unsigned d_off[NLD];
+    if constexpr (DMA) {
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            const int f = (((i * NW + wave_u) * 64) + (tid & 63)) * 4;   // float index in the buffer
+            const int prow = f / STRIDE, cf = f % STRIDE;
+            const int half = PAIRED && cf >= HALF ? 1 : 0;
+            const int col = cf - half * HALF;
+            const int ch = PAIRED ? (prow / WH) * 2 + half : prow / WH;
+            const int gy = y0 - R + prow % WH, gx = x0 - HL + col;
+            const bool ok = f < BUF && col < WW && gy >= 0 && gy < H && gx >= 0 && gx + VEC <= W;
+            d_off[i] = ok ? (unsigned)ch * (unsigned)(lplane * (long)sizeof(T)) +
+                                (unsigned)(gy * W + gx) * (unsigned)sizeof(T)
+                          : 0x80000000u;
+        }
+    }
     A st[NSTAGE];
-    // global -> registers for staged chunk j (key chunks first, then value)
+    // global -> registers (or straight into LDS buffer j&1) for staged chunk j (key chunks
+    // first, then value)
     auto stage_load = [&](int j) {
         const bool is_key = j < nKc;
         const T *src = is_key ? key : value;
         const int nch = is_key ? d : C;
         const int c0 = is_key ? j * CH : cbeg + (j - nKc) * CH;
+        if constexpr (DMA) {
+            // (device pass only: the host pass, which sees this body for the launch stub,
+            // knows neither the builtin nor the instructions of the chunk barrier)
+#if defined(__HIP_DEVICE_COMPILE__)
+            const int nleft = nch - c0 < CH ? nch - c0 : CH;
+            const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+                (void *)(src + ((long)n * nch + c0) * lplane), 0,
+                (int)((unsigned)nleft * (unsigned)(lplane * (long)sizeof(T))), 0x00020000);
+            A *dst = lds + (j & 1) * BUFA;
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) {
+                const int blk = i * NW + wave_u;
+                if ((i + 1) * NW <= NBLK || blk < NBLK)
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                        rsrc, (__attribute__((address_space(3))) void *)(dst + blk * 256), 16, d_off[i], 0, 0, 0);
+            }
+            // everything below is issued after these loads (the wait at the end of the
+            // chunk counts on it)
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+#endif
+            return;
+        }
         const T *base = src + (long)n * nch * lplane;
 #pragma unroll
         for (int ci = 0; ci < CPT; ++ci) {
             const int c = c0 + sl + ci * NSL;
-            const T *plane = base + (long)(c < nch ? c : nch - 1) * lplane;
+            const char *plane = (const char *)(base + (long)(c < nch ? c : nch - 1) * lplane);
 #pragma unroll
             for (int i = 0; i < NPOS; ++i) {
                 // unconditional load from the clamped address; the value is
                 // masked when it is stored to LDS, so that the load stays in
                 // flight across the FMAs of the current chunk
-                const VecV v = *(const VecV *)(plane + g_off[i]);
+                unsigned o = g_off[i];
+                asm volatile("" : "+v"(o));
+                const VecV v = *(const VecV *)(plane + o);
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) st[(ci * NPOS + i) * VEC + e] = (A)v.v[e];
             }
@@ -182,14 +259,15 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
     // registers -> LDS buffer j&1, zeroing what lies outside the image or
     // past the last channel
     auto stage_store = [&](int j) {
+        if constexpr (DMA) return;
         const bool is_key = j < nKc;
         const int nch = is_key ? d : C;
         const int c0 = is_key ? j * CH : cbeg + (j - nKc) * CH;
-        A *dst = lds + (j & 1) * BUF;
+        A *dst = lds + (j & 1) * BUFA;
 #pragma unroll
         for (int ci = 0; ci < CPT; ++ci) {
             const int ch = sl + ci * NSL;
-            A *dc = dst + (ch >> 1) * WH * STRIDE + (ch & 1) * HALF;
+            A *dc = dst + ch_off(ch);
 #pragma unroll
             for (int i = 0; i < NPOS; ++i) {
                 const unsigned m = c0 + ch < nch ? g_mask[i] : 0u;
@@ -221,13 +299,31 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
             }
     }
     stage_store(0);
-    __syncthreads();
+    // End of a chunk: the next chunk's window is in LDS and every wave is done with this one.
+    // (Direct-to-LDS: wait until only the operations issued after the staging loads are
+    // outstanding -- the counter retires in issue order -- so output stores stay in flight.)
+    auto chunk_barrier = [&](bool staged, bool first) {
+        if constexpr (DMA) {
+#if defined(__HIP_DEVICE_COMPILE__)
+            if (first) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            else if (staged) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NAFTER) : "memory");
+            asm volatile("s_barrier" ::: "memory");
+#endif
+        } else {
+            __syncthreads();
+        }
+    };
+    chunk_barrier(true, true);
 
     // this thread's window origin in buffer 0 (its neighbour kx = 0 column)
-    const A *win = lds + ly * STRIDE + lx + (HL - R);
+    const A *win = lds + ly * STRIDE + lx + (HL - R);   // (buffer 1 is BUFA floats further)
 
     if (DO_QK) {
-        const T *qp = q + (long)n * d * hplane + hpix_ld;
+        // (wave-uniform plane address + a 32-bit per-lane byte offset: no per-lane address arithmetic)
+        const char *qp = (const char *)(q + (long)n * d * hplane);
+        unsigned qoff[CY];
+#pragma unroll
+        for (int cy = 0; cy < CY; ++cy) qoff[cy] = (unsigned)((hpix_ld + (long)cy * hW) * (long)sizeof(T));
         const unsigned qmask = active ? 0xffffffffu : 0u;
         // q is fetched PF channels ahead of its use (a ring of PF x NJ
         // registers), so HBM latency hides behind the FMAs of PF channels.
@@ -243,8 +339,12 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
         auto load_q = [&](int c, A (&dst)[NJ]) {
 #pragma unroll
             for (int cy = 0; cy < CY; ++cy) {
-                const VecS v =
-                    load_stream<T, S>(qp + (long)(c < d ? c : d - 1) * hplane + (long)cy * hW);
+                const char *plane = qp + (long)(c < d ? c : d - 1) * hplane * (long)sizeof(T);
+                // (the offset is widened next to its use, or the compiler keeps a 64-bit copy
+                // of it and adds the plane address per lane)
+                unsigned o = qoff[cy];
+                asm volatile("" : "+v"(o));
+                const VecS v = load_stream<T, S>((const T *)(plane + o));
 #pragma unroll
                 for (int cx = 0; cx < S; ++cx) dst[cy * S + cx] = (A)v.v[cx];
             }
@@ -254,7 +354,7 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
         for (int j = 0; j < nKc; ++j) {
             if (j + 1 < ntot) stage_load(j + 1);
             const int c0 = j * CH;
-            const A *wb = win + (j & 1) * BUF;
+            const A *wb = win + (j & 1) * BUFA;
 #pragma unroll 1
             for (int ch0 = 0; ch0 < CH; ch0 += PF) {
 #pragma unroll
@@ -268,7 +368,11 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
                     for (int jj = 0; jj < NJ; ++jj)
                         qv[jj] = __uint_as_float(__float_as_uint(qr[u][jj]) & m);
                     load_q(c0 + ch + PF, qr[u]);
-                    const A *wc = wb + (ch >> 1) * WH * STRIDE + (ch & 1) * HALF;
+                    int co = ch_off(ch);
+#if SAPA_TILED_OPAQUE_BASE
+                    asm volatile("" : "+v"(co));
+#endif
+                    const A *wc = wb + co;
 #pragma unroll
                     for (int ky = 0; ky < K; ++ky)
 #pragma unroll
@@ -284,7 +388,7 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
                 }
             }
             if (j + 1 < ntot) stage_store(j + 1);
-            __syncthreads();
+            chunk_barrier(j + 1 < ntot, false);
         }
         if (DO_SOFTMAX) {
 #pragma unroll
@@ -348,13 +452,17 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
         for (int j = nKc; j < ntot; ++j) {
             if (j + 1 < ntot) stage_load(j + 1);
             const int c0 = cbeg + (j - nKc) * CH;
-            const A *wb = win + (j & 1) * BUF;
+            const A *wb = win + (j & 1) * BUFA;
             const int nleft = cend - c0 < CH ? cend - c0 : CH;
             const __amdgpu_buffer_rsrc_t orsrc = __builtin_amdgcn_make_buffer_rsrc(
                 (void *)(out + ((long)n * C + c0) * hplane), 0, (int)((unsigned)nleft * plane_bytes), 0x00020000);
 #pragma unroll
             for (int ch = 0; ch < CH; ++ch) {
-                const A *wc = wb + (ch >> 1) * WH * STRIDE + (ch & 1) * HALF;
+                int co = ch_off(ch);
+#if SAPA_TILED_OPAQUE_BASE
+                    asm volatile("" : "+v"(co));
+#endif
+                    const A *wc = wb + co;
                 A o[NJ];
 #pragma unroll
                 for (int jj = 0; jj < NJ; ++jj) o[jj] = 0;
@@ -380,7 +488,7 @@ sapa_b_tiled_kernel(const T *__restrict__ q, const T *__restrict__ key,
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (j + 1 < ntot) stage_store(j + 1);
-            __syncthreads();
+            chunk_barrier(j + 1 < ntot, false);
         }
     }
 }
@@ -481,16 +589,30 @@ static hipError_t launch_t(int mode, bool wide, const void *q, const void *key, 
         // show): two waves per band of parent rows, each thread with the two children of one
         // hi-res row (half the accumulators, twice the waves), 16-channel chunks (half the
         // barriers).  Measured at B=16, 25x42, d=64, C=256, fp32: 80 -> 59 us.
-        if (mode == TILED_FUSED && !wide && (long)B * H * W <= SAPA_TILED_SMALL_PARENTS)
+        // (fp32 windows of 16-wide tiles are also staged as 4-element vectors where the rows
+        // allow it, 4 columns wider: those go straight into LDS.  25x42-class shapes measured
+        // 59 -> 57 us, the 16 x 8 tiles 85 -> 73 us, the 16 x 16 tiles 66 -> 60 us.)
+        constexpr bool F32 = std::is_same<T, float>::value;
+        if (mode == TILED_FUSED && !wide && (long)B * H * W <= SAPA_TILED_SMALL_PARENTS) {
+            if constexpr (F32)
+                if (aligned(4))
+                    return launch_mode<T, 5, 2, 1, 1, 2, 16, 4, 16>(mode, wide, q, key, attn_in, value, out, B, d, C, H, W, st);
             return aligned(2)
                        ? launch_mode<T, 5, 2, 1, 1, 2, 16, 2, 16>(mode, wide, q, key, attn_in, value, out, B, d, C, H, W, st)
                        : launch_mode<T, 5, 2, 1, 1, 2, 16, 1, 16>(mode, wide, q, key, attn_in, value, out, B, d, C, H, W, st);
+        }
 #define SAPA_GEOM(NWX, NWY, VEC, WLX)                                                            \
     launch_mode<T, 5, 2, 2, NWX, NWY, 8, VEC, WLX>(mode, wide, q, key, attn_in, value, out, B, d, C, H, \
                                                    W, st)
         if (c22 <= c12 && c22 <= c14)
             return aligned(4) ? SAPA_GEOM(1, 4, 4, 32) : SAPA_GEOM(1, 4, 1, 32);
-        if (c14 <= c12) return aligned(2) ? SAPA_GEOM(1, 4, 2, 16) : SAPA_GEOM(1, 4, 1, 16);
+        if (c14 <= c12) {
+            if constexpr (F32)
+                if (aligned(4)) return SAPA_GEOM(1, 4, 4, 16);
+            return aligned(2) ? SAPA_GEOM(1, 4, 2, 16) : SAPA_GEOM(1, 4, 1, 16);
+        }
+        if constexpr (F32)
+            if (aligned(4)) return SAPA_GEOM(1, 2, 4, 16);
         return aligned(2) ? SAPA_GEOM(1, 2, 2, 16) : SAPA_GEOM(1, 2, 1, 16);
 #undef SAPA_GEOM
 #endif
