@@ -404,11 +404,15 @@ static hipError_t launch_t(int mode, const void *q, const void *key, const void 
                            int H, int W, int K, int s, hipStream_t st) {
     // fp32: the variant with the logits on the matrix pipe (sapa_b_nhwc_mm.hip) for the
     // large windows / up-factors, whose arithmetic shows: measured faster there (K = 7, s = 4
-    // at B=4, C=512, 64x64: 234 -> 194 us), 5 % slower at (5, 2) on large memory-bound shapes
-    // and 5-8 % faster on cache-resident ones.  The choice depends on (K, s) alone so that a
-    // batch and its images one by one take the same kernel (bit-identical results).
+    // at B=4, C=512, 64x64: 234 -> 194-206 us), 3-6 % slower at (5, 2).  The choice depends on
+    // (K, s) alone so that a batch and its images one by one take the same kernel
+    // (bit-identical results).
     if constexpr (std::is_same<T, float>::value)
+#ifdef SAPA_NHWC_MM_ALL
+        if (true)
+#else
         if (K == 7 || s == 4)
+#endif
             return launch_mm(mode, q, key, attn_in, value, qbias, out, B, d, C, H, W, K, s, st);
 #define SAPA_NHWC_KS(KV, SV)                                                                  \
     if (K == KV && s == SV)                                                                   \

@@ -25,9 +25,9 @@
 // Positions are 68 floats apart in LDS (64 of data): the 4 lanes of a quad read 4
 // consecutive positions and the 4 quads 4 blocks of 16 bytes, which then fall on
 // disjoint banks.  Measured against sapa_b_nhwc.hip on MI355X: faster where the
-// arithmetic shows (K = 7, s = 4: 234 -> 194 us at B=4, C=512, 64x64; cache-resident
-// (5, 2) shapes 5-8 %), 5 % slower at (5, 2) on large memory-bound shapes -- the launcher
-// of sapa_b_nhwc.hip sends K = 7 and s = 4 here.
+// arithmetic shows (K = 7, s = 4: 234 -> 194-206 us at B=4, C=512, 64x64), 3-6 % slower at
+// (5, 2) -- the launcher of sapa_b_nhwc.hip sends K = 7 and s = 4 here (SAPA_NHWC_MM_ALL
+// in a tuning build: everything).
 //
 // The channel sums run in the order above, not in the reference kernels' sequential
 // order: results agree with them to rounding (1e-5 relative), not bit for bit.
