@@ -431,7 +431,7 @@ static int nhwc_common(int mode, const void *query, const void *key, const void 
                                              dtype, (hipStream_t)stream));
 #endif
     if (e == hipErrorNotSupported)
-        e = took("sapa_b_nhwc_kernel", sapa_b_nhwc_launch(mode, query, key, attn, value, q_bias, out, B, d, C,
+        e = took(sapa_b_nhwc_kernel_name(K, s, dtype), sapa_b_nhwc_launch(mode, query, key, attn, value, q_bias, out, B, d, C,
                                                           H, W, K, s, dtype, (hipStream_t)stream));
     if (e == hipErrorNotSupported) return SAPA_ERR_UNSUPPORTED;
     return finish(e);

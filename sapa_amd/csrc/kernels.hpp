@@ -39,6 +39,8 @@ hipError_t sapa_b_tiled_launch(int mode, const void *q, const void *key, const v
 hipError_t sapa_b_nhwc_launch(int mode, const void *q, const void *key, const void *attn_in,
                               const void *value, const void *qbias, void *out, int B, int d, int C,
                               int H, int W, int K, int s, int dtype, hipStream_t st);
+// the kernel template sapa_b_nhwc_launch sends (K, s, dtype) to
+const char *sapa_b_nhwc_kernel_name(int K, int s, int dtype);
 
 // sapa_b_nhwc16.hip: the same four modes for f16 / bf16 channels-last tensors
 // on the 16-bit matrix instructions (hipErrorNotSupported for anything else)

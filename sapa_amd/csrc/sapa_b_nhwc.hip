@@ -398,6 +398,16 @@ static hipError_t launch_geom(int mode, const void *q, const void *key, const vo
     return hipGetLastError();
 }
 
+// fp32 cases of the kernel with the logits on the matrix pipe (SAPA_NHWC_MM_ALL in a tuning
+// build: all of them)
+static bool takes_mm(int K, int s) {
+#ifdef SAPA_NHWC_MM_ALL
+    return true;
+#else
+    return K == 7 || s == 4;
+#endif
+}
+
 template <typename T>
 static hipError_t launch_t(int mode, const void *q, const void *key, const void *attn_in,
                            const void *value, const void *qbias, void *out, int B, int d, int C,
@@ -408,11 +418,7 @@ static hipError_t launch_t(int mode, const void *q, const void *key, const void 
     // (K, s) alone so that a batch and its images one by one take the same kernel
     // (bit-identical results).
     if constexpr (std::is_same<T, float>::value)
-#ifdef SAPA_NHWC_MM_ALL
-        if (true)
-#else
-        if (K == 7 || s == 4)
-#endif
+        if (takes_mm(K, s))
             return launch_mm(mode, q, key, attn_in, value, qbias, out, B, d, C, H, W, K, s, st);
 #define SAPA_NHWC_KS(KV, SV)                                                                  \
     if (K == KV && s == SV)                                                                   \
@@ -424,6 +430,10 @@ static hipError_t launch_t(int mode, const void *q, const void *key, const void 
 }
 
 }  // namespace nhwc
+
+const char *sapa_b_nhwc_kernel_name(int K, int s, int dtype) {
+    return dtype == 0 && nhwc::takes_mm(K, s) ? "sapa_b_nhwc_mm_kernel" : "sapa_b_nhwc_kernel";
+}
 
 // Channels-last tensors (q [B, sH, sW, d], key [B, H, W, d], value [B, H, W, C],
 // attn [B, sH, sW, K*K], out like q with C or K*K channels), f32 / f16 / bf16,
