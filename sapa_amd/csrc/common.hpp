@@ -147,4 +147,37 @@ __device__ __forceinline__ void store_buffer(__amdgpu_buffer_rsrc_t r, unsigned 
     else __builtin_amdgcn_raw_buffer_store_b128(u.b, r, off, 0, NT_HINT);
 }
 
+// ---- butterfly step over lane distance 4 or 8 inside rows of 16 lanes (channels-last kernels)
+// For a pair of per-lane values (a, b): the lanes whose bit D is clear get a + (a of lane ^ D),
+// the others b + (b of lane ^ D) -- each lane keeps one of the two sums and adds what its
+// partner held of it.  Two DPP additions and no select: the lanes with the bit clear are
+// whole banks of 4 lanes (banks 0, 2 for distance 4; 0, 1 for distance 8), which the
+// instruction's bank mask can pick, and their partners are a row rotation away (by 12 / 4
+// lanes for distance 4, by 8 for distance 8).  Lanes outside the mask keep what the other
+// instruction wrote.  (s_nop 1: the two wait states a DPP read needs after the vector
+// instruction that wrote its source.)
+#ifndef SAPA_NHWC_DPP_HALVE
+#define SAPA_NHWC_DPP_HALVE 1
+#endif
+template <int D>
+__device__ __forceinline__ float pair_sum_dpp(float a, float b) {
+    static_assert(D == 4 || D == 8, "lane distance");
+    float r;
+#if defined(__HIP_DEVICE_COMPILE__)
+    if constexpr (D == 4)
+        asm volatile("s_nop 1\n\t"
+                     "v_add_f32_dpp %0, %1, %1 row_ror:12 row_mask:0xf bank_mask:0x5\n\t"
+                     "v_add_f32_dpp %0, %2, %2 row_ror:4 row_mask:0xf bank_mask:0xa"
+                     : "=&v"(r) : "v"(a), "v"(b));
+    else
+        asm volatile("s_nop 1\n\t"
+                     "v_add_f32_dpp %0, %1, %1 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+                     "v_add_f32_dpp %0, %2, %2 row_ror:8 row_mask:0xf bank_mask:0xc"
+                     : "=&v"(r) : "v"(a), "v"(b));
+#else
+    r = a + b;
+#endif
+    return r;
+}
+
 }  // namespace sapa

@@ -74,17 +74,25 @@ __device__ __forceinline__ float row_xor(float v, int lane) {
 // One butterfly step over lane distance D: n values per lane -> (n + 1) / 2.
 // The lane whose bit D is clear keeps the even-indexed sums, its partner the
 // odd-indexed ones; each adds what the other held of them.
-template <int D, int N>
+// Distances 4 and 8 take two DPP additions per result and no select (pair_sum_dpp) when
+// FROM_VALU says that the inputs were written by ordinary vector instructions: the wait
+// states inside pair_sum_dpp cover those, not a matrix instruction's result (the compiler
+// cannot see into the instruction text to add the longer wait itself).
+template <int D, int N, bool FROM_VALU = true>
 __device__ __forceinline__ void halve(const float (&in)[N], float (&out)[(N + 1) / 2], int lane) {
     const bool hi = lane & D;
+    (void)hi;
 #pragma unroll
     for (int m = 0; m < (N + 1) / 2; ++m) {
         const float a = in[2 * m], b = 2 * m + 1 < N ? in[2 * m + 1] : 0.f;
-        const float keep = hi ? b : a, send = hi ? a : b;
-        out[m] = keep + row_xor<D>(send, lane);
+        if constexpr (SAPA_NHWC_DPP_HALVE && FROM_VALU && (D == 4 || D == 8)) {
+            out[m] = pair_sum_dpp<D>(a, b);
+        } else {
+            const float keep = hi ? b : a, send = hi ? a : b;
+            out[m] = keep + row_xor<D>(send, lane);
+        }
     }
 }
-
 
 // sapa_b_nhwc_mm.hip: the same four modes with the logits on the matrix pipe (fp32 tensors)
 hipError_t launch_mm(int mode, const void *q, const void *key, const void *attn_in, const void *value,

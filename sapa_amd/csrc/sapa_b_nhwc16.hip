@@ -98,15 +98,22 @@ __device__ __forceinline__ float row_xor(float v, int lane) {
 }
 // One butterfly step over lane distance D: n values per lane -> n / 2.  The lane
 // whose bit D is clear keeps the even-indexed sums, its partner the odd-indexed
-// ones; each adds what the other held of them.
-template <int D, int N>
+// ones; each adds what the other held of them.  FROM_VALU: the inputs were written by
+// ordinary vector instructions -- then two DPP additions per result do it
+// (pair_sum_dpp, whose wait states cover those, not a matrix instruction's result).
+template <int D, int N, bool FROM_VALU>
 __device__ __forceinline__ void halve(const float (&in)[N], float (&out)[N / 2], int lane) {
     const bool hi = lane & D;
+    (void)hi;
 #pragma unroll
     for (int m = 0; m < N / 2; ++m) {
         const float a = in[2 * m], b = in[2 * m + 1];
-        const float keep = hi ? b : a, send = hi ? a : b;
-        out[m] = keep + row_xor<D>(send, lane);
+        if constexpr (SAPA_NHWC_DPP_HALVE && FROM_VALU) {
+            out[m] = pair_sum_dpp<D>(a, b);
+        } else {
+            const float keep = hi ? b : a, send = hi ? a : b;
+            out[m] = keep + row_xor<D>(send, lane);
+        }
     }
 }
 
@@ -289,8 +296,8 @@ sapa_b_nhwc16_kernel(const T *__restrict__ q, const T *__restrict__ key,
                     // summed over the 4 quads, tap 4 tau + bq stays in this lane
                     const float flat[4] = {a[0], a[1], a[2], a[3]};
                     float h1[2], h2[1];
-                    halve<4, 4>(flat, h1, lane);
-                    halve<8, 2>(h1, h2, lane);
+                    halve<4, 4, false>(flat, h1, lane);    // (inputs: a matrix instruction's result)
+                    halve<8, 2, true>(h1, h2, lane);
                     w[g * NTAU + tau] += h2[0];
                     // keeps the reads of at most two tap groups in flight (registers)
                     if (tau % 2 == 1) __builtin_amdgcn_sched_barrier(0);

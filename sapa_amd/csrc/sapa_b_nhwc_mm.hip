@@ -258,7 +258,7 @@ sapa_b_nhwc_mm_kernel(const T *__restrict__ q, const T *__restrict__ key,
                     // summed over the 4 quads of the row, tap 4 tau + bq stays in this lane
                     const float flat[4] = {a[0], a[1], a[2], a[3]};
                     float h1[2], h2[1];
-                    halve<4, 4>(flat, h1, lane);
+                    halve<4, 4, false>(flat, h1, lane);    // (inputs: a matrix instruction's result)
                     halve<8, 2>(h1, h2, lane);
                     w[g * NTAU + tau] += h2[0];
                     // keeps the reads of at most two tap groups in flight (registers)

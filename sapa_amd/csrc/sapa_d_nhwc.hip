@@ -81,15 +81,22 @@ __device__ __forceinline__ int row_bcast(int v) {
 }
 
 // One butterfly step over lane distance D: n values per lane -> n / 2; the
-// lane whose bit D is clear keeps the even-indexed sums, its partner the odd.
+// lane whose bit D is clear keeps the even-indexed sums, its partner the odd
+// (distances 4 and 8: two DPP additions per result, pair_sum_dpp -- the inputs
+// here are always results of ordinary vector instructions).
 template <int D, int N>
 __device__ __forceinline__ void halve(const float (&in)[N], float (&out)[N / 2], int lane) {
     const bool hi = lane & D;
+    (void)hi;
 #pragma unroll
     for (int m = 0; m < N / 2; ++m) {
         const float a = in[2 * m], b = in[2 * m + 1];
-        const float keep = hi ? b : a, send = hi ? a : b;
-        out[m] = keep + row_xor<D>(send, lane);
+        if constexpr (SAPA_NHWC_DPP_HALVE && (D == 4 || D == 8)) {
+            out[m] = pair_sum_dpp<D>(a, b);
+        } else {
+            const float keep = hi ? b : a, send = hi ? a : b;
+            out[m] = keep + row_xor<D>(send, lane);
+        }
     }
 }
 
