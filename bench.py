@@ -62,17 +62,17 @@ DEFORM_WORKLOADS = {
 MEASURED_TRAFFIC = {
     ('fpn_large', 'fp32', 'nchw'): (1831119034, 'profiles/sapa_b_fused_fpn_large_fp32.md', 'sapa_b_tiled_kernel'),
     ('fpn_large', 'bf16', 'nchw'): (999139434, 'profiles/sapa_b_fused_fpn_large_bf16.md', 'sapa_b_dot2_kernel'),
-    ('fpn_large', 'fp32', 'channels_last'): (1720500735, 'profiles/sapa_b_nhwc_fused_fpn_large_fp32.md',
+    ('fpn_large', 'fp32', 'channels_last'): (1720501334, 'profiles/sapa_b_nhwc_fused_fpn_large_fp32.md',
                                              'sapa_b_nhwc_kernel'),
-    ('fpn_large', 'bf16', 'channels_last'): (864607226, 'profiles/sapa_b_nhwc_fused_fpn_large_bf16.md',
+    ('fpn_large', 'bf16', 'channels_last'): (868223844, 'profiles/sapa_b_nhwc_fused_fpn_large_bf16.md',
                                              'sapa_b_nhwc16_kernel'),
     ('fpn_small', 'fp32', 'nchw'): (137685860, 'profiles/sapa_b_fused_fpn_small_fp32.md', 'sapa_b_tiled_kernel'),
     ('segformer_16', 'fp32', 'nchw'): (11936679, 'profiles/sapa_b_mfma_fused_segformer_16_fp32.md',
                                        'sapa_b_mfma_kernel'),
     ('stress', 'bf16', 'nchw'): (371333608, 'profiles/sapa_b_mfma_fused_stress_bf16.md', 'sapa_b_mfma_kernel'),
-    ('stress', 'fp32', 'channels_last'): (646238160, 'profiles/sapa_b_nhwc_mm_fused_stress_fp32.md',
+    ('stress', 'fp32', 'channels_last'): (647422060, 'profiles/sapa_b_nhwc_mm_fused_stress_fp32.md',
                                           'sapa_b_nhwc_mm_kernel'),
-    ('stress', 'bf16', 'channels_last'): (323149105, 'profiles/sapa_b_nhwc16_fused_stress_bf16.md',
+    ('stress', 'bf16', 'channels_last'): (323264189, 'profiles/sapa_b_nhwc16_fused_stress_bf16.md',
                                           'sapa_b_nhwc16_kernel'),
     ('deform_p25', 'fp32', 'nchw'): (459730983, 'profiles/sapa_d_wmat_fused_deform_p25_fp32_nchw.md',
                                      'deform_fused_wmat_kernel'),
