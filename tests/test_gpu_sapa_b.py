@@ -553,6 +553,42 @@ def test_window_staging_vector_widths(coracle, W):
     assert torch.equal(logits, coracle.qk(q, key, K, s, 'f32'))
 
 
+# (B, d, C, H, W): rows that are multiples of 4 elements at 16-byte aligned tensors, one case per tile
+# geometry the launcher picks for fp32 (32 x 8 tiles; 16 x 16; 16 x 8; the two-waves-per-band
+# geometry of small problems), with ragged tiles, channel counts off the chunk size and a sliced
+# value tensor
+LDS_DIRECT_SHAPES = [(2, 13, 21, 100, 168), (5, 9, 10, 128, 48), (4, 9, 10, 136, 48), (3, 20, 37, 19, 44),
+                     (1, 3, 2, 1, 4), (1, 64, 260, 10, 20)]
+
+
+@pytest.mark.parametrize('shape', LDS_DIRECT_SHAPES, ids=['-'.join(map(str, s)) for s in LDS_DIRECT_SHAPES])
+def test_windows_loaded_straight_into_lds(coracle, shape):
+    """fp32 windows whose rows allow 16-byte vectors go from global memory straight into LDS
+    (zero padding = the hardware's zero for an out-of-range offset): qk and av stay bit-exact,
+    the fused result within the stated bar, values at the image border included."""
+    B, d, C, H, W = shape
+    K, s = 5, 2
+    g = gen(121)
+    q, key, v = randn(g, B, d, H * s, W * s), randn(g, B, d, H, W), randn(g, B, C, H, W)
+    attn = F.softmax(randn(g, B, K * K, H * s, W * s), 1)
+    # large values on the border cells: a wrong padding or a shifted window row shows at once
+    # (in the two bit-exact comparisons only: in the fused one they would turn the bar, which
+    # is relative to the result, into one on cancelling terms 64 times its size)
+    def border(t, f):
+        t = t.clone()
+        t[:, :, 0, :] *= f
+        t[:, :, -1, :] *= f
+        t[:, :, :, 0] *= f
+        t[:, :, :, -1] *= f
+        return t
+    kb, vb = border(key, 64.0), border(v, 64.0)
+    assert torch.equal(sapa_amd.qk(*dev(q, kb), K, s).cpu(), coracle.qk(q, kb, K, s, 'f32'))
+    assert torch.equal(sapa_amd.av(*dev(attn, vb), K, s).cpu(), coracle.av(attn, vb, K, s, 'f32'))
+    got = sapa_amd.sapa_fused(*dev(q, key, v), K, s).cpu()
+    assert_f32_close(got, coracle.sapa_fused(q, key, v, K, s, 'f32'), f'fused {shape}')
+    assert sapa_amd._lib.last_kernel().startswith('sapa_b_tiled_kernel') or B * H * W <= 12288
+
+
 def test_module_with_folded_groupnorm_matches_two_step():
     """SAPA(fold_norm=True) = the same module with GroupNorm and the 1x1
     projections as separate steps (sapa_base.py:26-36), up to rounding."""
