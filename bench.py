@@ -386,9 +386,10 @@ def main():
         nhwc_ok = ((K, s) in ((3, 2), (5, 2), (7, 2), (5, 4), (7, 4))
                    and d % 4 == 0 and C % 4 == 0)
     if args.layout == 'channels_last':
-        if not nhwc_ok or args.direction == 'train':
-            sys.exit('bench.py: --layout channels_last covers the forward workloads with '
-                     '(K, s) in {(3,2), (5,2), (7,2), (5,4), (7,4)} (SAPA-B) / P <= 32 (SAPA-D)')
+        if not nhwc_ok or args.direction == 'module':
+            sys.exit('bench.py: --layout channels_last covers the workloads with '
+                     '(K, s) in {(3,2), (5,2), (7,2), (5,4), (7,4)} (SAPA-B) / P <= 32 (SAPA-D), '
+                     '--pass forward and --pass train')
         q, key, v, out = (t.contiguous(memory_format=torch.channels_last) for t in (q, key, v, out))
         if deform:
             off = off.contiguous(memory_format=torch.channels_last)
@@ -431,6 +432,11 @@ def main():
     if train:
         import sapa_amd
         go = torch.randn(B, C, H * s, W * s, device=dev).to(dtype)
+        if args.layout == 'channels_last':
+            # the forward runs on the channels-last kernels; the backward pass has no
+            # channels-last kernels: autograd copies its operands to contiguous order and
+            # the gradients come back in that order (the step below includes those copies)
+            go = go.contiguous(memory_format=torch.channels_last)
         leaves = [t.requires_grad_() for t in ((q, key, v, off) if deform else (q, key, v))]
         if deform:
             def step():
@@ -549,6 +555,8 @@ def main():
             abytes += esize * hi_px * 2 * (2 * G * P)
         what = what.replace('forward', 'forward + backward')
         kern = 'several (see profiles/)'
+        if args.layout == 'channels_last':
+            kern += '; forward on the channels-last kernels, backward through contiguous copies'
     traffic = traffic_source = None
     if not train:
         tlayout = 'nchw_reference_order' if deform and args.layout == 'nchw' and args.reference_order else args.layout

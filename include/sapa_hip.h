@@ -468,6 +468,20 @@ int sapa_project_nhwc(const void *x, const void *weight, const void *bias, void 
 
 /* ------------------------------------------------------------ calibration */
 
+/* Layout copy between the two memory orders the library serves: a dense
+ * [B, C, HW] tensor (contiguous, the reference's order) into channels-last
+ * order [B, HW, C] (to_channels_last = 1) or the other way (0), elements of
+ * esize = 2 or 4 bytes moved as they are.  No counterpart in the reference
+ * (which has no channels-last tensors); it is for the callers of the *_nhwc
+ * entry points whose backward pass runs on the contiguous kernels: one
+ * transposing launch (64 x 64-element tiles through LDS, 16-byte accesses on
+ * both sides where C, HW and the pointers allow) in place of a generic
+ * strided copy.  src and dst must not overlap.  SAPA_ERR_UNSUPPORTED for more
+ * than 65535 images or 4194240 rows of the side that is split into tiles
+ * (C for to_channels_last = 1, HW for 0). */
+int sapa_layout_copy(const void *src, void *dst, int B, int C, long long HW, int to_channels_last,
+                     int esize, void *stream);
+
 /* A kernel that only moves bytes, for putting the operators' measured rates
  * beside what the memory system gives a plain stream of the same read : write
  * mix.  No counterpart in the reference (which has no measurement code).

@@ -53,6 +53,7 @@ SIGNATURES = {
     'sapa_deform_qk_forward_from': [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_deform_av_forward_from': [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_stream_mix': [_vp, _vp, _ll, _i, _i, _i, _i, _vp],
+    'sapa_layout_copy': [_vp, _vp, _i, _i, _ll, _i, _i, _vp],
     'sapa_deform_fused_forward_from': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
 }
 
@@ -191,6 +192,32 @@ def memory_layout(**tensors):
         return 'channels_last'
     bad = [k for k, t in tensors.items() if t is not None and not t.is_contiguous()]
     raise RuntimeError(f'{bad[0]} must be contiguous (or every tensor in torch.channels_last order)')
+
+
+def is_channels_last(t):
+    """A 4-D tensor that is dense in torch.channels_last order and not in contiguous order."""
+    return (t is not None and t.dim() == 4 and not t.is_contiguous()
+            and t.is_contiguous(memory_format=torch.channels_last))
+
+
+def layout_copy(t, channels_last):
+    """`t` (4-D, dense in the other order) in contiguous / torch.channels_last order: the
+    library's transposing kernel for 2- and 4-byte elements on the device (the generic strided
+    copy behind Tensor.contiguous() runs at a small fraction of the memory rate on these
+    shapes), torch's copy for everything else."""
+    fmt = torch.channels_last if channels_last else torch.contiguous_format
+    if t.is_contiguous(memory_format=fmt):
+        return t
+    other = torch.contiguous_format if channels_last else torch.channels_last
+    if (t.is_cuda and t.dim() == 4 and t.element_size() in (2, 4) and t.is_contiguous(memory_format=other)
+            and not (t.requires_grad and torch.is_grad_enabled())):
+        out = torch.empty(t.shape, dtype=t.dtype, device=t.device, memory_format=fmt)
+        b, c, h, w = t.shape
+        status = call_status('sapa_layout_copy', t.device, ptr(t), ptr(out), b, c, h * w,
+                             1 if channels_last else 0, t.element_size())
+        if status != UNSUPPORTED:
+            return out
+    return t.contiguous(memory_format=fmt)
 
 
 def call_nhwc(name, device, *args):

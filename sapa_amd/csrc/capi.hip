@@ -736,6 +736,22 @@ int sapa_project_nhwc(const void *x, const void *weight, const void *bias, void 
     return finish(e);
 }
 
+int sapa_layout_copy(const void *src, void *dst, int B, int C, long long HW, int to_channels_last,
+                     int esize, void *stream) {
+    if (B < 0 || C < 0 || HW < 0 || (esize != 2 && esize != 4)) return SAPA_ERR_INVALID_ARGUMENT;
+    if ((long long)B * C * HW >= kMaxElems) return SAPA_ERR_TOO_LARGE;
+    if (B == 0 || C == 0 || HW == 0) return SAPA_OK;
+    if (!src || !dst || ((uintptr_t)src | (uintptr_t)dst) % (uintptr_t)esize != 0) return SAPA_ERR_INVALID_ARGUMENT;
+    // [B, rows, cols] -> [B, cols, rows]: the way back is the same transposition with the
+    // roles of C and HW exchanged
+    if (!to_channels_last && HW > 0x7fffffffLL) return SAPA_ERR_UNSUPPORTED;
+    const hipError_t e = to_channels_last
+        ? nchw_to_nhwc_launch(src, dst, C, nullptr, nullptr, 0, B, (long)HW, esize, (hipStream_t)stream)
+        : nchw_to_nhwc_launch(src, dst, (int)HW, nullptr, nullptr, 0, B, (long)C, esize, (hipStream_t)stream);
+    if (e == hipErrorNotSupported) return SAPA_ERR_UNSUPPORTED;
+    return finish(e);
+}
+
 int sapa_stream_mix(const void *src, void *dst, long long units, int reads, int writes, int reps,
                     int nontemporal, void *stream) {
     if (units < 0 || reads < 0 || writes < 0 || reps < 1 || (reads == 0 && writes == 0) || nontemporal < 0 || nontemporal > 7)

@@ -26,7 +26,7 @@ def _backward_16bit(entry, grad_output, a, low, offset, P, s, G, needs):
     configuration.  a: query (deform_qk) or attn (deform_av); low: key or value."""
     if low.dtype not in (torch.float16, torch.bfloat16):
         return None
-    go, a, low, off = (t.contiguous() for t in (grad_output, a, low, offset))
+    go, a, low, off = (_lib.layout_copy(t, False) for t in (grad_output, a, low, offset))
     _lib.require_cuda_contiguous(grad_output=go, a=a, low=low, offset=off)
     n, c, h, w = low.size()
     nbytes = _lib.lib().sapa_deform_backward_workspace(n, c, h, w, P, s, G, _lib.dtype_code(low))
@@ -45,7 +45,7 @@ def _deform_qk_backward(grad_output, query, key, offset, P, s, G, needs=(True, T
     if native is not None:
         return native
     cdt = _compute_dtype(query)
-    go, q, k, off = (t.contiguous().to(cdt) for t in (grad_output, query, key, offset))
+    go, q, k, off = (_lib.layout_copy(t, False).to(cdt) for t in (grad_output, query, key, offset))
     gq = _lib.new_out(q) if needs[0] else None
     gk = torch.zeros_like(k) if needs[1] else None
     goff = _lib.new_out(off) if needs[2] else None
@@ -63,7 +63,7 @@ def _deform_av_backward(grad_output, attn, value, offset, P, s, G, needs=(True, 
     if native is not None:
         return native
     cdt = _compute_dtype(value)
-    go, a, v, off = (t.contiguous().to(cdt) for t in (grad_output, attn, value, offset))
+    go, a, v, off = (_lib.layout_copy(t, False).to(cdt) for t in (grad_output, attn, value, offset))
     ga = _lib.new_out(a) if needs[0] else None
     gv = torch.zeros_like(v) if needs[1] else None
     goff = _lib.new_out(off) if needs[2] else None
@@ -223,17 +223,22 @@ def _deform_fused_backward(grad_output, query, key, value, offset, P, s, G, offs
     """Gradients of deform_av(softmax(deform_qk(q, k, off), dim=2), v, off)
     with respect to q, k, v and the offset tensor in its own layout."""
     with torch.no_grad():
-        # the gradient kernels take contiguous tensors: operands kept in
-        # channels-last order are copied here
-        query, key, value = query.contiguous(), key.contiguous(), value.contiguous()
-        grad_output = grad_output.contiguous()
-        offset = expand_offset(offset, s, offset_layout).contiguous()
+        # the gradient kernels take contiguous tensors: operands kept in channels-last order
+        # are transposed here by the library's layout kernel, and each gradient goes back in
+        # the order of the tensor it belongs to
+        cl = [_lib.is_channels_last(t) for t in (query, key, value, offset)]
+
+        def back(g, i):
+            return g if g is None or not cl[i] else _lib.layout_copy(g, True)
+        query, key, value = (_lib.layout_copy(t, False) for t in (query, key, value))
+        grad_output = _lib.layout_copy(grad_output, False)
+        offset = _lib.layout_copy(expand_offset(offset, s, offset_layout), False)
         native = _native_fused_backward(grad_output, query, key, value, offset, P, s, G, needs)
         if native is not None:
             gq, gk, gv, goff = native
             if goff is not None:
                 goff = _reduce_offset_grad(goff, s, offset_layout)
-            return gq, gk, gv, goff
+            return back(gq, 0), back(gk, 1), back(gv, 2), back(goff, 3)
         # 16-bit tensors: the logits are recomputed from fp32 copies so that, like
         # the forward kernel's, they are not rounded to 16 bits before the softmax
         wide = _compute_dtype(query)
@@ -244,7 +249,7 @@ def _deform_fused_backward(grad_output, query, key, value, offset, P, s, G, offs
         grad_logits = (a32 * (g32 - (g32 * a32).sum(dim=2, keepdim=True))).to(attn.dtype)
         gq, gk, goff_qk = _deform_qk_backward(grad_logits, query, key, offset, P, s, G)
         goff = _reduce_offset_grad(goff_av + goff_qk, s, offset_layout)
-    return gq, gk, gv, goff
+    return back(gq, 0), back(gk, 1), back(gv, 2), back(goff, 3)
 
 
 class DeformSAPAFusedFunction(Function):

@@ -16,13 +16,21 @@ def _check_odd_kernel(kernel_size):
     assert (kernel_size - 1) % 2 == 0 and kernel_size >= 1
 
 
+def _back(grad, channels_last):
+    """A gradient computed in contiguous order, in the order of the tensor it belongs to."""
+    return grad if grad is None or not channels_last else _lib.layout_copy(grad, True)
+
+
 def _qk_backward(grad_output, query, key, kernel_size, scale_factor, need_q=True, need_k=True):
     # the gradient kernels take contiguous tensors: operands kept in
     # channels-last order are copied here (the forward pass is the zero-copy one)
     # 16-bit tensors are read and written as they are (fp32 sums inside the
     # kernels), as the reference's half dispatch does (qk_cuda_kernel.cu:139-171)
-    query, key = query.contiguous(), key.contiguous()
-    grad_output = grad_output.contiguous()
+    # (_lib.layout_copy: the library's transposing kernel; the gradients go back in the order
+    # of the tensors they belong to)
+    cl_q, cl_k = _lib.is_channels_last(query), _lib.is_channels_last(key)
+    query, key = _lib.layout_copy(query, False), _lib.layout_copy(key, False)
+    grad_output = _lib.layout_copy(grad_output, False)
     grad_query = _lib.new_out(query) if need_q else None
     grad_key = _lib.new_out(key) if need_k else None
     _lib.require_cuda_contiguous(grad_output=grad_output, query=query, key=key)
@@ -30,12 +38,13 @@ def _qk_backward(grad_output, query, key, kernel_size, scale_factor, need_q=True
     _lib.call('sapa_qk_backward', key.device, _lib.ptr(grad_output), _lib.ptr(query),
               _lib.ptr(key), _lib.ptr(grad_query), _lib.ptr(grad_key), n, c, h, w,
               kernel_size, scale_factor, _lib.dtype_code(key))
-    return grad_query, grad_key
+    return _back(grad_query, cl_q), _back(grad_key, cl_k)
 
 
 def _av_backward(grad_output, attn, value, kernel_size, scale_factor, need_a=True, need_v=True):
-    attn, value = attn.contiguous(), value.contiguous()
-    grad_output = grad_output.contiguous()
+    cl_a, cl_v = _lib.is_channels_last(attn), _lib.is_channels_last(value)
+    attn, value = _lib.layout_copy(attn, False), _lib.layout_copy(value, False)
+    grad_output = _lib.layout_copy(grad_output, False)
     grad_attn = _lib.new_out(attn) if need_a else None
     grad_value = _lib.new_out(value) if need_v else None
     _lib.require_cuda_contiguous(grad_output=grad_output, attn=attn, value=value)
@@ -43,7 +52,7 @@ def _av_backward(grad_output, attn, value, kernel_size, scale_factor, need_a=Tru
     _lib.call('sapa_av_backward', value.device, _lib.ptr(grad_output), _lib.ptr(attn),
               _lib.ptr(value), _lib.ptr(grad_attn), _lib.ptr(grad_value), n, c, h, w,
               kernel_size, scale_factor, _lib.dtype_code(value))
-    return grad_attn, grad_value
+    return _back(grad_attn, cl_a), _back(grad_value, cl_v)
 
 
 class QKFunction(Function):
@@ -175,6 +184,15 @@ def _fused_backward(grad_output, query, key, value, K, s, needs=(True, True, Tru
     are recomputed (one launch) unless the forward pass kept them (`attn`, fp32),
     then the three operators' gradients chain."""
     need_q, need_k, need_v = needs
+    cl = [_lib.is_channels_last(t) for t in (query, key, value)]
+    if any(cl) or _lib.is_channels_last(grad_output) or _lib.is_channels_last(attn):
+        # the gradient kernels take contiguous tensors: operands in channels-last order are
+        # transposed by the library's layout kernel, and each gradient goes back in the order
+        # of the tensor it belongs to
+        grads = _fused_backward(_lib.layout_copy(grad_output, False), _lib.layout_copy(query, False),
+                                _lib.layout_copy(key, False), _lib.layout_copy(value, False), K, s, needs,
+                                None if attn is None else _lib.layout_copy(attn, False))
+        return tuple(_back(g, c) for g, c in zip(grads, cl))
     query, key, value = query.contiguous(), key.contiguous(), value.contiguous()
     grad_output = grad_output.contiguous()
     _lib.require_cuda_contiguous(grad_output=grad_output, query=query, key=key, value=value)

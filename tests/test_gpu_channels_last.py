@@ -175,6 +175,47 @@ def test_backward_through_channels_last_forward():
         torch.testing.assert_close(b, a, rtol=1e-4, atol=1e-5, msg=lambda m: f'grad_{name}: {m}')
 
 
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('shape', [(2, 8, 5, 7), (1, 3, 1, 35), (3, 64, 12, 20), (2, 260, 9, 4), (1, 1, 6, 6)])
+def test_layout_copy_kernel(shape, dtype):
+    """sapa_layout_copy both ways, on shapes that take its 16-byte form and its element form:
+    the same values as Tensor.contiguous(), in the requested order."""
+    from sapa_amd import _lib
+    x = randn(gen(330), *shape).to(dtype).to(DEV)
+    to_cl = _lib.layout_copy(x, True)
+    assert to_cl.is_contiguous(memory_format=CL) and torch.equal(to_cl, x)
+    src = x.contiguous(memory_format=CL)
+    back = _lib.layout_copy(src, False)
+    assert back.is_contiguous() and torch.equal(back, x)
+    if shape[1] > 1 and shape[2] * shape[3] > 1:
+        # the library's kernel did these, not torch's copy
+        out = torch.full_like(x, float('nan'))
+        _lib.call('sapa_layout_copy', x.device, src.data_ptr(), out.data_ptr(), shape[0], shape[1],
+                  shape[2] * shape[3], 0, x.element_size())
+        assert torch.equal(out, x)
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+def test_backward_of_channels_last_tensors_equals_contiguous(dtype):
+    """The backward pass of channels_last operands runs on the contiguous kernels after the
+    library's layout kernel: bit-identical gradients, each in the order of its tensor."""
+    B, d, C, H, W, K = 2, 16, 24, 12, 20, 5
+    q, key, v, _ = inputs(gen(331), B, d, C, H, W, K, dtype=dtype)
+    go = randn(gen(332), B, C, 2 * H, 2 * W).to(dtype)
+    grads = []
+    for fmt in (torch.contiguous_format, CL):
+        ts = [t.to(DEV).contiguous(memory_format=fmt).requires_grad_() for t in (q, key, v)]
+        # (the forward kernels of the two layouts sum in different orders; the gradients are
+        # taken with respect to the same operands either way)
+        out = sapa_amd.sapa_fused(*ts, K, 2)
+        gs = torch.autograd.grad(out, ts, go.to(DEV).contiguous(memory_format=fmt))
+        grads.append(gs)
+        for g in gs:
+            assert g.is_contiguous(memory_format=fmt)
+    for a, b, name in zip(grads[0], grads[1], ('query', 'key', 'value')):
+        assert torch.equal(a, b), f'grad_{name}'
+
+
 def test_module_in_channels_last_format():
     """A SAPA module in channels_last memory format: same result as the
     contiguous run, output in channels_last order, parameters get gradients."""
