@@ -132,6 +132,14 @@ def test_argument_validation_returns_codes():
     assert h.sapa_project_nhwc(p, None, p, p, 1, 256, 64, 100, 3, None) == -1
     assert h.sapa_project_nhwc(p, p, None, p, 1, 256, 64, 100, 0, None) == -2
     assert h.sapa_project_nhwc(None, None, None, None, 0, 256, 64, 100, 3, None) == 0
+    # layout copy: element size, negative extents, null / misaligned pointers, empty tensors,
+    # more rows than the tiled side holds
+    assert h.sapa_layout_copy(p, p, 1, 8, 64, 1, 3, None) == -1
+    assert h.sapa_layout_copy(p, p, 1, -1, 64, 1, 4, None) == -1
+    assert h.sapa_layout_copy(None, p, 1, 8, 64, 0, 4, None) == -1
+    assert h.sapa_layout_copy(ctypes.c_void_p(18), p, 1, 8, 64, 0, 4, None) == -1
+    assert h.sapa_layout_copy(None, None, 0, 8, 64, 1, 2, None) == 0
+    assert h.sapa_layout_copy(p, p, 1, 4, 5000000, 0, 4, None) == -2
     # GroupNorm fold: channels not divisible by the groups, null weight, empty batch
     assert h.sapa_groupnorm_fold(p, p, p, p, p, p, p, 1, 10, 4, 4, 1e-5, 0, None) == -1
     assert h.sapa_groupnorm_fold(p, p, p, None, p, p, p, 1, 8, 4, 4, 1e-5, 0, None) == -1
