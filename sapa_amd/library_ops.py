@@ -40,8 +40,11 @@ def _new_out(like, shape, *inputs):
 
 
 def _new_grad(t):
-    # the gradient kernels answer in contiguous order whatever the operand's order
-    return t.new_empty(t.shape)
+    # a gradient comes back in the order of the tensor it belongs to (the kernels work in
+    # contiguous order; channels-last operands and results are transposed around them)
+    cl = t.dim() == 4 and not t.is_contiguous() and t.is_contiguous(memory_format=torch.channels_last)
+    return torch.empty(t.shape, dtype=t.dtype, device=t.device,
+                       memory_format=torch.channels_last if cl else torch.contiguous_format)
 
 
 # ------------------------------------------------------------------ SAPA-B
@@ -74,7 +77,7 @@ def _qk_setup(ctx, inputs, output):
 
 def _qk_grad(ctx, grad_output):
     query, key = ctx.saved_tensors
-    gq, gk = qk_backward(grad_output.contiguous(), query, key, ctx.kernel_size, ctx.scale_factor)
+    gq, gk = qk_backward(grad_output, query, key, ctx.kernel_size, ctx.scale_factor)
     return gq, gk, None, None
 
 
@@ -110,7 +113,7 @@ def _av_setup(ctx, inputs, output):
 
 def _av_grad(ctx, grad_output):
     attn, value = ctx.saved_tensors
-    ga, gv = av_backward(grad_output.contiguous(), attn, value, ctx.kernel_size, ctx.scale_factor)
+    ga, gv = av_backward(grad_output, attn, value, ctx.kernel_size, ctx.scale_factor)
     return ga, gv, None, None
 
 
@@ -147,7 +150,7 @@ def _fused_setup(ctx, inputs, output):
 
 def _fused_grad(ctx, grad_output):
     query, key, value = ctx.saved_tensors
-    gq, gk, gv = sapa_fused_backward(grad_output.contiguous(), query, key, value,
+    gq, gk, gv = sapa_fused_backward(grad_output, query, key, value,
                                      ctx.kernel_size, ctx.scale_factor)
     return gq, gk, gv, None, None
 
@@ -270,7 +273,7 @@ def _dfused_setup(ctx, inputs, output):
 def _dfused_grad(ctx, grad_output):
     query, key, value, offset = ctx.saved_tensors
     gq, gk, gv, go = deform_sapa_fused_backward(
-        grad_output.contiguous(), query, key, value, offset, ctx.num_point, ctx.scale_factor,
+        grad_output, query, key, value, offset, ctx.num_point, ctx.scale_factor,
         ctx.groups, ctx.offset_layout)
     return gq, gk, gv, go, None, None, None, None
 

@@ -99,6 +99,12 @@ def test_channels_last_ops_and_compile():
     y_ref.backward(go)
     for a, b in zip(leaves, ref_leaves):
         assert torch.equal(a.grad, b.grad)
+    # the gradient ops answer in the order of their operands, and their shape-only
+    # implementations say so
+    gq, gk, gv = torch.ops.sapa_amd.sapa_fused_backward(go, q, key, v, 5, 2)
+    assert all(t.is_contiguous(memory_format=CL) for t in (gq, gk, gv))
+    torch.library.opcheck(torch.ops.sapa_amd.sapa_fused_backward.default, (go, q, key, v, 5, 2),
+                          test_utils=('test_schema', 'test_faketensor'))
     # SAPA-D: 4 channels per group so that the channels-last kernel takes it
     g = gen(402)
     B, G, H, W, P, s = 1, 2, 5, 6, 4, 2
