@@ -18,7 +18,7 @@ import torch.nn.functional as F
 
 from . import _lib
 from .deform_func import deform_av, deform_qk, deform_sapa_fused
-from .sapa_func import av, qk, sapa_fused
+from .sapa_func import av, in_memory_order, qk, sapa_fused
 
 
 def _needs_grad(*mods):
@@ -179,7 +179,7 @@ class SAPA(nn.Module):
             if not self.fused:
                 q, q_bias = q.add_(q_bias[:, :, None, None]), None
             (k,) = norm_project(x, nx, self.k, channels_last=True)
-            return self.attention(q, k, x.contiguous(memory_format=torch.channels_last), q_bias)
+            return self.attention(q, k, in_memory_order(x, torch.channels_last), q_bias)
         if self.norm and self.fold_norm:
             (q,), (k,) = norm_project(y, self.norm_y, self.q), norm_project(x, self.norm_x, self.k)
             return self.attention(q, k, x)
@@ -197,7 +197,7 @@ class SAPA(nn.Module):
         fmt = (torch.channels_last
                if not v.is_contiguous() and v.is_contiguous(memory_format=torch.channels_last)
                else torch.contiguous_format)
-        q, k, v = (t.contiguous(memory_format=fmt) for t in (q, k, v))
+        q, k, v = (in_memory_order(t, fmt) for t in (q, k, v))
         try:
             return self._attend(q, k, v, q_bias, fmt)
         except _lib.SapaUnsupported:
@@ -206,9 +206,9 @@ class SAPA(nn.Module):
         # a configuration the channels-last kernels do not cover (float64, other
         # (kernel, scale) pairs, channel counts that are no multiple of 4): one
         # layout copy each way and the contiguous kernels, which serve them all
-        out = self._attend(q.contiguous(), k.contiguous(), v.contiguous(), q_bias,
+        out = self._attend(*(in_memory_order(t, torch.contiguous_format) for t in (q, k, v)), q_bias,
                            torch.contiguous_format)
-        return out.contiguous(memory_format=torch.channels_last)
+        return in_memory_order(out, torch.channels_last)
 
     def _attend(self, q, k, v, q_bias, fmt):
         K, s = self.up_kernel_size, self.up_factor
@@ -263,7 +263,7 @@ class SAPADeform(nn.Module):
                 offset = F.pixel_shuffle(offset_lo, upscale_factor=self.up_factor)
             else:
                 offset = F.interpolate(offset_lo, scale_factor=self.up_factor)
-            return self.attention(q, k, x.contiguous(memory_format=torch.channels_last), offset)
+            return self.attention(q, k, in_memory_order(x, torch.channels_last), offset)
         if self.norm and self.fold_norm:
             (q,) = norm_project(y, self.norm_y, self.q)
             k, offset_lo = norm_project(x, self.norm_x, self.k, self.offset)
@@ -276,7 +276,7 @@ class SAPADeform(nn.Module):
                            or not x.is_contiguous(memory_format=torch.channels_last)):
             # the kernel reads the offset convolution's output in place
             try:
-                return deform_sapa_fused(q.contiguous(), k.contiguous(), x.contiguous(),
+                return deform_sapa_fused(*(in_memory_order(t, torch.contiguous_format) for t in (q, k, x)),
                                          offset_lo.contiguous(), self.num_point,
                                          self.up_factor, self.groups,
                                          'pixel_shuffle' if self.high_offset else 'nearest')
@@ -295,7 +295,7 @@ class SAPADeform(nn.Module):
             # model stays channels-last (the fused kernel serves that order)
             cl = not x.is_contiguous() and x.is_contiguous(memory_format=torch.channels_last)
             fmt = torch.channels_last if cl else torch.contiguous_format
-            q, k, x, offset = (t.contiguous(memory_format=fmt) for t in (q, k, x, offset))
+            q, k, x, offset = (in_memory_order(t, fmt) for t in (q, k, x, offset))
             try:
                 return deform_sapa_fused(q, k, x, offset, P, s, G)
             except _lib.SapaUnsupported:
@@ -303,14 +303,14 @@ class SAPADeform(nn.Module):
             # not covered in this memory order (float64, more than 32 points,
             # channel counts that are no multiple of 4 ...) or at all (more than 64
             # points): contiguous tensors, then the separate operators
-            q, k, x, offset = (t.contiguous() for t in (q, k, x, offset))
+            q, k, x, offset = (in_memory_order(t, torch.contiguous_format) for t in (q, k, x, offset))
             try:
                 out = deform_sapa_fused(q, k, x, offset, P, s, G)
             except _lib.SapaUnsupported:
                 attn = F.softmax(deform_qk(q, k, offset, P, s, G), dim=2)
                 out = deform_av(attn, x, offset, P, s, G)
-            return out.contiguous(memory_format=fmt)
+            return in_memory_order(out, fmt)
         # the separate operators take contiguous tensors only
-        q, k, x, offset = (t.contiguous() for t in (q, k, x, offset))
+        q, k, x, offset = (in_memory_order(t, torch.contiguous_format) for t in (q, k, x, offset))
         attn = F.softmax(deform_qk(q, k, offset, P, s, G), dim=2)
         return deform_av(attn, x, offset, P, s, G)

@@ -16,6 +16,33 @@ def _check_odd_kernel(kernel_size):
     assert (kernel_size - 1) % 2 == 0 and kernel_size >= 1
 
 
+class _MemoryOrder(Function):
+    """`t` in contiguous / torch.channels_last order with the library's transposing kernel
+    (_lib.layout_copy) in both passes: the gradient goes back in the order `t` had."""
+
+    @staticmethod
+    def forward(ctx, t, channels_last):
+        ctx.back_to_channels_last = _lib.is_channels_last(t)
+        with torch.no_grad():
+            return _lib.layout_copy(t, channels_last)
+
+    @staticmethod
+    def backward(ctx, grad):
+        return _lib.layout_copy(grad, ctx.back_to_channels_last), None
+
+
+def in_memory_order(t, memory_format):
+    """Tensor.contiguous(memory_format=...) for the feature maps of the modules: the tensor
+    itself when it is in that order already, else a transposed copy made by the library's
+    layout kernel (device tensors of 2- and 4-byte elements that are dense in the other order;
+    anything else takes Tensor.contiguous)."""
+    if t.is_contiguous(memory_format=memory_format):
+        return t
+    if not (t.is_cuda and t.dim() == 4 and t.element_size() in (2, 4)):
+        return t.contiguous(memory_format=memory_format)
+    return _MemoryOrder.apply(t, memory_format is torch.channels_last)
+
+
 def _back(grad, channels_last):
     """A gradient computed in contiguous order, in the order of the tensor it belongs to."""
     return grad if grad is None or not channels_last else _lib.layout_copy(grad, True)
