@@ -159,6 +159,27 @@ __device__ __forceinline__ void store_buffer(__amdgpu_buffer_rsrc_t r, unsigned 
 #ifndef SAPA_NHWC_DPP_HALVE
 #define SAPA_NHWC_DPP_HALVE 1
 #endif
+// (the same exchange as an all-to-partner maximum / sum of one value: every lane gets
+// max / sum of its own v and that of lane ^ D)
+template <int D>
+__device__ __forceinline__ float xor_max_dpp(float v) {
+    static_assert(D == 4 || D == 8, "lane distance");
+    float r;
+#if defined(__HIP_DEVICE_COMPILE__)
+    if constexpr (D == 4)
+        asm volatile("s_nop 1\n\t"
+                     "v_max_f32_dpp %0, %1, %1 row_ror:12 row_mask:0xf bank_mask:0x5\n\t"
+                     "v_max_f32_dpp %0, %1, %1 row_ror:4 row_mask:0xf bank_mask:0xa"
+                     : "=&v"(r) : "v"(v));
+    else
+        asm volatile("s_nop 1\n\t"
+                     "v_max_f32_dpp %0, %1, %1 row_ror:8 row_mask:0xf bank_mask:0xf"
+                     : "=&v"(r) : "v"(v));
+#else
+    r = v;
+#endif
+    return r;
+}
 template <int D>
 __device__ __forceinline__ float pair_sum_dpp(float a, float b) {
     static_assert(D == 4 || D == 8, "lane distance");

@@ -272,8 +272,13 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
 #pragma unroll
                     for (int m = 0; m < RPR; ++m)
                         if (ok[m]) mx = max_(mx, w[(ky * NG + g) * RPR + m]);
-                mx = max_(mx, row_xor<4>(mx, lane));
-                mx = max_(mx, row_xor<8>(mx, lane));
+                if constexpr (SAPA_NHWC_DPP_HALVE) {
+                    mx = xor_max_dpp<4>(mx);
+                    mx = xor_max_dpp<8>(mx);
+                } else {
+                    mx = max_(mx, row_xor<4>(mx, lane));
+                    mx = max_(mx, row_xor<8>(mx, lane));
+                }
                 float sum = 0.f;
 #pragma unroll
                 for (int ky = 0; ky < K; ++ky)
@@ -283,8 +288,13 @@ sapa_b_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
                         x = ok[m] ? exp_(x - mx) : 0.f;
                         sum += x;
                     }
-                sum += row_xor<4>(sum, lane);
-                sum += row_xor<8>(sum, lane);
+                if constexpr (SAPA_NHWC_DPP_HALVE) {
+                    sum = pair_sum_dpp<4>(sum, sum);
+                    sum = pair_sum_dpp<8>(sum, sum);
+                } else {
+                    sum += row_xor<4>(sum, lane);
+                    sum += row_xor<8>(sum, lane);
+                }
                 const float inv = 1.f / sum;
 #pragma unroll
                 for (int ky = 0; ky < K; ++ky)

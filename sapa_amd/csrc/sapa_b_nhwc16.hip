@@ -315,8 +315,13 @@ sapa_b_nhwc16_kernel(const T *__restrict__ q, const T *__restrict__ key,
 #pragma unroll
                 for (int m = 0; m < NTAU; ++m)
                     if (ok[m]) mx = max_(mx, w[g * NTAU + m]);
-                mx = max_(mx, row_xor<4>(mx, lane));
-                mx = max_(mx, row_xor<8>(mx, lane));
+                if constexpr (SAPA_NHWC_DPP_HALVE) {
+                    mx = xor_max_dpp<4>(mx);
+                    mx = xor_max_dpp<8>(mx);
+                } else {
+                    mx = max_(mx, row_xor<4>(mx, lane));
+                    mx = max_(mx, row_xor<8>(mx, lane));
+                }
                 float sum = 0.f;
 #pragma unroll
                 for (int m = 0; m < NTAU; ++m) {
@@ -324,8 +329,13 @@ sapa_b_nhwc16_kernel(const T *__restrict__ q, const T *__restrict__ key,
                     x = ok[m] ? exp_(x - mx) : 0.f;
                     sum += x;
                 }
-                sum += row_xor<4>(sum, lane);
-                sum += row_xor<8>(sum, lane);
+                if constexpr (SAPA_NHWC_DPP_HALVE) {
+                    sum = pair_sum_dpp<4>(sum, sum);
+                    sum = pair_sum_dpp<8>(sum, sum);
+                } else {
+                    sum += row_xor<4>(sum, lane);
+                    sum += row_xor<8>(sum, lane);
+                }
                 const float inv = 1.f / sum;
 #pragma unroll
                 for (int m = 0; m < NTAU; ++m) w[g * NTAU + m] *= inv;

@@ -311,20 +311,14 @@ deform_fused_nhwc_kernel(const T *__restrict__ q, const T *__restrict__ key,
 #pragma unroll
         for (int m = 1; m < MAXSETS; ++m)
             if (okp[m]) mx = max_(mx, att[m]);
-        mx = max_(mx, row_xor<1>(mx, lane));
-        mx = max_(mx, row_xor<2>(mx, lane));
-        mx = max_(mx, row_xor<4>(mx, lane));
-        mx = max_(mx, row_xor<8>(mx, lane));
+        mx = reduce_lanes<true, 16>(mx);      // (DPP steps: no exchange through LDS)
         float sum = 0.f;
 #pragma unroll
         for (int m = 0; m < MAXSETS; ++m) {
             att[m] = okp[m] ? exp_(att[m] - mx) : 0.f;
             sum += att[m];
         }
-        sum += row_xor<1>(sum, lane);
-        sum += row_xor<2>(sum, lane);
-        sum += row_xor<4>(sum, lane);
-        sum += row_xor<8>(sum, lane);
+        sum = reduce_lanes<false, 16>(sum);
         const float inv = 1.f / sum;
 #pragma unroll
         for (int m = 0; m < MAXSETS; ++m) att[m] *= inv;
