@@ -142,7 +142,19 @@ sapa_b_nhwc16_kernel(const T *__restrict__ q, const T *__restrict__ key,
     constexpr bool DO_AV = MODE == TILED_AV || MODE == TILED_FUSED;
     typedef Mma<T> M;
 
-    __shared__ __attribute__((aligned(16))) u32 lds[2 * BUF];
+    // The windows go from global memory straight into LDS (buffer loads with the LDS modifier:
+    // lane l of a wave's load fills the 16-byte slot l of 64 consecutive ones, 12 slots per
+    // position of which 8 hold its 64 channels): no staging registers, no LDS write
+    // instructions.  A buffer is a whole number of 64-slot blocks.
+#ifndef SAPA_NHWC16_DMA
+#define SAPA_NHWC16_DMA 1
+#endif
+    constexpr bool DMA = SAPA_NHWC16_DMA;
+    constexpr int SPP = PSW / 4;                                  // 16-byte slots per position
+    constexpr int BUFA = DMA ? (BUF + 255) / 256 * 256 : BUF;     // dwords per buffer
+    constexpr int NPD = (NPOS * SPP + NT - 1) / NT;               // direct loads per thread and chunk
+    static_assert(PSW % 4 == 0 && CHK == 64, "slot layout");
+    __shared__ __attribute__((aligned(16))) u32 lds[2 * BUFA];
 
     const int logical = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
     if (logical >= nblocks) return;
@@ -175,6 +187,32 @@ sapa_b_nhwc16_kernel(const T *__restrict__ q, const T *__restrict__ key,
         spix[p] = (pos < NPOS && gy >= 0 && gy < H && gx >= 0 && gx < W) ? gy * W + gx : -1;
     }
     const int sq = tid & 15;
+    // direct loads: pass p, thread t fills slot p * NT + t = 8 channels (slot % SPP < 8) of
+    // position slot / SPP; dpix: the position's pixel, -1 outside the image / for a spare
+    // slot / past the window
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    (void)wave_u;
+    int dpix[NPD], dq8[NPD];
+#pragma unroll
+    for (int p = 0; p < NPD; ++p) {
+        const int slot = p * NT + tid, pos = slot / SPP;
+        dq8[p] = slot % SPP;
+        const int gy = y0 - R + pos / WW, gx = x0 - R + pos % WW;
+        dpix[p] = (pos < NPOS && dq8[p] < 8 && gy >= 0 && gy < H && gx >= 0 && gx < W) ? gy * W + gx : -1;
+    }
+    // one chunk's loads from per-thread offsets `off`; (device pass only: the host pass, which
+    // sees this body for the launch stub, does not know the builtin)
+    auto direct_loads = [&](__amdgpu_buffer_rsrc_t r, int j, const u32 (&off)[NPD]) __attribute__((always_inline)) {
+#if defined(__HIP_DEVICE_COMPILE__)
+#pragma unroll
+        for (int p = 0; p < NPD; ++p) {
+            const int slot0 = p * NT + wave_u * 64;
+            if ((p + 1) * NT <= NPOS * SPP || slot0 < NPOS * SPP)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                    r, (__attribute__((address_space(3))) void *)(lds + (j & 1) * BUFA + slot0 * 4), 16, off[p], 0, 0, 0);
+        }
+#endif
+    };
     u32x2 st[NPASS];
     auto stage_load = [&](int j) __attribute__((always_inline)) {
         const bool is_key = j < nKc;
@@ -183,6 +221,17 @@ sapa_b_nhwc16_kernel(const T *__restrict__ q, const T *__restrict__ key,
         const T *base = (is_key ? key : value) + (long)n * lpix * nch;
         const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(
             (void *)base, 0, (int)(lpix * nch * (long)sizeof(T)), 0x00020000);
+        if constexpr (DMA) {
+            u32 off[NPD];
+#pragma unroll
+            for (int p = 0; p < NPD; ++p) {
+                const u32 c_bad = (u32)(nch - 1 - (c0 + 8 * dq8[p]));
+                off[p] = ((u32)(dpix[p] * nch + c0 + 8 * dq8[p]) * (u32)sizeof(T)) |
+                         ((c_bad | (u32)dpix[p]) & 0x80000000u);
+            }
+            direct_loads(r, j, off);
+            return;
+        }
         // bit 31 set = past the descriptor; pure arithmetic (sign bits of "channel
         // within the tensor" and "position within the image") instead of selects
         const u32 c_bad = (u32)(nch - 1 - (c0 + 4 * sq));
@@ -195,19 +244,36 @@ sapa_b_nhwc16_kernel(const T *__restrict__ q, const T *__restrict__ key,
     };
     // the same for value chunk jv from offsets prepared once (voff0, set up before
     // the aggregation): two instructions per load instead of the full address
-    u32 voff0[NPASS];
+    u32 voff0[DMA ? NPD : NPASS];
     auto stage_load_value = [&](int jv) __attribute__((always_inline)) {
         const T *base = value + (long)n * lpix * C;
         const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(
             (void *)base, 0, (int)(lpix * C * (long)sizeof(T)), 0x00020000);
+        if constexpr (DMA) {
+            u32 off[NPD];
+#pragma unroll
+            for (int p = 0; p < NPD; ++p)
+                off[p] = (voff0[p] + (u32)(jv * CHK) * (u32)sizeof(T)) |
+                         ((u32)(C - 1 - (jv * CHK + 8 * dq8[p])) & 0x80000000u);
+            direct_loads(r, nKc + jv, off);
+            return;
+        }
         const u32 c_bad = (u32)(C - 1 - (jv * CHK + 4 * sq)) & 0x80000000u;
 #pragma unroll
         for (int p = 0; p < NPASS; ++p)
             st[p] = __builtin_amdgcn_raw_buffer_load_b64(
                 r, (voff0[p] + (u32)(jv * CHK) * (u32)sizeof(T)) | c_bad, 0, 0);
     };
+    // registers -> LDS; direct loads: wait for them (the counter retires in issue order, so
+    // that is a wait for everything issued before them as well)
     auto stage_store = [&](int j) __attribute__((always_inline)) {
-        u32 *dst = lds + (j & 1) * BUF;
+        if constexpr (DMA) {
+#if defined(__HIP_DEVICE_COMPILE__)
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#endif
+            return;
+        }
+        u32 *dst = lds + (j & 1) * BUFA;
 #pragma unroll
         for (int p = 0; p < NPASS; ++p) {
             const int pos = p * (NT / 16) + tid / 16;
@@ -215,6 +281,18 @@ sapa_b_nhwc16_kernel(const T *__restrict__ q, const T *__restrict__ key,
         }
     };
 
+    // every wave is done with the current window and the next one is in LDS (direct loads:
+    // the bare barrier instruction -- the loads were waited for in stage_store, and a fence
+    // here would drain the output stores issued since)
+    auto chunk_barrier = [&]() __attribute__((always_inline)) {
+        if constexpr (DMA) {
+#if defined(__HIP_DEVICE_COMPILE__)
+            asm volatile("s_barrier" ::: "memory");
+#endif
+        } else {
+            __syncthreads();
+        }
+    };
     // this row's window origin: tap (ky, kx) of its parent sits at position
     // (wy + ky) * WW + 4 wx + row + kx.  Aggregation: lane li reads channels
     // 4 li .. 4 li + 3 (dwords 2 li, 2 li + 1 of the position); logits: lane
@@ -254,14 +332,14 @@ sapa_b_nhwc16_kernel(const T *__restrict__ q, const T *__restrict__ key,
     if (DO_QK) load_q(0, 0);
     stage_load(0);
     stage_store(0);
-    __syncthreads();
+    chunk_barrier();
 
     if (DO_QK) {
 #pragma unroll
         for (int i = 0; i < NR; ++i) w[i] = 0.f;
         for (int j = 0; j < nKc; ++j) {
             if (j + 1 < ntot) stage_load(j + 1);
-            const u32 *kb = kwin + (j & 1) * BUF;
+            const u32 *kb = kwin + (j & 1) * BUFA;
             // optional per-image bias of the query projection [B, d]: key . (q + b) =
             // key . q + key . b, the second product as four more instructions per tap
             // group with the bias as the B operand (same for the four children)
@@ -304,7 +382,7 @@ sapa_b_nhwc16_kernel(const T *__restrict__ q, const T *__restrict__ key,
                 });
             }
             if (j + 1 < ntot) stage_store(j + 1);
-            __syncthreads();
+            chunk_barrier();
         }
         if (DO_SOFTMAX) {
             // a child's taps lie in this lane's registers of its group and in the
@@ -386,13 +464,19 @@ sapa_b_nhwc16_kernel(const T *__restrict__ q, const T *__restrict__ key,
                     wlo[g][gi] = u32x2{pack2<T>(x[0], x[1]), pack2<T>(x[2], x[3])};
                 }
             }
+        if constexpr (DMA) {
 #pragma unroll
-        for (int p = 0; p < NPASS; ++p)
-            voff0[p] = ((u32)(spix[p] * C + 4 * sq) * (u32)sizeof(T)) | ((u32)spix[p] & 0x80000000u);
+            for (int p = 0; p < NPD; ++p)
+                voff0[p] = ((u32)(dpix[p] * C + 8 * dq8[p]) * (u32)sizeof(T)) | ((u32)dpix[p] & 0x80000000u);
+        } else {
+#pragma unroll
+            for (int p = 0; p < NPASS; ++p)
+                voff0[p] = ((u32)(spix[p] * C + 4 * sq) * (u32)sizeof(T)) | ((u32)spix[p] & 0x80000000u);
+        }
         for (int j = nKc; j < ntot; ++j) {
             if (j + 1 < ntot) stage_load_value(j + 1 - nKc);
             const int c0 = (j - nKc) * CHK;
-            const u32 *wb = win + (j & 1) * BUF;
+            const u32 *wb = win + (j & 1) * BUFA;
             // acc[g][u][i]: child 4g + i, channel c0 + 4 li + u
             f32x4 acc[NG][4];
 #pragma unroll
@@ -441,7 +525,7 @@ sapa_b_nhwc16_kernel(const T *__restrict__ q, const T *__restrict__ key,
                     __builtin_nontemporal_store(o, (u32x2 *)(out + child_pixel(jj) * C + c0 + 4 * li));
                 }
             }
-            __syncthreads();
+            chunk_barrier();
         }
     }
 }
