@@ -15,7 +15,7 @@ CSRC = os.path.join(HERE, 'csrc')
 OBJ = os.path.join(CSRC, '_obj')
 LIBDIR = os.path.join(HERE, 'lib')
 LIB = os.path.join(LIBDIR, 'libsapa_hip.so')
-SOURCES = ['capi.hip', 'sapa_b_generic.hip', 'sapa_b_tiled.hip', 'sapa_b_dot2.hip', 'sapa_b_nhwc.hip', 'sapa_b_nhwc_mm.hip', 'sapa_b_nhwc16.hip', 'sapa_b_mfma.hip', 'sapa_b_lowgrad.hip', 'sapa_d.hip', 'sapa_d_lowgrad.hip', 'sapa_d_nhwc.hip', 'sapa_d_wmat16.hip', 'sapa_d_backward.hip', 'sapa_d_bwdmat.hip', 'sapa_d_scatter.hip', 'sapa_moments.hip', 'sapa_project.hip', 'sapa_layout.hip', 'sapa_stream.hip',
+SOURCES = ['capi.hip', 'sapa_b_generic.hip', 'sapa_b_tiled.hip', 'sapa_b_dot2.hip', 'sapa_b_wmat16.hip', 'sapa_b_nhwc.hip', 'sapa_b_nhwc_mm.hip', 'sapa_b_nhwc16.hip', 'sapa_b_mfma.hip', 'sapa_b_lowgrad.hip', 'sapa_d.hip', 'sapa_d_lowgrad.hip', 'sapa_d_nhwc.hip', 'sapa_d_wmat16.hip', 'sapa_d_backward.hip', 'sapa_d_bwdmat.hip', 'sapa_d_scatter.hip', 'sapa_moments.hip', 'sapa_project.hip', 'sapa_layout.hip', 'sapa_stream.hip',
            'sapa_d_lds.hip']
 
 HIPCC = os.environ.get('HIPCC', '/opt/rocm/bin/hipcc')
@@ -23,10 +23,11 @@ HIPCC = os.environ.get('HIPCC', '/opt/rocm/bin/hipcc')
 FLAGS = ['-O3', '-std=c++17', '--offload-arch=gfx950', '-fPIC', '-fno-gpu-rdc',
          '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
          '-Wall', '-Wno-unused-function']
-# sapa_b_nhwc / sapa_b_nhwc_mm / sapa_b_nhwc16 / sapa_d_nhwc / sapa_d_wmat16 / sapa_d_bwdmat / sapa_d_scatter keep their MFMA accumulators in ordinary VGPRs: left to itself the
+# sapa_b_wmat16 / sapa_b_nhwc / sapa_b_nhwc_mm / sapa_b_nhwc16 / sapa_d_nhwc / sapa_d_wmat16 / sapa_d_bwdmat / sapa_d_scatter keep their MFMA accumulators in ordinary VGPRs: left to itself the
 # compiler moves them to the accumulation registers on top of an already full
 # VGPR budget, which costs the kernels a wave per SIMD
-SOURCE_FLAGS = {'sapa_b_nhwc.hip': ['-mllvm', '-amdgpu-mfma-vgpr-form'],
+SOURCE_FLAGS = {'sapa_b_wmat16.hip': ['-mllvm', '-amdgpu-mfma-vgpr-form'],
+                'sapa_b_nhwc.hip': ['-mllvm', '-amdgpu-mfma-vgpr-form'],
                 'sapa_b_nhwc_mm.hip': ['-mllvm', '-amdgpu-mfma-vgpr-form'],
                 'sapa_b_nhwc16.hip': ['-mllvm', '-amdgpu-mfma-vgpr-form'],
                 'sapa_d_nhwc.hip': ['-mllvm', '-amdgpu-mfma-vgpr-form'],

@@ -52,6 +52,11 @@ hipError_t tiled_launch(int mode, const void *q, const void *key, const void *at
     if (K == 5 && s == 2 && dtype != SAPA_F64 && mode == TILED_FUSED && (long)B * H * W <= kSmallFusedCells)
         e = took("sapa_b_mfma_kernel",
                  sapa_b_mfma_launch(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, dtype, st));
+#ifndef SAPA_WMAT16_OFF
+    if (e == hipErrorNotSupported)
+        e = took("sapa_b_wmat16_kernel",
+                 sapa_b_wmat16_launch(mode, q, key, value, out, B, d, C, H, W, K, s, dtype, st));
+#endif
     if (e == hipErrorNotSupported)
         e = took("sapa_b_dot2_kernel", sapa_b_dot2_launch(mode, q, key, attn_in, value, out, B,
                                                           d, C, H, W, K, s, dtype, st));

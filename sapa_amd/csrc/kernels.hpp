@@ -165,6 +165,12 @@ hipError_t sapa_b_dot2_launch(int mode, const void *q, const void *key, const vo
                               const void *value, void *out, int B, int d, int C, int H, int W,
                               int K, int s, int dtype, hipStream_t st, bool wide = false);
 
+// sapa_b_wmat16.hip: the fused forward for contiguous f16 / bf16 tensors (K = 5, s = 2) as two
+// dense products over the 8 x 8 window of each 4 x 4 block of parents, on the 16-bit matrix
+// instructions; hipErrorNotSupported otherwise.
+hipError_t sapa_b_wmat16_launch(int mode, const void *q, const void *key, const void *value, void *out, int B,
+                                int d, int C, int H, int W, int K, int s, int dtype, hipStream_t st);
+
 // sapa_b_mfma.hip: the same four modes on the matrix pipe (4x4x1 MFMA, one
 // block per parent); hipErrorNotSupported when (K, s, dtype) has no instance.
 hipError_t sapa_b_mfma_launch(int mode, const void *q, const void *key, const void *attn_in,
