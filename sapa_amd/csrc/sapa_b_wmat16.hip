@@ -26,15 +26,18 @@
 // The 4 x 4 output blocks go back through LDS so that global stores are 16 bytes per lane along
 // whole tile rows.
 //
-// All global -> LDS traffic is direct (buffer loads with the LDS modifier: 4-byte pieces of the
-// low-res windows, whose origin is 2 cells left of an aligned address, 16-byte pieces of q); an
-// offset of 2^31 is outside every descriptor and reads as zero.  The q / output tile is stored
-// with its 16-byte pieces XOR-swizzled so that transposing reads, accumulator writes and the
-// linear store pass are all free of 4-way bank conflicts without padding.
+// All global -> LDS traffic is direct (buffer loads with the LDS modifier, 16 bytes per lane); an
+// offset of 2^31 is outside every descriptor and reads as zero, which is the zero padding above
+// and below the image.  A window row starts 2 cells left of its block, so its 16-byte pieces are
+// only 4-byte aligned in memory and the first / last of a row run over the row's ends: what they
+// bring from the neighbouring row is put right in the registers (logit 0, weight 0 for a cell left
+// of x = 0 or right of x = W - 1).  The q / output tile is stored with its 16-byte pieces
+// XOR-swizzled so that transposing reads, accumulator writes and the linear store pass are all
+// free of 4-way bank conflicts without padding.
 //
-// A cell whose weight is zero still enters the aggregation as 0 * value: a non-finite value
-// spreads to every child of the 4 x 4 block whose window holds it rather than to the 25-cell
-// neighbourhoods only.
+// Masked cells still enter both products (a logit plus -inf, a weight of 0 times a value): a
+// non-finite key or value spreads to every child of the 4 x 4 block whose window holds it rather
+// than to the 25-cell neighbourhoods only.
 #include "kernels.hpp"
 
 namespace sapa {
@@ -51,9 +54,6 @@ constexpr int CHK = 16;            // channels per staged chunk
 constexpr int WROWS = 8;           // window rows = child rows of a block row
 constexpr u32 OUTSIDE = 0x80000000u;
 
-#ifndef SAPA_WM16_DEPTH
-#define SAPA_WM16_DEPTH 2
-#endif
 #ifndef SAPA_WM16_NSW
 #define SAPA_WM16_NSW 16
 #endif
@@ -100,7 +100,7 @@ __device__ __forceinline__ int swz(int ch, int r) { return ((ch & 7) << 1) | ((r
 // low-res windows, which neighbouring tiles re-read, out of the caches (fused FPN-large bf16, 860 MB:
 // 271 -> 213 us; at a quarter of the size, where everything fits the memory-side cache, 50 -> 58 us:
 // the launcher decides by size)
-template <typename T, int NSW, int ND, bool STREAM>
+template <typename T, int NSW, bool STREAM>
 __global__ __launch_bounds__(64 * NSW) void
 sapa_b_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key, const T *__restrict__ value,
                      T *__restrict__ out, int d, int C, int H, int W, int tiles_x, int tiles_y, int ns,
@@ -119,9 +119,10 @@ sapa_b_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key, const T
     static_assert(NSW == 16 || NSW == 8, "piece swizzle");
     constexpr int NPC = 2 * NSW / 2;                         // 16-byte pieces per tile row = NSW
 
-    // rings of ND buffers: chunk j lives in buffer j % ND and is requested ND - 1 chunks ahead
-    __shared__ __attribute__((aligned(16))) u32 lds[ND * (LOWBUF + HIBUF)];
-    u32 *const lowbuf = lds, *const hibuf = lds + ND * LOWBUF;
+    // two buffers of each kind (three, i.e. requests two chunks ahead, measured slower: 208 against
+    // 199 us at FPN-large)
+    __shared__ __attribute__((aligned(16))) u32 lds[2 * (LOWBUF + HIBUF)];
+    u32 *const lowbuf = lds, *const hibuf = lds + 2 * LOWBUF;
 
     const int logical = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
     if (logical >= nblocks) return;
@@ -173,92 +174,76 @@ sapa_b_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key, const T
         (void *)(out + (long)n * C * 4 * lpix), 0, (int)(C * hplane), 0x00020000);
 
     (void)rq, (void)rk, (void)rv;
-    // chunk j: key + q channels 16 j .. for j < nKc, value channels 16 (j - nKc) .. after; every
-    // wave issues the same number of loads for a chunk (the waits below count them).  A channel
-    // past the tensor's last lies past the descriptor: zeros.
-    auto stage = [&](int j) __attribute__((always_inline)) {
+    // Chunk j is the key + q channels 16 j .. for j < nKc and the value channels 16 (j - nKc) ..
+    // after; it lives in buffer j % 2 and is requested two chunks ahead, as soon as every wave is
+    // done with that buffer.  A channel past the tensor's last lies past the descriptor: zeros.
+    auto stage_low = [&](__amdgpu_buffer_rsrc_t r, u32 c0, int buf) __attribute__((always_inline)) {
 #if defined(__HIP_DEVICE_COMPILE__)
-        const bool is_key = j < nKc;
-        const u32 c0 = (u32)((is_key ? j : j - nKc) * CHK);
-        const __amdgpu_buffer_rsrc_t r = is_key ? rk : rv;
-        u32 *lb = lowbuf + (j % ND) * LOWBUF + wave * 256;
+        u32 *lb = lowbuf + buf * LOWBUF + wave * 256;
 #pragma unroll
         for (int i = 0; i < NLI; ++i)
             if ((i + 1) * NT <= NLP || i * NT + wave * 64 < NLP)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void *)(lb + i * NT * 4), 16,
                                                          off_low[i] + c0 * lplane, 0, 0, 0);
-        if (is_key) {
-            u32 *hb = hibuf + (j % ND) * HIBUF + wave * 256;
-#pragma unroll
-            for (int i = 0; i < NHI; ++i)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rq, (__attribute__((address_space(3))) void *)(hb + i * NT * 4),
-                                                         16, off_hi[i] + c0 * hplane, 0, 0, STREAM ? 2 : 0);
-        }
 #endif
     };
-    // vector-memory operations a wave issues for chunk i / the stores that follow iteration i
-    const int n_low = (NLP - wave * 64 + NT - 1) / NT;
-    auto n_loads = [&](int i) { return i >= ntot ? 0 : n_low + (i < nKc ? NHI : 0); };
-    auto n_stores = [&](int i) { return i >= nKc ? NHI : 0; };
-    // chunk j + 1 has landed in this wave's slots (the counter retires in issue order: all but
-    // the `after` operations issued after its loads may stay in flight), this wave's LDS writes
-    // are done; then every wave's
-    auto landed = [&](int after) __attribute__((always_inline)) {
+    auto stage_q = [&](u32 c0, int buf) __attribute__((always_inline)) {
+#if defined(__HIP_DEVICE_COMPILE__)
+        u32 *hb = hibuf + buf * HIBUF + wave * 256;
+#pragma unroll
+        for (int i = 0; i < NHI; ++i)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rq, (__attribute__((address_space(3))) void *)(hb + i * NT * 4), 16,
+                                                     off_hi[i] + c0 * hplane, 0, 0, STREAM ? 2 : 0);
+#endif
+    };
+    auto stage = [&](int j) __attribute__((always_inline)) {
+        if (j < nKc) {
+            stage_low(rk, (u32)(j * CHK), j & 1);
+            stage_q((u32)(j * CHK), j & 1);
+        } else if (j < ntot) {
+            stage_low(rv, (u32)((j - nKc) * CHK), j & 1);
+        }
+    };
+    // Waits are counted: the counter of vector-memory operations retires in issue order, so
+    // "at most N outstanding" means that everything but the last N issued is complete.  Written out
+    // because the compiler does not track a direct load's LDS write.
+    auto wait_all_but = [&](int after) __attribute__((always_inline)) {
 #if defined(__HIP_DEVICE_COMPILE__)
 #define SAPA_WM16_WAIT(N) case N: asm volatile("s_waitcnt vmcnt(" #N ")" ::: "memory"); break;
-        // (the two counts of the steady states first: a chain of scalar branches otherwise)
-        if (after == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        else if (after == NHI) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NHI) : "memory");
-        else switch (after) {
-            SAPA_WM16_WAIT(1) SAPA_WM16_WAIT(2) SAPA_WM16_WAIT(3) SAPA_WM16_WAIT(4) SAPA_WM16_WAIT(5)
-            SAPA_WM16_WAIT(6) SAPA_WM16_WAIT(7) SAPA_WM16_WAIT(8) SAPA_WM16_WAIT(9) SAPA_WM16_WAIT(10)
-            SAPA_WM16_WAIT(11) SAPA_WM16_WAIT(12) SAPA_WM16_WAIT(13) SAPA_WM16_WAIT(14) SAPA_WM16_WAIT(15)
-            SAPA_WM16_WAIT(16) SAPA_WM16_WAIT(17) SAPA_WM16_WAIT(18) SAPA_WM16_WAIT(19) SAPA_WM16_WAIT(20)
+        switch (after) {
+            SAPA_WM16_WAIT(1) SAPA_WM16_WAIT(2) SAPA_WM16_WAIT(3) SAPA_WM16_WAIT(4)
             default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
         }
 #undef SAPA_WM16_WAIT
 #endif
     };
-    // chunk jn has landed in this wave's slots: the 6 cells of the piece that has no address
-    // (first row of the image's first channel, tile at the left edge)
+    // chunk jn (the first of the keys or of the values) has landed in this wave's slots: the 6
+    // cells of the piece that has no address (first row of the image's first channel, tile at the
+    // left edge)
     auto patch_low = [&](int jn) __attribute__((always_inline)) {
-        if (tx == 0 && ty == 0 && (jn == 0 || jn == nKc) && jn < ntot) {
-            if (patch_slot >= 0) {
-                const __amdgpu_buffer_rsrc_t r = jn < nKc ? rk : rv;
-                u32 *dst = lowbuf + (jn % ND) * LOWBUF + patch_slot * 4;
+        if (tx == 0 && ty == 0 && patch_slot >= 0) {
+            const __amdgpu_buffer_rsrc_t r = jn < nKc ? rk : rv;
+            u32 *dst = lowbuf + (jn & 1) * LOWBUF + patch_slot * 4;
 #pragma unroll
-                for (int k = 1; k < 4; ++k) dst[k] = __builtin_amdgcn_raw_buffer_load_b32(r, 4 * (k - 1), 0, 0);
-            }
+            for (int k = 1; k < 4; ++k) dst[k] = __builtin_amdgcn_raw_buffer_load_b32(r, 4 * (k - 1), 0, 0);
         }
     };
+    // this wave's LDS writes are done; then every wave's (and every wave's landed loads)
     auto barrier = [&]() __attribute__((always_inline)) {
 #if defined(__HIP_DEVICE_COMPILE__)
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 #endif
     };
-    auto landed_barrier = [&](int after, int jn) __attribute__((always_inline)) {
-        landed(after);
-        patch_low(jn);
-        barrier();
-    };
-    // operations issued after chunk j + 1's loads by the time iteration j waits for them: the
-    // stores of iteration j + 1 - ND, then loads and stores of the iterations up to j - 1
-    auto after_next = [&](int j) {
-        int a = n_stores(j + 1 - ND);
-        for (int i = j + 2 - ND; i < j; ++i) a += n_loads(i + ND) + n_stores(i);
-        return a > 20 ? 0 : a;
-    };
 
     const bool active = wave < ns_here;
     const int t = wave;                                       // this wave's block of the tile
 
-    for (int i = 0; i < ND; ++i)
-        if (i < ntot) stage(i);
-    {
-        int a = 0;
-        for (int i = 1; i < ND; ++i) a += n_loads(i);
-        landed_barrier(a, 0);
-    }
+    stage(0);
+    stage(1);
+    // chunk 0: all but chunk 1's loads
+    wait_all_but(ntot < 2 ? 0 : (NLP - wave * 64 + NT - 1) / NT + (1 < nKc ? NHI : 0));
+    patch_low(0);
+    barrier();
 
     // ---- logits: Sim[cell][child], 4 x 4 accumulator blocks of 16 x 16 ----
     // block (mb, nb), lane (g, i16), element v: cell (row 2 mb + g / 2, column 4 (g % 2) + v) of the
@@ -273,7 +258,7 @@ sapa_b_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key, const T
     const int tch = 4 * g + (i16 >> 2), trow = (i16 & 3) >> 1, tcol = i16 & 1;
     for (int j = 0; j < nKc; ++j) {
         if (active) {
-            const u32 *kb = lowbuf + (j % ND) * LOWBUF, *qb = hibuf + (j % ND) * HIBUF;
+            const u32 *kb = lowbuf + (j & 1) * LOWBUF, *qb = hibuf + (j & 1) * HIBUF;
             u32x2 a[4], b[4];
 #pragma unroll
             for (int mb = 0; mb < 4; ++mb)
@@ -288,8 +273,11 @@ sapa_b_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key, const T
 #pragma unroll
                 for (int nb = 0; nb < 4; ++nb) sim[mb][nb] = Mma<T>::k16(a[mb], b[nb], sim[mb][nb]);
         }
-        landed_barrier(after_next(j), j + 1);
-        if (j + ND < ntot) stage(j + ND);
+        // chunk j + 1: nothing was issued after its loads
+        wait_all_but(0);
+        if (j + 1 == nKc) patch_low(nKc);
+        barrier();
+        stage(j + 2);
     }
 
     // ---- softmax over each child's 5 x 5 cells; the weights as A operands of the aggregation ----
@@ -377,7 +365,7 @@ sapa_b_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key, const T
         const u32 c0 = (u32)((j - nKc) * CHK);
         u32 *ob = hibuf + (j & 1) * HIBUF;                      // no loads into this ring any more
         if (active) {
-            const u32 *vb = lowbuf + (j % ND) * LOWBUF;
+            const u32 *vb = lowbuf + (j & 1) * LOWBUF;
             // B operand of step s: lane (g, channel i16) holds the cells of rows 4 s + g / 2 and
             // 4 s + 2 + g / 2, columns 4 (g % 2) .. + 3 -- the order the weights are held in
             u32x4 b[2];
@@ -401,8 +389,11 @@ sapa_b_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key, const T
                     u32x2{pack2<T>(acc[0], acc[1]), pack2<T>(acc[2], acc[3])};
             }
         }
-        landed_barrier(after_next(j), j + 1);
-        if (j + ND < ntot) stage(j + ND);
+        // chunk j + 1: its loads were the last operations issued
+#if defined(__HIP_DEVICE_COMPILE__)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#endif
+        barrier();
         // the tile's 16 channels x 8 rows, 16 bytes per lane, right after the barrier that completes
         // them (sending them behind the next chunk's matrix instructions measured slower); a piece
         // outside the tensor (ragged tile, channel past the last) lies outside the descriptor and
@@ -413,10 +404,12 @@ sapa_b_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key, const T
             if constexpr (STREAM) __builtin_amdgcn_raw_buffer_store_b128(o, ro, off_hi[i] + c0 * hplane, 0, 2);
             else __builtin_amdgcn_raw_buffer_store_b128(o, ro, off_hi[i] + c0 * hplane, 0, 0);
         }
+        // (the next request behind the stores: 208 us at FPN-large against 216 with the loads first)
+        if (j + 2 < ntot) stage_low(rv, (u32)((j + 2 - nKc) * CHK), j & 1);
     }
 }
 
-template <typename T, int NSW, int ND, bool STREAM>
+template <typename T, int NSW, bool STREAM>
 static hipError_t launch_geom(const void *q, const void *key, const void *value, void *out, int B, int d,
                               int C, int H, int W, hipStream_t st) {
     const int nsx = W / 4;
@@ -425,7 +418,7 @@ static hipError_t launch_geom(const void *q, const void *key, const void *value,
     const long nb = (long)tiles_x * tiles_y * B;
     if (nb > (1L << 30)) return hipErrorNotSupported;
     const int per_xcd = (int)((nb + 7) / 8);
-    hipLaunchKernelGGL((sapa_b_wmat16_kernel<T, NSW, ND, STREAM>), dim3(per_xcd * 8), dim3(64 * NSW), 0, st, (const T *)q,
+    hipLaunchKernelGGL((sapa_b_wmat16_kernel<T, NSW, STREAM>), dim3(per_xcd * 8), dim3(64 * NSW), 0, st, (const T *)q,
                        (const T *)key, (const T *)value, (T *)out, d, C, H, W, tiles_x, tiles_y, ns, (int)nb,
                        per_xcd);
     return hipGetLastError();
@@ -447,10 +440,10 @@ hipError_t sapa_b_wmat16_launch(int mode, const void *q, const void *key, const 
     // bytes read and written once; beyond the 256 MB memory-side cache they are streamed
     const bool stream = 2L * ((long)B * H * W * (5L * d + 5L * C)) > (256L << 20);
     if (dtype == 2)
-        return stream ? wm16::launch_geom<f16_t, SAPA_WM16_NSW, SAPA_WM16_DEPTH, true>(q, key, value, out, B, d, C, H, W, st)
-                      : wm16::launch_geom<f16_t, SAPA_WM16_NSW, SAPA_WM16_DEPTH, false>(q, key, value, out, B, d, C, H, W, st);
-    return stream ? wm16::launch_geom<bf16_t, SAPA_WM16_NSW, SAPA_WM16_DEPTH, true>(q, key, value, out, B, d, C, H, W, st)
-                  : wm16::launch_geom<bf16_t, SAPA_WM16_NSW, SAPA_WM16_DEPTH, false>(q, key, value, out, B, d, C, H, W, st);
+        return stream ? wm16::launch_geom<f16_t, SAPA_WM16_NSW, true>(q, key, value, out, B, d, C, H, W, st)
+                      : wm16::launch_geom<f16_t, SAPA_WM16_NSW, false>(q, key, value, out, B, d, C, H, W, st);
+    return stream ? wm16::launch_geom<bf16_t, SAPA_WM16_NSW, true>(q, key, value, out, B, d, C, H, W, st)
+                  : wm16::launch_geom<bf16_t, SAPA_WM16_NSW, false>(q, key, value, out, B, d, C, H, W, st);
 }
 
 }  // namespace sapa

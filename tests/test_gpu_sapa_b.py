@@ -196,6 +196,49 @@ def test_16bit_dot_product_kernels(coracle, shape, dtype, rel):
     assert_rel_rms_close(got.float(), coracle.sapa_fused(qf, kf, vf, K, s, 'f32a64'), rel, 'fused')
 
 
+# Fused, contiguous 16-bit tensors, K = 5, s = 2, W a multiple of 4, more than 12288 low-res cells (smaller
+# problems take the lane-per-child kernel): two dense products per 4 x 4 block of parents on the 16-bit matrix
+# instructions.  (B, d, C, H, W): one tile of 8 blocks; ragged tile rows, d and C off the 16-channel chunks;
+# a single tile of 13 blocks; 7 tiles in x; two unequal tiles; the FPN geometry (3 tiles of 14 blocks) with
+# odd channel counts.
+DENSE16_SHAPES = [(13, 16, 16, 32, 32), (2, 24, 40, 79, 80), (5, 40, 24, 51, 52), (1, 64, 48, 30, 420),
+                  (3, 32, 16, 66, 68), (1, 17, 19, 100, 168)]
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('shape', DENSE16_SHAPES, ids=['-'.join(map(str, s)) for s in DENSE16_SHAPES])
+def test_16bit_dense_window_kernel(coracle, shape, dtype):
+    """Products of 16-bit values are exact in fp32, sums and softmax are fp32, the weights enter the
+    aggregation as a 16-bit value plus a 16-bit remainder: what is left is the rounding of the result, at
+    most half a 16-bit spacing (2^-8 resp. 2^-11 of the value) against the double-precision oracle."""
+    B, d, C, H, W = shape
+    g = gen(131)
+    q, key, v = (randn(g, *sh).to(dtype) for sh in ((B, d, H * 2, W * 2), (B, d, H, W), (B, C, H, W)))
+    half_ulp = 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
+    got = sapa_amd.sapa_fused(*dev(q, key, v), 5, 2)
+    assert sapa_amd._lib.last_kernel() == 'sapa_b_wmat16_kernel'
+    assert got.dtype == dtype and got.shape == (B, C, 2 * H, 2 * W)
+    exact = torch.cat([coracle.sapa_fused(q[i:i + 1].float(), key[i:i + 1].float(), v[i:i + 1].float(), 5, 2, 'f32a64')
+                       for i in range(B)]).double()
+    err = (got.float().cpu().double() - exact).abs()
+    worst = (err / torch.maximum(exact.abs(), exact.square().mean().sqrt())).max().item()
+    assert worst <= 1.05 * half_ulp, f'{shape} {dtype}: {worst / half_ulp:.2f} half-spacings'
+    # zero query: every child weighs the 25 cells of its own window equally and the rest of the 8 x 8
+    # window not at all -- the box filter of the value, zero padding counted.  Positive values, large on
+    # the border cells, and a bar relative to each element: a cell too many or too few at an edge, a
+    # shifted window row or column shows at once.
+    vp = v.float().abs() + 0.5
+    for sl in ((slice(None), slice(None), 0), (slice(None), slice(None), -1),
+               (slice(None), slice(None), slice(None), 0), (slice(None), slice(None), slice(None), -1)):
+        vp[sl] *= 64.0
+    vp = vp.to(dtype)
+    got0 = sapa_amd.sapa_fused(torch.zeros_like(q).to(DEV), key.to(DEV), vp.to(DEV), 5, 2)
+    assert sapa_amd._lib.last_kernel() == 'sapa_b_wmat16_kernel'
+    box = F.interpolate(F.avg_pool2d(vp.double(), 5, 1, 2, count_include_pad=True), scale_factor=2)
+    rel = ((got0.float().cpu().double() - box).abs() / box).max().item()
+    assert rel <= 1.05 * half_ulp + 1e-6, f'{shape} {dtype} box filter: {rel / half_ulp:.2f} half-spacings'
+
+
 @pytest.mark.parametrize('shape', [SHAPES[0], SHAPES[6]], ids=[IDS[0], IDS[6]])
 def test_fp64(coracle, shape):
     B, d, C, H, W, K, s = shape
