@@ -45,18 +45,19 @@ const long kSmallFusedCells = 12288;
 hipError_t tiled_launch(int mode, const void *q, const void *key, const void *attn_in,
                         const void *value, void *out, int B, int d, int C, int H, int W, int K,
                         int s, int dtype, hipStream_t st) {
-    // small fused problems of the common window first: the matrix-pipe kernel's lane-per-child
-    // decomposition fills the chip where the thread-per-parent kernels leave it latency-bound
-    // (B=8, d=32, C=256, fp32: 16x16 32 -> 12 us, 32x32 32 -> 23 us)
+    // 16-bit fused problems of the common window first: both products on the 16-bit matrix
+    // instructions, whatever the size (B=8, d=32, C=256, bf16: 32x32 21 -> 16 us, 64x64 48 -> 20 us)
     hipError_t e = hipErrorNotSupported;
-    if (K == 5 && s == 2 && dtype != SAPA_F64 && mode == TILED_FUSED && (long)B * H * W <= kSmallFusedCells)
+#ifndef SAPA_WMAT16_OFF
+    e = took("sapa_b_wmat16_kernel", sapa_b_wmat16_launch(mode, q, key, value, out, B, d, C, H, W, K, s, dtype, st));
+#endif
+    // small fused problems next: the matrix-pipe kernel's lane-per-child decomposition fills the
+    // chip where the thread-per-parent kernels leave it latency-bound
+    // (B=8, d=32, C=256, fp32: 16x16 32 -> 12 us, 32x32 32 -> 23 us)
+    if (e == hipErrorNotSupported && K == 5 && s == 2 && dtype != SAPA_F64 && mode == TILED_FUSED &&
+        (long)B * H * W <= kSmallFusedCells)
         e = took("sapa_b_mfma_kernel",
                  sapa_b_mfma_launch(mode, q, key, attn_in, value, out, B, d, C, H, W, K, s, dtype, st));
-#ifndef SAPA_WMAT16_OFF
-    if (e == hipErrorNotSupported)
-        e = took("sapa_b_wmat16_kernel",
-                 sapa_b_wmat16_launch(mode, q, key, value, out, B, d, C, H, W, K, s, dtype, st));
-#endif
     if (e == hipErrorNotSupported)
         e = took("sapa_b_dot2_kernel", sapa_b_dot2_launch(mode, q, key, attn_in, value, out, B,
                                                           d, C, H, W, K, s, dtype, st));

@@ -54,9 +54,6 @@ constexpr int CHK = 16;            // channels per staged chunk
 constexpr int WROWS = 8;           // window rows = child rows of a block row
 constexpr u32 OUTSIDE = 0x80000000u;
 
-#ifndef SAPA_WM16_NSW
-#define SAPA_WM16_NSW 16
-#endif
 
 template <typename T> struct Mma;
 template <> struct Mma<f16_t> {
@@ -128,7 +125,7 @@ sapa_b_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key, const T
     if (logical >= nblocks) return;
     const int tx = logical % tiles_x, ty = (logical / tiles_x) % tiles_y, n = logical / (tiles_x * tiles_y);
     const int X0 = tx * 4 * ns, Y0 = ty * 4;                 // first parent of the tile
-    const int nsx = W / 4;
+    const int nsx = (W + 3) / 4;
     const int ns_here = nsx - tx * ns < ns ? nsx - tx * ns : ns;
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -144,6 +141,7 @@ sapa_b_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key, const T
     // that starts 2 cells before the image's first has no address: it reads as zeros and its 6
     // cells are fetched apart (patch_low).
     u32 off_low[NLI], off_hi[NHI];
+    bool half_piece[NHI];      // W % 4 == 2: a row's last 16-byte piece holds 4 of its children and 4 of the next row's
     int patch_slot = -1;
 #pragma unroll
     for (int i = 0; i < NLI; ++i) {
@@ -161,6 +159,7 @@ sapa_b_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key, const T
         const int cy = 2 * Y0 + r, cx = 2 * X0 + 8 * pc;
         const bool ok = pc < ns_here && cy < 2 * H && cx < 2 * W;
         off_hi[i] = ok ? (u32)(ch * 4 * lpix + (long)cy * 2 * W + cx) * (u32)sizeof(T) : OUTSIDE;
+        half_piece[i] = ok && cx + 8 > 2 * W;
     }
 
     const int nKc = (d + CHK - 1) / CHK, nVc = (C + CHK - 1) / CHK, ntot = nKc + nVc;
@@ -235,6 +234,7 @@ sapa_b_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key, const T
 #endif
     };
 
+    const bool row_tail = (W & 3) != 0 && X0 + 4 * ns_here > W;      // wave-uniform
     const bool active = wave < ns_here;
     const int t = wave;                                       // this wave's block of the tile
 
@@ -401,8 +401,13 @@ sapa_b_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key, const T
 #pragma unroll
         for (int i = 0; i < NHI; ++i) {
             const u32x4 o = *(const u32x4 *)(ob + (i * NT + tid) * 4);
-            if constexpr (STREAM) __builtin_amdgcn_raw_buffer_store_b128(o, ro, off_hi[i] + c0 * hplane, 0, 2);
-            else __builtin_amdgcn_raw_buffer_store_b128(o, ro, off_hi[i] + c0 * hplane, 0, 0);
+            u32 off = off_hi[i] + c0 * hplane;
+            if (row_tail && half_piece[i]) {
+                __builtin_amdgcn_raw_buffer_store_b64(u32x2{o[0], o[1]}, ro, off, 0, 0);
+                off = OUTSIDE;
+            }
+            if constexpr (STREAM) __builtin_amdgcn_raw_buffer_store_b128(o, ro, off, 0, 2);
+            else __builtin_amdgcn_raw_buffer_store_b128(o, ro, off, 0, 0);
         }
         // (the next request behind the stores: 208 us at FPN-large against 216 with the loads first)
         if (j + 2 < ntot) stage_low(rv, (u32)((j + 2 - nKc) * CHK), j & 1);
@@ -412,7 +417,7 @@ sapa_b_wmat16_kernel(const T *__restrict__ q, const T *__restrict__ key, const T
 template <typename T, int NSW, bool STREAM>
 static hipError_t launch_geom(const void *q, const void *key, const void *value, void *out, int B, int d,
                               int C, int H, int W, hipStream_t st) {
-    const int nsx = W / 4;
+    const int nsx = (W + 3) / 4;
     const int tiles_x = (nsx + NSW - 1) / NSW, tiles_y = (H + 3) / 4;
     const int ns = (nsx + tiles_x - 1) / tiles_x;             // blocks per tile, balanced over the row
     const long nb = (long)tiles_x * tiles_y * B;
@@ -426,24 +431,27 @@ static hipError_t launch_geom(const void *q, const void *key, const void *value,
 
 }  // namespace wm16
 
-// Fused forward only; f16 / bf16, K = 5, s = 2, W a multiple of 4, low-res tensors 4-byte and
+// Fused forward only; f16 / bf16, K = 5, s = 2, W even (rows of whole dwords), low-res tensors 4-byte and
 // high-res tensors 16-byte aligned, every image of every tensor below 2 GiB (32-bit offsets
 // inside an image); hipErrorNotSupported otherwise.
 hipError_t sapa_b_wmat16_launch(int mode, const void *q, const void *key, const void *value, void *out, int B,
                                 int d, int C, int H, int W, int K, int s, int dtype, hipStream_t st) {
-    if (mode != TILED_FUSED || K != 5 || s != 2 || W % 4 != 0 || W < 16) return hipErrorNotSupported;
+    if (mode != TILED_FUSED || K != 5 || s != 2 || W % 2 != 0 || W < 16) return hipErrorNotSupported;
     if (dtype != 2 && dtype != 3) return hipErrorNotSupported;
     const long hplane = (long)H * W * 8;
     if ((long)(d > C ? d : C) * hplane >= (1L << 31)) return hipErrorNotSupported;
     if (((uintptr_t)key | (uintptr_t)value) % 4 != 0 || ((uintptr_t)q | (uintptr_t)out) % 16 != 0)
         return hipErrorNotSupported;
-    // bytes read and written once; beyond the 256 MB memory-side cache they are streamed
+    // bytes read and written once; beyond the 256 MB memory-side cache they are streamed, in tiles of
+    // up to 16 blocks (longer rows per store); what fits the cache takes tiles of 8 blocks, two
+    // workgroups per CU (FPN 25x42 at B=16: 24 -> 19 us, SegFormer 64x64 at B=8: 25 -> 20 us).  The
+    // arithmetic of a child does not depend on the tiling: results are the same bit for bit.
     const bool stream = 2L * ((long)B * H * W * (5L * d + 5L * C)) > (256L << 20);
     if (dtype == 2)
-        return stream ? wm16::launch_geom<f16_t, SAPA_WM16_NSW, true>(q, key, value, out, B, d, C, H, W, st)
-                      : wm16::launch_geom<f16_t, SAPA_WM16_NSW, false>(q, key, value, out, B, d, C, H, W, st);
-    return stream ? wm16::launch_geom<bf16_t, SAPA_WM16_NSW, true>(q, key, value, out, B, d, C, H, W, st)
-                  : wm16::launch_geom<bf16_t, SAPA_WM16_NSW, false>(q, key, value, out, B, d, C, H, W, st);
+        return stream ? wm16::launch_geom<f16_t, 16, true>(q, key, value, out, B, d, C, H, W, st)
+                      : wm16::launch_geom<f16_t, 8, false>(q, key, value, out, B, d, C, H, W, st);
+    return stream ? wm16::launch_geom<bf16_t, 16, true>(q, key, value, out, B, d, C, H, W, st)
+                  : wm16::launch_geom<bf16_t, 8, false>(q, key, value, out, B, d, C, H, W, st);
 }
 
 }  // namespace sapa

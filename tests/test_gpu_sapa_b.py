@@ -196,13 +196,12 @@ def test_16bit_dot_product_kernels(coracle, shape, dtype, rel):
     assert_rel_rms_close(got.float(), coracle.sapa_fused(qf, kf, vf, K, s, 'f32a64'), rel, 'fused')
 
 
-# Fused, contiguous 16-bit tensors, K = 5, s = 2, W a multiple of 4, more than 12288 low-res cells (smaller
-# problems take the lane-per-child kernel): two dense products per 4 x 4 block of parents on the 16-bit matrix
-# instructions.  (B, d, C, H, W): one tile of 8 blocks; ragged tile rows, d and C off the 16-channel chunks;
+# Fused, contiguous 16-bit tensors, K = 5, s = 2, W even and at least 16: two dense products per 4 x 4 block
+# of parents on the 16-bit matrix instructions (small shapes of the lists above reach it as well).  (B, d, C, H, W): one tile of 8 blocks; ragged tile rows, d and C off the 16-channel chunks;
 # a single tile of 13 blocks; 7 tiles in x; two unequal tiles; the FPN geometry (3 tiles of 14 blocks) with
-# odd channel counts.
-DENSE16_SHAPES = [(13, 16, 16, 32, 32), (2, 24, 40, 79, 80), (5, 40, 24, 51, 52), (1, 64, 48, 30, 420),
-                  (3, 32, 16, 66, 68), (1, 17, 19, 100, 168)]
+# odd channel counts; rows that end inside a block and inside a 16-byte piece (W = 42: one tile, W = 70: two).
+DENSE16_SHAPES = [(1, 3, 5, 2, 16), (13, 16, 16, 32, 32), (2, 24, 40, 79, 80), (5, 40, 24, 51, 52), (1, 64, 48, 30, 420),
+                  (3, 32, 16, 66, 68), (1, 17, 19, 100, 168), (13, 20, 24, 25, 42), (2, 8, 8, 100, 70)]
 
 
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
