@@ -503,6 +503,27 @@ def main():
         err_cl = (cl[3][:1].float() - out[:1].float()).abs().max().item()
         del cl
 
+    half = None
+    if (not deform and args.dtype == 'fp32' and args.layout == 'nchw' and args.direction == 'forward'
+            and not args.only_main):
+        # the same workload and layout with bf16 tensors (the inputs rounded to bf16)
+        hq, hk, hv = (t.to(torch.bfloat16) for t in (q, key, v))
+        hout = torch.empty_like(out, dtype=torch.bfloat16)
+
+        def half_step():
+            _lib.check(lib.sapa_fused_forward(hq.data_ptr(), hk.data_ptr(), hv.data_ptr(), hout.data_ptr(), B, d, C,
+                                              H, W, K, s, 3, stream.cuda_stream), 'sapa_fused_forward')
+        ms_h, _ = timed(half_step)
+        hbytes = algorithmic_bytes(B, C, d, H, W, s, 2)
+        half = {'dtype': 'bf16', 'ms_per_step': ms_h, 'value': B * H * s * W * s / (ms_h * 1e-3) / 1e9,
+                'unit': 'Gpix/s', 'algorithmic_bytes': hbytes,
+                'roofline_frac': hbytes / (ms_h * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                'kernel': _lib.last_kernel() + ' (fused mode)',
+                'note': 'same workload, contiguous (NCHW) bf16 tensors (python bench.py --dtype bf16 makes this '
+                        'the main line); parity bar 1e-2 max(|b|, rms(b)), held by the tests to half a bf16 '
+                        'spacing of the double-precision result on the rounded inputs'}
+        del hq, hk, hv, hout
+
     reference_order = None
     if deform and main_is_ws and args.direction == 'forward' and not args.only_main:
         # the same contiguous tensors through the kernel that keeps the reference's order of sums
@@ -641,6 +662,8 @@ def main():
                            'the reference-order fp32 result printed and bounded there'),
             'note': 'same workload and algorithmic bytes, every tensor in torch.channels_last '
                     'order (python bench.py --layout channels_last makes this the main line)'}
+    if half is not None:
+        rec['bf16'] = half
     if reference_order is not None:
         reference_order['value'] = pix / (reference_order['ms_per_step'] * 1e-3) / 1e9
         reference_order['roofline_frac'] = abytes / (reference_order['ms_per_step'] * 1e-3) / 1e9 / HBM_PEAK_GBS
