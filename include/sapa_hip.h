@@ -153,8 +153,9 @@ int sapa_fused_backward(const void *grad_out, const void *query, const void *key
  * two passes, as the reference does (QKFunction / AVFunction save their operands,
  * sapa/sapa/sapa_func.py:28,73, and autograd keeps the softmax output):
  * sapa_fused_forward_attn writes attn [B,K*K,sH,sW] -- fp32 whatever `dtype` is --
- * next to out (two launches: the weights, then the aggregation with them; nothing
- * between them is rounded to 16 bits), and sapa_fused_backward_attn takes that
+ * next to out (two launches: the weights, then the aggregation with them -- for
+ * 16-bit tensors the one-launch forward, which forms the same fp32 weights itself;
+ * nothing between the two products is rounded to 16 bits either way), and sapa_fused_backward_attn takes that
  * tensor instead of recomputing it; its workspace holds grad_logits only
  * (sapa_fused_backward_attn_workspace bytes, half of the other's).  Same results
  * as sapa_fused_backward on the same operands, one launch less per step and a
