@@ -64,8 +64,8 @@ MEASURED_TRAFFIC = {
     ('fpn_large', 'bf16', 'nchw'): (944266161, 'profiles/sapa_b_fused_fpn_large_bf16.md', 'sapa_b_wmat16_kernel'),
     ('fpn_large', 'fp32', 'channels_last'): (1720501334, 'profiles/sapa_b_nhwc_fused_fpn_large_fp32.md',
                                              'sapa_b_nhwc_kernel'),
-    ('fpn_large', 'bf16', 'channels_last'): (868223844, 'profiles/sapa_b_nhwc_fused_fpn_large_bf16.md',
-                                             'sapa_b_nhwc16_kernel'),
+    ('fpn_large', 'bf16', 'channels_last'): (862391142, 'profiles/sapa_b_nhwc_fused_fpn_large_bf16.md',
+                                             'sapa_b_nhwc_wm16_kernel'),
     ('fpn_small', 'fp32', 'nchw'): (137685860, 'profiles/sapa_b_fused_fpn_small_fp32.md', 'sapa_b_tiled_kernel'),
     ('segformer_16', 'fp32', 'nchw'): (11936679, 'profiles/sapa_b_mfma_fused_segformer_16_fp32.md',
                                        'sapa_b_mfma_kernel'),

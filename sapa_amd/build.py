@@ -15,7 +15,7 @@ CSRC = os.path.join(HERE, 'csrc')
 OBJ = os.path.join(CSRC, '_obj')
 LIBDIR = os.path.join(HERE, 'lib')
 LIB = os.path.join(LIBDIR, 'libsapa_hip.so')
-SOURCES = ['capi.hip', 'sapa_b_generic.hip', 'sapa_b_tiled.hip', 'sapa_b_dot2.hip', 'sapa_b_wmat16.hip', 'sapa_b_nhwc.hip', 'sapa_b_nhwc_mm.hip', 'sapa_b_nhwc16.hip', 'sapa_b_mfma.hip', 'sapa_b_lowgrad.hip', 'sapa_d.hip', 'sapa_d_lowgrad.hip', 'sapa_d_nhwc.hip', 'sapa_d_wmat16.hip', 'sapa_d_backward.hip', 'sapa_d_bwdmat.hip', 'sapa_d_scatter.hip', 'sapa_moments.hip', 'sapa_project.hip', 'sapa_layout.hip', 'sapa_stream.hip',
+SOURCES = ['capi.hip', 'sapa_b_generic.hip', 'sapa_b_tiled.hip', 'sapa_b_dot2.hip', 'sapa_b_wmat16.hip', 'sapa_b_nhwc.hip', 'sapa_b_nhwc_mm.hip', 'sapa_b_nhwc16.hip', 'sapa_b_nhwc_wm16.hip', 'sapa_b_mfma.hip', 'sapa_b_lowgrad.hip', 'sapa_d.hip', 'sapa_d_lowgrad.hip', 'sapa_d_nhwc.hip', 'sapa_d_wmat16.hip', 'sapa_d_backward.hip', 'sapa_d_bwdmat.hip', 'sapa_d_scatter.hip', 'sapa_moments.hip', 'sapa_project.hip', 'sapa_layout.hip', 'sapa_stream.hip',
            'sapa_d_lds.hip']
 
 HIPCC = os.environ.get('HIPCC', '/opt/rocm/bin/hipcc')
@@ -27,6 +27,7 @@ FLAGS = ['-O3', '-std=c++17', '--offload-arch=gfx950', '-fPIC', '-fno-gpu-rdc',
 # compiler moves them to the accumulation registers on top of an already full
 # VGPR budget, which costs the kernels a wave per SIMD
 SOURCE_FLAGS = {'sapa_b_wmat16.hip': ['-mllvm', '-amdgpu-mfma-vgpr-form'],
+                'sapa_b_nhwc_wm16.hip': ['-mllvm', '-amdgpu-mfma-vgpr-form'],
                 'sapa_b_nhwc.hip': ['-mllvm', '-amdgpu-mfma-vgpr-form'],
                 'sapa_b_nhwc_mm.hip': ['-mllvm', '-amdgpu-mfma-vgpr-form'],
                 'sapa_b_nhwc16.hip': ['-mllvm', '-amdgpu-mfma-vgpr-form'],

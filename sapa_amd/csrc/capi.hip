@@ -437,10 +437,16 @@ static int nhwc_common(int mode, const void *query, const void *key, const void 
         return SAPA_ERR_INVALID_ARGUMENT;
     // 16-bit tensors: the kernel on the 16-bit matrix instructions first
     // (SAPA_NHWC16_OFF: a tuning build without it, for comparisons)
-#ifdef SAPA_NHWC16_OFF
     hipError_t e = hipErrorNotSupported;
-#else
-    hipError_t e = took("sapa_b_nhwc16_kernel",
+#ifndef SAPA_NHWC_WM16_OFF
+    // the fused forward without a query bias: dense window products (sapa_b_nhwc_wm16.hip;
+    // SAPA_NHWC_WM16_OFF: a tuning build without it, for comparisons)
+    e = took("sapa_b_nhwc_wm16_kernel", sapa_b_nhwc_wm16_launch(mode, query, key, value, q_bias, out, B, d, C, H, W,
+                                                                K, s, dtype, (hipStream_t)stream));
+#endif
+#ifndef SAPA_NHWC16_OFF
+    if (e == hipErrorNotSupported)
+        e = took("sapa_b_nhwc16_kernel",
                         sapa_b_nhwc16_launch(mode, query, key, attn, value, q_bias, out, B, d, C, H, W, K, s,
                                              dtype, (hipStream_t)stream));
 #endif

@@ -94,6 +94,46 @@ def test_16bit_vs_oracle(coracle, shape, dtype, rel):
     assert_rel_rms_close(got.float(), coracle.sapa_fused(qf, kf, vf, K, s, 'f32a64'), rel, 'fused')
 
 
+# Fused, channels-last 16-bit tensors, K = 5, s = 2, d and C multiples of 8, no query bias: two dense
+# products per 4 x 4 block of parents on the 16-bit matrix instructions.  (B, d, C, H, W): a single block; one
+# tile of 4 blocks; ragged tiles and partial 64-channel chunks; more than one key chunk; the FPN geometries.
+DENSE16_CL_SHAPES = [(1, 8, 8, 4, 4), (2, 64, 64, 8, 16), (2, 24, 40, 13, 22), (1, 72, 136, 30, 50),
+                     (1, 136, 24, 9, 10), (3, 64, 256, 25, 42), (1, 16, 32, 100, 168)]
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('shape', DENSE16_CL_SHAPES, ids=['-'.join(map(str, s)) for s in DENSE16_CL_SHAPES])
+def test_16bit_dense_window_kernel(coracle, shape, dtype):
+    """Products of 16-bit values are exact in fp32, sums and softmax are fp32, the weights enter the
+    aggregation as a 16-bit value plus a 16-bit remainder: what is left is the rounding of the result, at
+    most half a 16-bit spacing (2^-8 resp. 2^-11 of the value) against the double-precision oracle."""
+    B, d, C, H, W = shape
+    g = gen(341)
+    q, key, v = (randn(g, *sh).to(dtype) for sh in ((B, d, H * 2, W * 2), (B, d, H, W), (B, C, H, W)))
+    half_ulp = 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
+    got = sapa_amd.sapa_fused(*cl(q, key, v), 5, 2)
+    assert sapa_amd._lib.last_kernel() == 'sapa_b_nhwc_wm16_kernel'
+    assert got.dtype == dtype and got.shape == (B, C, 2 * H, 2 * W) and got.is_contiguous(memory_format=CL)
+    exact = torch.cat([coracle.sapa_fused(q[i:i + 1].float(), key[i:i + 1].float(), v[i:i + 1].float(), 5, 2, 'f32a64')
+                       for i in range(B)]).double()
+    err = (got.float().cpu().double() - exact).abs()
+    worst = (err / torch.maximum(exact.abs(), exact.square().mean().sqrt())).max().item()
+    assert worst <= 1.05 * half_ulp, f'{shape} {dtype}: {worst / half_ulp:.2f} half-spacings'
+    # zero query: every child weighs the 25 cells of its own window equally and the rest of the 8 x 8
+    # window not at all -- the box filter of the value, zero padding counted.  Positive values, large on
+    # the border cells, and a bar relative to each element.
+    vp = v.float().abs() + 0.5
+    for sl in ((slice(None), slice(None), 0), (slice(None), slice(None), -1),
+               (slice(None), slice(None), slice(None), 0), (slice(None), slice(None), slice(None), -1)):
+        vp[sl] *= 64.0
+    vp = vp.to(dtype)
+    got0 = sapa_amd.sapa_fused(*cl(torch.zeros_like(q), key, vp), 5, 2)
+    assert sapa_amd._lib.last_kernel() == 'sapa_b_nhwc_wm16_kernel'
+    box = F.interpolate(F.avg_pool2d(vp.double(), 5, 1, 2, count_include_pad=True), scale_factor=2)
+    rel = ((got0.float().cpu().double() - box).abs() / box).max().item()
+    assert rel <= 1.05 * half_ulp + 1e-6, f'{shape} {dtype} box filter: {rel / half_ulp:.2f} half-spacings'
+
+
 @pytest.mark.parametrize('dtype,rel', [(torch.bfloat16, BF16_REL), (torch.float16, F16_REL)])
 @pytest.mark.parametrize('K,s', [(5, 2), (7, 4)])
 def test_16bit_matches_contiguous_path_at_a_larger_shape(dtype, rel, K, s):
