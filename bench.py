@@ -522,6 +522,22 @@ def main():
                 'note': 'same workload, contiguous (NCHW) bf16 tensors (python bench.py --dtype bf16 makes this '
                         'the main line); parity bar 1e-2 max(|b|, rms(b)), held by the tests to half a bf16 '
                         'spacing of the double-precision result on the rounded inputs'}
+        if nhwc_ok:
+            # and with every tensor in torch.channels_last order
+            hc = [t.contiguous(memory_format=torch.channels_last) for t in (hq, hk, hv, hout)]
+
+            def half_cl_step():
+                _lib.check(lib.sapa_fused_forward_nhwc(hc[0].data_ptr(), hc[1].data_ptr(), hc[2].data_ptr(),
+                                                       hc[3].data_ptr(), B, d, C, H, W, K, s, 3, stream.cuda_stream),
+                           'sapa_fused_forward_nhwc')
+            ms_hc, _ = timed(half_cl_step)
+            half['channels_last'] = {
+                'ms_per_step': ms_hc, 'value': B * H * s * W * s / (ms_hc * 1e-3) / 1e9, 'unit': 'Gpix/s',
+                'roofline_frac': hbytes / (ms_hc * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                'kernel': _lib.last_kernel() + ' (fused mode)',
+                'max_abs_diff_vs_nchw_image0': (hc[3][:1].float() - hout[:1].float()).abs().max().item(),
+                'note': 'python bench.py --dtype bf16 --layout channels_last makes this the main line'}
+            del hc
         del hq, hk, hv, hout
 
     reference_order = None

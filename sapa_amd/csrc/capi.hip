@@ -439,7 +439,7 @@ static int nhwc_common(int mode, const void *query, const void *key, const void 
     // (SAPA_NHWC16_OFF: a tuning build without it, for comparisons)
     hipError_t e = hipErrorNotSupported;
 #ifndef SAPA_NHWC_WM16_OFF
-    // the fused forward without a query bias: dense window products (sapa_b_nhwc_wm16.hip;
+    // the fused forward: dense window products (sapa_b_nhwc_wm16.hip;
     // SAPA_NHWC_WM16_OFF: a tuning build without it, for comparisons)
     e = took("sapa_b_nhwc_wm16_kernel", sapa_b_nhwc_wm16_launch(mode, query, key, value, q_bias, out, B, d, C, H, W,
                                                                 K, s, dtype, (hipStream_t)stream));

@@ -47,7 +47,7 @@ const char *sapa_b_nhwc_kernel_name(int K, int s, int dtype);
 hipError_t sapa_b_nhwc16_launch(int mode, const void *q, const void *key, const void *attn_in,
                                 const void *value, const void *qbias, void *out, int B, int d,
                                 int C, int H, int W, int K, int s, int dtype, hipStream_t st);
-// sapa_b_nhwc_wm16.hip: the fused forward of channels-last f16 / bf16 tensors (K = 5, s = 2, no query
+// sapa_b_nhwc_wm16.hip: the fused forward of channels-last f16 / bf16 tensors (K = 5, s = 2, optional query
 // bias) as dense window products on the 16-bit matrix instructions; hipErrorNotSupported otherwise.
 hipError_t sapa_b_nhwc_wm16_launch(int mode, const void *q, const void *key, const void *value, const void *qbias,
                                    void *out, int B, int d, int C, int H, int W, int K, int s, int dtype,

@@ -76,10 +76,12 @@ __device__ __forceinline__ u32x2 read_tr(const u32 *p) {
 // dword offset of the 16-byte piece `piece` (0..7) of cell / child `idx` in a [idx][64 channels] array
 __device__ __forceinline__ int piece_at(int idx, int piece) { return idx * CELL + ((piece ^ (idx & 7)) << 2); }
 
-template <typename T, int NSW, bool STREAM>
+// QB: a per-image bias [B, d] of the query projection: key . (q + b) = key . q + key . b, the second
+// product with the bias as the operand of every child (nothing is rounded in between)
+template <typename T, int NSW, bool STREAM, bool QB>
 __global__ __launch_bounds__(64 * NSW) void
 sapa_b_nhwc_wm16_kernel(const T *__restrict__ q, const T *__restrict__ key, const T *__restrict__ value,
-                        T *__restrict__ out, int d, int C, int H, int W, int tiles_x, int tiles_y, int ns,
+                        const T *__restrict__ qbias, T *__restrict__ out, int d, int C, int H, int W, int tiles_x, int tiles_y, int ns,
                         int nblocks, int per_xcd) {
     constexpr int NT = 64 * NSW;
     constexpr int WC = 4 * NSW + 4;                          // window cells per row of the tile
@@ -164,6 +166,17 @@ sapa_b_nhwc_wm16_kernel(const T *__restrict__ q, const T *__restrict__ key, cons
 
     stage(0);
     stage(1);
+    // One barrier per chunk: a wave computes on chunk j, waits until chunk j + 1 has landed in its own
+    // slots, meets the others (chunk j + 1 complete, buffer j % 2 free) and requests chunk j + 2.
+    auto landed_barrier = [&](bool stores_after) __attribute__((always_inline)) {
+#if defined(__HIP_DEVICE_COMPILE__)
+        // (the 8 stores a wave issues per chunk of the aggregation come after the loads waited for)
+        if (stores_after) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#endif
+        barrier();
+    };
+    landed_barrier(false);
 
     // this lane's child of block nb: row 2 nb + i16 / 8, column i16 % 8 of the block's 8 x 8 children
     // (pixel offset of nb = 0; nb adds two rows)
@@ -180,8 +193,15 @@ sapa_b_nhwc_wm16_kernel(const T *__restrict__ q, const T *__restrict__ key, cons
         for (int nb = 0; nb < 4; ++nb) sim[mb][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
     for (int j = 0; j < nKc; ++j) {
         // q of this chunk: B operand of reduction step s = channels 32 s + 8 g .. + 7 of the child
-        u32x4 qb[4][2];
+        u32x4 qb[4][2], bb[2];
         if (active) {
+            if constexpr (QB) {
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    const int c = j * CHK + 32 * s + 8 * g;
+                    bb[s] = c < d ? *(const u32x4 *)(qbias + (long)n * d + c) : u32x4{0u, 0u, 0u, 0u};
+                }
+            }
 #pragma unroll
             for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
@@ -193,13 +213,6 @@ sapa_b_nhwc_wm16_kernel(const T *__restrict__ q, const T *__restrict__ key, cons
                     qb[nb][s] = __builtin_amdgcn_raw_buffer_load_b128(rq, off, 0, STREAM_AUX);
                 }
         }
-        // chunk j has landed: what this wave issued after its loads may stay in flight (chunk
-        // j + 1's loads, then the q loads above)
-#if defined(__HIP_DEVICE_COMPILE__)
-        if (j == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // (prologue: both chunks; simplest)
-        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#endif
-        barrier();
         if (active) {
             const u32 *kb = lowbuf + (j & 1) * LOWBUF;
 #pragma unroll
@@ -213,10 +226,13 @@ sapa_b_nhwc_wm16_kernel(const T *__restrict__ q, const T *__restrict__ key, cons
 #pragma unroll
                 for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
-                    for (int nb = 0; nb < 4; ++nb) sim[mb][nb] = Mma<T>::k32(a[mb], qb[nb][s], sim[mb][nb]);
+                    for (int nb = 0; nb < 4; ++nb) {
+                        sim[mb][nb] = Mma<T>::k32(a[mb], qb[nb][s], sim[mb][nb]);
+                        if constexpr (QB) sim[mb][nb] = Mma<T>::k32(a[mb], bb[s], sim[mb][nb]);
+                    }
             }
         }
-        barrier();                      // every wave is done with buffer j % 2
+        landed_barrier(false);
         stage(j + 2);
     }
 
@@ -293,12 +309,6 @@ sapa_b_nhwc_wm16_kernel(const T *__restrict__ q, const T *__restrict__ key, cons
     }
     for (int j = nKc; j < ntot; ++j) {
         const int c0 = (j - nKc) * CHK;
-        // chunk j has landed: the loads of chunk j + 1 were issued after it, and nothing since
-        // (inactive waves: no stores either)
-#if defined(__HIP_DEVICE_COMPILE__)
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#endif
-        barrier();
         if (active) {
             const u32 *vb = lowbuf + (j & 1) * LOWBUF;
             // A operand of (channel block mk, step s): lane (g, channel i16) holds the cells of rows
@@ -345,13 +355,13 @@ sapa_b_nhwc_wm16_kernel(const T *__restrict__ q, const T *__restrict__ key, cons
                 }
             }
         }
-        barrier();                      // every wave is done with buffer j % 2
+        landed_barrier(active);
         stage(j + 2);
     }
 }
 
 template <typename T, int NSW, bool STREAM>
-static hipError_t launch_geom(const void *q, const void *key, const void *value, void *out, int B, int d,
+static hipError_t launch_geom(const void *q, const void *key, const void *value, const void *qbias, void *out, int B, int d,
                               int C, int H, int W, hipStream_t st) {
     const int nsx = (W + 3) / 4;
     const int tiles_x = (nsx + NSW - 1) / NSW, tiles_y = (H + 3) / 4;
@@ -359,29 +369,35 @@ static hipError_t launch_geom(const void *q, const void *key, const void *value,
     const long nb = (long)tiles_x * tiles_y * B;
     if (nb > (1L << 30)) return hipErrorNotSupported;
     const int per_xcd = (int)((nb + 7) / 8);
-    hipLaunchKernelGGL((sapa_b_nhwc_wm16_kernel<T, NSW, STREAM>), dim3(per_xcd * 8), dim3(64 * NSW), 0, st,
-                       (const T *)q, (const T *)key, (const T *)value, (T *)out, d, C, H, W, tiles_x, tiles_y, ns,
-                       (int)nb, per_xcd);
+    if (qbias)
+        hipLaunchKernelGGL((sapa_b_nhwc_wm16_kernel<T, NSW, STREAM, true>), dim3(per_xcd * 8), dim3(64 * NSW), 0, st,
+                           (const T *)q, (const T *)key, (const T *)value, (const T *)qbias, (T *)out, d, C, H, W,
+                           tiles_x, tiles_y, ns, (int)nb, per_xcd);
+    else
+        hipLaunchKernelGGL((sapa_b_nhwc_wm16_kernel<T, NSW, STREAM, false>), dim3(per_xcd * 8), dim3(64 * NSW), 0, st,
+                           (const T *)q, (const T *)key, (const T *)value, (const T *)nullptr, (T *)out, d, C, H, W,
+                           tiles_x, tiles_y, ns, (int)nb, per_xcd);
     return hipGetLastError();
 }
 
 }  // namespace cwm16
 
-// Fused forward only, no query bias; f16 / bf16, K = 5, s = 2, d and C multiples of 8, tensors
+// Fused forward only (qbias: optional [B, d], aligned to 16 bytes); f16 / bf16, K = 5, s = 2, d and C multiples of 8, tensors
 // aligned to 16 bytes, every image of every tensor below 2 GiB; hipErrorNotSupported otherwise.
 hipError_t sapa_b_nhwc_wm16_launch(int mode, const void *q, const void *key, const void *value, const void *qbias,
                                    void *out, int B, int d, int C, int H, int W, int K, int s, int dtype,
                                    hipStream_t st) {
-    if (mode != TILED_FUSED || qbias || K != 5 || s != 2 || d % 8 != 0 || C % 8 != 0) return hipErrorNotSupported;
+    if (mode != TILED_FUSED || K != 5 || s != 2 || d % 8 != 0 || C % 8 != 0) return hipErrorNotSupported;
     if (dtype != 2 && dtype != 3) return hipErrorNotSupported;
     if ((long)(d > C ? d : C) * H * W * 8 >= (1L << 31)) return hipErrorNotSupported;
-    if (((uintptr_t)q | (uintptr_t)key | (uintptr_t)value | (uintptr_t)out) % 16 != 0) return hipErrorNotSupported;
+    if (((uintptr_t)q | (uintptr_t)key | (uintptr_t)value | (uintptr_t)out | (uintptr_t)qbias) % 16 != 0)
+        return hipErrorNotSupported;
     const bool stream = 2L * ((long)B * H * W * (5L * d + 5L * C)) > (256L << 20);
     if (dtype == 2)
-        return stream ? cwm16::launch_geom<f16_t, 4, true>(q, key, value, out, B, d, C, H, W, st)
-                      : cwm16::launch_geom<f16_t, 4, false>(q, key, value, out, B, d, C, H, W, st);
-    return stream ? cwm16::launch_geom<bf16_t, 4, true>(q, key, value, out, B, d, C, H, W, st)
-                  : cwm16::launch_geom<bf16_t, 4, false>(q, key, value, out, B, d, C, H, W, st);
+        return stream ? cwm16::launch_geom<f16_t, 4, true>(q, key, value, qbias, out, B, d, C, H, W, st)
+                      : cwm16::launch_geom<f16_t, 4, false>(q, key, value, qbias, out, B, d, C, H, W, st);
+    return stream ? cwm16::launch_geom<bf16_t, 4, true>(q, key, value, qbias, out, B, d, C, H, W, st)
+                  : cwm16::launch_geom<bf16_t, 4, false>(q, key, value, qbias, out, B, d, C, H, W, st);
 }
 
 }  // namespace sapa
