@@ -226,10 +226,16 @@ sapa_b_nhwc_wm16_kernel(const T *__restrict__ q, const T *__restrict__ key, cons
 #pragma unroll
                 for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
-                    for (int nb = 0; nb < 4; ++nb) {
-                        sim[mb][nb] = Mma<T>::k32(a[mb], qb[nb][s], sim[mb][nb]);
-                        if constexpr (QB) sim[mb][nb] = Mma<T>::k32(a[mb], bb[s], sim[mb][nb]);
+                    for (int nb = 0; nb < 4; ++nb) sim[mb][nb] = Mma<T>::k32(a[mb], qb[nb][s], sim[mb][nb]);
+                if constexpr (QB) {
+                    // key . b is the same for every child: one product per block of cells, added to all four
+#pragma unroll
+                    for (int mb = 0; mb < 4; ++mb) {
+                        const f32x4 kb4 = Mma<T>::k32(a[mb], bb[s], f32x4{0.f, 0.f, 0.f, 0.f});
+#pragma unroll
+                        for (int nb = 0; nb < 4; ++nb) sim[mb][nb] += kb4;
                     }
+                }
             }
         }
         landed_barrier(false);
@@ -388,6 +394,11 @@ hipError_t sapa_b_nhwc_wm16_launch(int mode, const void *q, const void *key, con
                                    void *out, int B, int d, int C, int H, int W, int K, int s, int dtype,
                                    hipStream_t st) {
     if (mode != TILED_FUSED || K != 5 || s != 2 || d % 8 != 0 || C % 8 != 0) return hipErrorNotSupported;
+    // small images: the kernel with a workgroup per 4 x 4 parents has four times the workgroups and a
+    // shorter chain per workgroup (B=8, 32x32: 9 against 12 us; B=16, 25x42: 15 against 17 us; from
+    // 64x64 on this one wins: 19 against 25 us).  By image size, not batch size: a batch and its images
+    // one by one take the same kernel.
+    if ((long)H * W < 2048) return hipErrorNotSupported;
     if (dtype != 2 && dtype != 3) return hipErrorNotSupported;
     if ((long)(d > C ? d : C) * H * W * 8 >= (1L << 31)) return hipErrorNotSupported;
     if (((uintptr_t)q | (uintptr_t)key | (uintptr_t)value | (uintptr_t)out | (uintptr_t)qbias) % 16 != 0)

@@ -94,11 +94,12 @@ def test_16bit_vs_oracle(coracle, shape, dtype, rel):
     assert_rel_rms_close(got.float(), coracle.sapa_fused(qf, kf, vf, K, s, 'f32a64'), rel, 'fused')
 
 
-# Fused, channels-last 16-bit tensors, K = 5, s = 2, d and C multiples of 8, no query bias: two dense
-# products per 4 x 4 block of parents on the 16-bit matrix instructions.  (B, d, C, H, W): a single block; one
-# tile of 4 blocks; ragged tiles and partial 64-channel chunks; more than one key chunk; the FPN geometries.
-DENSE16_CL_SHAPES = [(1, 8, 8, 4, 4), (2, 64, 64, 8, 16), (2, 24, 40, 13, 22), (1, 72, 136, 30, 50),
-                     (1, 136, 24, 9, 10), (3, 64, 256, 25, 42), (1, 16, 32, 100, 168)]
+# Fused, channels-last 16-bit tensors, K = 5, s = 2, d and C multiples of 8, images of at least 2048 low-res
+# cells: two dense products per 4 x 4 block of parents on the 16-bit matrix instructions.  (B, d, C, H, W): one
+# 64-channel chunk of each; whole tiles; ragged tiles (H % 4 = 1, W % 4 = 2) and partial chunks; partial
+# chunks of key and value; more than one key chunk; the FPN geometry.
+DENSE16_CL_SHAPES = [(1, 8, 8, 46, 46), (2, 64, 64, 32, 64), (2, 24, 40, 45, 50), (1, 72, 136, 40, 56),
+                     (1, 136, 24, 47, 44), (1, 16, 32, 100, 168)]
 
 
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
@@ -132,6 +133,17 @@ def test_16bit_dense_window_kernel(coracle, shape, dtype):
     box = F.interpolate(F.avg_pool2d(vp.double(), 5, 1, 2, count_include_pad=True), scale_factor=2)
     rel = ((got0.float().cpu().double() - box).abs() / box).max().item()
     assert rel <= 1.05 * half_ulp + 1e-6, f'{shape} {dtype} box filter: {rel / half_ulp:.2f} half-spacings'
+    # a per-image bias of the query: key . (q + b) with nothing rounded in between
+    if B * H * W <= 6000:
+        bias = (randn(g, B, d) * 0.7).to(dtype)
+        got_b = sapa_amd.sapa_fused(*cl(q, key, v), 5, 2, bias.to(DEV))
+        assert sapa_amd._lib.last_kernel() == 'sapa_b_nhwc_wm16_kernel'
+        qb = q.float() + bias.float()[:, :, None, None]
+        exact_b = torch.cat([coracle.sapa_fused(qb[i:i + 1], key[i:i + 1].float(), v[i:i + 1].float(), 5, 2, 'f32a64')
+                             for i in range(B)]).double()
+        err = (got_b.float().cpu().double() - exact_b).abs()
+        worst = (err / torch.maximum(exact_b.abs(), exact_b.square().mean().sqrt())).max().item()
+        assert worst <= 1.05 * half_ulp, f'{shape} {dtype} with bias: {worst / half_ulp:.2f} half-spacings'
 
 
 @pytest.mark.parametrize('dtype,rel', [(torch.bfloat16, BF16_REL), (torch.float16, F16_REL)])
