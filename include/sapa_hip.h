@@ -461,9 +461,13 @@ int sapa_groupnorm_fold(const float *mean_var, const void *gamma, const void *be
  * x [B,HW,C], weight [B,O,C] (sapa_groupnorm_fold's output), bias [B,O] or NULL,
  * out [B,HW,O] -- self.q(norm_y(y)) / self.k(norm_x(x)) of the reference
  * (sapa/sapa/sapa_base.py:32-35; Conv2d and GroupNorm, ATen calls there) as one
- * stream over the feature.  SAPA_F16 / SAPA_BF16, C in {64,128,256,512}, O in
- * {32,64,128} (not every pair), pointers aligned to 16 bytes;
- * SAPA_ERR_UNSUPPORTED otherwise. */
+ * stream over the feature.  SAPA_F16 / SAPA_BF16 / SAPA_F32, C in {64,128,256,512},
+ * O in {32,64,128} (not every pair; SAPA_F32: the pairs with 6 * C * O bytes of
+ * weights within the LDS, e.g. (256,64), (512,32)), pointers aligned to 16 bytes;
+ * SAPA_ERR_UNSUPPORTED otherwise.  SAPA_F32 multiplies on the bf16 matrix
+ * instruction, each product as six products of bf16 pieces with fp32 sums: the
+ * result of an fp32 dot product to rounding, in another order of summation than a
+ * library GEMM's. */
 int sapa_project_nhwc(const void *x, const void *weight, const void *bias, void *out,
                       int B, int C, int O, long long HW, int dtype, void *stream);
 

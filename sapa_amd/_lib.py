@@ -311,12 +311,13 @@ def groupnorm_fold(mean_var, norm, conv, dtype):
 
 def project_nhwc(x, weight, bias=None):
     """out[b, :, h, w] = weight[b] @ x[b, :, h, w] (+ bias[b]) for a channels_last
-    16-bit CUDA feature x [B, C, H, W] and per-image weights [B, O, C]: a
+    f16 / bf16 / fp32 CUDA feature x [B, C, H, W] and per-image weights [B, O, C]: a
     channels_last tensor [B, O, H, W], or None if the kernel does not cover the
     configuration (the caller then uses a library GEMM)."""
     B, C, H, W = x.shape
     O = weight.shape[1]
-    if x.dtype not in (torch.float16, torch.bfloat16) or weight.dtype != x.dtype or x.numel() == 0:
+    if (x.dtype not in (torch.float16, torch.bfloat16, torch.float32) or weight.dtype != x.dtype
+            or x.numel() == 0):
         return None
     if not x.is_contiguous(memory_format=torch.channels_last):
         return None

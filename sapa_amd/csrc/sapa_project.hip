@@ -15,6 +15,17 @@
 //     operand layout of v_mfma_f32_16x16x16 (row = pixel);
 //   * the 16 x 16 results per output tile go back through LDS, so that a lane
 //     stores 16 contiguous bytes and the wave one contiguous run of 32 O bytes.
+//
+// fp32 features (project32_kernel) take the same stream through the bf16 matrix
+// instruction: every fp32 number is the exact sum of three bf16 numbers (8 + 8 + 8
+// significant bits), a product of two bf16 numbers is exact in fp32, and of the nine
+// piece products of x * w the six largest are kept (the other three are below 2^-23 of
+// the product): six v_mfma_f32_16x16x32_bf16 per fp32 matrix step, fp32 sums -- an
+// fp32 dot product to fp32 rounding at 32 / 6 times the rate of the fp32 matrix
+// instruction, which leaves the kernel waiting for memory, not arithmetic.  The image's
+// weights are taken apart once per workgroup into three bf16 planes in LDS; x goes
+// from global memory straight into the A-operand registers (a lane reads two 16-byte
+// pieces of its pixel's record per step of 32 channels) and is taken apart there.
 #include "kernels.hpp"
 
 namespace sapa {
@@ -174,6 +185,202 @@ static hipError_t launch_co(const void *x, const void *w, const void *bias, void
     return hipGetLastError();
 }
 
+// ---- fp32 ----
+// the three bf16 pieces of two fp32 numbers, each pair packed in a dword (x0 in the low half)
+struct Pieces {
+    u32 hi, mid, lo;
+};
+__device__ __forceinline__ Pieces split2(float x0, float x1) {
+    const u32 TOP = 0xffff0000u, SEL = 0x07060302u;        // SEL: the upper halves of two dwords
+    const u32 u0 = __builtin_bit_cast(u32, x0), u1 = __builtin_bit_cast(u32, x1);
+    const float r0 = x0 - __builtin_bit_cast(float, u0 & TOP), r1 = x1 - __builtin_bit_cast(float, u1 & TOP);
+    const u32 v0 = __builtin_bit_cast(u32, r0), v1 = __builtin_bit_cast(u32, r1);
+    const float l0 = r0 - __builtin_bit_cast(float, v0 & TOP), l1 = r1 - __builtin_bit_cast(float, v1 & TOP);
+    Pieces p;
+    p.hi = __builtin_amdgcn_perm(u1, u0, SEL);
+    p.mid = __builtin_amdgcn_perm(v1, v0, SEL);
+    p.lo = __builtin_amdgcn_perm(__builtin_bit_cast(u32, l1), __builtin_bit_cast(u32, l0), SEL);
+    return p;
+}
+__device__ __forceinline__ f32x4 mma32(u32x4 a, u32x4 b, f32x4 c) {
+    typedef __bf16 v8 __attribute__((ext_vector_type(8)));
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8, a), __builtin_bit_cast(v8, b), c, 0, 0, 0);
+}
+
+// C input channels (a multiple of 32), O outputs (a multiple of 16); 8 waves, tiles of 32
+// pixels (two blocks of 16 matrix rows share every weight operand read from LDS).
+// Reduction step ks takes channels 32 ks ..; inside it lane group kg holds channels
+// 4 kg .. + 3 and 16 + 4 kg .. + 3 (two 16-byte pieces of memory; the 16 lanes of a piece
+// read 64 contiguous bytes per pixel) -- the weight planes are stored in that order.
+template <int C, int O>
+__global__ void __launch_bounds__(512)
+project32_kernel(const float *__restrict__ x, const float *__restrict__ w, const float *__restrict__ bias,
+                 float *__restrict__ out, long HW, int tiles_per_wave) {
+    constexpr int NW = 8;
+    constexpr int RW = C / 2 + 4;                 // dwords per padded row of C bf16 values
+    constexpr int PLANE = O * RW;                 // dwords per piece plane
+    constexpr int NT = O / 16;                    // output tiles of 16 columns
+    constexpr int OS = O + 4;                     // floats per padded row of the result tile
+    constexpr int KS = C / 32;                    // reduction steps
+    constexpr int RING = KS < 4 ? KS : 4;         // steps of x in flight
+    static_assert(KS % RING == 0, "the ring of x registers is indexed by the step");
+    extern __shared__ __attribute__((aligned(16))) u32 sh[];
+    u32 *wl = sh;                                 // weights: 3 planes of O rows of RW dwords
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    float *rt = (float *)(sh + 3 * PLANE) + wave * 16 * OS;     // this wave's result tile: 16 rows of OS floats
+    const int b = blockIdx.y;
+
+    // the image's weights, taken apart, -> LDS (two neighbouring channels per thread and step)
+    {
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        const f32x2 *src = (const f32x2 *)(w + (long)b * O * C);
+        for (int i = threadIdx.x; i < O * C / 2; i += 64 * NW) {
+            const int o = i / (C / 2), c = 2 * (i % (C / 2)), cs = c % 32;
+            const int pos = 32 * (c / 32) + 8 * ((cs % 16) / 4) + 4 * (cs / 16) + cs % 4;
+            const f32x2 v = src[i];
+            const Pieces pc = split2(v[0], v[1]);
+            u32 *dst = wl + o * RW + pos / 2;
+            dst[0] = pc.hi;
+            dst[PLANE] = pc.mid;
+            dst[2 * PLANE] = pc.lo;
+        }
+    }
+    __syncthreads();
+
+    const long ntiles = (HW + 31) / 32;
+    const long t0 = ((long)blockIdx.x * NW + wave) * tiles_per_wave;
+    const long t1 = t0 + tiles_per_wave < ntiles ? t0 + tiles_per_wave : ntiles;
+    if (t0 >= t1) return;
+    const int r16 = lane & 15, kg = lane >> 4;    // row / column of a 16 x 16 tile, k group
+    float bv[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) bv[nt] = bias ? bias[(long)b * O + 16 * nt + r16] : 0.f;
+
+    // byte offsets inside the image: out of range = past the last pixel = zeros / dropped
+    const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(x + (long)b * HW * C), 0, (int)(HW * C * 4), 0x00020000);
+    const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(out + (long)b * HW * O), 0, (int)(HW * O * 4), 0x00020000);
+    const u32 xoff = (u32)(r16 * C + 4 * kg) * 4u;            // pixel r16 of block 0, first piece
+    // step (t, ks) of x: 2 blocks x 2 pieces of 16 bytes per lane
+    u32x4 raw[RING][2][2];
+    auto load_step = [&](int slot, long t, int ks) __attribute__((always_inline)) {
+        const u32 so = (u32)((t * 32 * C + 32 * ks) * 4);
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                raw[slot][mb][h] = __builtin_amdgcn_raw_buffer_load_b128(rx, xoff + (u32)((mb * 16 * C + 16 * h) * 4), so, 0);
+    };
+#pragma unroll
+    for (int k = 0; k < RING; ++k) load_step(k, t0, k);
+    for (long t = t0; t < t1; ++t) {
+        f32x4 acc[2][NT];
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) acc[mb][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            u32x4 ahi[2], amid[2], alo[2];
+#pragma unroll
+            for (int mb = 0; mb < 2; ++mb) {
+                const f32x4 p0 = __builtin_bit_cast(f32x4, raw[ks % RING][mb][0]);
+                const f32x4 p1 = __builtin_bit_cast(f32x4, raw[ks % RING][mb][1]);
+                const Pieces s0 = split2(p0[0], p0[1]), s1 = split2(p0[2], p0[3]);
+                const Pieces s2 = split2(p1[0], p1[1]), s3 = split2(p1[2], p1[3]);
+                ahi[mb] = u32x4{s0.hi, s1.hi, s2.hi, s3.hi};
+                amid[mb] = u32x4{s0.mid, s1.mid, s2.mid, s3.mid};
+                alo[mb] = u32x4{s0.lo, s1.lo, s2.lo, s3.lo};
+            }
+            // the ring slot is free: the step RING further on (of this tile or of the next)
+            if (ks + RING < KS) load_step(ks % RING, t, ks + RING);
+            else if (t + 1 < t1) load_step(ks % RING, t + 1, ks + RING - KS);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const u32 *wp = wl + (16 * nt + r16) * RW + 16 * ks + 4 * kg;
+                const u32x4 bhi = *(const u32x4 *)wp, bmid = *(const u32x4 *)(wp + PLANE), blo = *(const u32x4 *)(wp + 2 * PLANE);
+#pragma unroll
+                for (int mb = 0; mb < 2; ++mb) {
+                    // smallest terms first
+                    f32x4 a = mma32(ahi[mb], blo, acc[mb][nt]);
+                    a = mma32(alo[mb], bhi, a);
+                    a = mma32(amid[mb], bmid, a);
+                    a = mma32(ahi[mb], bmid, a);
+                    a = mma32(amid[mb], bhi, a);
+                    acc[mb][nt] = mma32(ahi[mb], bhi, a);
+                }
+            }
+        }
+        // acc[mb][nt][i]: pixel 16 mb + 4 kg + i, output 16 nt + r16 -> the wave's tile, then 16
+        // rows of 4 O bytes -> one contiguous run of 64 O bytes per block
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) rt[(4 * kg + i) * OS + 16 * nt + r16] = acc[mb][nt][i] + bv[nt];
+            const u32 obase = (u32)((t * 32 + 16 * mb) * O * 4);
+#pragma unroll
+            for (int j = 0; j < (16 * O / 4 + 63) / 64; ++j) {
+                const int i = j * 64 + lane, row = i / (O / 4), col = i % (O / 4);
+                if (16 * O / 4 % 64 == 0 || i < 16 * O / 4)
+                    __builtin_amdgcn_raw_buffer_store_b128(*(const u32x4 *)(rt + row * OS + 4 * col), ro, (u32)(i * 16), obase, 2);
+            }
+        }
+    }
+}
+
+template <int C, int O>
+static hipError_t launch32_co(const void *x, const void *w, const void *bias, void *out, int B, long HW,
+                              hipStream_t st) {
+    constexpr size_t lds = (size_t)(3 * O * (C / 2 + 4) + 8 * 16 * (O + 4)) * 4;
+    static_assert(lds <= 160 * 1024, "weights and tiles must fit LDS");
+    // 32-bit byte offsets inside an image
+    if (HW * (long)(C > O ? C : O) * 4 >= (1L << 31)) return hipErrorNotSupported;
+    const long ntiles = (HW + 31) / 32;
+    // One workgroup is resident per CU (its weight planes fill most of the LDS) and the part has
+    // 256 CUs: two full rounds of workgroups where that leaves a wave 8 tiles or more, else one
+    // (16 images: 200x336 pixels 301 us in two rounds against 315 in one; 100x168 pixels 71 us in
+    // one round against 98 in 272 workgroups)
+    const long slots = 256;
+    long blocks = 2 * slots / B > 1 ? 2 * slots / B : 1;
+    long per = (ntiles + 8 * blocks - 1) / (8 * blocks);
+    if (per < 8) {
+        blocks = slots / B > 1 ? slots / B : 1;
+        per = (ntiles + 8 * blocks - 1) / (8 * blocks);
+    }
+    blocks = (ntiles + 8 * per - 1) / (8 * per);
+    if (blocks > 65535 * 32L || B > 65535) return hipErrorNotSupported;
+    auto kern = project32_kernel<C, O>;
+    if (lds > 64 * 1024) {
+        int dev = 0, most = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&most, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess ||
+            (size_t)most < lds ||
+            hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds) != hipSuccess) {
+            (void)hipGetLastError();
+            return hipErrorNotSupported;
+        }
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks, B), dim3(512), lds, st, (const float *)x, (const float *)w,
+                       (const float *)bias, (float *)out, HW, (int)per);
+    return hipGetLastError();
+}
+
+static hipError_t launch32(const void *x, const void *w, const void *bias, void *out, int B, int C, int O,
+                           long HW, hipStream_t st) {
+#define SAPA_PROJECT_CASE(CV, OV) \
+    if (C == CV && O == OV) return launch32_co<CV, OV>(x, w, bias, out, B, HW, st);
+    SAPA_PROJECT_CASE(64, 32) SAPA_PROJECT_CASE(64, 64)
+    SAPA_PROJECT_CASE(128, 32) SAPA_PROJECT_CASE(128, 64)
+    SAPA_PROJECT_CASE(256, 32) SAPA_PROJECT_CASE(256, 64)
+    SAPA_PROJECT_CASE(512, 32)
+#undef SAPA_PROJECT_CASE
+    return hipErrorNotSupported;
+}
+
 template <typename T>
 static hipError_t launch_t(const void *x, const void *w, const void *bias, void *out, int B, int C,
                            int O, long HW, hipStream_t st) {
@@ -189,14 +396,16 @@ static hipError_t launch_t(const void *x, const void *w, const void *bias, void 
 
 }  // namespace project
 
-// x [B, HW, C], w [B, O, C], bias [B, O] or null, out [B, HW, O]; f16 / bf16;
-// (C, O) among the instantiated pairs (C in {64, 128, 256, 512}, O in {32, 64, 128});
-// every pointer aligned to 16 bytes.  hipErrorNotSupported otherwise.
+// x [B, HW, C], w [B, O, C], bias [B, O] or null, out [B, HW, O]; f16 / bf16 / fp32;
+// (C, O) among the instantiated pairs (C in {64, 128, 256, 512}, O in {32, 64, 128}; fp32:
+// those whose three weight planes fit LDS); every pointer aligned to 16 bytes.
+// hipErrorNotSupported otherwise.
 hipError_t project_nhwc_launch(const void *x, const void *w, const void *bias, void *out, int B,
                                int C, int O, long HW, int dtype, hipStream_t st) {
     const void *ptrs[3] = {x, w, out};
     for (const void *p : ptrs)
         if ((uintptr_t)p % 16 != 0) return hipErrorNotSupported;
+    if (dtype == 0) return project::launch32(x, w, bias, out, B, C, O, HW, st);
     if (dtype == 2) return project::launch_t<f16_t>(x, w, bias, out, B, C, O, HW, st);
     if (dtype == 3) return project::launch_t<bf16_t>(x, w, bias, out, B, C, O, HW, st);
     return hipErrorNotSupported;

@@ -118,8 +118,9 @@ def norm_project(x, norm, *convs, channels_last=False, defer_bias=False):
         # GEMM, then the bias in place: measurably faster than baddbmm here, which
         # first spreads the bias over the whole output
         if channels_last:
-            # a 16-bit channels_last feature that needs no gradient: the library's
-            # streaming projection kernel (bias in its epilogue); else a library GEMM
+            # a channels_last feature (f16 / bf16 / fp32) that needs no gradient: the
+            # library's streaming projection kernel (bias in its epilogue); else a
+            # library GEMM
             out = None
             if x_cl and x.is_cuda and not torch.is_grad_enabled():
                 out = _lib.project_nhwc(x, w_b, None if defer_bias else b_b)

@@ -127,10 +127,10 @@ def test_argument_validation_returns_codes():
     big = (2, 1024, 1 << 22, 1)
     assert h.sapa_channel_moments_workspace(*big) > h.sapa_channel_moments_static_capacity()
     assert h.sapa_channel_moments_static(p, p, big[0], big[1], big[2], big[3], 0, None) == -3
-    # projection: extents, null pointers, fp32 (no kernel), empty batch
+    # projection: extents, null pointers, fp64 (no kernel), empty batch
     assert h.sapa_project_nhwc(p, p, p, p, 1, 0, 64, 100, 3, None) == -1
     assert h.sapa_project_nhwc(p, None, p, p, 1, 256, 64, 100, 3, None) == -1
-    assert h.sapa_project_nhwc(p, p, None, p, 1, 256, 64, 100, 0, None) == -2
+    assert h.sapa_project_nhwc(p, p, None, p, 1, 256, 64, 100, 1, None) == -2
     assert h.sapa_project_nhwc(None, None, None, None, 0, 256, 64, 100, 3, None) == 0
     # layout copy: element size, negative extents, null / misaligned pointers, empty tensors,
     # more rows than the tiled side holds

@@ -485,4 +485,36 @@ def test_projection_kernel(dtype, tol, shape):
         ref = want if bias is None else want + bias.double().cpu()[:, :, None, None]
         torch.testing.assert_close(out.double().cpu(), ref, rtol=tol, atol=tol)
     assert _lib.project_nhwc(x[:, :48].contiguous(memory_format=CL), w[:, :, :48].contiguous()) is None
-    assert _lib.project_nhwc(x.float(), w.float()) is None
+    assert _lib.project_nhwc(x.double(), w.double()) is None
+
+
+@pytest.mark.parametrize('shape', [(2, 256, 64, 9, 11), (1, 128, 32, 40, 33), (3, 64, 64, 5, 7), (1, 512, 32, 4, 4),
+                                   (2, 256, 32, 1, 1), (1, 256, 64, 130, 129), (2, 64, 32, 17, 3)])
+def test_projection_kernel_fp32(shape):
+    """The fp32 form of the streaming projection: every product as six products of bf16
+    pieces on the matrix instruction, fp32 sums.  Against float64 arithmetic on the same
+    values it must stand where an fp32 dot product stands: the bound is the error of
+    torch's own fp32 product on these values (with a factor for its different order of
+    summation) and, outright, the stated 1e-5 relative to the operands' scale."""
+    from sapa_amd import _lib
+    B, C, O, H, W = shape
+    g = gen(361)
+    x = (randn(g, B, C, H, W) * 3 + 0.5).to(DEV).contiguous(memory_format=CL)
+    w = (randn(g, B, O, C) * 0.1).to(DEV)
+    b = randn(g, B, O).to(DEV)
+    want = torch.einsum('boc,bchw->bohw', w.double().cpu(), x.double().cpu())
+    e32 = (torch.einsum('boc,bchw->bohw', w.cpu(), x.cpu()).double() - want).abs().max().item()
+    # sum over c of |w x|: what the rounding of an fp32 dot product scales with
+    scale = torch.einsum('boc,bchw->bohw', w.double().abs().cpu(), x.double().abs().cpu()).max().item()
+    for bias in (None, b):
+        out = _lib.project_nhwc(x, w, bias)
+        assert out is not None and out.dtype == torch.float32 and out.shape == (B, O, H, W)
+        assert out.is_contiguous(memory_format=CL)
+        ref = want if bias is None else want + bias.double().cpu()[:, :, None, None]
+        err = (out.double().cpu() - ref).abs().max().item()
+        assert err <= max(3 * e32, 1e-6 * scale), (err, e32, scale)
+        assert err <= 1e-5 * scale
+    # pairs whose three weight planes do not fit the LDS go to the caller's library GEMM
+    if C == 256 and O == 64:
+        w2 = torch.cat([w, w], 1).contiguous()
+        assert _lib.project_nhwc(x, w2) is None
