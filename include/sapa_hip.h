@@ -471,6 +471,17 @@ int sapa_groupnorm_fold(const float *mean_var, const void *gamma, const void *be
 int sapa_project_nhwc(const void *x, const void *weight, const void *bias, void *out,
                       int B, int C, int O, long long HW, int dtype, void *stream);
 
+/* The same projection of a contiguous feature x [B,C,HW] (the reference's layout:
+ * self.q(norm_y(y)) on an NCHW tensor, sapa/sapa/sapa_base.py:32-35): out [B,O,HW],
+ * or [B,HW,O] (channels-last, what the channels-last operator takes) when
+ * out_channels_last is non-zero.  SAPA_F32 only, the (C,O) pairs of
+ * sapa_project_nhwc's SAPA_F32 form, HW a multiple of 4 for a [B,O,HW] result, x and
+ * out aligned to 16 bytes; SAPA_ERR_UNSUPPORTED otherwise (the caller uses a library
+ * GEMM). */
+int sapa_project_nchw(const void *x, const void *weight, const void *bias, void *out,
+                      int B, int C, int O, long long HW, int out_channels_last, int dtype,
+                      void *stream);
+
 /* ------------------------------------------------------------ calibration */
 
 /* Layout copy between the two memory orders the library serves: a dense

@@ -22,6 +22,7 @@ _vp, _i, _ll = ctypes.c_void_p, ctypes.c_int, ctypes.c_longlong
 SIGNATURES = {
     'sapa_fused_forward_nhwc_qbias': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_project_nhwc': [_vp, _vp, _vp, _vp, _i, _i, _i, _ll, _i, _vp],
+    'sapa_project_nchw': [_vp, _vp, _vp, _vp, _i, _i, _i, _ll, _i, _i, _vp],
     'sapa_channel_moments': [_vp, _vp, _vp, _i, _i, _ll, _i, _i, _vp],
     'sapa_channel_moments_static': [_vp, _vp, _i, _i, _ll, _i, _i, _vp],
     'sapa_groupnorm_fold': [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, ctypes.c_float, _i, _vp],
@@ -307,6 +308,31 @@ def groupnorm_fold(mean_var, norm, conv, dtype):
         return None
     check(status, 'sapa_groupnorm_fold')
     return w_out, b_out
+
+
+def project_nchw(x, weight, bias=None, channels_last_out=False):
+    """out[b, :, h, w] = weight[b] @ x[b, :, h, w] (+ bias[b]) for a contiguous fp32
+    CUDA feature x [B, C, H, W] and per-image weights [B, O, C]: a contiguous (or, with
+    channels_last_out, a channels_last) tensor [B, O, H, W], or None if the kernel does
+    not cover the configuration (the caller then uses a library GEMM)."""
+    B, C, H, W = x.shape
+    O = weight.shape[1]
+    if x.dtype != torch.float32 or weight.dtype != x.dtype or x.numel() == 0 or not x.is_contiguous():
+        return None
+    weight = weight.contiguous()
+    if bias is not None:
+        bias = bias.to(x.dtype).contiguous()
+    with torch.cuda.device(x.device):
+        out = torch.empty(B, O, H, W, dtype=x.dtype, device=x.device,
+                          memory_format=torch.channels_last if channels_last_out else torch.contiguous_format)
+        status = lib().sapa_project_nchw(
+            x.data_ptr(), weight.data_ptr(), None if bias is None else bias.data_ptr(), out.data_ptr(),
+            B, C, O, H * W, 1 if channels_last_out else 0, DTYPES[x.dtype],
+            torch.cuda.current_stream(x.device).cuda_stream)
+    if status == UNSUPPORTED:
+        return None
+    check(status, 'sapa_project_nchw')
+    return out
 
 
 def project_nhwc(x, weight, bias=None):

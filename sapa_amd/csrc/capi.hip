@@ -756,6 +756,18 @@ int sapa_project_nhwc(const void *x, const void *weight, const void *bias, void 
     return finish(e);
 }
 
+int sapa_project_nchw(const void *x, const void *weight, const void *bias, void *out, int B, int C,
+                      int O, long long HW, int out_channels_last, int dtype, void *stream) {
+    if (!dtype_ok(dtype) || B < 0 || C <= 0 || O <= 0 || HW <= 0) return SAPA_ERR_INVALID_ARGUMENT;
+    if ((long long)B * HW * (C > O ? C : O) >= kMaxElems) return SAPA_ERR_TOO_LARGE;
+    if (B == 0) return SAPA_OK;
+    if (!x || !weight || !out) return SAPA_ERR_INVALID_ARGUMENT;
+    const hipError_t e = project_nchw_launch(x, weight, bias, out, B, C, O, (long)HW, out_channels_last,
+                                             dtype, (hipStream_t)stream);
+    if (e == hipErrorNotSupported) return SAPA_ERR_UNSUPPORTED;
+    return finish(e);
+}
+
 int sapa_layout_copy(const void *src, void *dst, int B, int C, long long HW, int to_channels_last,
                      int esize, void *stream) {
     if (B < 0 || C < 0 || HW < 0 || (esize != 2 && esize != 4)) return SAPA_ERR_INVALID_ARGUMENT;

@@ -80,6 +80,9 @@ hipError_t stream_split_launch(const void *src, void *dst, long groups, int reps
 // sapa_project.hip: 1x1 projection of a channels-last 16-bit feature with per-image weights
 hipError_t project_nhwc_launch(const void *x, const void *w, const void *bias, void *out, int B,
                                int C, int O, long HW, int dtype, hipStream_t st);
+// ... of a contiguous feature [B, C, HW] into [B, HW, O] (out_channels_last) or [B, O, HW]; fp32
+hipError_t project_nchw_launch(const void *x, const void *w, const void *bias, void *out, int B,
+                               int C, int O, long HW, int out_channels_last, int dtype, hipStream_t st);
 
 // sapa_d_nhwc.hip: fused SAPA-D forward for tensors in channels-last memory
 // order (offsets [B, sH, sW, 2GP]); f32 / f16 / bf16, s in {1, 2, 4}, P <= 32,

@@ -212,22 +212,35 @@ __device__ __forceinline__ f32x4 mma32(u32x4 a, u32x4 b, f32x4 c) {
 // Reduction step ks takes channels 32 ks ..; inside it lane group kg holds channels
 // 4 kg .. + 3 and 16 + 4 kg .. + 3 (two 16-byte pieces of memory; the 16 lanes of a piece
 // read 64 contiguous bytes per pixel) -- the weight planes are stored in that order.
-template <int C, int O>
+//
+// IN_CL = false: x is [B, C, HW] (contiguous planes).  A lane fetches 4 neighbouring pixels of
+// one channel (a wave: 8 channels x 128 bytes per load), four such loads per step, and the step's
+// 32 channels x 32 pixels pass through a wave-private LDS tile from which the A operands are read
+// as single dwords (the 16-pixel halves of a row swapped for every other group of 4 channels, so
+// that the two channel groups of a half-wave read disjoint banks).  OUT_CL = false: out is
+// [B, O, HW]; a block of 16 outputs x 32 pixels goes back through LDS and leaves as 128-byte rows
+// (HW a multiple of 4: a 16-byte piece never runs from one plane into the next).
+template <int C, int O, bool IN_CL, bool OUT_CL>
 __global__ void __launch_bounds__(512)
 project32_kernel(const float *__restrict__ x, const float *__restrict__ w, const float *__restrict__ bias,
                  float *__restrict__ out, long HW, int tiles_per_wave) {
+    static_assert(IN_CL ? OUT_CL : true, "channels-last features give channels-last projections");
     constexpr int NW = 8;
     constexpr int RW = C / 2 + 4;                 // dwords per padded row of C bf16 values
     constexpr int PLANE = O * RW;                 // dwords per piece plane
     constexpr int NT = O / 16;                    // output tiles of 16 columns
-    constexpr int OS = O + 4;                     // floats per padded row of the result tile
+    constexpr int OS = O + 4;                     // floats per padded row of the result tile (channels-last)
+    constexpr int PS = 32 + 4;                    // ... of a block of 16 outputs x 32 pixels (planes)
+    constexpr int XB = IN_CL ? 0 : 32 * 32;       // floats of the wave's x tile
+    constexpr int RT = OUT_CL ? 16 * OS : 16 * PS;
+    constexpr int WF = RT > XB ? RT : XB;         // floats of a wave's LDS (x tile, then results)
     constexpr int KS = C / 32;                    // reduction steps
     constexpr int RING = KS < 4 ? KS : 4;         // steps of x in flight
     static_assert(KS % RING == 0, "the ring of x registers is indexed by the step");
     extern __shared__ __attribute__((aligned(16))) u32 sh[];
     u32 *wl = sh;                                 // weights: 3 planes of O rows of RW dwords
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    float *rt = (float *)(sh + 3 * PLANE) + wave * 16 * OS;     // this wave's result tile: 16 rows of OS floats
+    float *rt = (float *)(sh + 3 * PLANE) + wave * WF;          // this wave's x tile / result tile
     const int b = blockIdx.y;
 
     // the image's weights, taken apart, -> LDS (two neighbouring channels per thread and step)
@@ -261,17 +274,25 @@ project32_kernel(const float *__restrict__ x, const float *__restrict__ w, const
         (void *)(x + (long)b * HW * C), 0, (int)(HW * C * 4), 0x00020000);
     const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(
         (void *)(out + (long)b * HW * O), 0, (int)(HW * O * 4), 0x00020000);
-    const u32 xoff = (u32)(r16 * C + 4 * kg) * 4u;            // pixel r16 of block 0, first piece
-    // step (t, ks) of x: 2 blocks x 2 pieces of 16 bytes per lane
+    // step (t, ks) of x, 4 pieces of 16 bytes per lane.  Channels-last: blocks mb = 0, 1 x pieces
+    // h = 0, 1 of pixel r16's record.  Planes: piece j = pixels 4 (lane % 8) .. + 3 of channel
+    // 8 j + lane / 8 of the step
+    const u32 xoff = IN_CL ? (u32)(r16 * C + 4 * kg) * 4u : (u32)((lane >> 3) * HW + 4 * (lane & 7)) * 4u;
+    const u32 xstride = IN_CL ? 0u : (u32)(8 * HW * 4);
     u32x4 raw[RING][2][2];
     auto load_step = [&](int slot, long t, int ks) __attribute__((always_inline)) {
-        const u32 so = (u32)((t * 32 * C + 32 * ks) * 4);
+        const u32 so = IN_CL ? (u32)((t * 32 * C + 32 * ks) * 4) : (u32)((32L * ks * HW + t * 32) * 4);
 #pragma unroll
         for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
             for (int h = 0; h < 2; ++h)
-                raw[slot][mb][h] = __builtin_amdgcn_raw_buffer_load_b128(rx, xoff + (u32)((mb * 16 * C + 16 * h) * 4), so, 0);
+                raw[slot][mb][h] = __builtin_amdgcn_raw_buffer_load_b128(
+                    rx, IN_CL ? xoff + (u32)((mb * 16 * C + 16 * h) * 4) : xoff + (u32)(2 * mb + h) * xstride, so, 0);
     };
+    // (planes) the x tile [32 channels][32 pixels]: where this lane writes its pieces, and where it
+    // reads channel 4 kg (+ 16) of pixel r16 (+ 16)
+    float *const xw = rt + (lane >> 3) * 32 + (((lane & 7) ^ ((lane >> 5) << 2)) << 2);
+    const float *const xr = rt + 4 * kg * 32 + ((((r16 >> 2)) ^ ((kg & 1) << 2)) << 2) + (r16 & 3);
 #pragma unroll
     for (int k = 0; k < RING; ++k) load_step(k, t0, k);
     for (long t = t0; t < t1; ++t) {
@@ -283,10 +304,24 @@ project32_kernel(const float *__restrict__ x, const float *__restrict__ w, const
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             u32x4 ahi[2], amid[2], alo[2];
+            if (!IN_CL) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) *(u32x4 *)(xw + 8 * j * 32) = raw[ks % RING][j >> 1][j & 1];
+            }
 #pragma unroll
             for (int mb = 0; mb < 2; ++mb) {
-                const f32x4 p0 = __builtin_bit_cast(f32x4, raw[ks % RING][mb][0]);
-                const f32x4 p1 = __builtin_bit_cast(f32x4, raw[ks % RING][mb][1]);
+                f32x4 p0, p1;
+                if (IN_CL) {
+                    p0 = __builtin_bit_cast(f32x4, raw[ks % RING][mb][0]);
+                    p1 = __builtin_bit_cast(f32x4, raw[ks % RING][mb][1]);
+                } else {
+                    // (block mb: the other 16-pixel half of the row, i.e. piece index bit 2 flipped)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        p0[e] = xr[e * 32 + (mb ? 16 - 32 * (kg & 1) : 0)];
+                        p1[e] = xr[(16 + e) * 32 + (mb ? 16 - 32 * (kg & 1) : 0)];
+                    }
+                }
                 const Pieces s0 = split2(p0[0], p0[1]), s1 = split2(p0[2], p0[3]);
                 const Pieces s2 = split2(p1[0], p1[1]), s3 = split2(p1[2], p1[3]);
                 ahi[mb] = u32x4{s0.hi, s1.hi, s2.hi, s3.hi};
@@ -312,8 +347,30 @@ project32_kernel(const float *__restrict__ x, const float *__restrict__ w, const
                 }
             }
         }
-        // acc[mb][nt][i]: pixel 16 mb + 4 kg + i, output 16 nt + r16 -> the wave's tile, then 16
-        // rows of 4 O bytes -> one contiguous run of 64 O bytes per block
+        // acc[mb][nt][i]: pixel 16 mb + 4 kg + i, output 16 nt + r16
+        if (!OUT_CL) {
+            // planes: a block of 16 outputs x 32 pixels -> the wave's tile (a lane holds 4
+            // neighbouring pixels), then 16 rows of 128 bytes; pieces past the plane's end are dropped
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+                for (int mb = 0; mb < 2; ++mb) {
+                    const f32x4 v = {acc[mb][nt][0] + bv[nt], acc[mb][nt][1] + bv[nt], acc[mb][nt][2] + bv[nt],
+                                     acc[mb][nt][3] + bv[nt]};
+                    *(f32x4 *)(rt + r16 * PS + 16 * mb + 4 * kg) = v;
+                }
+                const u32 obase = (u32)((16L * nt * HW + t * 32) * 4);
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int row = 8 * j + (lane >> 3), col = lane & 7;
+                    const u32 off = t * 32 + 4 * col < HW ? (u32)(row * HW + 4 * col) * 4u : 0x80000000u;
+                    __builtin_amdgcn_raw_buffer_store_b128(*(const u32x4 *)(rt + row * PS + 4 * col), ro, off, obase, 2);
+                }
+            }
+            continue;
+        }
+        // channels-last: the wave's tile, then 16 rows of 4 O bytes -> one contiguous run of 64 O
+        // bytes per block
 #pragma unroll
         for (int mb = 0; mb < 2; ++mb) {
 #pragma unroll
@@ -331,10 +388,12 @@ project32_kernel(const float *__restrict__ x, const float *__restrict__ w, const
     }
 }
 
-template <int C, int O>
+template <int C, int O, bool IN_CL, bool OUT_CL>
 static hipError_t launch32_co(const void *x, const void *w, const void *bias, void *out, int B, long HW,
                               hipStream_t st) {
-    constexpr size_t lds = (size_t)(3 * O * (C / 2 + 4) + 8 * 16 * (O + 4)) * 4;
+    constexpr int RT = OUT_CL ? 16 * (O + 4) : 16 * 36, XB = IN_CL ? 0 : 32 * 32;
+    constexpr size_t lds = (size_t)(3 * O * (C / 2 + 4) + 8 * (RT > XB ? RT : XB)) * 4;
+    if (!OUT_CL && HW % 4 != 0) return hipErrorNotSupported;
     static_assert(lds <= 160 * 1024, "weights and tiles must fit LDS");
     // 32-bit byte offsets inside an image
     if (HW * (long)(C > O ? C : O) * 4 >= (1L << 31)) return hipErrorNotSupported;
@@ -352,7 +411,7 @@ static hipError_t launch32_co(const void *x, const void *w, const void *bias, vo
     }
     blocks = (ntiles + 8 * per - 1) / (8 * per);
     if (blocks > 65535 * 32L || B > 65535) return hipErrorNotSupported;
-    auto kern = project32_kernel<C, O>;
+    auto kern = project32_kernel<C, O, IN_CL, OUT_CL>;
     if (lds > 64 * 1024) {
         int dev = 0, most = 0;
         if (hipGetDevice(&dev) != hipSuccess ||
@@ -369,10 +428,11 @@ static hipError_t launch32_co(const void *x, const void *w, const void *bias, vo
     return hipGetLastError();
 }
 
+template <bool IN_CL, bool OUT_CL>
 static hipError_t launch32(const void *x, const void *w, const void *bias, void *out, int B, int C, int O,
                            long HW, hipStream_t st) {
 #define SAPA_PROJECT_CASE(CV, OV) \
-    if (C == CV && O == OV) return launch32_co<CV, OV>(x, w, bias, out, B, HW, st);
+    if (C == CV && O == OV) return launch32_co<CV, OV, IN_CL, OUT_CL>(x, w, bias, out, B, HW, st);
     SAPA_PROJECT_CASE(64, 32) SAPA_PROJECT_CASE(64, 64)
     SAPA_PROJECT_CASE(128, 32) SAPA_PROJECT_CASE(128, 64)
     SAPA_PROJECT_CASE(256, 32) SAPA_PROJECT_CASE(256, 64)
@@ -405,10 +465,24 @@ hipError_t project_nhwc_launch(const void *x, const void *w, const void *bias, v
     const void *ptrs[3] = {x, w, out};
     for (const void *p : ptrs)
         if ((uintptr_t)p % 16 != 0) return hipErrorNotSupported;
-    if (dtype == 0) return project::launch32(x, w, bias, out, B, C, O, HW, st);
+    if (dtype == 0) return project::launch32<true, true>(x, w, bias, out, B, C, O, HW, st);
     if (dtype == 2) return project::launch_t<f16_t>(x, w, bias, out, B, C, O, HW, st);
     if (dtype == 3) return project::launch_t<bf16_t>(x, w, bias, out, B, C, O, HW, st);
     return hipErrorNotSupported;
+}
+
+// The same projection of a contiguous feature x [B, C, HW] (planes): out [B, HW, O]
+// (out_channels_last) or [B, O, HW]; fp32, the (C, O) pairs of the fp32 kernel above, HW a
+// multiple of 4 for a planar result, x and out aligned to 16 bytes.  hipErrorNotSupported
+// otherwise.
+hipError_t project_nchw_launch(const void *x, const void *w, const void *bias, void *out, int B, int C,
+                               int O, long HW, int out_channels_last, int dtype, hipStream_t st) {
+    const void *ptrs[3] = {x, w, out};
+    for (const void *p : ptrs)
+        if ((uintptr_t)p % 16 != 0) return hipErrorNotSupported;
+    if (dtype != 0) return hipErrorNotSupported;
+    return out_channels_last ? project::launch32<false, true>(x, w, bias, out, B, C, O, HW, st)
+                             : project::launch32<false, false>(x, w, bias, out, B, C, O, HW, st);
 }
 
 }  // namespace sapa

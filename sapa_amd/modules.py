@@ -122,18 +122,26 @@ def norm_project(x, norm, *convs, channels_last=False, defer_bias=False):
             # library's streaming projection kernel (bias in its epilogue); else a
             # library GEMM
             out = None
-            if x_cl and x.is_cuda and not torch.is_grad_enabled():
-                out = _lib.project_nhwc(x, w_b, None if defer_bias else b_b)
+            if x.is_cuda and not torch.is_grad_enabled():
+                if x_cl:
+                    out = _lib.project_nhwc(x, w_b, None if defer_bias else b_b)
+                else:
+                    # (a contiguous fp32 feature: the same kernel reading planes)
+                    out = _lib.project_nchw(x, w_b, None if defer_bias else b_b, channels_last_out=True)
             if out is None:
                 out = torch.bmm(x3.transpose(1, 2), w_b.transpose(1, 2))      # [B, HW, O]
                 if not defer_bias:
                     out.add_(b_b.unsqueeze(1))
                 out = out.view(B, H, W, O).permute(0, 3, 1, 2)
         else:
-            out = torch.bmm(w_b, x3)                                     # [B, O, HW]
-            if not defer_bias:
-                out.add_(b_b.unsqueeze(2))
-            out = out.view(B, O, H, W)
+            out = None
+            if x.is_cuda and not x_cl and not torch.is_grad_enabled():
+                out = _lib.project_nchw(x, w_b, None if defer_bias else b_b)
+            if out is None:
+                out = torch.bmm(w_b, x3)                                 # [B, O, HW]
+                if not defer_bias:
+                    out.add_(b_b.unsqueeze(2))
+                out = out.view(B, O, H, W)
         outs.append((out, b_b) if defer_bias else out)
     return outs
 

@@ -518,3 +518,36 @@ def test_projection_kernel_fp32(shape):
     if C == 256 and O == 64:
         w2 = torch.cat([w, w], 1).contiguous()
         assert _lib.project_nhwc(x, w2) is None
+
+
+@pytest.mark.parametrize('shape', [(2, 256, 64, 9, 12), (1, 128, 32, 40, 33), (3, 64, 64, 5, 8), (1, 512, 32, 4, 4),
+                                   (2, 256, 32, 1, 4), (1, 256, 64, 130, 129), (2, 64, 32, 17, 3)])
+def test_projection_kernel_fp32_contiguous_feature(shape):
+    """The fp32 projection reading a contiguous feature (planes), writing a channels_last
+    or a contiguous result (the latter for plane sizes that are multiples of 4; None
+    otherwise): same bound as the channels_last form, and the two results bit for bit
+    the same (one arithmetic, two store patterns)."""
+    from sapa_amd import _lib
+    B, C, O, H, W = shape
+    g = gen(362)
+    x = (randn(g, B, C, H, W) * 3 + 0.5).to(DEV)
+    w = (randn(g, B, O, C) * 0.1).to(DEV)
+    b = randn(g, B, O).to(DEV)
+    want = torch.einsum('boc,bchw->bohw', w.double().cpu(), x.double().cpu())
+    e32 = (torch.einsum('boc,bchw->bohw', w.cpu(), x.cpu()).double() - want).abs().max().item()
+    scale = torch.einsum('boc,bchw->bohw', w.double().abs().cpu(), x.double().abs().cpu()).max().item()
+    for bias in (None, b):
+        ref = want if bias is None else want + bias.double().cpu()[:, :, None, None]
+        out_cl = _lib.project_nchw(x, w, bias, channels_last_out=True)
+        assert out_cl is not None and out_cl.shape == (B, O, H, W) and out_cl.is_contiguous(memory_format=CL)
+        err = (out_cl.double().cpu() - ref).abs().max().item()
+        assert err <= max(3 * e32, 1e-6 * scale) and err <= 1e-5 * scale, (err, e32, scale)
+        out = _lib.project_nchw(x, w, bias)
+        if (H * W) % 4:
+            assert out is None
+        else:
+            assert out.is_contiguous() and torch.equal(out, out_cl)
+        # ... and the same bits as the channels_last feature's kernel
+        assert torch.equal(_lib.project_nhwc(x.contiguous(memory_format=CL), w, bias), out_cl)
+    assert _lib.project_nchw(x.bfloat16(), w.bfloat16()) is None
+    assert _lib.project_nchw(x.contiguous(memory_format=CL), w) is None
