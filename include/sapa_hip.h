@@ -474,10 +474,10 @@ int sapa_project_nhwc(const void *x, const void *weight, const void *bias, void 
 /* The same projection of a contiguous feature x [B,C,HW] (the reference's layout:
  * self.q(norm_y(y)) on an NCHW tensor, sapa/sapa/sapa_base.py:32-35): out [B,O,HW],
  * or [B,HW,O] (channels-last, what the channels-last operator takes) when
- * out_channels_last is non-zero.  SAPA_F32 only, the (C,O) pairs of
- * sapa_project_nhwc's SAPA_F32 form, HW a multiple of 4 for a [B,O,HW] result, x and
- * out aligned to 16 bytes; SAPA_ERR_UNSUPPORTED otherwise (the caller uses a library
- * GEMM). */
+ * out_channels_last is non-zero.  SAPA_F32 / SAPA_F16 / SAPA_BF16, the (C,O) pairs of
+ * sapa_project_nhwc's SAPA_F32 form; SAPA_F32: HW a multiple of 4 for a [B,O,HW]
+ * result; 16-bit: HW a multiple of 8; x and out aligned to 16 bytes;
+ * SAPA_ERR_UNSUPPORTED otherwise (the caller uses a library GEMM). */
 int sapa_project_nchw(const void *x, const void *weight, const void *bias, void *out,
                       int B, int C, int O, long long HW, int out_channels_last, int dtype,
                       void *stream);

@@ -311,13 +311,14 @@ def groupnorm_fold(mean_var, norm, conv, dtype):
 
 
 def project_nchw(x, weight, bias=None, channels_last_out=False):
-    """out[b, :, h, w] = weight[b] @ x[b, :, h, w] (+ bias[b]) for a contiguous fp32
-    CUDA feature x [B, C, H, W] and per-image weights [B, O, C]: a contiguous (or, with
-    channels_last_out, a channels_last) tensor [B, O, H, W], or None if the kernel does
-    not cover the configuration (the caller then uses a library GEMM)."""
+    """out[b, :, h, w] = weight[b] @ x[b, :, h, w] (+ bias[b]) for a contiguous f16 /
+    bf16 / fp32 CUDA feature x [B, C, H, W] and per-image weights [B, O, C]: a contiguous
+    (or, with channels_last_out, a channels_last) tensor [B, O, H, W], or None if the
+    kernel does not cover the configuration (the caller then uses a library GEMM)."""
     B, C, H, W = x.shape
     O = weight.shape[1]
-    if x.dtype != torch.float32 or weight.dtype != x.dtype or x.numel() == 0 or not x.is_contiguous():
+    if (x.dtype not in (torch.float16, torch.bfloat16, torch.float32) or weight.dtype != x.dtype
+            or x.numel() == 0 or not x.is_contiguous()):
         return None
     weight = weight.contiguous()
     if bias is not None:

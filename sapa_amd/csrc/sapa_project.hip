@@ -53,6 +53,20 @@ template <> struct Mma<bf16_t> {
     }
 };
 
+template <typename T> struct Mma32;
+template <> struct Mma32<f16_t> {
+    static __device__ __forceinline__ f32x4 run(u32x4 a, u32x4 b, f32x4 c) {
+        typedef _Float16 v8 __attribute__((ext_vector_type(8)));
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8, a), __builtin_bit_cast(v8, b), c, 0, 0, 0);
+    }
+};
+template <> struct Mma32<bf16_t> {
+    static __device__ __forceinline__ f32x4 run(u32x4 a, u32x4 b, f32x4 c) {
+        typedef __bf16 v8 __attribute__((ext_vector_type(8)));
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8, a), __builtin_bit_cast(v8, b), c, 0, 0, 0);
+    }
+};
+
 template <typename T>
 __device__ __forceinline__ u32 pack2(float a, float b) {
     typedef float f32x2 __attribute__((ext_vector_type(2)));
@@ -183,6 +197,180 @@ static hipError_t launch_co(const void *x, const void *w, const void *bias, void
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks, B), dim3(256), lds, st, (const T *)x, (const T *)w,
                        (const T *)bias, (T *)out, HW, (int)per);
     return hipGetLastError();
+}
+
+// ---- 16-bit, contiguous feature (planes) ----
+// x [B, C, HW]: a lane fetches 8 neighbouring pixels of one channel (a wave: 8 channels x 128
+// bytes per load); a reduction step's 32 channels x 64 pixels pass through a wave-private LDS
+// tile [channel][pixel] from which ds_read_tr16_b64 hands every lane its pixel's 4 channels (rows
+// of 160 bytes: the four rows of a transposing read lie on disjoint banks).  Same order of the
+// channels inside a step as in the fp32 kernel below; weights [O][C] in that order in LDS.
+// Tiles of 64 pixels (four blocks of 16 matrix rows).  OUT_CL: out [B, HW, O], else [B, O, HW].
+// HW a multiple of 8 (16-byte pieces never run from one plane into the next).
+template <typename T, int C, int O, bool OUT_CL>
+__global__ void __launch_bounds__(256)
+project16p_kernel(const T *__restrict__ x, const T *__restrict__ w, const T *__restrict__ bias,
+                  T *__restrict__ out, long HW, int tiles_per_wave) {
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    constexpr int NW = 4;
+    constexpr int RW = C / 2 + 4;                 // dwords per padded row of C 16-bit values
+    constexpr int NT = O / 16;                    // output tiles of 16 columns
+    constexpr int OW = O / 2 + 4;                 // dwords per padded row of the result tile (channels-last)
+    constexpr int PW = 64 / 2 + 4;                // ... of a block of 16 outputs x 64 pixels (planes)
+    constexpr int XS = 64 / 2 + 8;                // dwords per row of the x tile: 160 bytes
+    constexpr int KS = C / 32;                    // reduction steps
+    constexpr int RING = KS < 4 ? KS : 4;         // steps of x in flight
+    constexpr int RT = OUT_CL ? 16 * OW : 16 * PW;
+    constexpr int WF = RT > 32 * XS ? RT : 32 * XS;
+    static_assert(KS % RING == 0, "the ring of x registers is indexed by the step");
+    extern __shared__ __attribute__((aligned(16))) u32 sh[];
+    u32 *wl = sh;                                 // weights: O rows of RW dwords
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    u32 *xt = sh + O * RW + wave * WF;            // this wave's x tile / result tile
+    const int b = blockIdx.y;
+
+    // the image's weights -> LDS, 8 channels per thread and step: two groups of 4, which lie 8
+    // places apart in the step's order
+    {
+        const u32x4 *src = (const u32x4 *)(w + (long)b * O * C);
+        for (int i = threadIdx.x; i < O * C / 8; i += 64 * NW) {
+            const int o = i / (C / 8), c = 8 * (i % (C / 8)), cs = c % 32;
+            const int pos = 32 * (c / 32) + 8 * ((cs % 16) / 4) + 4 * (cs / 16);
+            const u32x4 v = src[i];
+            u32 *dst = wl + o * RW + pos / 2;
+            *(u32x2 *)dst = u32x2{v[0], v[1]};
+            *(u32x2 *)(dst + 4) = u32x2{v[2], v[3]};
+        }
+    }
+    __syncthreads();
+
+    const long ntiles = (HW + 63) / 64;
+    const long t0 = ((long)blockIdx.x * NW + wave) * tiles_per_wave;
+    const long t1 = t0 + tiles_per_wave < ntiles ? t0 + tiles_per_wave : ntiles;
+    if (t0 >= t1) return;
+    const int r16 = lane & 15, kg = lane >> 4;
+    float bv[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) bv[nt] = bias ? (float)bias[(long)b * O + 16 * nt + r16] : 0.f;
+
+    const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(x + (long)b * HW * C), 0, (int)(HW * C * 2), 0x00020000);
+    const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(out + (long)b * HW * O), 0, (int)(HW * O * 2), 0x00020000);
+    // step (t, ks) of x: piece j = pixels 8 (lane % 8) .. + 7 of channel 8 j + lane / 8 of the step
+    const u32 xoff = (u32)((lane >> 3) * HW + 8 * (lane & 7)) * 2u, xstride = (u32)(8 * HW * 2);
+    u32x4 raw[RING][4];
+    auto load_step = [&](int slot, long t, int ks) __attribute__((always_inline)) {
+        const u32 so = (u32)((32L * ks * HW + t * 64) * 2);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            raw[slot][j] = __builtin_amdgcn_raw_buffer_load_b128(rx, xoff + (u32)j * xstride, so, 0);
+    };
+    u32 *const xw = xt + (lane >> 3) * XS + 4 * (lane & 7);
+    // transposing reads: lane L of a 16-lane block addresses row L / 4, pixels 4 (L % 4) .. + 3 of
+    // the block's 16 and receives pixel L's value of the 4 rows; block kg takes channels 4 kg ..
+    // (and 16 + 4 kg ..) of the step
+    const u32 *const xr = xt + (4 * kg + (r16 >> 2)) * XS + 2 * (r16 & 3);
+#pragma unroll
+    for (int k = 0; k < RING; ++k) load_step(k, t0, k);
+    for (long t = t0; t < t1; ++t) {
+        f32x4 acc[4][NT];
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) acc[mb][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) *(u32x4 *)(xw + 8 * j * XS) = raw[ks % RING][j];
+            if (ks + RING < KS) load_step(ks % RING, t, ks + RING);
+            else if (t + 1 < t1) load_step(ks % RING, t + 1, ks + RING - KS);
+            u32x4 a[4];
+#pragma unroll
+            for (int mb = 0; mb < 4; ++mb) {
+                const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                                     (s16x4 __attribute__((address_space(3))) *)(xr + 8 * mb)));
+                const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                                     (s16x4 __attribute__((address_space(3))) *)(xr + 16 * XS + 8 * mb)));
+                a[mb] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+            }
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const u32x4 bm = *(const u32x4 *)(wl + (16 * nt + r16) * RW + 16 * ks + 4 * kg);
+#pragma unroll
+                for (int mb = 0; mb < 4; ++mb) acc[mb][nt] = Mma32<T>::run(a[mb], bm, acc[mb][nt]);
+            }
+        }
+        // acc[mb][nt][i]: pixel 16 mb + 4 kg + i, output 16 nt + r16
+        if (OUT_CL) {
+            // 16 rows of 2 O bytes per block -> one contiguous run of 32 O bytes
+            unsigned short *rt = (unsigned short *)xt;
+#pragma unroll
+            for (int mb = 0; mb < 4; ++mb) {
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        rt[(4 * kg + i) * (2 * OW) + 16 * nt + r16] = (unsigned short)pack2<T>(acc[mb][nt][i] + bv[nt], 0.f);
+                const u32 obase = (u32)((t * 64 + 16 * mb) * O * 2);
+#pragma unroll
+                for (int j = 0; j < (16 * O / 8 + 63) / 64; ++j) {
+                    const int i = j * 64 + lane, row = i / (O / 8), col = i % (O / 8);
+                    if (16 * O / 8 % 64 == 0 || i < 16 * O / 8)
+                        __builtin_amdgcn_raw_buffer_store_b128(*(const u32x4 *)(xt + row * OW + 4 * col), ro, (u32)(i * 16), obase, 2);
+                }
+            }
+        } else {
+            // a block of 16 outputs x 64 pixels (a lane holds 4 neighbouring pixels), then 16 rows of
+            // 128 bytes; pieces past the plane's end are dropped
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+                for (int mb = 0; mb < 4; ++mb)
+                    *(u32x2 *)(xt + r16 * PW + 8 * mb + 2 * kg) =
+                        u32x2{pack2<T>(acc[mb][nt][0] + bv[nt], acc[mb][nt][1] + bv[nt]),
+                              pack2<T>(acc[mb][nt][2] + bv[nt], acc[mb][nt][3] + bv[nt])};
+                const u32 obase = (u32)((16L * nt * HW + t * 64) * 2);
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int row = 8 * j + (lane >> 3), col = lane & 7;
+                    const u32 off = t * 64 + 8 * col < HW ? (u32)(row * HW + 8 * col) * 2u : 0x80000000u;
+                    __builtin_amdgcn_raw_buffer_store_b128(*(const u32x4 *)(xt + row * PW + 4 * col), ro, off, obase, 2);
+                }
+            }
+        }
+    }
+}
+
+template <typename T, int C, int O, bool OUT_CL>
+static hipError_t launch16p_co(const void *x, const void *w, const void *bias, void *out, int B, long HW,
+                               hipStream_t st) {
+    constexpr int RT = OUT_CL ? 16 * (O / 2 + 4) : 16 * 36, XT = 32 * 40;
+    constexpr size_t lds = (size_t)(O * (C / 2 + 4) + 4 * (RT > XT ? RT : XT)) * 4;
+    static_assert(lds <= 64 * 1024, "weights and tiles within the default LDS of a workgroup");
+    if (HW % 8 != 0 || HW * (long)(C > O ? C : O) * 2 >= (1L << 31)) return hipErrorNotSupported;
+    const long ntiles = (HW + 63) / 64;
+    // about 3 workgroups per CU over the whole launch (256 CUs), at least 2 tiles per wave
+    long per = (ntiles * B + 4L * 768 - 1) / (4L * 768);
+    if (per < 2) per = 2;
+    const long blocks = (ntiles + 4 * per - 1) / (4 * per);
+    if (blocks > 65535 * 32L || B > 65535) return hipErrorNotSupported;
+    hipLaunchKernelGGL((project16p_kernel<T, C, O, OUT_CL>), dim3((unsigned)blocks, B), dim3(256), lds, st,
+                       (const T *)x, (const T *)w, (const T *)bias, (T *)out, HW, (int)per);
+    return hipGetLastError();
+}
+
+template <typename T, bool OUT_CL>
+static hipError_t launch16p(const void *x, const void *w, const void *bias, void *out, int B, int C, int O,
+                            long HW, hipStream_t st) {
+#define SAPA_PROJECT_CASE(CV, OV) \
+    if (C == CV && O == OV) return launch16p_co<T, CV, OV, OUT_CL>(x, w, bias, out, B, HW, st);
+    SAPA_PROJECT_CASE(64, 32) SAPA_PROJECT_CASE(64, 64)
+    SAPA_PROJECT_CASE(128, 32) SAPA_PROJECT_CASE(128, 64)
+    SAPA_PROJECT_CASE(256, 32) SAPA_PROJECT_CASE(256, 64)
+    SAPA_PROJECT_CASE(512, 32)
+#undef SAPA_PROJECT_CASE
+    return hipErrorNotSupported;
 }
 
 // ---- fp32 ----
@@ -472,14 +660,20 @@ hipError_t project_nhwc_launch(const void *x, const void *w, const void *bias, v
 }
 
 // The same projection of a contiguous feature x [B, C, HW] (planes): out [B, HW, O]
-// (out_channels_last) or [B, O, HW]; fp32, the (C, O) pairs of the fp32 kernel above, HW a
-// multiple of 4 for a planar result, x and out aligned to 16 bytes.  hipErrorNotSupported
-// otherwise.
+// (out_channels_last) or [B, O, HW]; the (C, O) pairs of the fp32 kernel above; fp32: HW a
+// multiple of 4 for a planar result; f16 / bf16: HW a multiple of 8; x and out aligned to 16
+// bytes.  hipErrorNotSupported otherwise.
 hipError_t project_nchw_launch(const void *x, const void *w, const void *bias, void *out, int B, int C,
                                int O, long HW, int out_channels_last, int dtype, hipStream_t st) {
     const void *ptrs[3] = {x, w, out};
     for (const void *p : ptrs)
         if ((uintptr_t)p % 16 != 0) return hipErrorNotSupported;
+    if (dtype == 2)
+        return out_channels_last ? project::launch16p<f16_t, true>(x, w, bias, out, B, C, O, HW, st)
+                                 : project::launch16p<f16_t, false>(x, w, bias, out, B, C, O, HW, st);
+    if (dtype == 3)
+        return out_channels_last ? project::launch16p<bf16_t, true>(x, w, bias, out, B, C, O, HW, st)
+                                 : project::launch16p<bf16_t, false>(x, w, bias, out, B, C, O, HW, st);
     if (dtype != 0) return hipErrorNotSupported;
     return out_channels_last ? project::launch32<false, true>(x, w, bias, out, B, C, O, HW, st)
                              : project::launch32<false, false>(x, w, bias, out, B, C, O, HW, st);

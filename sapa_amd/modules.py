@@ -126,7 +126,7 @@ def norm_project(x, norm, *convs, channels_last=False, defer_bias=False):
                 if x_cl:
                     out = _lib.project_nhwc(x, w_b, None if defer_bias else b_b)
                 else:
-                    # (a contiguous fp32 feature: the same kernel reading planes)
+                    # (a contiguous feature: the same kernels reading planes)
                     out = _lib.project_nchw(x, w_b, None if defer_bias else b_b, channels_last_out=True)
             if out is None:
                 out = torch.bmm(x3.transpose(1, 2), w_b.transpose(1, 2))      # [B, HW, O]

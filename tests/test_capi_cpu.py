@@ -134,7 +134,8 @@ def test_argument_validation_returns_codes():
     assert h.sapa_project_nhwc(None, None, None, None, 0, 256, 64, 100, 3, None) == 0
     assert h.sapa_project_nchw(p, p, p, p, 1, 256, 0, 100, 0, 0, None) == -1
     assert h.sapa_project_nchw(p, p, p, None, 1, 256, 64, 100, 1, 0, None) == -1
-    assert h.sapa_project_nchw(p, p, None, p, 1, 256, 64, 100, 0, 3, None) == -2
+    assert h.sapa_project_nchw(p, p, None, p, 1, 256, 64, 100, 0, 1, None) == -2     # fp64
+    assert h.sapa_project_nchw(p, p, None, p, 1, 256, 64, 100, 0, 3, None) == -2     # 16-bit planes of 100 pixels
     assert h.sapa_project_nchw(p, p, None, p, 1, 256, 64, 102, 0, 0, None) == -2     # planes of 102 pixels
     assert h.sapa_project_nchw(None, None, None, None, 0, 256, 64, 100, 1, 0, None) == 0
     # layout copy: element size, negative extents, null / misaligned pointers, empty tensors,

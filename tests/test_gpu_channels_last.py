@@ -549,5 +549,35 @@ def test_projection_kernel_fp32_contiguous_feature(shape):
             assert out.is_contiguous() and torch.equal(out, out_cl)
         # ... and the same bits as the channels_last feature's kernel
         assert torch.equal(_lib.project_nhwc(x.contiguous(memory_format=CL), w, bias), out_cl)
-    assert _lib.project_nchw(x.bfloat16(), w.bfloat16()) is None
+    assert _lib.project_nchw(x.double(), w.double()) is None
     assert _lib.project_nchw(x.contiguous(memory_format=CL), w) is None
+
+
+@pytest.mark.parametrize('dtype,tol', [(torch.bfloat16, 2e-2), (torch.float16, 3e-3)])
+@pytest.mark.parametrize('shape', [(2, 256, 64, 9, 16), (1, 128, 32, 40, 34), (3, 64, 64, 5, 8), (1, 512, 32, 4, 4),
+                                   (2, 256, 32, 1, 8), (1, 256, 64, 130, 132), (2, 64, 32, 17, 3)])
+def test_projection_kernel_16bit_contiguous_feature(dtype, tol, shape):
+    """The 16-bit projection reading a contiguous feature (planes of a multiple of 8
+    pixels; None otherwise), writing a channels_last or a contiguous result: against
+    float64 arithmetic on the same values, the two results bit for bit the same, and the
+    same bits as the channels_last feature's kernel gives (fp32 sums in the same order
+    would not be needed for that bar; they are what the kernels do)."""
+    from sapa_amd import _lib
+    B, C, O, H, W = shape
+    g = gen(363)
+    x = randn(g, B, C, H, W).to(dtype).to(DEV)
+    w = (randn(g, B, O, C) * 0.1).to(dtype).to(DEV)
+    b = randn(g, B, O).to(dtype).to(DEV)
+    want = torch.einsum('boc,bchw->bohw', w.double().cpu(), x.double().cpu())
+    for bias in (None, b):
+        out_cl = _lib.project_nchw(x, w, bias, channels_last_out=True)
+        out = _lib.project_nchw(x, w, bias)
+        if (H * W) % 8:
+            assert out_cl is None and out is None
+            continue
+        assert out_cl.is_contiguous(memory_format=CL) and out.is_contiguous() and out.dtype == dtype
+        ref = want if bias is None else want + bias.double().cpu()[:, :, None, None]
+        torch.testing.assert_close(out_cl.double().cpu(), ref, rtol=tol, atol=tol)
+        assert torch.equal(out, out_cl)
+        torch.testing.assert_close(_lib.project_nhwc(x.contiguous(memory_format=CL), w, bias).float(), out_cl.float(),
+                                   rtol=2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10, atol=1e-6)
