@@ -249,13 +249,11 @@ def cpu_baseline(fn, tensors, pix_per_image, median_budget_s=8.0, batch_budget_s
     return rec, out
 
 
-def module_pass(args, dev, dtype, stream):
-    """The caller of the hot path: SAPA.forward(y, x) = GroupNorm(32) on both
-    features, 1x1 q / k projections, fused operator (sapa_base.py:26-40), timed
-    as the reference composes it and with the projections of this build."""
+def module_cases(args, dev, dtype, stream, only=None, warmup=None, steps=None):
+    """SAPA.forward(y, x) = GroupNorm(32) on both features, 1x1 q / k projections,
+    fused operator (sapa_base.py:26-40), timed as the reference composes it and with
+    the projections of this build: {case: {'ms', 'max_abs_diff_vs_first_image0'}}."""
     import sapa_amd
-    if args.workload not in WORKLOADS:
-        sys.exit('bench.py: --pass module covers the SAPA-B workloads')
     B, C, d, H, W, K, s = WORKLOADS[args.workload]
     g = torch.Generator(device=dev).manual_seed(0)
     y = torch.randn(B, C, H * s, W * s, generator=g, device=dev).to(dtype)
@@ -268,8 +266,10 @@ def module_pass(args, dev, dtype, stream):
              ('channels_last=True, contiguous features', {'channels_last': True}, (y, x)),
              ('channels_last=True, channels_last features', {'channels_last': True}, (ycl, xcl)),
              ('GroupNorm -> Conv2d -> fused operator, channels_last features', {}, (ycl, xcl))]
-    if args.module_case >= 0:
-        cases = cases[args.module_case:args.module_case + 1]
+    if only is not None:
+        cases = [cases[i] for i in only]
+    warmup = max(args.warmup // 10, 3) if warmup is None else warmup
+    steps = max(args.steps // 10, 5) if steps is None else steps
     res, ref = {}, None
     with torch.no_grad():
         for name, kw, feats in cases:
@@ -278,17 +278,27 @@ def module_pass(args, dev, dtype, stream):
             if ref is None:
                 ref = out[:1].float()
             err = (out[:1].float() - ref).abs().max().item()
-            for _ in range(max(args.warmup // 10, 3)):
+            for _ in range(warmup):
                 m(*feats)
             torch.cuda.synchronize()
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            n = max(args.steps // 10, 5)
+            n = steps
             e0.record(stream)
             for _ in range(n):
                 m(*feats)
             e1.record(stream)
             torch.cuda.synchronize()
             res[name] = {'ms': e0.elapsed_time(e1) / n, 'max_abs_diff_vs_first_image0': err}
+    return res
+
+
+def module_pass(args, dev, dtype, stream):
+    """The caller of the hot path (module_cases) as the main line."""
+    if args.workload not in WORKLOADS:
+        sys.exit('bench.py: --pass module covers the SAPA-B workloads')
+    B, C, d, H, W, K, s = WORKLOADS[args.workload]
+    res = module_cases(args, dev, dtype, stream,
+                       only=[args.module_case] if args.module_case >= 0 else None)
     pix = B * H * s * W * s
     best = min(res, key=lambda k: res[k]['ms'] if 'contiguous features' in k or len(res) == 1 else 1e9)
     print(json.dumps({
@@ -540,6 +550,17 @@ def main():
             del hc
         del hq, hk, hv, hout
 
+    module = None
+    if (not deform and args.dtype == 'fp32' and args.layout == 'nchw' and args.direction == 'forward'
+            and not args.only_main):
+        # the caller of the hot path: the whole SAPA module forward on this workload's features (the
+        # reference's composition, and GroupNorm folded into this library's projection kernels)
+        module = {'unit': 'ms per forward', 'note': 'python bench.py --pass module [--dtype bf16] makes this the main line',
+                  'fp32': {k: round(v['ms'], 4) for k, v in module_cases(
+                      args, dev, torch.float32, stream, only=[0, 1, 3], warmup=5, steps=10).items()},
+                  'bf16': {k: round(v['ms'], 4) for k, v in module_cases(
+                      args, dev, torch.bfloat16, stream, only=[0, 1, 3], warmup=5, steps=10).items()}}
+
     reference_order = None
     if deform and main_is_ws and args.direction == 'forward' and not args.only_main:
         # the same contiguous tensors through the kernel that keeps the reference's order of sums
@@ -680,6 +701,8 @@ def main():
                     'order (python bench.py --layout channels_last makes this the main line)'}
     if half is not None:
         rec['bf16'] = half
+    if module is not None:
+        rec['module_forward'] = module
     if reference_order is not None:
         reference_order['value'] = pix / (reference_order['ms_per_step'] * 1e-3) / 1e9
         reference_order['roofline_frac'] = abytes / (reference_order['ms_per_step'] * 1e-3) / 1e9 / HBM_PEAK_GBS
