@@ -317,6 +317,7 @@ def project_nchw(x, weight, bias=None, channels_last_out=False):
     kernel does not cover the configuration (the caller then uses a library GEMM)."""
     B, C, H, W = x.shape
     O = weight.shape[1]
+    assert weight.shape == (B, O, C) and (bias is None or bias.shape == (B, O)), 'per-image weights [B, O, C], bias [B, O]'
     if (x.dtype not in (torch.float16, torch.bfloat16, torch.float32) or weight.dtype != x.dtype
             or x.numel() == 0 or not x.is_contiguous()):
         return None
@@ -343,6 +344,7 @@ def project_nhwc(x, weight, bias=None):
     configuration (the caller then uses a library GEMM)."""
     B, C, H, W = x.shape
     O = weight.shape[1]
+    assert weight.shape == (B, O, C) and (bias is None or bias.shape == (B, O)), 'per-image weights [B, O, C], bias [B, O]'
     if (x.dtype not in (torch.float16, torch.bfloat16, torch.float32) or weight.dtype != x.dtype
             or x.numel() == 0):
         return None
