@@ -175,9 +175,11 @@ static hipError_t launch_co(const void *x, const void *w, const void *bias, void
     constexpr size_t lds = (size_t)(O * RW + 4 * XT) * 4;
     static_assert(lds <= 160 * 1024, "weights and tiles must fit LDS");
     const long ntiles = (HW + 15) / 16;
-    // about 8 workgroups per CU over the whole launch, at least 8 tiles per wave
-    long per = (ntiles * B + 4L * 2048 - 1) / (4L * 2048);
-    if (per < 8) per = 8;
+    // two workgroups are resident per CU (LDS) and the part has 256 CUs: one round of at most 512
+    // workgroups, at least 2 tiles per wave (16 images of 100 x 168 pixels, 256 -> 64: 37 us against
+    // 46 with a fixed 8 tiles per wave; 200 x 336 pixels: 141 against 146)
+    long per = (ntiles * B + 4L * 512 - 1) / (4L * 512);
+    if (per < 2) per = 2;
     const long blocks = (ntiles + 4 * per - 1) / (4 * per);
     if (blocks > 65535 * 32L || B > 65535) return hipErrorNotSupported;
     auto kern = project_kernel<T, C, O>;
@@ -350,8 +352,10 @@ static hipError_t launch16p_co(const void *x, const void *w, const void *bias, v
     static_assert(lds <= 64 * 1024, "weights and tiles within the default LDS of a workgroup");
     if (HW % 8 != 0 || HW * (long)(C > O ? C : O) * 2 >= (1L << 31)) return hipErrorNotSupported;
     const long ntiles = (HW + 63) / 64;
-    // about 3 workgroups per CU over the whole launch (256 CUs), at least 2 tiles per wave
-    long per = (ntiles * B + 4L * 768 - 1) / (4L * 768);
+    // two workgroups are resident per CU (their registers) and the part has 256 CUs: one round of
+    // at most 512 workgroups, at least 2 tiles per wave (q projection at 16 x 200 x 336 pixels:
+    // 140 us against 152 with 704 workgroups)
+    long per = (ntiles * B + 4L * 512 - 1) / (4L * 512);
     if (per < 2) per = 2;
     const long blocks = (ntiles + 4 * per - 1) / (4 * per);
     if (blocks > 65535 * 32L || B > 65535) return hipErrorNotSupported;
