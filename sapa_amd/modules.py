@@ -63,38 +63,45 @@ def norm_project(x, norm, *convs, channels_last=False, defer_bias=False):
         acc = torch.float64 if x.dtype == torch.float64 else torch.float32
         if x.is_cuda and not (torch.is_grad_enabled() and x.requires_grad):
             mom = _lib.channel_moments(x)
-        if mom is not None:
-            mean_ch, var_ch = (mom[..., i].reshape(B, G, per_c) for i in (0, 1))
-            mean = mean_ch.mean(dim=2)
-            var = (var_ch + (mean_ch - mean.unsqueeze(2)).square()).mean(dim=2)
-        elif x_cl:
-            # per-channel moments, then per group: no layout copy of x
-            m1 = x.mean(dim=(2, 3), dtype=acc).reshape(B, G, per_c)
-            m2 = (torch.linalg.vector_norm(x, dim=(2, 3), dtype=acc).square()
-                  / (H * W)).reshape(B, G, per_c)
-            mean = m1.mean(dim=2)
-            var = (m2.mean(dim=2) - mean * mean).clamp_min(0)
-        else:
-            xg = x.reshape(B, G, -1)
-            if x.dtype in (torch.float16, torch.bfloat16):
-                # fp32 accumulation straight from the 16-bit tensor (no fp32 copy)
-                mean = xg.mean(dim=2, dtype=torch.float32)
-                sq = torch.linalg.vector_norm(xg, dim=2, dtype=torch.float32).square() / xg.shape[2]
-                var = (sq - mean * mean).clamp_min(0)
+        # the per-(image, channel) scale and shift of the normalisation as torch tensors: only the
+        # projections that do not go through the library's fold kernel below need them (a dozen
+        # small launches otherwise spent for nothing)
+        def affine():
+            if mom is not None:
+                mean_ch, var_ch = (mom[..., i].reshape(B, G, per_c) for i in (0, 1))
+                mean = mean_ch.mean(dim=2)
+                var = (var_ch + (mean_ch - mean.unsqueeze(2)).square()).mean(dim=2)
+            elif x_cl:
+                # per-channel moments, then per group: no layout copy of x
+                m1 = x.mean(dim=(2, 3), dtype=acc).reshape(B, G, per_c)
+                m2 = (torch.linalg.vector_norm(x, dim=(2, 3), dtype=acc).square()
+                      / (H * W)).reshape(B, G, per_c)
+                mean = m1.mean(dim=2)
+                var = (m2.mean(dim=2) - mean * mean).clamp_min(0)
             else:
-                var, mean = torch.var_mean(xg.to(acc), dim=2, unbiased=False)
-        rstd = torch.rsqrt(var + norm.eps)
-        rstd_c = rstd.repeat_interleave(per_c, dim=1)                    # [B, C]
-        mean_c = mean.repeat_interleave(per_c, dim=1)
-        gamma = norm.weight.to(acc) if norm.weight is not None else x.new_ones(C, dtype=acc)
-        beta = norm.bias.to(acc) if norm.bias is not None else x.new_zeros(C, dtype=acc)
-        scale = gamma.unsqueeze(0) * rstd_c                              # [B, C]
-        shift = beta.unsqueeze(0) - mean_c * scale                       # [B, C]
+                xg = x.reshape(B, G, -1)
+                if x.dtype in (torch.float16, torch.bfloat16):
+                    # fp32 accumulation straight from the 16-bit tensor (no fp32 copy)
+                    mean = xg.mean(dim=2, dtype=torch.float32)
+                    sq = torch.linalg.vector_norm(xg, dim=2, dtype=torch.float32).square() / xg.shape[2]
+                    var = (sq - mean * mean).clamp_min(0)
+                else:
+                    var, mean = torch.var_mean(xg.to(acc), dim=2, unbiased=False)
+            rstd = torch.rsqrt(var + norm.eps)
+            rstd_c = rstd.repeat_interleave(per_c, dim=1)                    # [B, C]
+            mean_c = mean.repeat_interleave(per_c, dim=1)
+            gamma = norm.weight.to(acc) if norm.weight is not None else x.new_ones(C, dtype=acc)
+            beta = norm.bias.to(acc) if norm.bias is not None else x.new_zeros(C, dtype=acc)
+            scale = gamma.unsqueeze(0) * rstd_c                              # [B, C]
+            shift = beta.unsqueeze(0) - mean_c * scale                       # [B, C]
+            return scale, shift
     else:
         mom = None
         acc = torch.float64 if x.dtype == torch.float64 else torch.float32
-        scale = x.new_ones(B, C, dtype=acc)
-        shift = x.new_zeros(B, C, dtype=acc)
+
+        def affine():
+            return x.new_ones(B, C, dtype=acc), x.new_zeros(B, C, dtype=acc)
+    scale_shift = None
     # [B, C, HW] view of x in either memory order
     x3 = x.permute(0, 2, 3, 1).reshape(B, H * W, C).transpose(1, 2) if x_cl else x.reshape(B, C, H * W)
     outs = []
@@ -109,6 +116,9 @@ def norm_project(x, norm, *convs, channels_last=False, defer_bias=False):
         if folded is not None:
             w_b, b_b = folded
         else:
+            if scale_shift is None:
+                scale_shift = affine()
+            scale, shift = scale_shift
             w = conv.weight.reshape(O, C).to(acc)
             w_b = (w.unsqueeze(0) * scale.unsqueeze(1)).to(x.dtype)      # [B, O, C]
             b_b = torch.einsum('oc,bc->bo', w, shift)
