@@ -482,6 +482,25 @@ int sapa_project_nchw(const void *x, const void *weight, const void *bias, void 
                       int B, int C, int O, long long HW, int out_channels_last, int dtype,
                       void *stream);
 
+/* self.q(self.norm_y(y)) / self.k(self.norm_x(x)) (sapa/sapa/sapa_base.py:27-35; GroupNorm and a
+ * 1x1 Conv2d, ATen calls there) in one call: sapa_channel_moments, sapa_groupnorm_fold and
+ * sapa_project_nhwc (x_channels_last != 0; the result is channels-last) or sapa_project_nchw
+ * (result [B,O,HW], or [B,HW,O] when out_channels_last != 0) on one stream -- four launches,
+ * the normalised feature never written.  gamma / beta [C] (NULL: 1 / 0), weight [O,C], bias
+ * [O] or NULL, all of type `dtype`.  scratch: sapa_norm_project_scratch(...) bytes, aligned
+ * to 16 (intermediates; nothing to keep).  bias_out, if not NULL, receives the folded
+ * per-image bias [B,O] and the projection is written WITHOUT it (for
+ * sapa_fused_forward_nhwc_qbias); if NULL the bias is added.  Nothing is launched and
+ * SAPA_ERR_UNSUPPORTED returned unless every step has a kernel for the configuration
+ * (SAPA_F32 / F16 / BF16, C a multiple of groups and <= 8192, the (C,O) pairs and extents
+ * of the projection entry points, x and out aligned to 16 bytes). */
+long long sapa_norm_project_scratch(int B, int C, int O, long long HW, int x_channels_last,
+                                    int dtype);
+int sapa_norm_project(const void *x, const void *gamma, const void *beta, const void *weight,
+                      const void *bias, void *scratch, void *out, void *bias_out, int B, int C,
+                      int O, long long HW, int groups, float eps, int x_channels_last,
+                      int out_channels_last, int dtype, void *stream);
+
 /* ------------------------------------------------------------ calibration */
 
 /* Layout copy between the two memory orders the library serves: a dense

@@ -23,6 +23,8 @@ SIGNATURES = {
     'sapa_fused_forward_nhwc_qbias': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     'sapa_project_nhwc': [_vp, _vp, _vp, _vp, _i, _i, _i, _ll, _i, _vp],
     'sapa_project_nchw': [_vp, _vp, _vp, _vp, _i, _i, _i, _ll, _i, _i, _vp],
+    'sapa_norm_project': [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _ll, _i, ctypes.c_float, _i, _i, _i,
+                          _vp],
     'sapa_channel_moments': [_vp, _vp, _vp, _i, _i, _ll, _i, _i, _vp],
     'sapa_channel_moments_static': [_vp, _vp, _i, _i, _ll, _i, _i, _vp],
     'sapa_groupnorm_fold': [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, ctypes.c_float, _i, _vp],
@@ -97,6 +99,8 @@ def lib():
             fn.argtypes = argtypes
         handle.sapa_channel_moments_workspace.restype = _ll
         handle.sapa_channel_moments_workspace.argtypes = [_i, _i, _ll, _i]
+        handle.sapa_norm_project_scratch.restype = _ll
+        handle.sapa_norm_project_scratch.argtypes = [_i, _i, _i, _ll, _i, _i]
         handle.sapa_fused_backward_workspace.restype = _ll
         handle.sapa_fused_backward_workspace.argtypes = [_i, _i, _i, _i, _i]
         handle.sapa_fused_backward_attn_workspace.restype = _ll
@@ -308,6 +312,45 @@ def groupnorm_fold(mean_var, norm, conv, dtype):
         return None
     check(status, 'sapa_groupnorm_fold')
     return w_out, b_out
+
+
+def norm_project(x, norm, conv, channels_last_out=False, defer_bias=False):
+    """conv(norm(x)) for a GroupNorm and a 1x1 convolution on a CUDA feature x [B, C, H, W]
+    (contiguous or channels_last; f16 / bf16 / fp32) in one library call (moments, fold,
+    projection: four launches): (out, None), or with defer_bias (out without the bias,
+    per-image bias [B, O]); out is channels_last for a channels_last x or with
+    channels_last_out.  None if some step has no kernel for the configuration (nothing was
+    launched then; the caller takes the steps one by one)."""
+    B, C, H, W = x.shape
+    O = conv.out_channels
+    dtype = x.dtype
+    params = [norm.weight, norm.bias, conv.weight, conv.bias]
+    if (dtype not in DTYPES or x.numel() == 0 or conv.weight.numel() != O * C
+            or any(p is not None and (p.dtype != dtype or not p.is_contiguous()) for p in params)):
+        return None
+    if x.is_contiguous():
+        cl = 0
+    elif x.is_contiguous(memory_format=torch.channels_last):
+        cl = 1
+    else:
+        return None
+    out_cl = 1 if (cl or channels_last_out) else 0
+    handle = lib()
+    ptr = lambda t: None if t is None else t.data_ptr()
+    with torch.cuda.device(x.device):
+        nbytes = handle.sapa_norm_project_scratch(B, C, O, H * W, cl, DTYPES[dtype])
+        scratch = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
+        out = torch.empty(B, O, H, W, dtype=dtype, device=x.device,
+                          memory_format=torch.channels_last if out_cl else torch.contiguous_format)
+        b_out = torch.empty(B, O, dtype=dtype, device=x.device) if defer_bias else None
+        status = handle.sapa_norm_project(
+            x.data_ptr(), ptr(norm.weight), ptr(norm.bias), conv.weight.data_ptr(), ptr(conv.bias),
+            scratch.data_ptr(), out.data_ptr(), ptr(b_out), B, C, O, H * W, norm.num_groups, float(norm.eps),
+            cl, out_cl, DTYPES[dtype], torch.cuda.current_stream(x.device).cuda_stream)
+    if status == UNSUPPORTED:
+        return None
+    check(status, 'sapa_norm_project')
+    return out, b_out
 
 
 def project_nchw(x, weight, bias=None, channels_last_out=False):

@@ -768,6 +768,49 @@ int sapa_project_nchw(const void *x, const void *weight, const void *bias, void 
     return finish(e);
 }
 
+namespace {
+long long round256(long long n) { return (n + 255) / 256 * 256; }
+long long esize_of(int dtype) { return dtype == SAPA_F32 ? 4 : dtype == SAPA_F64 ? 8 : 2; }
+}  // namespace
+
+long long sapa_norm_project_scratch(int B, int C, int O, long long HW, int x_channels_last, int dtype) {
+    if (B <= 0 || C <= 0 || O <= 0 || HW <= 0 || !dtype_ok(dtype)) return 0;
+    return round256(channel_moments_workspace(B, C, (long)HW, x_channels_last != 0)) + round256((long long)B * C * 8) +
+           round256((long long)B * O * C * esize_of(dtype)) + round256((long long)B * O * esize_of(dtype));
+}
+
+int sapa_norm_project(const void *x, const void *gamma, const void *beta, const void *weight, const void *bias,
+                      void *scratch, void *out, void *bias_out, int B, int C, int O, long long HW, int groups,
+                      float eps, int x_channels_last, int out_channels_last, int dtype, void *stream) {
+    if (!dtype_ok(dtype) || B < 0 || C <= 0 || O <= 0 || HW <= 0 || groups <= 0) return SAPA_ERR_INVALID_ARGUMENT;
+    if ((long long)B * HW * (C > O ? C : O) >= kMaxElems) return SAPA_ERR_TOO_LARGE;
+    if (B == 0) return SAPA_OK;
+    if (!x || !weight || !scratch || !out) return SAPA_ERR_INVALID_ARGUMENT;
+    // nothing is launched unless every step has a kernel for the configuration
+    if (dtype == SAPA_F64 || C % groups != 0 || C > 8192 ||
+        !project_supported(C, O, (long)HW, x_channels_last != 0, out_channels_last != 0, dtype) ||
+        ((uintptr_t)x | (uintptr_t)out | (uintptr_t)scratch) % 16 != 0)
+        return SAPA_ERR_UNSUPPORTED;
+    char *p = (char *)scratch;
+    void *ws = p;
+    p += round256(channel_moments_workspace(B, C, (long)HW, x_channels_last != 0));
+    float *mean_var = (float *)p;
+    p += round256((long long)B * C * 8);
+    void *w_b = p;
+    p += round256((long long)B * O * C * esize_of(dtype));
+    void *b_b = bias_out ? bias_out : (void *)p;
+    hipStream_t st = (hipStream_t)stream;
+    hipError_t e = channel_moments_launch(x, ws, mean_var, B, C, (long)HW, x_channels_last != 0, dtype, st);
+    if (e == hipSuccess)
+        e = groupnorm_fold_launch(mean_var, gamma, beta, weight, bias, w_b, b_b, B, C, O, groups, eps, dtype, st);
+    if (e == hipSuccess)
+        e = x_channels_last ? project_nhwc_launch(x, w_b, bias_out ? nullptr : b_b, out, B, C, O, (long)HW, dtype, st)
+                            : project_nchw_launch(x, w_b, bias_out ? nullptr : b_b, out, B, C, O, (long)HW,
+                                                  out_channels_last, dtype, st);
+    if (e == hipErrorNotSupported) return SAPA_ERR_UNSUPPORTED;
+    return finish(e);
+}
+
 int sapa_layout_copy(const void *src, void *dst, int B, int C, long long HW, int to_channels_last,
                      int esize, void *stream) {
     if (B < 0 || C < 0 || HW < 0 || (esize != 2 && esize != 4)) return SAPA_ERR_INVALID_ARGUMENT;

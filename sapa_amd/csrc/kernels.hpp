@@ -83,6 +83,8 @@ hipError_t project_nhwc_launch(const void *x, const void *w, const void *bias, v
 // ... of a contiguous feature [B, C, HW] into [B, HW, O] (out_channels_last) or [B, O, HW]; fp32
 hipError_t project_nchw_launch(const void *x, const void *w, const void *bias, void *out, int B,
                                int C, int O, long HW, int out_channels_last, int dtype, hipStream_t st);
+// whether one of the two has a kernel for the configuration (pointer alignment aside)
+bool project_supported(int C, int O, long HW, bool x_channels_last, bool out_channels_last, int dtype);
 
 // sapa_d_nhwc.hip: fused SAPA-D forward for tensors in channels-last memory
 // order (offsets [B, sH, sW, 2GP]); f32 / f16 / bf16, s in {1, 2, 4}, P <= 32,

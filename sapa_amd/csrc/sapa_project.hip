@@ -683,4 +683,19 @@ hipError_t project_nchw_launch(const void *x, const void *w, const void *bias, v
                              : project::launch32<false, false>(x, w, bias, out, B, C, O, HW, st);
 }
 
+// Whether project_nhwc_launch (x_channels_last; the result is channels-last then) / project_nchw_launch
+// has a kernel for the configuration, pointer alignment aside.
+bool project_supported(int C, int O, long HW, bool x_channels_last, bool out_channels_last, int dtype) {
+    const bool small_pair = (C == 64 && (O == 32 || O == 64)) || (C == 128 && (O == 32 || O == 64)) ||
+                            (C == 256 && (O == 32 || O == 64)) || (C == 512 && O == 32);
+    if (dtype == 2 || dtype == 3) {
+        if (x_channels_last)
+            return out_channels_last && (small_pair || (C == 128 && O == 128) || (C == 256 && O == 128) || (C == 512 && O == 64));
+        return small_pair && HW % 8 == 0 && HW * (long)(C > O ? C : O) * 2 < (1L << 31);
+    }
+    if (dtype != 0 || !small_pair || HW * (long)(C > O ? C : O) * 4 >= (1L << 31)) return false;
+    if (x_channels_last) return out_channels_last;
+    return out_channels_last || HW % 4 == 0;
+}
+
 }  // namespace sapa

@@ -53,6 +53,13 @@ def norm_project(x, norm, *convs, channels_last=False, defer_bias=False):
     that adds the bias itself)."""
     B, C, H, W = x.shape
     x_cl = not x.is_contiguous() and x.is_contiguous(memory_format=torch.channels_last)
+    if (norm is not None and len(convs) == 1 and x.is_cuda and not torch.is_grad_enabled()
+            and convs[0].kernel_size == (1, 1) and convs[0].groups == 1 and (channels_last or not x_cl)):
+        # inference on the GPU, one projection of the feature: moments, fold and projection in one
+        # library call (the same four launches as below, a third of the host time)
+        res = _lib.norm_project(x, norm, convs[0], channels_last_out=channels_last, defer_bias=defer_bias)
+        if res is not None:
+            return [res if defer_bias else res[0]]
     if norm is not None:
         G = norm.num_groups
         per_c = C // G

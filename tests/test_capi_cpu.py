@@ -31,6 +31,7 @@ def test_library_exports_every_declared_symbol():
     # (the workspace query returns a size, not a status: bound separately)
     ops = [n for n in names if not n.startswith('sapa_hip_')
            and n not in ('sapa_channel_moments_workspace', 'sapa_channel_moments_static_capacity',
+                         'sapa_norm_project_scratch',
                          'sapa_fused_backward_workspace', 'sapa_fused_backward_attn_workspace',
                          'sapa_deform_fused_forward_workspace',
                          'sapa_deform_fused_backward_workspace', 'sapa_deform_backward_workspace')]
@@ -138,6 +139,20 @@ def test_argument_validation_returns_codes():
     assert h.sapa_project_nchw(p, p, None, p, 1, 256, 64, 100, 0, 3, None) == -2     # 16-bit planes of 100 pixels
     assert h.sapa_project_nchw(p, p, None, p, 1, 256, 64, 102, 0, 0, None) == -2     # planes of 102 pixels
     assert h.sapa_project_nchw(None, None, None, None, 0, 256, 64, 100, 1, 0, None) == 0
+    # moments + fold + projection in one call: scratch = moments workspace + [B,C,2] fp32 + folded
+    # weights + folded bias, each rounded to 256 bytes; extents, null pointers; configurations without
+    # a kernel are refused before anything is launched
+    assert (h.sapa_norm_project_scratch(16, 256, 64, 67200, 1, 3)
+            == (h.sapa_channel_moments_workspace(16, 256, 67200, 1) + 255) // 256 * 256
+            + 16 * 256 * 8 + 16 * 64 * 256 * 2 + 16 * 64 * 2)
+    assert h.sapa_norm_project_scratch(0, 256, 64, 67200, 1, 3) == 0
+    assert h.sapa_norm_project(p, p, p, p, p, p, p, p, 1, 256, 64, 100, 0, 1e-5, 1, 1, 3, None) == -1
+    assert h.sapa_norm_project(p, p, p, p, p, None, p, p, 1, 256, 64, 100, 32, 1e-5, 1, 1, 3, None) == -1
+    assert h.sapa_norm_project(p, p, p, p, p, p, p, p, 1, 256, 64, 100, 32, 1e-5, 1, 1, 1, None) == -2     # fp64
+    assert h.sapa_norm_project(p, p, p, p, p, p, p, p, 1, 256, 48, 100, 32, 1e-5, 1, 1, 3, None) == -2     # no (256, 48)
+    assert h.sapa_norm_project(p, p, p, p, p, p, p, p, 1, 256, 64, 100, 32, 1e-5, 0, 0, 3, None) == -2     # 16-bit planes of 100
+    assert h.sapa_norm_project(p, p, p, p, p, p, p, p, 1, 256, 64, 100, 48, 1e-5, 1, 1, 3, None) == -2     # 256 % 48
+    assert h.sapa_norm_project(None, None, None, None, None, None, None, None, 0, 256, 64, 100, 32, 1e-5, 1, 1, 3, None) == 0
     # layout copy: element size, negative extents, null / misaligned pointers, empty tensors,
     # more rows than the tiled side holds
     assert h.sapa_layout_copy(p, p, 1, 8, 64, 1, 3, None) == -1

@@ -553,6 +553,40 @@ def test_projection_kernel_fp32_contiguous_feature(shape):
     assert _lib.project_nchw(x.contiguous(memory_format=CL), w) is None
 
 
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('shape', [(2, 256, 64, 9, 16), (1, 128, 32, 40, 34), (3, 64, 64, 5, 8), (2, 64, 48, 6, 8)])
+def test_norm_project_in_one_call(dtype, shape):
+    """Moments, fold and projection through the single entry point: the same bits as the
+    three entry points one after the other (it launches the same kernels), for both
+    memory orders of the feature, with the bias added and with it handed back; None --
+    and nothing launched -- for a channel pair without a projection kernel."""
+    from sapa_amd import _lib
+    B, C, O, H, W = shape
+    torch.manual_seed(11)
+    norm = torch.nn.GroupNorm(32, C).to(DEV).to(dtype)
+    conv = torch.nn.Conv2d(C, O, 1).to(DEV).to(dtype)
+    torch.nn.init.normal_(norm.weight, 1.0, 0.2)
+    torch.nn.init.normal_(norm.bias, 0.0, 0.2)
+    x = (randn(gen(364), B, C, H, W) * 1.5 + 0.3).to(dtype).to(DEV)
+    for feat, cl_out in ((x, False), (x, True), (x.contiguous(memory_format=CL), True)):
+        got = _lib.norm_project(feat, norm, conv, channels_last_out=cl_out)
+        got_d = _lib.norm_project(feat, norm, conv, channels_last_out=cl_out, defer_bias=True)
+        if O == 48:
+            assert got is None and got_d is None
+            continue
+        w_b, b_b = _lib.groupnorm_fold(_lib.channel_moments(feat), norm, conv, dtype)
+        if feat.is_contiguous():
+            want, want_d = (_lib.project_nchw(feat, w_b, b, channels_last_out=cl_out) for b in (b_b, None))
+        else:
+            want, want_d = (_lib.project_nhwc(feat, w_b, b) for b in (b_b, None))
+        assert got[1] is None and torch.equal(got[0], want) and got[0].stride() == want.stride()
+        assert torch.equal(got_d[0], want_d) and torch.equal(got_d[1], b_b)
+        # and the composition it stands for
+        ref = conv(norm(x)).float()
+        tol = 2e-4 if dtype == torch.float32 else 6e-2 if dtype == torch.bfloat16 else 1e-2
+        torch.testing.assert_close(got[0].float(), ref, rtol=tol, atol=tol)
+
+
 @pytest.mark.parametrize('dtype,tol', [(torch.bfloat16, 2e-2), (torch.float16, 3e-3)])
 @pytest.mark.parametrize('shape', [(2, 256, 64, 9, 16), (1, 128, 32, 40, 34), (3, 64, 64, 5, 8), (1, 512, 32, 4, 4),
                                    (2, 256, 32, 1, 8), (1, 256, 64, 130, 132), (2, 64, 32, 17, 3)])
