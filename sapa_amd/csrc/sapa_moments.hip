@@ -176,10 +176,19 @@ finish_kernel(const T *__restrict__ x, const float *__restrict__ part, float *__
     if (i >= (long)B * C) return;
     const int b = (int)(i / C), c = (int)(i % C);
     float s1 = 0.f, s2 = 0.f;
-    for (int k = 0; k < chunks; ++k) {
-        const float *p = CL ? part + (((long)b * chunks + k) * C + c) * 2 : part + (i * chunks + k) * 2;
-        s1 += p[0];
-        s2 += p[1];
+    auto at = [&](int k) { return CL ? part + (((long)b * chunks + k) * C + c) * 2 : part + (i * chunks + k) * 2; };
+    // (eight chunks' loads in flight at a time; the additions in the chunks' order)
+    int k = 0;
+    for (; k + 8 <= chunks; k += 8) {
+        float a[8], q[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) a[u] = at(k + u)[0], q[u] = at(k + u)[1];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) s1 += a[u], s2 += q[u];
+    }
+    for (; k < chunks; ++k) {
+        s1 += at(k)[0];
+        s2 += at(k)[1];
     }
     const float shift = (float)(CL ? x[(long)b * HW * C + c] : x[i * HW]);
     const float m = s1 / (float)HW;
